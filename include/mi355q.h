@@ -1,0 +1,94 @@
+/*
+ * mi355q -- C ABI of the MI355X (gfx950) quantized-linear kernels.
+ *
+ * Every entry point takes raw device pointers, explicit sizes and a HIP
+ * stream (passed as void*, it is a hipStream_t; NULL = the null stream),
+ * enqueues its work asynchronously on that stream and returns 0 on success
+ * or a non-zero code; mi355q_last_error() then describes the failure
+ * (thread-local).  Nothing here synchronises with the host and nothing
+ * allocates device memory: every output and workspace belongs to the caller.
+ *
+ * Each declaration names the operator of the reference (EnflameTechnology/
+ * vllm-gcu) whose vendor-library call it replaces.
+ */
+#ifndef MI355Q_H
+#define MI355Q_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of activations / outputs */
+enum { MI355Q_F16 = 0, MI355Q_BF16 = 1, MI355Q_F32 = 2 };
+
+/* how zero-points are handed to the W4A16 kernels */
+enum {
+  MI355Q_ZP_NONE = 0,      /* symmetric int4: z = 8 everywhere                      */
+  MI355Q_ZP_PACKED = 1,    /* int32 [K/g, N/8], nibble j of column c = z[g, 8c+j]   */
+  MI355Q_ZP_PRESCALED = 2  /* activation-dtype [K/g, N] holding z*scale (the form   */
+                           /* the reference's GPTQ loader produces,                 */
+                           /* vllm_gcu/kernels/quantization/rearrange.py:33-34)     */
+};
+
+/* source formats understood by the int4 repack kernels */
+enum {
+  MI355Q_W4_SRC_GPTQ = 0,      /* int32 [K/8, N], nibble i of row r = k 8r+i (rearrange.py:13-21)     */
+  MI355Q_W4_SRC_AWQ = 1,       /* int32 [K, N/8], AWQ interleave (rearrange.py:66-95)                 */
+  MI355Q_W4_SRC_REF_KN = 2,    /* uint8 [K/2, N] reference half-group layout (rearrange.py:36-56)     */
+  MI355Q_W4_SRC_REF_NK = 3     /* uint8 [N, K/2] the same, stored transposed for MoE experts          */
+                               /* (vllm_gcu/kernels/quantization/moe_wna16.py:464-466)                */
+};
+
+const char* mi355q_last_error(void);
+int mi355q_abi_version(void);
+
+/* ---- int4 weight formats (load time) ------------------------------------
+ * Replaces the CPU repack of rearrange_uint4_int32_uint8_gptq / _awq
+ * (vllm_gcu/kernels/quantization/rearrange.py:6-133) by device kernels that
+ * produce this library's slab layout: int32 [K/8, N] flat stream
+ * [N/128][K/128][8 tiles][64 lanes][4 words]; word s of lane l (c = l%16,
+ * kq = l/16) of tile t holds, in nibble {0,4,1,5,2,6,3,7}[j], the weight at
+ * k = 128g + 32s + 8kq + j, n = 128S + 8c + t.  K and N must be multiples of
+ * 128.  `batch` matrices are converted back to back (MoE experts). */
+int mi355q_w4_repack(const void* src, int src_format, int32_t* dst,
+                     int batch, int K, int N, void* stream);
+/* zero-points -> MI355Q_ZP_PACKED.  src_format GPTQ: int32 [G, N/8] with the
+ * "+1" convention (rearrange.py:24-29); AWQ: int32 [G, N/8] interleaved
+ * (rearrange.py:96-101). */
+int mi355q_w4_repack_zeros(const int32_t* src, int src_format, int32_t* dst,
+                           int batch, int G, int N, void* stream);
+/* debug / parity: slab layout -> uint8 [K, N] (one value per byte) */
+int mi355q_w4_unpack(const int32_t* packed, uint8_t* dst, int batch, int K, int N,
+                     void* stream);
+
+/* ---- W4A16 GEMM ----------------------------------------------------------
+ * Replaces topsatenGemmQuant as called by gptq_gemm_gcu / awq_gemm_gcu
+ * (csrc/src/gptq_gemm_gcu.cpp:27-48, csrc/src/awq_gemm_gcu.cpp:27-47):
+ *   out[M, N] = x[M, K] @ ((q - z) * s)[K, N] (+ bias[N]),  fp32 accumulate.
+ * x, out, scales, bias share `dtype` (F16 or BF16); qweight is the slab
+ * layout; scales [K/g, N]; group_size a multiple of 32 dividing K (or -1 for
+ * one group).  M <= 64 runs the split-K streaming kernel, larger M the
+ * LDS-staged MFMA kernel.  `workspace` must hold
+ * mi355q_w4a16_workspace_bytes() bytes, be zero-filled once before first use,
+ * and must not be shared by launches that may overlap in time. */
+size_t mi355q_w4a16_workspace_bytes(int M, int K, int N);
+int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight,
+                      const void* scales, const void* zeros, int zeros_kind,
+                      const void* bias, int M, int K, int N, int group_size,
+                      int dtype, void* workspace, size_t workspace_bytes,
+                      void* stream);
+/* tuning hook used by the benchmark: force the split-K factor (0 = auto) and
+ * the kernel family (0 = auto, 1 = streaming, 2 = LDS/MFMA) */
+int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
+                         const void* scales, const void* zeros, int zeros_kind,
+                         const void* bias, int M, int K, int N, int group_size,
+                         int dtype, void* workspace, size_t workspace_bytes,
+                         int split_k, int family, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355Q_H */

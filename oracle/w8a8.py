@@ -1,0 +1,99 @@
+"""W8A8 int8 path on the CPU (numpy / CPU torch).  Test infrastructure only.
+
+* per-token dynamic int8 quantisation
+  (csrc/src/dynamic_scaled_int8_quant.cpp:12-19; the arithmetic is upstream
+  vLLM's: ``scale = absmax / 127``, ``q = sat_s8(rne(x * (127 / absmax)))``),
+* static int8 quantisation (csrc/src/static_scaled_int8_quant.cpp:12-28:
+  the reciprocal of the scale is taken and rounded to the *input* dtype, then
+  ``q = sat_s8(rne(x * inv))``),
+* exact int32 GEMM and the scaled epilogue of ``cutlass_scaled_mm`` /
+  ``dot_bias_quant`` (csrc/src/cutlass_scaled_mm.cpp:12-36,
+  csrc/src/dot_bias_quant.cpp:12-24).
+"""
+import numpy as np
+import torch
+
+
+def dynamic_scaled_int8_quant(x: np.ndarray):
+    """x float [M, K] -> (q int8 [M, K], scales float32 [M, 1]).
+
+    All arithmetic in float32.  A row of zeros has scale 0 and quantises to 0
+    (upstream: 0 * inf = nan converts to 0).
+    """
+    xf = x.astype(np.float32)
+    absmax = np.max(np.abs(xf), axis=-1, keepdims=True).astype(np.float32)
+    scales = (absmax / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        inv = (np.float32(127.0) / absmax).astype(np.float32)
+        y = (xf * inv).astype(np.float32)
+    y = np.where(np.isnan(y), np.float32(0), y)
+    q = np.clip(np.rint(y), -128, 127).astype(np.int8)
+    return q, scales
+
+
+def static_scaled_int8_quant(x: np.ndarray, scale: np.ndarray):
+    """x float16/float32 [M, K]; scale float32 scalar or [K] -> int8 [M, K].
+
+    The reciprocal is rounded to x's dtype (static_scaled_int8_quant.cpp:21,
+    24); the product is evaluated in float32 and rounded half-to-even.
+    """
+    inv = (np.float32(1.0) / np.asarray(scale, dtype=np.float32)).astype(x.dtype)
+    y = x.astype(np.float32) * inv.astype(np.float32)
+    return np.clip(np.rint(y), -128, 127).astype(np.int8)
+
+
+def int8_gemm_i32(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """Exact ``a[M, K] @ b[K, N]`` in int32 for int8 operands.
+
+    Evaluated as float32 matmuls over K-chunks of 1024: every partial sum is
+    an integer below 1024 * 128 * 128 = 2**24, hence exact in float32; the
+    chunks are then added in int64.
+    """
+    M, K = a.shape
+    K2, N = b.shape
+    assert K == K2
+    acc = np.zeros((M, N), dtype=np.int64)
+    bt = torch.from_numpy(np.ascontiguousarray(b))
+    at = torch.from_numpy(np.ascontiguousarray(a))
+    for k0 in range(0, K, 1024):
+        pa = at[:, k0:k0 + 1024].float()
+        pb = bt[k0:k0 + 1024].float()
+        acc += torch.matmul(pa, pb).numpy().astype(np.int64)
+    assert np.abs(acc).max(initial=0) < 2 ** 31
+    return acc.astype(np.int32)
+
+
+def scaled_mm_epilogue(acc: np.ndarray, x_scale, w_scale, bias=None) -> np.ndarray:
+    """float32 ``acc * x_scale[M or 1] * w_scale[N or 1] (+ bias)``.
+
+    x_scale: scalar, [1], [M] or [M, 1]; w_scale: scalar, [1], [N] or [N, 1]
+    (cutlass_scaled_mm.cpp:23-32 unsqueezes a 0-d x_scale and squeezes an
+    [N, 1] w_scale).  The product is formed as ``(float(acc) * x_scale) *
+    w_scale`` in float32; the caller casts to the output dtype.
+    """
+    xs = np.asarray(x_scale, dtype=np.float32).reshape(-1, 1)
+    ws = np.asarray(w_scale, dtype=np.float32).reshape(1, -1)
+    out = (acc.astype(np.float32) * xs).astype(np.float32) * ws
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=np.float32).reshape(1, -1)
+    return out.astype(np.float32)
+
+
+def weight_only_int8(x: np.ndarray, w_nk: np.ndarray, scale: np.ndarray,
+                     group_size: int, bias=None) -> np.ndarray:
+    """W8A16: ``x @ (w[N, K] * scale).T`` in float32
+    (csrc/src/weight_only_quant.cpp:28-101); scale [N] (per channel,
+    group_size -1) or [K/g, N]."""
+    N, K = w_nk.shape
+    wf = w_nk.astype(np.float32)
+    if group_size in (-1, 0) or scale.ndim == 1:
+        wd = wf * scale.astype(np.float32).reshape(N, 1)
+    else:
+        g = group_size
+        wd = (wf.reshape(N, K // g, g) *
+              scale.astype(np.float32).T.reshape(N, K // g, 1)).reshape(N, K)
+    out = torch.matmul(torch.from_numpy(x.astype(np.float32)),
+                       torch.from_numpy(np.ascontiguousarray(wd.T))).numpy()
+    if bias is not None:
+        out = out + bias.astype(np.float32)[None, :]
+    return out

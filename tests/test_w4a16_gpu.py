@@ -1,0 +1,187 @@
+"""GPU parity of the int4 format kernels and the W4A16 GEMM against the CPU
+oracle.  Integer unpack is bit-exact; fp16/bf16 GEMM outputs are within
+rtol 1e-2 / atol 1e-2 of ``x.float() @ ((q - z) * s)`` (fp32 accumulation),
+and bit-exact in the special cases where every partial sum is representable."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import w4 as ow4
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from vllm_gcu_amd.kernels import _custom_ops
+    return _custom_ops
+
+
+@pytest.fixture(scope="module")
+def rearrange():
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    return rearrange
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def make_case(seed, M, K, N, g, dtype=np.float16, exact=False):
+    rng = np.random.default_rng(seed)
+    G = K // (K if g == -1 else g)
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(G, N), dtype=np.uint8)
+    if exact:
+        s = (2.0 ** -rng.integers(4, 8, size=(G, N))).astype(np.float32)
+        x = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    else:
+        s = rng.uniform(0.001, 0.01, size=(G, N)).astype(np.float32)
+        x = rng.standard_normal((M, K)).astype(np.float32)
+    return q, z, s, x
+
+
+def to_act(a, dtype):
+    return torch.from_numpy(a).to(dtype)
+
+
+# ------------------------------------------------------------ formats ----
+@pytest.mark.parametrize("K,N", [(128, 128), (512, 384), (4096, 4096)])
+def test_repack_all_sources_bit_exact(rearrange, K, N):
+    print(f"case repack K={K} N={N}", flush=True)
+    rng = np.random.default_rng(K + N)
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    want = ow4.native_pack(q)
+    w_gptq, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
+    w_awq, _ = rearrange.rearrange_uint4_int32_awq(dev(ow4.awq_pack(q)), None)
+    w_kn = rearrange.from_reference_layout(dev(ow4.ref_halfgroup_pack(q)))
+    nk = np.ascontiguousarray(ow4.ref_halfgroup_pack(q).T)
+    w_nk = rearrange.from_reference_layout(dev(nk), transposed=True)
+    for name, got in [("gptq", w_gptq), ("awq", w_awq), ("ref_kn", w_kn), ("ref_nk", w_nk)]:
+        assert got.shape == (K // 8, N) and got.dtype == torch.int32
+        assert np.array_equal(got.cpu().numpy(), want), name
+    assert np.array_equal(rearrange.unpack_slab(w_gptq).cpu().numpy(), q)
+
+
+def test_repack_batched_experts_and_zeros(rearrange):
+    rng = np.random.default_rng(11)
+    E, K, N, G = 3, 256, 128, 2
+    q = rng.integers(0, 16, size=(E, K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(E, G, N), dtype=np.uint8)
+    z[0, 0, :16] = np.arange(16)
+    qw = np.stack([ow4.gptq_pack_weight(q[e]) for e in range(E)])
+    qz = np.stack([ow4.gptq_pack_zeros(z[e]) for e in range(E)])
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(qw), dev(qz))
+    assert np.array_equal(rearrange.unpack_slab(w).cpu().numpy(), q)
+    want_z = np.stack([ow4.native_pack_zeros(z[e]) for e in range(E)])
+    assert np.array_equal(zp.cpu().numpy(), want_z)
+    az = np.stack([ow4.awq_pack(z[e]) for e in range(E)])
+    _, zp2 = rearrange.rearrange_uint4_int32_awq(dev(np.stack([ow4.awq_pack(q[e]) for e in range(E)])), dev(az))
+    assert np.array_equal(zp2.cpu().numpy(), want_z)
+    assert np.array_equal(rearrange.pack_int8_zeros(dev(z.astype(np.int8))).cpu().numpy(), want_z)
+
+
+# --------------------------------------------------------------- GEMM ----
+def run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=None, split_k=0, family=0):
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    out = ops.w4a16_gemm(to_act(x, dtype).cuda(), w, to_act(s, dtype).cuda(), zp,
+                         None if bias is None else to_act(bias, dtype).cuda(), g, split_k=split_k, family=family)
+    torch.cuda.synchronize()
+    return out
+
+
+def oracle(q, z, s, x, g, dtype, bias=None):
+    xs = to_act(x, dtype).float().numpy()
+    ss = to_act(s, dtype).float().numpy()
+    b = None if bias is None else to_act(bias, dtype).float().numpy()
+    return ow4.w4a16_gemm(xs, q, z, ss, g, bias=b)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_stream_gemm_parity(ops, rearrange, M, dtype):
+    K, N, g = 1024, 384, 128
+    print(f"case stream M={M} K={K} N={N} {dtype}", flush=True)
+    q, z, s, x = make_case(M, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, dtype).float().cpu().numpy()
+    want = oracle(q, z, s, x, g, dtype)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("split_k", [1, 2, 3, 8])
+def test_stream_gemm_exact_and_split_invariant(ops, rearrange, split_k):
+    # power-of-two scales + small integer activations: every product and every
+    # partial sum is exact in fp32, so any split / summation order must give
+    # the same bits as the oracle
+    M, K, N, g = 16, 2048, 256, 128
+    print(f"case exact split_k={split_k}", flush=True)
+    q, z, s, x = make_case(7, M, K, N, g, exact=True)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, split_k=split_k)
+    want = torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("g", [32, 64, 128, 256, -1])
+def test_stream_gemm_group_sizes_and_bias(ops, rearrange, g):
+    M, K, N = 5, 512, 128
+    print(f"case group g={g}", flush=True)
+    q, z, s, x = make_case(100 + g, M, K, N, g)
+    bias = np.random.default_rng(5).standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias).float().cpu().numpy()
+    want = oracle(q, z, s, x, g, torch.float16, bias=bias)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+def test_config0_full_size_and_determinism(ops, rearrange):
+    # BASELINE config 0: x f16 [16, 4096], int4 [4096, 4096], g = 128
+    M, K, N, g = 16, 4096, 4096, 128
+    print("case config0", flush=True)
+    q, z, s, x = make_case(0, M, K, N, g)
+    a = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16)
+    b = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16)
+    assert torch.equal(a, b), "split-K result depends on scheduling"
+    want = oracle(q, z, s, x, g, torch.float16)
+    np.testing.assert_allclose(a.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_symmetric_default_zero_point(ops, rearrange):
+    M, K, N, g = 4, 256, 128, 128
+    q, z, s, x = make_case(21, M, K, N, g)
+    w, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
+    out = ops.gptq_gemm_gcu(to_act(x, torch.float16).cuda(), w, torch.empty(0, dtype=torch.int32, device="cuda"),
+                            to_act(s, torch.float16).cuda(), torch.empty(0, dtype=torch.int32, device="cuda"),
+                            4, None, g)
+    want = oracle(q, None, s, x, g, torch.float16)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("M", [2, 48])
+def test_reference_layout_drop_in(ops, M):
+    # exactly what the reference's GPTQ loader leaves on the layer
+    # (gptq.py:229-261): uint8 half-group weights, fp16 zeros = z * scales
+    K, N, g = 512, 256, 128
+    print(f"case reference-layout M={M}", flush=True)
+    q, z, s, x = make_case(31 + M, M, K, N, g)
+    s16 = s.astype(np.float16)
+    rweight, zeros_f = ow4.rearrange_gptq(ow4.gptq_pack_weight(q), ow4.gptq_pack_zeros(z), s16)
+    out = ops.gptq_gemm_gcu(to_act(x, torch.float16).cuda().reshape(1, M, K), dev(rweight), dev(zeros_f),
+                            dev(s16), torch.arange(K, dtype=torch.int32, device="cuda") // g, 4, None, g)
+    assert out.shape == (1, M, N)
+    xs = to_act(x, torch.float16).float().numpy()
+    want = xs @ ow4.dequantize_prescaled_zeros(q, zeros_f, s16, g)
+    np.testing.assert_allclose(out.float().cpu().numpy()[0], want, rtol=RTOL, atol=ATOL)
+    # AWQ form: int8 zero-points kept as integers (awq.py:80-106)
+    rw8, z8 = ow4.rearrange_awq(ow4.awq_pack(q), ow4.awq_pack(z), s16, zeros_in_int8=True)
+    out2 = ops.awq_gemm_gcu(to_act(x, torch.float16).cuda(), dev(rw8), dev(s16), dev(z8), 8, None, g)
+    want2 = oracle(q, z, s, x, g, torch.float16)
+    np.testing.assert_allclose(out2.float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
+
+
+def test_empty_input_returns_empty(ops, rearrange):
+    q, z, s, x = make_case(1, 1, 128, 128, 128)
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    out = ops.w4a16_gemm(torch.empty(0, 128, dtype=torch.float16, device="cuda"), w,
+                         to_act(s, torch.float16).cuda(), zp, None, 128)
+    assert out.shape == (0, 128)

@@ -1,0 +1,60 @@
+"""ctypes binding of ``libmi355q.so`` (the C ABI declared in include/mi355q.h).
+
+There is deliberately no fallback: if the shared library is missing or a call
+fails, an exception is raised.
+"""
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, c_float
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355q.so")
+
+F16, BF16, F32 = 0, 1, 2
+ZP_NONE, ZP_PACKED, ZP_PRESCALED = 0, 1, 2
+W4_SRC_GPTQ, W4_SRC_AWQ, W4_SRC_REF_KN, W4_SRC_REF_NK = 0, 1, 2, 3
+
+# name -> (restype, argtypes); must list every symbol include/mi355q.h declares
+SIGNATURES = {
+    "mi355q_last_error": (c_char_p, []),
+    "mi355q_abi_version": (c_int, []),
+    "mi355q_w4_repack": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "mi355q_w4_repack_zeros": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "mi355q_w4_unpack": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "mi355q_w4a16_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "mi355q_w4a16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                  c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "mi355q_w4a16_gemm_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                     c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_int,
+                                     c_int, c_void_p]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the library once; raise ImportError with build instructions if absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build it first with "
+            "`python -c 'import __graft_entry__ as g; g.build()'` (needs hipcc)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what=""):
+    if rc != 0:
+        msg = load().mi355q_last_error().decode(errors="replace")
+        raise RuntimeError(f"mi355q {what} failed (code {rc}): {msg}")
+
+
+def call(name, *args):
+    check(getattr(load(), name)(*args), name)

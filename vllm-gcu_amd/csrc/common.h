@@ -1,0 +1,86 @@
+// Shared helpers for the gfx950 kernels: error reporting, vector types,
+// small device utilities.  Everything here is internal to the library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/mi355q.h"
+
+namespace mi355q {
+
+// ---- host-side error plumbing ---------------------------------------------
+void set_error(const char* fmt, ...);
+
+#define MQ_REQUIRE(cond, ...)                 \
+  do {                                        \
+    if (!(cond)) {                            \
+      ::mi355q::set_error(__VA_ARGS__);       \
+      return 1;                               \
+    }                                         \
+  } while (0)
+
+#define MQ_LAUNCH_CHECK(what)                                              \
+  do {                                                                     \
+    hipError_t e__ = hipGetLastError();                                    \
+    if (e__ != hipSuccess) {                                               \
+      ::mi355q::set_error("%s: launch failed: %s", what,                   \
+                          hipGetErrorString(e__));                         \
+      return 2;                                                            \
+    }                                                                      \
+  } while (0)
+
+// ---- vector types ----------------------------------------------------------
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef short s8v __attribute__((ext_vector_type(8)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef int i4 __attribute__((ext_vector_type(4)));
+typedef int i16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+template <typename T, typename U>
+__device__ __forceinline__ T bitcast(const U& u) {
+  static_assert(sizeof(T) == sizeof(U), "bitcast size");
+  return __builtin_bit_cast(T, u);
+}
+
+// bf16 <-> f32 by bit manipulation (round to nearest even on the way down)
+__device__ __forceinline__ float bf16_to_f32(uint16_t v) {
+  return bitcast<float>((uint32_t)v << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = bitcast<uint32_t>(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <int DT> struct Elem;            // activation element traits
+template <> struct Elem<MI355Q_F16> {
+  typedef _Float16 type;
+  static __device__ __forceinline__ float to_f32(uint16_t raw) {
+    return (float)bitcast<_Float16>(raw);
+  }
+  static __device__ __forceinline__ uint16_t from_f32(float f) {
+    return bitcast<uint16_t>((_Float16)f);
+  }
+};
+template <> struct Elem<MI355Q_BF16> {
+  typedef __bf16 type;
+  static __device__ __forceinline__ float to_f32(uint16_t raw) { return bf16_to_f32(raw); }
+  static __device__ __forceinline__ uint16_t from_f32(float f) { return f32_to_bf16(f); }
+};
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+int device_cu_count();
+
+}  // namespace mi355q

@@ -1,0 +1,59 @@
+// W4A16 GEMM entry points: argument checks and the choice between the
+// streaming (small M) and the LDS-staged MFMA (large M) kernels.
+#include "common.h"
+
+namespace mi355q {
+int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                        const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
+                        int group_size, int dtype, void* workspace, size_t workspace_bytes,
+                        int split_k, hipStream_t st);
+size_t w4a16_stream_workspace_bytes(int M, int N);
+int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                      const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
+                      int group_size, int dtype, hipStream_t st);
+}  // namespace mi355q
+
+using namespace mi355q;
+
+extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
+  (void)K;
+  if (M <= 0 || N <= 0) return 0;
+  return w4a16_stream_workspace_bytes(M > 64 ? 64 : M, N);
+}
+
+extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
+                                    const void* scales, const void* zeros, int zeros_kind,
+                                    const void* bias, int M, int K, int N, int group_size,
+                                    int dtype, void* workspace, size_t workspace_bytes,
+                                    int split_k, int family, void* stream) {
+  MQ_REQUIRE(M >= 0 && K > 0 && N > 0, "w4a16_gemm: bad shape M=%d K=%d N=%d", M, K, N);
+  if (M == 0) return 0;
+  MQ_REQUIRE(out && x && qweight && scales, "w4a16_gemm: null pointer");
+  MQ_REQUIRE(K % 128 == 0 && N % 128 == 0,
+             "w4a16_gemm: K=%d and N=%d must be multiples of 128 (slab layout)", K, N);
+  MQ_REQUIRE(dtype == MI355Q_F16 || dtype == MI355Q_BF16, "w4a16_gemm: dtype %d not supported", dtype);
+  if (group_size <= 0) group_size = K;
+  MQ_REQUIRE(group_size % 32 == 0 && K % group_size == 0,
+             "w4a16_gemm: group_size=%d must be a multiple of 32 dividing K=%d", group_size, K);
+  MQ_REQUIRE(group_size % 128 == 0 || 128 % group_size == 0,
+             "w4a16_gemm: group_size=%d must divide or be a multiple of 128", group_size);
+  MQ_REQUIRE(zeros_kind >= MI355Q_ZP_NONE && zeros_kind <= MI355Q_ZP_PRESCALED,
+             "w4a16_gemm: unknown zeros_kind %d", zeros_kind);
+  MQ_REQUIRE(zeros_kind == MI355Q_ZP_NONE || zeros, "w4a16_gemm: zeros pointer missing");
+  MQ_REQUIRE(family >= 0 && family <= 2, "w4a16_gemm: unknown kernel family %d", family);
+  if (family == 0) family = (M <= 64) ? 1 : 2;
+  MQ_REQUIRE(family != 1 || M <= 64, "w4a16_gemm: streaming kernel handles M <= 64, got %d", M);
+  if (family == 1)
+    return w4a16_stream_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size,
+                               dtype, workspace, workspace_bytes, split_k, as_stream(stream));
+  return w4a16_tile_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
+                           as_stream(stream));
+}
+
+extern "C" int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight, const void* scales,
+                                 const void* zeros, int zeros_kind, const void* bias, int M, int K,
+                                 int N, int group_size, int dtype, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  return mi355q_w4a16_gemm_ex(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size,
+                              dtype, workspace, workspace_bytes, 0, 0, stream);
+}

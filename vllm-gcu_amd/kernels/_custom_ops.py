@@ -1,0 +1,182 @@
+"""Operator surface of the quantized-linear path.
+
+Registers, with ``torch.library``, implementations for the same operator names
+and schemas that the reference registers in csrc/torch_bindings.cpp (library
+fragments ``_C`` and ``_moe_C``) and exposes the same Python wrappers as
+vllm_gcu/kernels/_custom_ops.py.  A schema is defined only when no other
+extension has defined the name already (the reference's ``findSchema`` guard,
+torch_bindings.cpp:114-117); the implementation is registered for the GPU
+dispatch key ("CUDA" is the HIP device on PyTorch-ROCm).  Every implementation
+converts tensors to raw pointers and calls the C ABI of ``libmi355q.so``.
+"""
+from typing import List, Optional, Tuple
+
+import torch
+
+from .. import _lib
+from . import _runtime as rt
+from .quantization import rearrange
+
+_lib.load()          # fail at import time when the HIP library is missing
+
+_libs = {
+    "_C": torch.library.Library("_C", "FRAGMENT"),
+    "_moe_C": torch.library.Library("_moe_C", "FRAGMENT"),
+}
+# operator name -> schema text, as registered by this module
+SCHEMAS = {}
+
+
+def _schema_exists(qualname: str) -> bool:
+    try:
+        torch._C._dispatch_find_schema_or_throw(qualname, "")
+        return True
+    except RuntimeError:
+        return False
+
+
+def _register(ns: str, name: str, schema: str, fn, tags=()):
+    SCHEMAS[f"{ns}::{name}"] = name + schema
+    if not _schema_exists(f"{ns}::{name}"):
+        _libs[ns].define(name + schema, tags=tags)
+    _libs[ns].impl(name, fn, "CUDA")
+
+
+# ---------------------------------------------------------------------------
+# W4A16 (csrc/torch_bindings.cpp:770-788)
+# ---------------------------------------------------------------------------
+_ref_layout_cache = {}
+
+
+def _slab_weight(qweight: torch.Tensor) -> torch.Tensor:
+    """Return the slab-layout tensor for ``qweight``.
+
+    int32 tensors are this build's layout already.  uint8/int8 ``[K/2, N]``
+    tensors are the reference's half-group layout (rearrange.py:44-56); they
+    are converted on the device once and remembered per storage, so a caller
+    that keeps the reference's loader still works (at the cost of holding both
+    copies).
+    """
+    if qweight.dtype == torch.int32:
+        return qweight
+    if qweight.dtype not in (torch.uint8, torch.int8):
+        raise TypeError(f"int4 weights must be int32 (slab) or uint8/int8 (reference), got {qweight.dtype}")
+    key = (qweight.data_ptr(), tuple(qweight.shape), qweight.device.index, qweight._version)
+    hit = _ref_layout_cache.get(key)
+    if hit is None:
+        hit = rearrange.from_reference_layout(qweight)
+        _ref_layout_cache[key] = hit
+    return hit
+
+
+def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype):
+    """-> (tensor or None, zeros_kind)"""
+    if zeros is None or zeros.numel() == 0:
+        return None, _lib.ZP_NONE
+    if zeros.dtype == torch.int32:
+        return zeros, _lib.ZP_PACKED
+    if zeros.dtype in (torch.int8, torch.uint8):
+        key = (zeros.data_ptr(), tuple(zeros.shape), zeros.device.index, zeros._version)
+        hit = _ref_layout_cache.get(key)
+        if hit is None:
+            hit = rearrange.pack_int8_zeros(zeros)
+            _ref_layout_cache[key] = hit
+        return hit, _lib.ZP_PACKED
+    if zeros.dtype == act_dtype:
+        return zeros, _lib.ZP_PRESCALED
+    raise TypeError(f"zero-points of dtype {zeros.dtype} do not match activations of dtype {act_dtype}")
+
+
+def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
+               zeros: Optional[torch.Tensor], bias: Optional[torch.Tensor], group_size: int,
+               split_k: int = 0, family: int = 0) -> torch.Tensor:
+    """out[M, N] = x[M, K] @ dequant(qweight) (+ bias); allocates the output
+    like gptq_gemm_gcu (csrc/src/gptq_gemm_gcu.cpp:35)."""
+    rt.require_gpu(x, qweight, scales, zeros, bias)
+    if x.dim() != 2:
+        raise RuntimeError(f"w4a16_gemm expects a 2-D activation, got {tuple(x.shape)}")
+    qw = _slab_weight(qweight)
+    M, K = x.shape
+    N = qw.shape[-1]
+    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if x.numel() == 0:
+        return out
+    if qw.shape[-2] * 8 != K:
+        raise RuntimeError(f"w4a16_gemm: activation K={K} does not match weight K={qw.shape[-2] * 8}")
+    x = x.contiguous()
+    scales = scales.contiguous()
+    if scales.dtype != x.dtype:
+        scales = scales.to(x.dtype)
+    z, zk = _zero_points(zeros, x.dtype)
+    if z is not None:
+        z = z.contiguous()
+    if bias is not None:
+        bias = bias.to(x.dtype).contiguous()
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        ws_bytes = lib.mi355q_w4a16_workspace_bytes(M, K, N)
+        ws = rt.workspace(x.device, ws_bytes)
+        _lib.check(lib.mi355q_w4a16_gemm_ex(
+            out.data_ptr(), x.data_ptr(), qw.data_ptr(), scales.data_ptr(), rt.ptr(z), zk, rt.ptr(bias),
+            M, K, N, int(group_size), rt.dtype_code(x.dtype), ws.data_ptr(), ws.numel(),
+            int(split_k), int(family), rt.stream_ptr()), "w4a16_gemm")
+    return out
+
+
+def _gptq_gemm_gcu_impl(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bit, bias, group_size):
+    if bit != 4:
+        raise RuntimeError("gptq_gemm_gcu: only bit == 4 takes this operator "
+                           "(8-bit goes through weight_only_quant)")
+    return w4a16_gemm(a, b_q_weight, b_gptq_scales, b_gptq_qzeros, bias, group_size)
+
+
+def _awq_gemm_gcu_impl(_in_feats, _kernel, _scaling_factors, _zeros, split_k_iters, bias, group_size):
+    return w4a16_gemm(_in_feats, _kernel, _scaling_factors, _zeros, bias, group_size)
+
+
+_register("_C", "gptq_gemm_gcu",
+          "(Tensor a, Tensor b_q_weight, Tensor b_gptq_qzeros, Tensor b_gptq_scales, Tensor b_g_idx, "
+          "int bit, Tensor? bias, int group_size) -> Tensor", _gptq_gemm_gcu_impl)
+_register("_C", "awq_gemm_gcu",
+          "(Tensor _in_feats, Tensor _kernel, Tensor _scaling_factors, Tensor _zeros, "
+          "SymInt split_k_iters, Tensor? bias, int group_size) -> Tensor", _awq_gemm_gcu_impl)
+
+
+# awq (vllm_gcu/kernels/_custom_ops.py:213-238; the reference's parameter names
+# for scales / zeros are swapped relative to the schema, positions are kept)
+def awq_gemm_gcu(input: torch.Tensor, qweight: torch.Tensor, qzeros: torch.Tensor,
+                 scales: torch.Tensor, split_k_iters: int, bias=None, group_size=128) -> torch.Tensor:
+    return torch.ops._C.awq_gemm_gcu(input, qweight, qzeros, scales, split_k_iters, bias, group_size)
+
+
+@torch.library.register_fake("_C::awq_gemm_gcu")
+def _awq_gemm_gcu_fake(input, qweight, qzeros, scales, split_k_iters, bias=None, group_size=128):
+    out_shape = input.shape[:-1] + (qweight.shape[-1],)
+    return torch.empty(out_shape, dtype=input.dtype, device=input.device)
+
+
+# gptq (vllm_gcu/kernels/_custom_ops.py:242-293)
+def gptq_gemm_gcu(a: torch.Tensor, b_q_weight: torch.Tensor, b_gptq_qzeros: torch.Tensor,
+                  b_gptq_scales: torch.Tensor, b_g_idx: torch.Tensor, bit: int, bias=None,
+                  group_size=128) -> torch.Tensor:
+    assert bit in [4, 8]
+    if bit == 4:
+        out_shape = a.shape[:-1] + (b_q_weight.shape[-1],)
+        reshaped_a = a.reshape(-1, a.shape[-1])
+        output = torch.ops._C.gptq_gemm_gcu(reshaped_a, b_q_weight, b_gptq_qzeros, b_gptq_scales,
+                                            b_g_idx, bit, bias, group_size)
+        return output.reshape(out_shape)
+    out_shape = a.shape[:-1] + (b_q_weight.shape[0],)
+    output = torch.empty(out_shape, dtype=a.dtype, device=a.device)
+    torch.ops._C.weight_only_quant(output, a, b_q_weight, bias, b_gptq_scales, group_size)
+    return output
+
+
+@torch.library.register_fake("_C::gptq_gemm_gcu")
+def _gptq_gemm_gcu_fake(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bit, bias=None,
+                        group_size=128):
+    if bit == 4:
+        out_shape = a.shape[:-1] + (b_q_weight.shape[-1],)
+    else:
+        out_shape = a.shape[:-1] + (b_q_weight.shape[0],)
+    return torch.empty(out_shape, dtype=a.dtype, device=a.device)

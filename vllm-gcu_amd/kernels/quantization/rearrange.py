@@ -1,0 +1,107 @@
+"""int4 weight repack at load time, on the device.
+
+Counterpart of vllm_gcu/kernels/quantization/rearrange.py:6-133.  The
+reference unpacks GPTQ / AWQ checkpoints on the CPU into a ``uint8 [K/2, N]``
+half-group layout for the GCU; here the same checkpoints (or tensors already in
+the reference layout) are converted by HIP kernels into the MI355X slab layout
+the W4A16 kernels stream (see include/mi355q.h), and zero-points are kept as
+packed int4 instead of being pre-multiplied by the scales.
+"""
+import torch
+
+from .. import _runtime as rt
+from ... import _lib
+
+
+def _repack(src: torch.Tensor, fmt: int, batch: int, K: int, N: int) -> torch.Tensor:
+    rt.require_gpu(src)
+    src = src.contiguous()
+    shape = (K // 8, N) if batch is None else (batch, K // 8, N)
+    dst = torch.empty(shape, dtype=torch.int32, device=src.device)
+    with torch.cuda.device(src.device):
+        _lib.call("mi355q_w4_repack", src.data_ptr(), fmt, dst.data_ptr(),
+                  1 if batch is None else batch, K, N, rt.stream_ptr())
+    return dst
+
+
+def _repack_zeros(src: torch.Tensor, fmt: int) -> torch.Tensor:
+    rt.require_gpu(src)
+    src = src.contiguous()
+    assert src.dtype == torch.int32
+    batch = 1 if src.dim() == 2 else src.shape[0]
+    G, N8 = src.shape[-2], src.shape[-1]
+    dst = torch.empty_like(src)
+    with torch.cuda.device(src.device):
+        _lib.call("mi355q_w4_repack_zeros", src.data_ptr(), fmt, dst.data_ptr(), batch, G, N8 * 8,
+                  rt.stream_ptr())
+    return dst
+
+
+def rearrange_uint4_int32_gptq(qweight: torch.Tensor, qzeros, scales=None):
+    """GPTQ checkpoint tensors -> (slab-layout qweight int32 [K/8, N], packed
+    zero-points int32 [K/g, N/8] with the "+1" applied).
+
+    qweight int32 [K/8, N] (or [E, K/8, N]); qzeros int32 [K/g, N/8] or None.
+    Same inputs as rearrange_uint4_int32_uint8_gptq (rearrange.py:6-58).
+    """
+    assert qweight.dtype == torch.int32
+    batch = None if qweight.dim() == 2 else qweight.shape[0]
+    K, N = qweight.shape[-2] * 8, qweight.shape[-1]
+    w = _repack(qweight, _lib.W4_SRC_GPTQ, batch, K, N)
+    z = None if qzeros is None else _repack_zeros(qzeros, _lib.W4_SRC_GPTQ)
+    return w, z
+
+
+def rearrange_uint4_int32_awq(qweight: torch.Tensor, qzeros, scales=None):
+    """AWQ checkpoint tensors (qweight int32 [K, N/8], qzeros int32 [K/g, N/8])
+    -> (slab-layout qweight, packed zero-points).  Same inputs as
+    rearrange_uint4_int32_uint8_awq (rearrange.py:61-133)."""
+    assert qweight.dtype == torch.int32
+    batch = None if qweight.dim() == 2 else qweight.shape[0]
+    K, N = qweight.shape[-2], qweight.shape[-1] * 8
+    w = _repack(qweight, _lib.W4_SRC_AWQ, batch, K, N)
+    z = None if qzeros is None else _repack_zeros(qzeros, _lib.W4_SRC_AWQ)
+    return w, z
+
+
+def from_reference_layout(rweight: torch.Tensor, transposed: bool = False) -> torch.Tensor:
+    """Reference device layout -> slab layout.
+
+    ``rweight`` is uint8/int8 ``[K/2, N]`` (dense, rearrange.py:44-56) or, with
+    ``transposed=True``, ``[N, K/2]`` / ``[E, N, K/2]`` (MoE experts,
+    moe_wna16.py:464-466).  The result keeps the GPTQ checkpoint shape
+    ``[K/8, N]`` (``[E, K/8, N]``), dtype int32.
+    """
+    assert rweight.dtype in (torch.uint8, torch.int8)
+    batch = None if rweight.dim() == 2 else rweight.shape[0]
+    if transposed:
+        N, K = rweight.shape[-2], rweight.shape[-1] * 2
+        fmt = _lib.W4_SRC_REF_NK
+    else:
+        K, N = rweight.shape[-2] * 2, rweight.shape[-1]
+        fmt = _lib.W4_SRC_REF_KN
+    return _repack(rweight, fmt, batch, K, N)
+
+
+def pack_int8_zeros(z: torch.Tensor) -> torch.Tensor:
+    """int8/uint8 zero-points [..., G, N] (the AWQ ``zeros_in_int8`` form,
+    awq.py:80-106) -> packed int32 [..., G, N/8]."""
+    v = z.to(torch.int32) & 15
+    v = v.reshape(*z.shape[:-1], z.shape[-1] // 8, 8)
+    shifts = torch.arange(0, 32, 4, device=z.device, dtype=torch.int32)
+    return (v << shifts).sum(dim=-1).to(torch.int32)
+
+
+def unpack_slab(packed: torch.Tensor) -> torch.Tensor:
+    """Slab layout int32 [K/8, N] -> uint8 [K, N], one int4 value per byte
+    (parity/debug helper)."""
+    rt.require_gpu(packed)
+    assert packed.dtype == torch.int32
+    batch = None if packed.dim() == 2 else packed.shape[0]
+    K, N = packed.shape[-2] * 8, packed.shape[-1]
+    shape = (K, N) if batch is None else (batch, K, N)
+    dst = torch.empty(shape, dtype=torch.uint8, device=packed.device)
+    with torch.cuda.device(packed.device):
+        _lib.call("mi355q_w4_unpack", packed.contiguous().data_ptr(), dst.data_ptr(),
+                  1 if batch is None else batch, K, N, rt.stream_ptr())
+    return dst
