@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Default workload (BASELINE.json configs[1]): the W4A16 GEMM at the four
+Llama-3-8B linear shapes (qkv, o, gate_up, down) with M = 16 fp16 activations,
+int4 weights, group size 128.  One *step* = one pass over the four layers.
+Weights rotate through enough distinct copies to exceed twice the 256 MB
+Infinity Cache, so every step streams its weights from HBM.  Steps are captured
+in a HIP graph (launch gaps would otherwise dominate microsecond kernels) and
+timed with HIP events on the launch stream.
+
+Prints ONE JSON line: whole-job GB/s of algorithmic bytes, the roofline
+fraction of the dominant kernel, and the CPU oracle timed on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+LLAMA3_8B = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
+GROUP = 128
+HBM_PEAK_GBPS = 8000.0
+FP16_PEAK_TFLOPS = 2500.0
+INT8_PEAK_TOPS = 5000.0
+
+
+def w4a16_bytes(M, K, N, g=GROUP):
+    """Algorithmic bytes of one W4A16 GEMM: packed weights + fp16 scales +
+    packed int4 zeros + fp16 activations in + fp16 out."""
+    return K * N // 2 + (K // g) * N * 2 + (K // g) * N // 2 + 2 * M * K + 2 * M * N
+
+
+def make_layer(K, N, copies, dev, seed):
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    layers = []
+    for c in range(copies):
+        # random bits are as good as any int4 matrix; they are in slab order already
+        qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, generator=g).to(dev)
+        zp = torch.randint(-2**31, 2**31 - 1, (K // GROUP, N // 8), dtype=torch.int32, generator=g).to(dev)
+        sc = (torch.rand(K // GROUP, N, generator=g) * 0.009 + 0.001).to(torch.float16).to(dev)
+        layers.append((qw, zp, sc))
+    return layers
+
+
+def time_graph(fn_list, steps, warmup, stream):
+    """Time exactly `steps` steps, step i running fn_list[i % len(fn_list)].
+
+    One HIP graph holds len(fn_list) consecutive steps (so the kernels run back
+    to back without host launch gaps); it is replayed steps // len times and a
+    second graph holds the remainder.  HIP events on `stream` bracket the timed
+    region.  Returns seconds for all steps."""
+    import torch
+    n = len(fn_list)
+
+    def capture(k):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(k):
+                fn_list[i]()
+        return g
+
+    with torch.cuda.stream(stream):
+        for fn in fn_list:
+            fn()                                    # warm (allocates workspaces on this stream)
+        stream.synchronize()
+        full = capture(n)
+        rem = capture(steps % n) if steps % n else None
+        for _ in range(max(1, -(-warmup // n))):
+            full.replay()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps // n):
+            full.replay()
+        if rem is not None:
+            rem.replay()
+        e1.record(stream)
+        e1.synchronize()
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3
+
+
+def cpu_baseline_w4a16(M, budget_s=20.0):
+    """The CPU oracle (dequantize + torch.matmul, fp32) on the same four
+    shapes, all host threads.  Returns GB/s of the same algorithmic bytes."""
+    import numpy as np
+    import torch
+    from oracle import w4 as ow4
+    torch.set_num_threads(os.cpu_count() or 1)
+    rng = np.random.default_rng(0)
+    tot_b, tot_t, done = 0, 0.0, []
+    t_start = time.time()
+    for name, K, N in LLAMA3_8B:
+        q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+        z = rng.integers(0, 16, size=(K // GROUP, N), dtype=np.uint8)
+        s = rng.uniform(0.001, 0.01, size=(K // GROUP, N)).astype(np.float16)
+        x = rng.standard_normal((M, K)).astype(np.float16)
+        t0 = time.time()
+        ow4.w4a16_gemm(x, q, z, s, GROUP)
+        dt = time.time() - t0
+        tot_b += w4a16_bytes(M, K, N)
+        tot_t += dt
+        done.append(name)
+        if time.time() - t_start > budget_s:
+            break
+    return {"value": round(tot_b / tot_t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"one pass of oracle.w4.w4a16_gemm (numpy dequantize + torch fp32 matmul) over "
+                      f"layers {','.join(done)} at M={M}; {tot_t:.2f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--m", type=int, default=16, help="activation rows of the default workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sweep", action="store_true", help="also time every (shape, M) of the config")
+    ap.add_argument("--split-k", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no sharding, no collectives); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream(device=dev)
+    M = args.m
+
+    set_bytes = sum(K * N // 2 for _, K, N in LLAMA3_8B)
+    copies = max(2, -(-2 * 256 * 2**20 // set_bytes) + 1)
+    layers = {name: make_layer(K, N, copies, dev, seed=i) for i, (name, K, N) in enumerate(LLAMA3_8B)}
+    xs = {K: torch.randn(M, K, dtype=torch.float16, device=dev) for K in {k for _, k, _ in LLAMA3_8B}}
+
+    def layer_call(name, K, c):
+        qw, zp, sc = layers[name][c]
+        return ops.w4a16_gemm(xs[K], qw, sc, zp, None, GROUP, split_k=args.split_k)
+
+    def make_step(c):
+        def step():
+            for name, K, N in LLAMA3_8B:
+                layer_call(name, K, c)
+        return step
+
+    step_fns = [make_step(c) for c in range(copies)]
+    secs = time_graph(step_fns, args.steps, args.warmup, stream)
+    step_bytes = sum(w4a16_bytes(M, K, N) for _, K, N in LLAMA3_8B)
+    ms_per_step = secs / args.steps * 1e3
+    value = step_bytes * args.steps / secs / 1e9
+
+    # dominant kernel: the streaming kernel on the largest layer (gate_up)
+    per_layer = {}
+    for name, K, N in LLAMA3_8B:
+        fns = [(lambda name=name, K=K, c=c: layer_call(name, K, c)) for c in range(copies)]
+        n = max(args.steps, 100)
+        t = time_graph(fns, n, args.warmup, stream) / n
+        b = w4a16_bytes(M, K, N)
+        per_layer[name] = {"K": K, "N": N, "us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
+                           "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBPS, 4)}
+    dom = max(per_layer, key=lambda k: per_layer[k]["us"])
+    domK, domN = per_layer[dom]["K"], per_layer[dom]["N"]
+    roofline = {"bound": "hbm", "kernel": "w4a16_stream_kernel", "layer": dom,
+                "achieved": per_layer[dom]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": per_layer[dom]["frac_hbm"], "traffic": None,
+                "algorithmic_bytes": w4a16_bytes(M, domK, domN)}
+
+    out = {
+        "metric": "W4A16 GEMM HBM GB/s (algorithmic bytes / time), Llama-3-8B linear shapes",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"W4A16 GEMM, Llama-3-8B shapes qkv/o/gate_up/down, M={M}, int4 g=128, "
+                               f"fp16 act, fp32 accumulate; one step = the 4 layers once",
+                   "weight_copies_rotated": copies, "bytes_per_step": step_bytes},
+        "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "per_layer": per_layer,
+        "roofline": roofline,
+    }
+    if args.sweep:
+        out["sweep"] = sweep(ops, dev, stream, args)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_w4a16(M)
+    print(json.dumps(out))
+
+
+def sweep(ops, dev, stream, args):
+    """Every (shape, M) of BASELINE configs[1]: GB/s and TFLOP/s."""
+    import torch
+    res = []
+    for name, K, N in LLAMA3_8B:
+        copies = max(2, -(-2 * 256 * 2**20 // (K * N // 2)) + 1)
+        lay = make_layer(K, N, copies, dev, seed=7)
+        for M in (1, 8, 16, 32, 128, 2048):
+            x = torch.randn(M, K, dtype=torch.float16, device=dev)
+            fns = [(lambda c=c: ops.w4a16_gemm(x, lay[c][0], lay[c][2], lay[c][1], None, GROUP))
+                   for c in range(copies)]
+            try:
+                n = 200 if M <= 128 else 30
+                t = time_graph(fns, n, 10, stream) / n
+            except RuntimeError as e:       # kernel family not available for this M
+                res.append({"layer": name, "M": M, "error": str(e)[:80]})
+                continue
+            b, fl = w4a16_bytes(M, K, N), 2.0 * M * K * N
+            res.append({"layer": name, "K": K, "N": N, "M": M, "us": round(t * 1e6, 2),
+                        "GBps": round(b / t / 1e9, 1), "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBPS, 4),
+                        "TFLOPs": round(fl / t / 1e12, 2),
+                        "frac_fp16_mfma": round(fl / t / 1e12 / FP16_PEAK_TFLOPS, 4)})
+        del lay
+        torch.cuda.empty_cache()
+    return res
+
+
+if __name__ == "__main__":
+    main()

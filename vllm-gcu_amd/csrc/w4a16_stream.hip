@@ -28,61 +28,113 @@ struct StreamArgs {
   int* counters;     // [N/128], zero between launches
 };
 
+// (a & mask) | orv.  Callers launder `mask` into an SGPR and `orv` into a VGPR
+// (see launder_*) so the compiler cannot fold them into literals and selects
+// the single VOP3 v_and_or_b32 instead of an and + or pair.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
+  return (a & mask) | orv;
+}
+__device__ __forceinline__ uint32_t launder_sgpr(uint32_t v) {
+  asm volatile("" : "+s"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t launder_vgpr(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// Per activation type: the MFMA, and how packed nibbles become B operands
+// WITHOUT per-weight arithmetic.  A nibble q is OR-ed into the mantissa of a
+// constant, giving base + q (or base + 16 q for the odd nibble of a byte in
+// fp16, whose A elements are pre-multiplied by 1/16).  The MFMA therefore
+// accumulates  sum_k x_k q_k + CORR  where CORR depends only on row sums of x;
+// CORR and the zero-point term z * sum_k x_k are removed once per group from
+// the fp32 accumulator.
 template <int DT> struct Mma;
 template <> struct Mma<MI355Q_F16> {
   typedef h8 vec;
+  static constexpr bool kScaledA = true;      // needs the separate correction MFMA
+  static constexpr float kBase = 1024.0f;
   static __device__ __forceinline__ f4 run(vec a, vec b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ vec from_h2(h2 r0, h2 r1, h2 r2, h2 r3) {
-    return (h8){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
-  }
-  static __device__ __forceinline__ vec splat_one() {
-    const _Float16 o = (_Float16)1.0f;
+  static __device__ __forceinline__ vec splat(float v) {
+    const _Float16 o = (_Float16)v;
     return (h8){o, o, o, o, o, o, o, o};
   }
+  // elements (2,3) and (6,7) meet the "16 q" nibbles: scale them by 1/16
+  static __device__ __forceinline__ vec prep_a(u4 raw) {
+    const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+    raw[1] = bitcast<uint32_t>(bitcast<h2>(raw[1]) * sixteenth);
+    raw[3] = bitcast<uint32_t>(bitcast<h2>(raw[3]) * sixteenth);
+    return bitcast<vec>(raw);
+  }
+  static __device__ __forceinline__ vec make_b(uint32_t w, uint32_t magic, uint32_t mlo, uint32_t mhi) {
+    uint32_t w8 = w >> 8;
+    u4 v = {and_or(w, mlo, magic), and_or(w, mhi, magic), and_or(w8, mlo, magic), and_or(w8, mhi, magic)};
+    return bitcast<vec>(v);
+  }
+  static __device__ __forceinline__ uint32_t magic() { return 0x64006400u; }   // 1024.0 x2
 };
 template <> struct Mma<MI355Q_BF16> {
   typedef b8 vec;
+  static constexpr bool kScaledA = false;
+  static constexpr float kBase = 128.0f;
   static __device__ __forceinline__ f4 run(vec a, vec b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
-  // small integers held exactly in fp16 -> the same integers in bf16
-  static __device__ __forceinline__ uint32_t cvt(h2 r) {
-    uint32_t lo = bitcast<uint32_t>((float)r.x), hi = bitcast<uint32_t>((float)r.y);
-    return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+  static __device__ __forceinline__ vec splat(float v) {
+    uint32_t h = bitcast<uint32_t>(v) >> 16;
+    h |= h << 16;
+    u4 r = {h, h, h, h};
+    return bitcast<vec>(r);
   }
-  static __device__ __forceinline__ vec from_h2(h2 r0, h2 r1, h2 r2, h2 r3) {
-    u4 v = {cvt(r0), cvt(r1), cvt(r2), cvt(r3)};
+  static __device__ __forceinline__ vec prep_a(u4 raw) { return bitcast<vec>(raw); }
+  static __device__ __forceinline__ vec make_b(uint32_t w, uint32_t magic, uint32_t mlo, uint32_t) {
+    u4 v = {and_or(w, mlo, magic), and_or(w >> 4, mlo, magic), and_or(w >> 8, mlo, magic),
+            and_or(w >> 12, mlo, magic)};
     return bitcast<vec>(v);
   }
-  static __device__ __forceinline__ vec splat_one() {
-    u4 v = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
-    return bitcast<vec>(v);
-  }
+  static __device__ __forceinline__ uint32_t magic() { return 0x43004300u; }   // 128.0 x2
 };
 
-// one 32-bit word (8 nibbles) -> four packed pairs of exact (q - z)
-// zlo = (1024 + z, 1024 + z), zhi = (64 + z, 64 + z)
-__device__ __forceinline__ void dequant_word(uint32_t w, h2 zlo, h2 zhi, h2& r0, h2& r1, h2& r2,
-                                             h2& r3) {
-  const uint32_t MAGIC = 0x64006400u;            // fp16 1024.0 twice
-  const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-  uint32_t w8 = w >> 8;
-  h2 a0 = bitcast<h2>((w & 0x000f000fu) | MAGIC);    // 1024 + q
-  h2 a1 = bitcast<h2>((w & 0x00f000f0u) | MAGIC);    // 1024 + 16 q
-  h2 a2 = bitcast<h2>((w8 & 0x000f000fu) | MAGIC);
-  h2 a3 = bitcast<h2>((w8 & 0x00f000f0u) | MAGIC);
-  r0 = a0 - zlo;
-  r1 = __builtin_elementwise_fma(a1, sixteenth, -zhi);
-  r2 = a2 - zlo;
-  r3 = __builtin_elementwise_fma(a3, sixteenth, -zhi);
+__device__ __forceinline__ void store_partial(float* p, const float* v) {
+  // device-scope relaxed stores: written through to memory, no cache flush
+#pragma unroll
+  for (int t = 0; t < 8; t += 2) {
+    uint64_t bits = (uint64_t)bitcast<uint32_t>(v[t]) | ((uint64_t)bitcast<uint32_t>(v[t + 1]) << 32);
+    __hip_atomic_store((uint64_t*)(p + t), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+__device__ __forceinline__ void load_partial_add(const float* p, float* v) {
+#pragma unroll
+  for (int t = 0; t < 8; t += 2) {
+    uint64_t bits = __hip_atomic_load((const uint64_t*)(p + t), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v[t] += bitcast<float>((uint32_t)bits);
+    v[t + 1] += bitcast<float>((uint32_t)(bits >> 32));
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void store_out_row(uint16_t* out, const uint16_t* bias, int ncol, const float* v) {
+  u4 o;
+#pragma unroll
+  for (int t = 0; t < 8; t += 2) {
+    float v0 = v[t], v1 = v[t + 1];
+    if (bias) {
+      v0 += Elem<DT>::to_f32(bias[ncol + t]);
+      v1 += Elem<DT>::to_f32(bias[ncol + t + 1]);
+    }
+    o[t >> 1] = (uint32_t)Elem<DT>::from_f32(v0) | ((uint32_t)Elem<DT>::from_f32(v1) << 16);
+  }
+  *(u4*)out = o;
 }
 
 template <int DT, int MT, int ZK, int SPF>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, MT == 1 ? 2 : 1)
 w4a16_stream_kernel(StreamArgs a) {
-  typedef typename Mma<DT>::vec vec;
+  typedef Mma<DT> MM;
+  typedef typename MM::vec vec;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, kq = lane >> 4;
   const int slab = blockIdx.x, split = blockIdx.y;
@@ -100,97 +152,103 @@ w4a16_stream_kernel(StreamArgs a) {
 
   const u4* wbase = a.qw + (size_t)slab * G * 512 + lane;
   const int ncol = 128 * slab + 8 * c;               // first of this lane's 8 columns
+  const uint32_t magic = launder_vgpr(MM::magic());
+  const uint32_t mlo = launder_sgpr(0x000f000fu), mhi = launder_sgpr(0x00f000f0u);
 
+  // Everything a block's arithmetic needs is loaded together and one block
+  // ahead, so the only memory wait inside the compute phase is for the block
+  // being consumed while the next block's loads stay in flight (the wait
+  // counter retires in order: a late load would drain the prefetch too).
   struct Block {
     u4 w[8];
-    vec av[MT == 1 ? 4 : 1];
+    u4 sraw[4 / SPF];
+    u4 zraw[ZK == MI355Q_ZP_PRESCALED ? 4 / SPF : 1];
+    uint32_t zword[4 / SPF];
+    u4 xr[MT == 1 ? 4 : 1];
   };
   auto load_block = [&](Block& b, int g) {
     const u4* p = wbase + (size_t)g * 512;
 #pragma unroll
     for (int t = 0; t < 8; ++t) b.w[t] = __builtin_nontemporal_load(p + t * 64);
-    if (MT == 1) {
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        u4 v = {0u, 0u, 0u, 0u};
-        if (c < a.M) v = *(const u4*)(a.x + (size_t)c * K + 128 * g + 32 * s + 8 * kq);
-        b.av[s] = bitcast<vec>(v);
-      }
-    }
-  };
-
-  auto compute_block = [&](const Block& b, int g) {
-    vec av[MT][4];
-    if (MT == 1) {
-#pragma unroll
-      for (int s = 0; s < 4; ++s) av[0][s] = b.av[s];
-    } else {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          u4 v = {0u, 0u, 0u, 0u};
-          int row = 16 * mt + c;
-          if (row < a.M) v = *(const u4*)(a.x + (size_t)row * K + 128 * g + 32 * s + 8 * kq);
-          av[mt][s] = bitcast<vec>(v);
-        }
-    }
 #pragma unroll
     for (int f = 0; f < 4 / SPF; ++f) {
       const int qrow = (128 * g + 32 * SPF * f) / a.gs;
-      // 8 scales, 8 zero-points for this lane's columns
-      u4 sraw = *(const u4*)(a.scales + (size_t)qrow * N + ncol);
-      float sc[8];
+      b.sraw[f] = *(const u4*)(a.scales + (size_t)qrow * N + ncol);
+      b.zword[f] = 0x88888888u;
+      if (ZK == MI355Q_ZP_PACKED) b.zword[f] = ((const uint32_t*)a.zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)];
+      if (ZK == MI355Q_ZP_PRESCALED) b.zraw[f] = *(const u4*)((const uint16_t*)a.zeros + (size_t)qrow * N + ncol);
+    }
+    if (MT == 1) {
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        uint32_t word = sraw[t >> 1];
-        sc[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (word >> 16) : (word & 0xffffu)));
+      for (int s = 0; s < 4; ++s) {
+        // rows past M repeat the last row: output rows are independent and
+        // rows >= M are never stored, so no predicated load is needed
+        b.xr[s] = *(const u4*)(a.x + (size_t)min(c, a.M - 1) * K + 128 * g + 32 * s + 8 * kq);
       }
-      uint32_t zword = 0x88888888u;
-      float zs[8];
-      if (ZK == MI355Q_ZP_PACKED) zword = ((const uint32_t*)a.zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)];
-      if (ZK == MI355Q_ZP_PRESCALED) {
-        zword = 0u;
-        u4 zraw = *(const u4*)((const uint16_t*)a.zeros + (size_t)qrow * N + ncol);
+    }
+  };
+  // activations of block g for MT > 1 (too many registers to carry a block ahead)
+  struct Acts { u4 xr[MT == 1 ? 1 : MT][4]; };
+  auto load_acts = [&](Acts& x, int g) {
+    if (MT == 1) return;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          uint32_t word = zraw[t >> 1];
-          zs[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (word >> 16) : (word & 0xffffu)));
-        }
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int row = min(16 * mt + c, a.M - 1);
+        x.xr[mt][s] = *(const u4*)(a.x + (size_t)row * K + 128 * g + 32 * s + 8 * kq);
       }
-      // row sums of x over this scale group (only the pre-scaled-zero form needs them)
-      f4 xsum[MT];
-      if (ZK == MI355Q_ZP_PRESCALED) {
+  };
+
+  auto compute_block = [&](const Block& b, const Acts& xa) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          xsum[mt] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (int f = 0; f < 4 / SPF; ++f) {
+      const u4 sraw = b.sraw[f];
+      const uint32_t zword = b.zword[f];
+      // per row of x over this scale group: xs = sum x, corr = what the
+      // mantissa trick added to the accumulator
+      vec av[MT][SPF];
+      f4 xs[MT], corr[MT];
 #pragma unroll
-          for (int s = 0; s < SPF; ++s)
-            xsum[mt] = Mma<DT>::run(av[mt][SPF * f + s], Mma<DT>::splat_one(), xsum[mt]);
-        }
-      }
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const float zf = (float)((zword >> (4 * t)) & 15u);
-        const _Float16 zl = (_Float16)(1024.0f + zf), zh = (_Float16)(64.0f + zf);
-        const h2 zlo = {zl, zl}, zhi = {zh, zh};
-        f4 part[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) part[mt] = (f4){0.f, 0.f, 0.f, 0.f};
+      for (int mt = 0; mt < MT; ++mt) {
+        xs[mt] = (f4){0.f, 0.f, 0.f, 0.f};
+        corr[mt] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < SPF; ++s) {
-          h2 r0, r1, r2, r3;
-          dequant_word(b.w[t][SPF * f + s], zlo, zhi, r0, r1, r2, r3);
-          vec bv = Mma<DT>::from_h2(r0, r1, r2, r3);
+          const u4 raw = (MT == 1) ? b.xr[MT == 1 ? SPF * f + s : 0] : xa.xr[MT == 1 ? 0 : mt][SPF * f + s];
+          av[mt][s] = MM::prep_a(raw);
+          xs[mt] = MM::run(bitcast<vec>(raw), MM::splat(1.0f), xs[mt]);
+          if (MM::kScaledA) corr[mt] = MM::run(av[mt][s], MM::splat(MM::kBase), corr[mt]);
+        }
+        if (!MM::kScaledA) corr[mt] = MM::kBase * xs[mt];
+      }
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) part[mt] = Mma<DT>::run(av[mt][SPF * f + s], bv, part[mt]);
+      for (int t = 0; t < 8; ++t) {
+        const uint32_t sword = sraw[t >> 1];
+        const float sc = Elem<DT>::to_f32((uint16_t)((t & 1) ? (sword >> 16) : (sword & 0xffffu)));
+        f4 part[MT];
+        if (ZK == MI355Q_ZP_PRESCALED) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) part[mt] = -corr[mt];
+        } else {
+          const float zf = (float)((zword >> (4 * t)) & 15u);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) part[mt] = -zf * xs[mt] - corr[mt];
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          if (ZK == MI355Q_ZP_PRESCALED)
-            acc[mt][t] += sc[t] * part[mt] - zs[t] * xsum[mt];
-          else
-            acc[mt][t] += sc[t] * part[mt];
+        for (int s = 0; s < SPF; ++s) {
+          vec bv = MM::make_b(b.w[t][SPF * f + s], magic, mlo, mhi);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) part[mt] = MM::run(av[mt][s], bv, part[mt]);
+        }
+        if (ZK == MI355Q_ZP_PRESCALED) {
+          const uint32_t zw = b.zraw[f][t >> 1];
+          const float zsf = Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu)));
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt][t] += sc * part[mt] - zsf * xs[mt];
+        } else {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt][t] += sc * part[mt];
         }
       }
     }
@@ -198,16 +256,30 @@ w4a16_stream_kernel(StreamArgs a) {
 
   {
     Block b0, b1;
+    Acts xa;
     int g = gb + wave;
     if (g < ge) {
+      // the prefetch is unconditional (the last one re-reads this wave's own
+      // final block) so the loop body is straight-line code and the compiler
+      // can wait for exactly the block being consumed
+      const int glast = g + ((ge - 1 - g) & ~3);
       load_block(b0, g);
       while (true) {
-        if (g + 4 < ge) load_block(b1, g + 4);
-        compute_block(b0, g);
+        // sched_barrier: keep the prefetch ahead of the arithmetic, the
+        // instruction scheduler would otherwise sink the loads next to
+        // their first use one iteration later
+        load_acts(xa, g);
+        load_block(b1, min(g + 4, glast));
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(b0, xa);
+        __builtin_amdgcn_sched_barrier(0);
         g += 4;
         if (g >= ge) break;
-        if (g + 4 < ge) load_block(b0, g + 4);
-        compute_block(b1, g);
+        load_acts(xa, g);
+        load_block(b0, min(g + 4, glast));
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(b1, xa);
+        __builtin_amdgcn_sched_barrier(0);
         g += 4;
         if (g >= ge) break;
       }
@@ -217,6 +289,7 @@ w4a16_stream_kernel(StreamArgs a) {
   // ---- reduce the 4 wavefronts through LDS; wave w finishes rows 4*kq + w ----
   __shared__ float red[4][32][64];
   const int Mpad = 16 * MT;
+  float fin[MT][8];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -224,70 +297,45 @@ w4a16_stream_kernel(StreamArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) red[wave][i * 8 + t][lane] = acc[mt][t][i];
     __syncthreads();
-    float v[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t)
-      v[t] = ((red[0][wave * 8 + t][lane] + red[1][wave * 8 + t][lane]) +
-              red[2][wave * 8 + t][lane]) + red[3][wave * 8 + t][lane];
+      fin[mt][t] = ((red[0][wave * 8 + t][lane] + red[1][wave * 8 + t][lane]) +
+                    red[2][wave * 8 + t][lane]) + red[3][wave * 8 + t][lane];
     __syncthreads();
     const int m = 16 * mt + 4 * kq + wave;
-    if (a.splits == 1) {
-      if (m < a.M) {
-        u4 o;
-#pragma unroll
-        for (int t = 0; t < 8; t += 2) {
-          float v0 = v[t], v1 = v[t + 1];
-          if (a.bias) {
-            v0 += Elem<DT>::to_f32(a.bias[ncol + t]);
-            v1 += Elem<DT>::to_f32(a.bias[ncol + t + 1]);
-          }
-          o[t >> 1] = (uint32_t)Elem<DT>::from_f32(v0) | ((uint32_t)Elem<DT>::from_f32(v1) << 16);
-        }
-        *(u4*)(a.out + (size_t)m * N + ncol) = o;
-      }
-    } else {
-      float* p = a.partial + ((size_t)split * Mpad + m) * N + ncol;
-      *(f4*)p = (f4){v[0], v[1], v[2], v[3]};
-      *(f4*)(p + 4) = (f4){v[4], v[5], v[6], v[7]};
+    if (m < a.M) {
+      if (a.splits == 1)
+        store_out_row<DT>(a.out + (size_t)m * N + ncol, a.bias, ncol, fin[mt]);
+      else
+        store_partial(a.partial + ((size_t)split * Mpad + m) * N + ncol, fin[mt]);
     }
   }
   if (a.splits == 1) return;
 
-  // ---- cross-workgroup split-K: last arriver adds the partial tiles in order ----
+  // ---- cross-workgroup split-K ---------------------------------------------
+  // Partial tiles travel as device-scope relaxed accesses (they bypass the
+  // per-XCD L2 instead of flushing it); the barrier's wait for outstanding
+  // stores orders them before the arrival count.  The last workgroup to
+  // arrive adds the tiles in split order, so the sum is reproducible.
   __shared__ int is_last;
-  __threadfence();
   __syncthreads();
   if (threadIdx.x == 0) {
-    int old = __hip_atomic_fetch_add(a.counters + slab, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    int old = __hip_atomic_fetch_add(a.counters + slab, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     is_last = (old == a.splits - 1);
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + 4 * kq + wave;
     if (m >= a.M) continue;
-    f4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < a.splits; ++sp) {
-      const float* p = a.partial + ((size_t)sp * Mpad + m) * N + ncol;
-      s0 += __builtin_nontemporal_load((const f4*)p);
-      s1 += __builtin_nontemporal_load((const f4*)(p + 4));
-    }
-    float v[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-    u4 o;
-#pragma unroll
-    for (int t = 0; t < 8; t += 2) {
-      float v0 = v[t], v1 = v[t + 1];
-      if (a.bias) {
-        v0 += Elem<DT>::to_f32(a.bias[ncol + t]);
-        v1 += Elem<DT>::to_f32(a.bias[ncol + t + 1]);
-      }
-      o[t >> 1] = (uint32_t)Elem<DT>::from_f32(v0) | ((uint32_t)Elem<DT>::from_f32(v1) << 16);
-    }
-    *(u4*)(a.out + (size_t)m * N + ncol) = o;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < a.splits; ++sp)
+      load_partial_add(a.partial + ((size_t)sp * Mpad + m) * N + ncol, v);
+    store_out_row<DT>(a.out + (size_t)m * N + ncol, a.bias, ncol, v);
   }
-  if (threadIdx.x == 0) a.counters[slab] = 0;
+  if (threadIdx.x == 0)
+    __hip_atomic_store(a.counters + slab, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int DT, int MT, int ZK>
@@ -313,14 +361,17 @@ static void launch_mt(const StreamArgs& a, int zk, hipStream_t st) {
   else launch_zk<DT, 4>(a, zk, st);
 }
 
-// split-K choice: enough workgroups to cover the CUs about twice while every
-// wavefront still streams at least two K blocks
+// split-K choice.  Exchanging partial tiles between workgroups costs two
+// dependent trips to memory, so K is split only while the grid would leave
+// most CUs idle: aim at about 0.6 workgroups per CU and keep at least two K
+// blocks per wavefront (measured on MI355X at M = 16: 224 slabs -> 1 split,
+// 48 slabs -> 3, 32 slabs -> 4..5).
 int w4a16_stream_auto_splits(int M, int K, int N) {
   const int slabs = N / 128, G = K / 128;
-  const int cus = device_cu_count();
-  int want = (2 * cus + slabs - 1) / slabs;
-  int maxs = G / 8 > 0 ? G / 8 : 1;        // >= 8 K blocks (2 per wavefront) per workgroup
-  int s = want < maxs ? want : maxs;
+  const int target = (device_cu_count() * 5) / 8;
+  int s = (target + slabs / 2) / slabs;
+  int maxs = G / 8 > 0 ? G / 8 : 1;
+  if (s > maxs) s = maxs;
   if (s < 1) s = 1;
   if (s > 32) s = 32;
   (void)M;

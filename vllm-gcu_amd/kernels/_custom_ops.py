@@ -45,28 +45,33 @@ def _register(ns: str, name: str, schema: str, fn, tags=()):
 # ---------------------------------------------------------------------------
 # W4A16 (csrc/torch_bindings.cpp:770-788)
 # ---------------------------------------------------------------------------
-_ref_layout_cache = {}
+def _converted(t: torch.Tensor, convert):
+    """Convert ``t`` once and keep the result on the tensor object itself (so
+    it lives exactly as long as the source and can never be confused with a
+    later allocation at the same address).  Re-converts if the source was
+    written in place or re-pointed since."""
+    tag = (t.data_ptr(), t._version, tuple(t.shape))
+    hit = getattr(t, "_mi355q_converted", None)
+    if hit is None or hit[0] != tag:
+        hit = (tag, convert(t))
+        t._mi355q_converted = hit
+    return hit[1]
 
 
-def _slab_weight(qweight: torch.Tensor) -> torch.Tensor:
+def _slab_weight(qweight: torch.Tensor, transposed: bool = False) -> torch.Tensor:
     """Return the slab-layout tensor for ``qweight``.
 
-    int32 tensors are this build's layout already.  uint8/int8 ``[K/2, N]``
-    tensors are the reference's half-group layout (rearrange.py:44-56); they
-    are converted on the device once and remembered per storage, so a caller
-    that keeps the reference's loader still works (at the cost of holding both
-    copies).
+    int32 tensors are this build's layout already.  uint8/int8 tensors are the
+    reference's half-group layout (``[K/2, N]`` dense, rearrange.py:44-56, or
+    ``[E, N, K/2]`` for MoE experts with ``transposed=True``); they are
+    converted on the device once, so a caller that keeps the reference's
+    loader still works (at the cost of holding both copies).
     """
     if qweight.dtype == torch.int32:
         return qweight
     if qweight.dtype not in (torch.uint8, torch.int8):
         raise TypeError(f"int4 weights must be int32 (slab) or uint8/int8 (reference), got {qweight.dtype}")
-    key = (qweight.data_ptr(), tuple(qweight.shape), qweight.device.index, qweight._version)
-    hit = _ref_layout_cache.get(key)
-    if hit is None:
-        hit = rearrange.from_reference_layout(qweight)
-        _ref_layout_cache[key] = hit
-    return hit
+    return _converted(qweight, lambda t: rearrange.from_reference_layout(t, transposed=transposed))
 
 
 def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype):
@@ -76,12 +81,7 @@ def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype):
     if zeros.dtype == torch.int32:
         return zeros, _lib.ZP_PACKED
     if zeros.dtype in (torch.int8, torch.uint8):
-        key = (zeros.data_ptr(), tuple(zeros.shape), zeros.device.index, zeros._version)
-        hit = _ref_layout_cache.get(key)
-        if hit is None:
-            hit = rearrange.pack_int8_zeros(zeros)
-            _ref_layout_cache[key] = hit
-        return hit, _lib.ZP_PACKED
+        return _converted(zeros, rearrange.pack_int8_zeros), _lib.ZP_PACKED
     if zeros.dtype == act_dtype:
         return zeros, _lib.ZP_PRESCALED
     raise TypeError(f"zero-points of dtype {zeros.dtype} do not match activations of dtype {act_dtype}")
