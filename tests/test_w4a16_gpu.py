@@ -185,3 +185,52 @@ def test_empty_input_returns_empty(ops, rearrange):
     out = ops.w4a16_gemm(torch.empty(0, 128, dtype=torch.float16, device="cuda"), w,
                          to_act(s, torch.float16).cuda(), zp, None, 128)
     assert out.shape == (0, 128)
+
+
+# ------------------------------------------------------- MFMA tile kernel ----
+@pytest.mark.parametrize("M,K,N", [(65, 256, 256), (128, 512, 384), (200, 1024, 512), (2048, 4096, 4096)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_tile_gemm_parity(ops, rearrange, M, K, N, dtype):
+    if dtype == torch.bfloat16 and M == 2048:
+        pytest.skip("one full-size case is enough")
+    g = 128
+    print(f"case tile M={M} K={K} N={N} {dtype}", flush=True)
+    q, z, s, x = make_case(M + K, M, K, N, g)
+    bias = np.random.default_rng(9).standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias).float().cpu().numpy()
+    want = oracle(q, z, s, x, g, dtype, bias=bias)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+def test_tile_gemm_exact_and_agrees_with_stream(ops, rearrange):
+    # exact case: both kernel families must reproduce the oracle bit for bit
+    M, K, N, g = 64, 512, 256, 128
+    q, z, s, x = make_case(3, M, K, N, g, exact=True)
+    want = torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16)
+    a = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=1)
+    b = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=2)
+    assert torch.equal(a.cpu(), want) and torch.equal(b.cpu(), want)
+
+
+def test_tile_gemm_zero_kinds_and_group_256(ops, rearrange):
+    M, K, N, g = 130, 512, 256, 256
+    q, z, s, x = make_case(77, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).float().cpu().numpy()
+    np.testing.assert_allclose(got, oracle(q, z, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)
+    # symmetric default (no zero-points) and the reference's pre-scaled fp16 zeros
+    w, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
+    xs = to_act(x, torch.float16).cuda()
+    out = ops.w4a16_gemm(xs, w, to_act(s, torch.float16).cuda(), None, None, g)
+    np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, None, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)
+    s16 = s.astype(np.float16)
+    zs = (z.astype(np.float32) * s16.astype(np.float32)).astype(np.float16)
+    out = ops.w4a16_gemm(xs, w, dev(s16), dev(zs), None, g)
+    want = to_act(x, torch.float16).float().numpy() @ ow4.dequantize_prescaled_zeros(q, zs, s16, g)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):
+    M, K, N, g = 150, 256, 128, 64
+    q, z, s, x = make_case(5, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).float().cpu().numpy()
+    np.testing.assert_allclose(got, oracle(q, z, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)

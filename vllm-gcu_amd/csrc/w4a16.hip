@@ -41,11 +41,25 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
              "w4a16_gemm: unknown zeros_kind %d", zeros_kind);
   MQ_REQUIRE(zeros_kind == MI355Q_ZP_NONE || zeros, "w4a16_gemm: zeros pointer missing");
   MQ_REQUIRE(family >= 0 && family <= 2, "w4a16_gemm: unknown kernel family %d", family);
-  if (family == 0) family = (M <= 64) ? 1 : 2;
-  MQ_REQUIRE(family != 1 || M <= 64, "w4a16_gemm: streaming kernel handles M <= 64, got %d", M);
-  if (family == 1)
-    return w4a16_stream_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size,
-                               dtype, workspace, workspace_bytes, split_k, as_stream(stream));
+  // bf16: the MFMA kernel rounds every dequantised weight to bf16 (8
+  // significant bits), which can exceed the 1e-2 parity bound on long dot
+  // products; bf16 therefore stays on the exact-integer streaming kernel
+  if (family == 0) family = (M <= 64 || group_size % 128 != 0 || dtype == MI355Q_BF16) ? 1 : 2;
+  MQ_REQUIRE(family != 2 || group_size % 128 == 0,
+             "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
+  if (family == 1) {
+    // the streaming kernel covers 64 rows per launch; taller inputs (only
+    // reached with group sizes below 128) go through it in row chunks
+    const size_t esz = 2;
+    for (int m0 = 0; m0 < M; m0 += 64) {
+      const int mc = M - m0 < 64 ? M - m0 : 64;
+      int rc = w4a16_stream_launch((char*)out + (size_t)m0 * N * esz, (const char*)x + (size_t)m0 * K * esz,
+                                   qweight, scales, zeros, zeros_kind, bias, mc, K, N, group_size, dtype,
+                                   workspace, workspace_bytes, split_k, as_stream(stream));
+      if (rc) return rc;
+    }
+    return 0;
+  }
   return w4a16_tile_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
                            as_stream(stream));
 }
