@@ -126,6 +126,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also time every (shape, M) of the config")
     ap.add_argument("--split-k", type=int, default=0)
+    ap.add_argument("--no-w8a8", action="store_true", help="skip the W8A8 int8 GEMM leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); "
@@ -189,11 +190,35 @@ def main():
         "per_layer": per_layer,
         "roofline": roofline,
     }
+    if not args.no_w8a8:
+        out["w8a8_int8"] = w8a8_gemm_bench(ops, dev, stream)
     if args.sweep:
         out["sweep"] = sweep(ops, dev, stream, args)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_w4a16(M)
     print(json.dumps(out))
+
+
+def w8a8_gemm_bench(ops, dev, stream, iters=20):
+    """BASELINE configs[2]: W8A8 int8 GEMM, M=2048, K=8192, N=28672 (one
+    Llama-3-70B MLP layer), per-token x per-channel scales fused, fp16 out."""
+    import torch
+    M, K, N = 2048, 8192, 28672
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(M, K, generator=g).to(torch.float16).to(dev)
+    xq, xs, _ = ops.scaled_int8_quant(x)
+    w_nk = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g).to(dev)
+    ws = (torch.rand(N, generator=g) * 0.019 + 0.001).float().to(dev)
+    out = torch.empty(M, N, dtype=torch.float16, device=dev)
+    wt = w_nk.t()
+    t = time_graph([lambda: torch.ops._C.cutlass_scaled_mm(out, xq, wt, xs, ws, None)], iters, 3, stream) / iters
+    tq = time_graph([lambda: ops.scaled_int8_quant(x)], iters, 3, stream) / iters
+    ops_ = 2.0 * M * K * N
+    return {"workload": "W8A8 int8 GEMM M=2048 K=8192 N=28672, fused per-token x per-channel scales, fp16 out",
+            "gemm_us": round(t * 1e6, 1), "TOPs": round(ops_ / t / 1e12, 1),
+            "frac_int8_mfma_peak": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
+            "dynamic_quant_us": round(tq * 1e6, 1),
+            "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1)}
 
 
 def sweep(ops, dev, stream, args):

@@ -88,6 +88,33 @@ int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          int dtype, void* workspace, size_t workspace_bytes,
                          int split_k, int family, void* stream);
 
+/* ---- W8A8 int8 -------------------------------------------------------------
+ * Replaces topsatenDotBiasQuant as called by cutlass_scaled_mm
+ * (csrc/src/cutlass_scaled_mm.cpp:12-36) and dot_bias_quant
+ * (csrc/src/dot_bias_quant.cpp:12-24):
+ *   out[m, n] = (sum_k x[m, k] * w[n, k]  in int32) * x_scale[m or 0] * w_scale[n or 0] (+ bias[n])
+ * x is [M, K] int8 with row stride ldx bytes; w is [N, K] int8 (K contiguous)
+ * with row stride ldw bytes -- the physical layout of a checkpoint's [N, K]
+ * weight, i.e. the `weight.t()` view the compressed-tensors path passes.
+ * Scale pointers may be NULL (= 1.0); *_per_row / *_per_col select a vector
+ * or a single value.  bias is in the output dtype, or fp32 when bias_f32.
+ * acc_out (optional) receives the raw int32 accumulators [M, N] for parity
+ * checks.  K %% 128 == 0, N %% 4 == 0. */
+int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* x, const int8_t* w,
+                          const float* x_scale, int x_scale_per_row, const float* w_scale,
+                          int w_scale_per_col, const void* bias, int bias_f32, int M, int N, int K,
+                          long ldx, long ldw, long ldo, int out_dtype, void* stream);
+/* Replaces topsvllmDynamicScaledInt8Quant (csrc/src/dynamic_scaled_int8_quant.cpp:12-19):
+ * per row scale = absmax / 127 (fp32 [M]), q = sat_s8(rne(x * (127 / absmax))).
+ * valid_rows (optional device int32[1]) limits the rows processed. */
+int mi355q_dynamic_int8_quant(int8_t* out, float* scales, const void* x, int M, int K, int dtype,
+                              const int32_t* valid_rows, void* stream);
+/* Replaces topsatenQuantize as called by static_scaled_int8_quant
+ * (csrc/src/static_scaled_int8_quant.cpp:12-28): q = sat_s8(rne(x * (1/scale)))
+ * with the reciprocal rounded to the input dtype; scale is one value or [K]. */
+int mi355q_static_int8_quant(int8_t* out, const void* x, const float* scale, int per_channel, int M,
+                             int K, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

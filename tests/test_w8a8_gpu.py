@@ -1,0 +1,138 @@
+"""GPU parity of the W8A8 int8 path: quantisers and int32 accumulators are
+bit-exact against the CPU oracle; scaled fp16/bf16 outputs within rtol 1e-2 /
+atol 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import w8a8 as o8
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from vllm_gcu_amd.kernels import _custom_ops
+    return _custom_ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,K", [(1, 128), (37, 1000), (64, 8192)])
+def test_dynamic_int8_quant_bit_exact(ops, dtype, M, K):
+    print(f"case dyn-quant {M}x{K} {dtype}", flush=True)
+    rng = np.random.default_rng(M * K)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    if M > 1:
+        x[1] = 0                       # all-zero row: scale 0, q 0
+        x[2, 5] = 40.0                 # outlier
+    q, s, azp = ops.scaled_int8_quant(x.cuda())
+    assert azp is None and q.dtype == torch.int8 and s.shape == (M, 1) and s.dtype == torch.float32
+    qo, so = o8.dynamic_scaled_int8_quant(x.float().numpy())
+    assert np.array_equal(s.cpu().numpy(), so)
+    assert np.array_equal(q.cpu().numpy(), qo)
+
+
+def test_dynamic_int8_quant_3d_input(ops):
+    x = torch.randn(3, 5, 256, dtype=torch.float16)
+    q, s, _ = ops.scaled_int8_quant(x.cuda())
+    qo, so = o8.dynamic_scaled_int8_quant(x.float().numpy().reshape(15, 256))
+    assert q.shape == x.shape and s.shape == (15, 1)
+    assert np.array_equal(q.cpu().numpy().reshape(15, 256), qo) and np.array_equal(s.cpu().numpy(), so)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_static_int8_quant_bit_exact(ops, dtype):
+    rng = np.random.default_rng(1)
+    x = torch.from_numpy((rng.standard_normal((33, 512)) * 3).astype(np.float32)).to(dtype)
+    x[0, 0] = 1000.0
+    x[0, 1] = -1000.0
+    np_x = x.numpy() if dtype == torch.float32 else x.numpy().astype(np.float16)
+    scale = torch.tensor(0.037, dtype=torch.float32)
+    q, s, _ = ops.scaled_int8_quant(x.cuda(), scale.cuda())
+    assert np.array_equal(q.cpu().numpy(), o8.static_scaled_int8_quant(np_x, scale.numpy()))
+    ch = torch.from_numpy(rng.uniform(0.01, 0.1, 512).astype(np.float32))
+    q, _, _ = ops.scaled_int8_quant(x.cuda(), ch.cuda())
+    assert np.array_equal(q.cpu().numpy(), o8.static_scaled_int8_quant(np_x, ch.numpy()))
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 128, 4), (7, 256, 36), (300, 1024, 520), (256, 512, 256), (513, 2048, 1028)])
+def test_int8_gemm_accumulators_bit_exact_both_layouts(ops, M, K, N):
+    print(f"case i8 acc {M}x{K}x{N}", flush=True)
+    rng = np.random.default_rng(M + K + N)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    x[0, :] = -128
+    w_nk[0, :] = -127
+    want = o8.int8_gemm_i32(x, np.ascontiguousarray(w_nk.T))
+    # [K, N] view of an [N, K] checkpoint tensor (compressed-tensors path)
+    acc = ops.int8_gemm_accumulators(dev(x), dev(w_nk).t())
+    assert acc.dtype == torch.int32 and np.array_equal(acc.cpu().numpy(), want)
+    # physically [K, N] weight (w8a8_gcu path, w8a8.py:152-155)
+    acc2 = ops.int8_gemm_accumulators(dev(x), dev(np.ascontiguousarray(w_nk.T)))
+    assert np.array_equal(acc2.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_cutlass_scaled_mm_epilogue(ops, dtype):
+    rng = np.random.default_rng(3)
+    M, K, N = 130, 512, 260
+    xf = rng.standard_normal((M, K)).astype(np.float16)
+    xq, xs = o8.dynamic_scaled_int8_quant(xf)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    acc = o8.int8_gemm_i32(xq, np.ascontiguousarray(w_nk.T))
+    for b, sa, sb in [(None, dev(xs), dev(ws)), (torch.from_numpy(bias).to(dtype).cuda(), dev(xs), dev(ws).reshape(N, 1)),
+                      (None, dev(xs[:1, 0]).reshape(()), dev(ws[:1]))]:
+        out = ops.cutlass_scaled_mm(dev(xq), dev(w_nk).t(), sa, sb, dtype, b)
+        want = o8.scaled_mm_epilogue(acc, sa.cpu().numpy(), sb.cpu().numpy(),
+                                     None if b is None else b.float().cpu().numpy())
+        assert out.dtype == dtype and out.shape == (M, N)
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_dot_bias_quant_single_scale(ops):
+    rng = np.random.default_rng(4)
+    M, K, N = 20, 256, 132
+    xq = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_kn = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    sc = rng.uniform(1e-4, 1e-3, N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float16)
+    out = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    ops.dot_bias_quant(out, dev(xq), dev(w_kn), dev(sc), dev(bias))
+    want = o8.scaled_mm_epilogue(o8.int8_gemm_i32(xq, w_kn), 1.0, sc, bias.astype(np.float32))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    ops.cutlass_scaled_mm(torch.empty(0, K, dtype=torch.int8, device="cuda"), dev(w_kn), dev(sc[:1]), dev(sc), torch.float16)
+
+
+def test_config2_full_size_sampled_rows(ops):
+    # BASELINE config 2: x f16 [2048, 8192] -> per-token int8; W int8 [8192, 28672];
+    # int32 accumulate bit-exact.  The oracle checks 96 rows spread over every
+    # 256-row tile, all 28672 columns.
+    M, K, N = 2048, 8192, 28672
+    print("case config2", flush=True)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(M, K, generator=g).to(torch.float16)
+    w_nk = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g)
+    ws = (torch.rand(N, generator=g) * 0.019 + 0.001).float()
+    xq, xs, _ = ops.scaled_int8_quant(x.cuda())
+    wd = w_nk.cuda()
+    acc = ops.int8_gemm_accumulators(xq, wd.t())
+    out = ops.cutlass_scaled_mm(xq, wd.t(), xs, ws.cuda(), torch.float16)
+    rows = np.unique(np.concatenate([np.arange(0, M, 256), np.arange(255, M, 256),
+                                     np.random.default_rng(0).integers(0, M, 80)]))
+    xq_o, xs_o = o8.dynamic_scaled_int8_quant(x[rows].float().numpy())
+    assert np.array_equal(xq[rows].cpu().numpy(), xq_o)
+    want_acc = o8.int8_gemm_i32(xq_o, np.ascontiguousarray(w_nk.numpy().T))
+    assert np.array_equal(acc[rows].cpu().numpy(), want_acc)
+    want = o8.scaled_mm_epilogue(want_acc, xs_o, ws.numpy())
+    np.testing.assert_allclose(out[rows].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # size-independent property on the full result: linearity in the weights'
+    # sign (negating W negates every accumulator exactly)
+    acc_neg = ops.int8_gemm_accumulators(xq, (-wd).t())
+    assert torch.equal(acc_neg, -acc)

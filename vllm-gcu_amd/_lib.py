@@ -5,7 +5,7 @@ fails, an exception is raised.
 """
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, c_float
+from ctypes import c_char_p, c_int, c_long, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi355q.so")
@@ -27,6 +27,11 @@ SIGNATURES = {
     "mi355q_w4a16_gemm_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_int,
                                      c_int, c_void_p]),
+    "mi355q_w8a8_int8_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                      c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_int,
+                                      c_void_p]),
+    "mi355q_dynamic_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None

@@ -180,3 +180,155 @@ def _gptq_gemm_gcu_fake(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bi
     else:
         out_shape = a.shape[:-1] + (b_q_weight.shape[0],)
     return torch.empty(out_shape, dtype=a.dtype, device=a.device)
+
+
+# ---------------------------------------------------------------------------
+# W8A8 int8 (csrc/torch_bindings.cpp:734-766, 1002-1019)
+# ---------------------------------------------------------------------------
+def _int8_weight_nk(weight: torch.Tensor):
+    """-> (tensor whose memory is [N, K] K-contiguous, row stride in bytes).
+
+    ``weight`` is the operator's ``[K, N]`` argument.  The compressed-tensors
+    path hands over ``w.t()`` of an ``[N, K]`` checkpoint tensor (strides
+    ``(1, K)``, csrc/torch_bindings.cpp:1013-1017 tags the op flexible_layout),
+    which already is the layout the int8 MFMA consumes.  A physically ``[K, N]``
+    tensor (w8a8.py:152-155 transposes at load time) is transposed back once.
+    """
+    if weight.dim() != 2 or weight.dtype != torch.int8:
+        raise RuntimeError(f"int8 weight must be a 2-D int8 tensor, got {weight.dtype} {tuple(weight.shape)}")
+    if weight.stride(0) == 1 and weight.stride(1) >= weight.shape[0] and weight.stride(1) % 16 == 0:
+        return weight, weight.stride(1)
+    wt = _converted(weight, lambda t: t.t().contiguous())
+    return wt, wt.stride(0)
+
+
+def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
+    rt.require_gpu(out, x, weight, x_scale, w_scale, bias)
+    if x.numel() == 0:
+        return
+    if x.dtype != torch.int8:
+        raise RuntimeError(f"scaled int8 matmul needs int8 activations, got {x.dtype}")
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or x2.stride(0) % 16 != 0:
+        x2 = x2.contiguous()
+    M, K = x2.shape
+    if weight.shape[0] != K:
+        raise RuntimeError(f"weight is {tuple(weight.shape)} but activations have K={K}")
+    N = weight.shape[1]
+    w, ldw = _int8_weight_nk(weight)
+    out2 = out.reshape(-1, N)
+    if out2.data_ptr() != out.data_ptr() or out2.stride(-1) != 1:
+        raise RuntimeError("output must be a dense [.., N] tensor")
+    xs = ws = None
+    xs_row = ws_col = 0
+    if x_scale is not None:
+        xs = x_scale.to(torch.float32).reshape(-1).contiguous()
+        xs_row = int(xs.numel() > 1)
+        if xs_row and xs.numel() != M:
+            raise RuntimeError(f"x_scale has {xs.numel()} entries for M={M}")
+    if w_scale is not None:
+        ws = w_scale.to(torch.float32).reshape(-1).contiguous()
+        ws_col = int(ws.numel() > 1)
+        if ws_col and ws.numel() != N:
+            raise RuntimeError(f"w_scale has {ws.numel()} entries for N={N}")
+    bias_f32 = 0
+    if bias is not None:
+        bias_f32 = int(bias.dtype == torch.float32)
+        if not bias_f32 and bias.dtype != out.dtype:
+            bias = bias.to(torch.float32)
+            bias_f32 = 1
+        bias = bias.contiguous()
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_w8a8_int8_gemm", out2.data_ptr(), rt.ptr(acc_out), x2.data_ptr(), w.data_ptr(),
+                  rt.ptr(xs), xs_row, rt.ptr(ws), ws_col, rt.ptr(bias), bias_f32, M, N, K,
+                  x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.stream_ptr())
+
+
+def _cutlass_scaled_mm_impl(out, x, weight, x_scale, w_scale, bias):
+    _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias)
+
+
+def _dot_bias_quant_impl(out, lhs, rhs, scale, bias):
+    # single scale[N]: the activation scale is pre-folded (w8a8.py:157-171);
+    # bias is promoted to fp32 (dot_bias_quant.cpp:19-21)
+    _scaled_int8_mm(out, lhs, rhs, None, scale, None if bias is None else bias.to(torch.float32))
+
+
+def _dynamic_scaled_int8_quant_impl(output, input, scales, azp):
+    rt.require_gpu(output, input, scales)
+    if azp is not None:
+        raise RuntimeError("dynamic_scaled_int8_quant: asymmetric quantisation (azp) is not supported")
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    K = x.shape[-1]
+    M = x.numel() // K
+    if not output.is_contiguous() or not scales.is_contiguous() or scales.dtype != torch.float32:
+        raise RuntimeError("dynamic_scaled_int8_quant: output and fp32 scales must be contiguous")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_dynamic_int8_quant", output.data_ptr(), scales.data_ptr(), x.data_ptr(), M, K,
+                  rt.dtype_code(x.dtype), 0, rt.stream_ptr())
+
+
+def _static_scaled_int8_quant_impl(result, input, scale, azp):
+    rt.require_gpu(result, input, scale)
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    K = x.shape[-1]
+    M = x.numel() // K
+    sc = scale.to(torch.float32).reshape(-1).contiguous()
+    if sc.numel() not in (1, K):
+        raise RuntimeError(f"static_scaled_int8_quant: scale must have 1 or K={K} entries, got {sc.numel()}")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_static_int8_quant", result.data_ptr(), x.data_ptr(), sc.data_ptr(),
+                  int(sc.numel() > 1), M, K, rt.dtype_code(x.dtype), rt.stream_ptr())
+
+
+_register("_C", "cutlass_scaled_mm",
+          "(Tensor! out, Tensor x, Tensor weight, Tensor x_scale, Tensor w_scale, Tensor? bias) -> ()",
+          _cutlass_scaled_mm_impl, tags=(torch.Tag.flexible_layout,))
+_register("_C", "dot_bias_quant", "(Tensor! out, Tensor lhs, Tensor rhs, Tensor scale, Tensor? bias) -> ()",
+          _dot_bias_quant_impl)
+# `azp` is a plain Tensor in the reference's schema and Python passes None for
+# it (modular_experts.py:246); when this module owns the schema it is optional
+_register("_C", "dynamic_scaled_int8_quant",
+          "(Tensor! output, Tensor input, Tensor! scales, Tensor? azp) -> ()", _dynamic_scaled_int8_quant_impl)
+_register("_C", "static_scaled_int8_quant",
+          "(Tensor! result, Tensor input, Tensor scale, Tensor? azp) -> ()", _static_scaled_int8_quant_impl)
+
+
+def scaled_int8_quant(input: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                      azp: Optional[torch.Tensor] = None, symmetric: bool = True):
+    """vLLM's ``ops.scaled_int8_quant`` as the reference calls it (w8a8.py:164;
+    patch/patch_0_9_2/utils.py:13-15): static when ``scale`` is given, else
+    dynamic per token.  Returns ``(q int8, scales f32 [.., 1], azp None)``."""
+    output = torch.empty_like(input, dtype=torch.int8)
+    if scale is not None:
+        torch.ops._C.static_scaled_int8_quant(output, input, scale, azp)
+        return output, scale, azp
+    scales = torch.empty((input.numel() // input.shape[-1], 1), device=input.device, dtype=torch.float32)
+    torch.ops._C.dynamic_scaled_int8_quant(output, input.contiguous(), scales, None)
+    return output, scales, None
+
+
+def cutlass_scaled_mm(a: torch.Tensor, b: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
+                      out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """vLLM's ``ops.cutlass_scaled_mm`` (compressed_tensor.py:32-36): allocates
+    ``out [M, N]`` and calls the operator."""
+    out = torch.empty((a.shape[0], b.shape[1]), dtype=out_dtype, device=a.device)
+    torch.ops._C.cutlass_scaled_mm(out, a, b, scale_a, scale_b, bias)
+    return out
+
+
+def dot_bias_quant(out: torch.Tensor, lhs: torch.Tensor, rhs: torch.Tensor, scale: torch.Tensor,
+                   bias: Optional[torch.Tensor] = None) -> None:
+    torch.ops._C.dot_bias_quant(out, lhs, rhs, scale, bias)
+
+
+def int8_gemm_accumulators(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """Raw int32 accumulators of the int8 GEMM (parity/debug helper)."""
+    acc = torch.empty((x.shape[0], weight.shape[1]), dtype=torch.int32, device=x.device)
+    out = torch.empty((x.shape[0], weight.shape[1]), dtype=torch.float32, device=x.device)
+    _scaled_int8_mm(out, x, weight, None, None, None, acc_out=acc)
+    return acc
