@@ -115,6 +115,61 @@ int mi355q_dynamic_int8_quant(int8_t* out, float* scales, const void* x, int M, 
 int mi355q_static_int8_quant(int8_t* out, const void* x, const float* scale, int per_channel, int M,
                              int K, int dtype, void* stream);
 
+/* ---- MoE routing ------------------------------------------------------------
+ * Replaces topsvllm's topk_softmax (csrc/src/topk_softmax.cpp:27-34):
+ * softmax over E experts in fp32, top-k descending (ties to the lower index);
+ * token_expert_indices[row, k] = k * M + row (may be NULL).  `renormalize`
+ * divides by the row sum (done in Python by the reference's caller).  gating
+ * is [M, E] of `dtype` (f16 / bf16 / f32).  E <= 1024, topk <= 64. */
+int mi355q_topk_softmax(float* topk_weights, int32_t* topk_ids, int32_t* token_expert_indices,
+                        const void* gating, int M, int E, int topk, int renormalize, int dtype,
+                        void* stream);
+/* Replaces topsvllmGroupedTopk, both overloads (csrc/src/fused_grouped_topk.cpp:22-44):
+ * scores = softmax | sigmoid; with `bias` selection uses scores + bias and a
+ * group's score is the sum of its two best; without it the group's max; the
+ * `topk_group` best groups are kept, top-k taken among them, weights come from
+ * the un-biased scores.  bias may be NULL. */
+int mi355q_grouped_topk(float* topk_weights, int32_t* topk_ids, const void* gating, const float* bias,
+                        int M, int E, int topk, int renormalize, int num_expert_group, int topk_group,
+                        int scoring_sigmoid, int dtype, void* stream);
+/* Replaces the vendor kernel behind moe_align_block_size, moe_align_block_size_pad,
+ * sgl_moe_align_block_size and exts_moe_align_block_size
+ * (csrc/src/moe_align_block_size.cpp:30-105, moe_align_block_size_pad.cpp:30-110,
+ * exts_moe_align_block_size.cpp:16-101): stable counting sort of the flat
+ * (token, slot) ids by expert, runs padded to block_size.  sorted_token_ids has
+ * numel + E*(block_size-1) entries (pads = numel), expert_ids one entry per
+ * block, num_tokens_post_pad one int.  valid_rows (device int32[1], optional):
+ * only that many rows of topk_ids are valid.  expert_map (device int32[E],
+ * optional) is applied to expert_ids. */
+int mi355q_moe_align_block_size(const void* topk_ids, int ids_are_int64, int numel, int topk,
+                                const int32_t* valid_rows, int num_experts, int block_size,
+                                const int32_t* expert_map, int32_t* sorted_token_ids,
+                                int32_t* expert_ids, int32_t* num_tokens_post_pad, void* stream);
+
+/* ---- activation glue --------------------------------------------------------
+ * silu_and_mul / silu_and_mul_pad (csrc/src/silu_and_mul.cpp:29-109,
+ * silu_and_mul_pad.cpp:27-90): out[r, :d] = silu(x[r, :d]) * x[r, d:2d]. */
+int mi355q_silu_and_mul(void* out, const void* x, long rows, int d, int dtype,
+                        const int32_t* valid_rows, void* stream);
+/* dynamic_per_token_group_fp8_quant(_with_size) and, with fuse_silu_mul,
+ * silu_mul_per_token_group_quant(_with_size)
+ * (csrc/src/dynamic_per_token_group_fp8_quant.cpp:15-84,
+ * silu_mul_per_token_group_quant_with_size.cpp:15-89): per (row, group)
+ * s = max(absmax, 1e-10) / 448, q = e4m3fn(clamp(x / s)).  x is [rows, K]
+ * (or [rows, 2K] when fused); scales [rows, K / group_size] row-major. */
+int mi355q_fp8_group_quant(uint8_t* out, float* scales, const void* x, long rows, int K, int group_size,
+                           int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream);
+/* dynamic_per_token_scaled_fp8_quant (csrc/src/dynamic_per_token_scaled_fp8_quant.cpp): one scale per row */
+int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x, int rows, int K, int dtype,
+                           const int32_t* valid_rows, void* stream);
+/* static_scaled_fp8_quant and silu_mul_static_fp8_quant (csrc/torch_bindings.cpp:291, 714):
+ * q = e4m3fn(clamp(x / scale)) with one fp32 scale */
+int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, long rows, int K,
+                            int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream);
+/* moe_sum_pad (csrc/src/moe_sum.cpp:64-131): out[m, :] = sum_t in[m, t, :], fp32 accumulate */
+int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in_dtype, int out_dtype,
+                   const int32_t* valid_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

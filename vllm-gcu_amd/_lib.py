@@ -32,6 +32,17 @@ SIGNATURES = {
                                       c_void_p]),
     "mi355q_dynamic_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "mi355q_topk_softmax": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "mi355q_grouped_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_int, c_void_p]),
+    "mi355q_moe_align_block_size": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_void_p]),
+    "mi355q_silu_and_mul": (c_int, [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_fp8_group_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p,
+                                       c_void_p]),
+    "mi355q_fp8_token_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_fp8_static_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_moe_sum": (c_int, [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
 }
 
 _lib = None

@@ -1,0 +1,306 @@
+// Elementwise glue between the GEMMs: SiLU-gate, fp8-e4m3fn activation
+// quantisers (per token group, per token, static), the fused SiLU-gate + group
+// quantiser, and the top-k sum.  All are HBM-bound: 16-byte loads per lane,
+// fp32 arithmetic, one pass over the data.  Every kernel takes an optional
+// device int32 `valid_rows` so padded (graph-captured) batches skip dead rows
+// without a host synchronisation.
+#include "common.h"
+
+namespace mi355q {
+namespace {
+
+constexpr float FP8_MAX = 448.0f;
+
+template <int DT> struct E16 { typedef Elem<DT> T; };
+
+template <int DT>
+__device__ __forceinline__ void unpack8(const u4& v, float* f) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = Elem<DT>::to_f32((uint16_t)(v[i] & 0xffffu));
+    f[2 * i + 1] = Elem<DT>::to_f32((uint16_t)(v[i] >> 16));
+  }
+}
+template <int DT>
+__device__ __forceinline__ u4 pack8(const float* f) {
+  u4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    v[i] = (uint32_t)Elem<DT>::from_f32(f[2 * i]) | ((uint32_t)Elem<DT>::from_f32(f[2 * i + 1]) << 16);
+  return v;
+}
+template <int DT>
+__device__ __forceinline__ float round_act(float f) {
+  return Elem<DT>::to_f32(Elem<DT>::from_f32(f));
+}
+
+__device__ __forceinline__ float silu_mul(float a, float b) {
+  return a * (1.0f / (1.0f + expf(-a))) * b;      // left * sigmoid(left) * right
+}
+
+// 8 floats (already within +-448) -> 8 e4m3fn codes, round to nearest even
+__device__ __forceinline__ u2 to_fp8x8(const float* y) {
+  u2 r;
+  int w0 = 0, w1 = 0;
+  w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], w0, false);
+  w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+  w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], w1, false);
+  w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+  r.x = (uint32_t)w0;
+  r.y = (uint32_t)w1;
+  return r;
+}
+
+__device__ __forceinline__ float clamp448(float y) { return fminf(fmaxf(y, -FP8_MAX), FP8_MAX); }
+
+// ---- silu_and_mul: out[r, :d] = silu(x[r, :d]) * x[r, d:] -------------------
+template <int DT>
+__global__ void __launch_bounds__(256)
+silu_and_mul_kernel(uint16_t* out, const uint16_t* x, long rows, int d, const int* valid_rows) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+  const int chunks = d / 8;
+  const long total = nrow * chunks;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long r = i / chunks;
+    const int c = (int)(i - r * chunks);
+    float a[8], b[8], y[8];
+    unpack8<DT>(*(const u4*)(x + r * 2 * d + 8 * c), a);
+    unpack8<DT>(*(const u4*)(x + r * 2 * d + d + 8 * c), b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = silu_mul(a[e], b[e]);
+    *(u4*)(out + r * d + 8 * c) = pack8<DT>(y);
+  }
+}
+
+// ---- per-token-group fp8 quantisation (optionally fused behind SiLU-gate) ---
+// A group of `gs` elements is handled by gs/8 adjacent lanes (gs in 64,128,256,512).
+template <int DT, bool SILU>
+__global__ void __launch_bounds__(256)
+group_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, long rows, int K, int gs,
+                       const int* valid_rows) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+  const int chunks = K / 8;                      // 8-element chunks per output row
+  const int lpg = gs / 8;                        // lanes per group (power of two <= 64)
+  const long total = nrow * chunks;
+  const long stride = (long)gridDim.x * 256;
+  for (long i0 = (long)blockIdx.x * 256; i0 < total; i0 += stride) {
+    const long i = i0 + threadIdx.x;
+    const bool live = i < total;
+    const long r = live ? i / chunks : 0;
+    const int c = live ? (int)(i - r * chunks) : 0;
+    float y[8];
+    if (SILU) {
+      float a[8], b[8];
+      unpack8<DT>(*(const u4*)(x + r * 2 * K + 8 * c), a);
+      unpack8<DT>(*(const u4*)(x + r * 2 * K + K + 8 * c), b);
+      // the unfused sequence stores the gate output in the activation dtype
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = round_act<DT>(silu_mul(a[e], b[e]));
+    } else {
+      unpack8<DT>(*(const u4*)(x + r * K + 8 * c), y);
+    }
+    float mx = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(y[e]));
+    if (!live) mx = 0.f;
+    for (int o = 1; o < lpg; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    const float s = fmaxf(mx, 1e-10f) / FP8_MAX;
+    float q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q[e] = clamp448(y[e] / s);
+    if (live) {
+      *(u2*)(out + r * K + 8 * c) = to_fp8x8(q);
+      if ((c % lpg) == 0) scales[r * (K / gs) + c / lpg] = s;
+    }
+  }
+}
+
+// ---- per-token fp8 (one workgroup per row) and static fp8 --------------------
+template <int DT>
+__global__ void __launch_bounds__(256)
+token_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, int K, const int* valid_rows) {
+  const long row = blockIdx.x;
+  if (valid_rows && row >= *valid_rows) return;
+  __shared__ float red[4];
+  float mx = 0.f;
+  for (int k = threadIdx.x; k < K; k += 256) mx = fmaxf(mx, fabsf(Elem<DT>::to_f32(x[row * K + k])));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float s = fmaxf(mx, 1e-10f) / FP8_MAX;
+  if (threadIdx.x == 0) scales[row] = s;
+  for (int k = threadIdx.x; k < K; k += 256) {
+    const float y = clamp448(Elem<DT>::to_f32(x[row * K + k]) / s);
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
+    out[row * K + k] = (uint8_t)(w & 0xff);
+  }
+}
+
+template <int DT, bool SILU>
+__global__ void __launch_bounds__(256)
+static_fp8_quant_kernel(uint8_t* out, const uint16_t* x, const float* scale, long rows, int K,
+                        const int* valid_rows) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+  const long total = nrow * K;
+  const float s = *scale;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    float v;
+    if (SILU) {
+      const long r = i / K;
+      const int c = (int)(i - r * K);
+      v = round_act<DT>(silu_mul(Elem<DT>::to_f32(x[r * 2 * K + c]), Elem<DT>::to_f32(x[r * 2 * K + K + c])));
+    } else {
+      v = Elem<DT>::to_f32(x[i]);
+    }
+    const float y = clamp448(v / s);
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
+    out[i] = (uint8_t)(w & 0xff);
+  }
+}
+
+// ---- moe_sum: out[m, :] = sum_t in[m, t, :] in fp32 --------------------------
+template <int DT_IN, int DT_OUT>
+__global__ void __launch_bounds__(256)
+moe_sum_kernel(void* out, const uint16_t* in, long rows, int T, int K, const int* valid_rows) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+  const int chunks = K / 8;
+  const long total = nrow * chunks;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long r = i / chunks;
+    const int c = (int)(i - r * chunks);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < T; ++t) {
+      float v[8];
+      unpack8<DT_IN>(*(const u4*)(in + (r * T + t) * K + 8 * c), v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += v[e];
+    }
+    if (DT_OUT == MI355Q_F32) {
+      float* o = (float*)out + r * K + 8 * c;
+      *(f4*)o = (f4){acc[0], acc[1], acc[2], acc[3]};
+      *(f4*)(o + 4) = (f4){acc[4], acc[5], acc[6], acc[7]};
+    } else {
+      *(u4*)((uint16_t*)out + r * K + 8 * c) = pack8<DT_OUT == MI355Q_F32 ? MI355Q_F16 : DT_OUT>(acc);
+    }
+  }
+}
+
+inline unsigned grid_for(long items) {
+  long b = (items + 255) / 256;
+  long cap = (long)device_cu_count() * 16;
+  return (unsigned)(b < 1 ? 1 : (b > cap ? cap : b));
+}
+
+}  // namespace
+}  // namespace mi355q
+
+using namespace mi355q;
+
+#define MQ_DISPATCH_16(dtype, CALL_F16, CALL_BF16, what)             \
+  do {                                                               \
+    if ((dtype) == MI355Q_F16) { CALL_F16; }                         \
+    else if ((dtype) == MI355Q_BF16) { CALL_BF16; }                  \
+    else MQ_REQUIRE(false, what ": dtype %d must be f16 or bf16", (int)(dtype)); \
+  } while (0)
+
+extern "C" int mi355q_silu_and_mul(void* out, const void* x, long rows, int d, int dtype,
+                                   const int32_t* valid_rows, void* stream) {
+  MQ_REQUIRE(rows >= 0 && d > 0 && d % 8 == 0, "silu_and_mul: bad shape rows=%ld d=%d (d %% 8 == 0)", rows, d);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && x, "silu_and_mul: null pointer");
+  hipStream_t st = as_stream(stream);
+  unsigned g = grid_for(rows * (d / 8));
+  MQ_DISPATCH_16(dtype,
+    hipLaunchKernelGGL((silu_and_mul_kernel<MI355Q_F16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint16_t*)x, rows, d, valid_rows),
+    hipLaunchKernelGGL((silu_and_mul_kernel<MI355Q_BF16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint16_t*)x, rows, d, valid_rows),
+    "silu_and_mul");
+  MQ_LAUNCH_CHECK("silu_and_mul");
+  return 0;
+}
+
+extern "C" int mi355q_fp8_group_quant(uint8_t* out, float* scales, const void* x, long rows, int K,
+                                      int group_size, int fuse_silu_mul, int dtype,
+                                      const int32_t* valid_rows, void* stream) {
+  MQ_REQUIRE(rows >= 0 && K > 0, "fp8_group_quant: bad shape rows=%ld K=%d", rows, K);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && scales && x, "fp8_group_quant: null pointer");
+  MQ_REQUIRE(group_size == 64 || group_size == 128 || group_size == 256 || group_size == 512,
+             "fp8_group_quant: group_size=%d must be 64, 128, 256 or 512", group_size);
+  MQ_REQUIRE(K % group_size == 0, "fp8_group_quant: K=%d must be a multiple of group_size=%d", K, group_size);
+  hipStream_t st = as_stream(stream);
+  // whole groups must sit inside one workgroup pass: 256 lanes cover 2048 elements
+  unsigned g = grid_for(rows * (K / 8));
+  if (fuse_silu_mul) {
+    MQ_DISPATCH_16(dtype,
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_F16, true>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_BF16, true>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
+      "fp8_group_quant");
+  } else {
+    MQ_DISPATCH_16(dtype,
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_F16, false>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_BF16, false>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
+      "fp8_group_quant");
+  }
+  MQ_LAUNCH_CHECK("fp8_group_quant");
+  return 0;
+}
+
+extern "C" int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x, int rows, int K, int dtype,
+                                      const int32_t* valid_rows, void* stream) {
+  MQ_REQUIRE(rows >= 0 && K > 0, "fp8_token_quant: bad shape rows=%d K=%d", rows, K);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && scales && x, "fp8_token_quant: null pointer");
+  hipStream_t st = as_stream(stream);
+  MQ_DISPATCH_16(dtype,
+    hipLaunchKernelGGL((token_fp8_quant_kernel<MI355Q_F16>), dim3(rows), dim3(256), 0, st, out, scales, (const uint16_t*)x, K, valid_rows),
+    hipLaunchKernelGGL((token_fp8_quant_kernel<MI355Q_BF16>), dim3(rows), dim3(256), 0, st, out, scales, (const uint16_t*)x, K, valid_rows),
+    "fp8_token_quant");
+  MQ_LAUNCH_CHECK("fp8_token_quant");
+  return 0;
+}
+
+extern "C" int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, long rows, int K,
+                                       int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream) {
+  MQ_REQUIRE(rows >= 0 && K > 0, "fp8_static_quant: bad shape rows=%ld K=%d", rows, K);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && scale && x, "fp8_static_quant: null pointer");
+  hipStream_t st = as_stream(stream);
+  unsigned g = grid_for(rows * K);
+  if (fuse_silu_mul) {
+    MQ_DISPATCH_16(dtype,
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, true>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, true>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      "fp8_static_quant");
+  } else {
+    MQ_DISPATCH_16(dtype,
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, false>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, false>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      "fp8_static_quant");
+  }
+  MQ_LAUNCH_CHECK("fp8_static_quant");
+  return 0;
+}
+
+extern "C" int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in_dtype,
+                              int out_dtype, const int32_t* valid_rows, void* stream) {
+  MQ_REQUIRE(rows >= 0 && topk > 0 && K > 0 && K % 8 == 0, "moe_sum: bad shape rows=%ld topk=%d K=%d (K %% 8 == 0)", rows, topk, K);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && in, "moe_sum: null pointer");
+  MQ_REQUIRE(in_dtype == MI355Q_F16 || in_dtype == MI355Q_BF16, "moe_sum: input dtype %d must be f16 or bf16", in_dtype);
+  MQ_REQUIRE(out_dtype == in_dtype || out_dtype == MI355Q_F32, "moe_sum: output dtype %d must equal the input's or be f32", out_dtype);
+  hipStream_t st = as_stream(stream);
+  unsigned g = grid_for(rows * (K / 8));
+  const uint16_t* p = (const uint16_t*)in;
+  if (in_dtype == MI355Q_F16 && out_dtype == MI355Q_F16)
+    hipLaunchKernelGGL((moe_sum_kernel<MI355Q_F16, MI355Q_F16>), dim3(g), dim3(256), 0, st, out, p, rows, topk, K, valid_rows);
+  else if (in_dtype == MI355Q_F16)
+    hipLaunchKernelGGL((moe_sum_kernel<MI355Q_F16, MI355Q_F32>), dim3(g), dim3(256), 0, st, out, p, rows, topk, K, valid_rows);
+  else if (out_dtype == MI355Q_BF16)
+    hipLaunchKernelGGL((moe_sum_kernel<MI355Q_BF16, MI355Q_BF16>), dim3(g), dim3(256), 0, st, out, p, rows, topk, K, valid_rows);
+  else
+    hipLaunchKernelGGL((moe_sum_kernel<MI355Q_BF16, MI355Q_F32>), dim3(g), dim3(256), 0, st, out, p, rows, topk, K, valid_rows);
+  MQ_LAUNCH_CHECK("moe_sum");
+  return 0;
+}

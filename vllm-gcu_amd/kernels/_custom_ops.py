@@ -332,3 +332,339 @@ def int8_gemm_accumulators(x: torch.Tensor, weight: torch.Tensor) -> torch.Tenso
     out = torch.empty((x.shape[0], weight.shape[1]), dtype=torch.float32, device=x.device)
     _scaled_int8_mm(out, x, weight, None, None, None, acc_out=acc)
     return acc
+
+
+# ---------------------------------------------------------------------------
+# MoE routing / align (csrc/torch_bindings.cpp:803-809, 1052-1063, 1178-1189,
+# 1390-1431)
+# ---------------------------------------------------------------------------
+def _topk_softmax_impl(topk_weights, topk_indices, token_expert_indices, gating_output):
+    rt.require_gpu(topk_weights, topk_indices, token_expert_indices, gating_output)
+    if gating_output.numel() == 0:
+        return
+    g = gating_output.contiguous()
+    M, E = g.shape
+    k = topk_weights.shape[-1]
+    if topk_weights.dtype != torch.float32 or topk_indices.dtype != torch.int32:
+        raise RuntimeError("topk_softmax: topk_weights must be float32 and topk_indices int32")
+    if not (topk_weights.is_contiguous() and topk_indices.is_contiguous()):
+        raise RuntimeError("topk_softmax: outputs must be contiguous")
+    tei = token_expert_indices
+    if tei is not None and (tei.dtype != torch.int32 or not tei.is_contiguous()):
+        raise RuntimeError("topk_softmax: token_expert_indices must be contiguous int32")
+    with torch.cuda.device(g.device):
+        _lib.call("mi355q_topk_softmax", topk_weights.data_ptr(), topk_indices.data_ptr(), rt.ptr(tei),
+                  g.data_ptr(), M, E, k, 0, rt.dtype_code(g.dtype), rt.stream_ptr())
+
+
+def _fused_grouped_topk_impl(topk_weights, topk_ids, gating_output, topk, renormalize, num_expert_group,
+                             topk_group, e_score_correction_bias, scoring_func):
+    rt.require_gpu(topk_weights, topk_ids, gating_output, e_score_correction_bias)
+    if gating_output.numel() == 0:
+        return
+    if scoring_func not in ("softmax", "sigmoid"):
+        raise RuntimeError(f"fused_grouped_topk: unsupported scoring function {scoring_func!r}")
+    g = gating_output.contiguous()
+    M, E = g.shape
+    bias = e_score_correction_bias
+    if bias is not None:
+        bias = bias.to(torch.float32).contiguous()
+    if topk_weights.dtype != torch.float32 or topk_ids.dtype != torch.int32:
+        raise RuntimeError("fused_grouped_topk: topk_weights must be float32 and topk_ids int32")
+    with torch.cuda.device(g.device):
+        _lib.call("mi355q_grouped_topk", topk_weights.data_ptr(), topk_ids.data_ptr(), g.data_ptr(),
+                  rt.ptr(bias), M, E, int(topk), int(bool(renormalize)), int(num_expert_group),
+                  int(topk_group), int(scoring_func == "sigmoid"), rt.dtype_code(g.dtype), rt.stream_ptr())
+
+
+def _align(topk_ids, valid_rows, num_experts, block_size, expert_map, sorted_token_ids, experts_ids,
+           num_tokens_post_pad):
+    rt.require_gpu(topk_ids, valid_rows, expert_map, sorted_token_ids, experts_ids, num_tokens_post_pad)
+    ids = topk_ids.contiguous()
+    if ids.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError(f"moe_align_block_size: topk_ids must be int32 or int64, got {ids.dtype}")
+    numel = ids.numel()
+    top = ids.shape[-1] if ids.dim() > 1 else 1
+    cap = numel + num_experts * (block_size - 1)
+    if sorted_token_ids.numel() < cap or experts_ids.numel() < cap // block_size:
+        raise RuntimeError("moe_align_block_size: output buffers are smaller than "
+                           "numel + num_experts * (block_size - 1)")
+    for t in (sorted_token_ids, experts_ids, num_tokens_post_pad):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("moe_align_block_size: outputs must be contiguous int32")
+    if valid_rows is not None and valid_rows.dtype != torch.int32:
+        valid_rows = valid_rows.to(torch.int32)
+    if expert_map is not None:
+        expert_map = expert_map.to(torch.int32).contiguous()
+    with torch.cuda.device(ids.device):
+        _lib.call("mi355q_moe_align_block_size", ids.data_ptr(), int(ids.dtype == torch.int64), numel, top,
+                  rt.ptr(valid_rows), int(num_experts), int(block_size), rt.ptr(expert_map),
+                  sorted_token_ids.data_ptr(), experts_ids.data_ptr(), num_tokens_post_pad.data_ptr(),
+                  rt.stream_ptr())
+
+
+def _moe_align_block_size_impl(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                               num_tokens_post_pad):
+    _align(topk_ids, None, num_experts, block_size, None, sorted_token_ids, experts_ids, num_tokens_post_pad)
+
+
+def _moe_align_block_size_pad_impl(topk_ids, topk_ids_size, num_experts, block_size, sorted_token_ids,
+                                   experts_ids, num_tokens_post_pad):
+    _align(topk_ids, topk_ids_size, num_experts, block_size, None, sorted_token_ids, experts_ids,
+           num_tokens_post_pad)
+
+
+def _exts_moe_align_block_size_impl(sorted_token_ids, experts_ids, num_tokens_post_pad, topk_ids,
+                                    real_token_num, expert_map, num_experts, block_size):
+    _align(topk_ids, real_token_num, num_experts, block_size, expert_map, sorted_token_ids, experts_ids,
+           num_tokens_post_pad)
+
+
+_register("_moe_C", "topk_softmax",
+          "(Tensor! topk_weights, Tensor! topk_indices, Tensor! token_expert_indices, Tensor gating_output) -> ()",
+          _topk_softmax_impl)
+# e_score_correction_bias is a plain Tensor in the reference and Python passes
+# None (fused_moe.py:256-266); optional where this module owns the schema
+_register("_C", "fused_grouped_topk",
+          "(Tensor! topk_weights, Tensor! topk_ids, Tensor gating_output, SymInt topk, bool renormalize, "
+          "SymInt num_expert_group, SymInt topk_group, Tensor? e_score_correction_bias, str scoring_func) -> ()",
+          _fused_grouped_topk_impl)
+_register("_moe_C", "moe_align_block_size",
+          "(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, Tensor! experts_ids, "
+          "Tensor! num_tokens_post_pad) -> ()", _moe_align_block_size_impl)
+_register("_moe_C", "sgl_moe_align_block_size",
+          "(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, Tensor! experts_ids, "
+          "Tensor! num_tokens_post_pad) -> ()", _moe_align_block_size_impl)
+# registered from a C++ function pointer in the reference, hence positional-only
+# callers (torch_bindings.cpp:803-809, moe_align_block_size_pad.cpp:43-47)
+_register("_C", "moe_align_block_size_pad",
+          "(Tensor topk_ids, Tensor topk_ids_size, int num_experts, int block_size, Tensor! sorted_token_ids, "
+          "Tensor! experts_ids, Tensor! num_tokens_post_pad) -> ()", _moe_align_block_size_pad_impl)
+_register("_C", "exts_moe_align_block_size",
+          "(Tensor(a!) sorted_token_ids, Tensor(a!) experts_ids, Tensor(a!) num_tokens_post_pad, Tensor topk_ids, "
+          "Tensor real_token_num, Tensor expert_map, int num_experts, int block_size) -> ()",
+          _exts_moe_align_block_size_impl)
+
+
+def topk_softmax(topk_weights, topk_ids, token_expert_indices, gating_output) -> None:
+    torch.ops._moe_C.topk_softmax(topk_weights, topk_ids, token_expert_indices, gating_output)
+
+
+def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int, renormalize: bool):
+    """vLLM's ``fused_topk`` as used by ``FusedMoE.select_experts``
+    (moe_wna16.py:612-623): softmax -> top-k (descending) -> optional renorm."""
+    M = gating_output.shape[0]
+    topk_weights = torch.empty(M, topk, dtype=torch.float32, device=gating_output.device)
+    topk_ids = torch.empty(M, topk, dtype=torch.int32, device=gating_output.device)
+    token_expert_indices = torch.empty(M, topk, dtype=torch.int32, device=gating_output.device)
+    topk_softmax(topk_weights, topk_ids, token_expert_indices, gating_output.float())
+    if renormalize:
+        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+    return topk_weights, topk_ids
+
+
+# fused moe (vllm_gcu/kernels/_custom_ops.py:490-543)
+def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                         num_tokens_post_pad) -> None:
+    torch.ops._moe_C.moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                                          num_tokens_post_pad)
+
+
+def sgl_moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                             num_tokens_post_pad) -> None:
+    torch.ops._moe_C.sgl_moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids,
+                                              experts_ids, num_tokens_post_pad)
+
+
+def moe_align_block_size_pad(topk_ids, topk_ids_size, num_experts, block_size, sorted_token_ids,
+                             experts_ids, num_tokens_post_pad):
+    torch.ops._C.moe_align_block_size_pad(topk_ids, topk_ids_size, num_experts, block_size,
+                                          sorted_token_ids, experts_ids, num_tokens_post_pad)
+
+
+# ---------------------------------------------------------------------------
+# activation glue (csrc/torch_bindings.cpp:163-175, 291, 714-766, 1083-1153,
+# 1404-1410)
+# ---------------------------------------------------------------------------
+def _rows_last(t: torch.Tensor):
+    return t.numel() // t.shape[-1], t.shape[-1]
+
+
+def _silu_and_mul_common(out, input, size):
+    rt.require_gpu(out, input, size)
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    rows, d2 = _rows_last(x)
+    if not out.is_contiguous() or out.shape[-1] * 2 != d2 or out.dtype != x.dtype:
+        raise RuntimeError("silu_and_mul: out must be contiguous [..., d] of the input dtype for input [..., 2d]")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_silu_and_mul", out.data_ptr(), x.data_ptr(), rows, d2 // 2, rt.dtype_code(x.dtype),
+                  rt.ptr(size), rt.stream_ptr())
+
+
+def _silu_and_mul_impl(result, input):
+    _silu_and_mul_common(result, input, None)
+
+
+def _silu_and_mul_pad_impl(out, input, size):
+    _silu_and_mul_common(out, input, size.to(torch.int32) if size.dtype != torch.int32 else size)
+
+
+def _fp8_out_ok(out, shape):
+    if out.dtype not in (torch.float8_e4m3fn, torch.uint8) or not out.is_contiguous() or tuple(out.shape) != tuple(shape):
+        raise RuntimeError(f"fp8 output must be a contiguous float8_e4m3fn tensor of shape {tuple(shape)}")
+
+
+def _group_quant_common(out, scale, input, real_size, group_size, fuse):
+    rt.require_gpu(out, scale, input, real_size)
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    rows, kin = _rows_last(x)
+    K = kin // 2 if fuse else kin
+    _fp8_out_ok(out, x.shape[:-1] + (K,))
+    if scale.dtype != torch.float32 or not scale.is_contiguous() or scale.numel() != rows * (K // group_size):
+        raise RuntimeError("per-token-group quant: scale must be contiguous float32 [..., K / group_size]")
+    if real_size is not None and real_size.dtype != torch.int32:
+        real_size = real_size.to(torch.int32)
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_fp8_group_quant", out.data_ptr(), scale.data_ptr(), x.data_ptr(), rows, K,
+                  int(group_size), int(fuse), rt.dtype_code(x.dtype), rt.ptr(real_size), rt.stream_ptr())
+
+
+def _dynamic_per_token_group_fp8_quant_impl(out, scale, input, group_size):
+    _group_quant_common(out, scale, input, None, group_size, False)
+
+
+def _dynamic_per_token_group_fp8_quant_with_size_impl(out, scale, input, real_size, group_size):
+    _group_quant_common(out, scale, input, real_size, group_size, False)
+
+
+def _silu_mul_per_token_group_quant_impl(out, scale, input, group_size):
+    _group_quant_common(out, scale, input, None, group_size, True)
+
+
+def _silu_mul_per_token_group_quant_with_size_impl(out, scale, input, size, group_size):
+    # `size` counts rows of the leading dimension; the kernel works on flattened rows
+    x = input
+    lead = x.shape[0]
+    inner = (x.numel() // x.shape[-1]) // max(lead, 1)
+    rows_valid = size.to(torch.int32) * inner if inner != 1 else size
+    _group_quant_common(out, scale, input, rows_valid, group_size, True)
+
+
+def _dynamic_per_token_scaled_fp8_quant_impl(result, input, scale, scale_ub):
+    # scale_ub is ignored, as in the reference (dynamic_per_token_scaled_fp8_quant.cpp:32-34)
+    rt.require_gpu(result, input, scale)
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    rows, K = _rows_last(x)
+    _fp8_out_ok(result, x.shape)
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_fp8_token_quant", result.data_ptr(), scale.data_ptr(), x.data_ptr(), rows, K,
+                  rt.dtype_code(x.dtype), 0, rt.stream_ptr())
+
+
+def _static_fp8_common(out, input, scale, real_rows, fuse):
+    rt.require_gpu(out, input, scale, real_rows)
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    rows, kin = _rows_last(x)
+    K = kin // 2 if fuse else kin
+    _fp8_out_ok(out, x.shape[:-1] + (K,))
+    sc = scale.to(torch.float32).reshape(-1)
+    if sc.numel() != 1:
+        raise RuntimeError("static fp8 quant takes a single scale")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_fp8_static_quant", out.data_ptr(), x.data_ptr(), sc.data_ptr(), rows, K, int(fuse),
+                  rt.dtype_code(x.dtype), rt.ptr(real_rows), rt.stream_ptr())
+
+
+def _static_scaled_fp8_quant_impl(result, input, scale):
+    _static_fp8_common(result, input, scale, None, False)
+
+
+def _silu_mul_static_fp8_quant_impl(out, input, scale, real_num_tokens):
+    lead = input.shape[0]
+    inner = (input.numel() // input.shape[-1]) // max(lead, 1)
+    rows_valid = real_num_tokens.to(torch.int32) * inner if inner != 1 else real_num_tokens.to(torch.int32)
+    _static_fp8_common(out, input, scale, rows_valid, True)
+
+
+def _moe_sum_pad_impl(out, input, size, dim, keepdim):
+    rt.require_gpu(out, input, size)
+    if input.numel() == 0:
+        return
+    if input.dim() != 3 or dim != 1 or keepdim:
+        raise RuntimeError("moe_sum_pad: expects input [M, topk, K], dim=1, keepdim=False")
+    x = input.contiguous()
+    M, T, K = x.shape
+    if not out.is_contiguous() or tuple(out.shape) != (M, K):
+        raise RuntimeError("moe_sum_pad: out must be contiguous [M, K]")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_moe_sum", out.data_ptr(), x.data_ptr(), M, T, K, rt.dtype_code(x.dtype),
+                  rt.dtype_code(out.dtype), rt.ptr(None if size is None else size.to(torch.int32)),
+                  rt.stream_ptr())
+
+
+_register("_C", "silu_and_mul", "(Tensor! result, Tensor input) -> ()", _silu_and_mul_impl)
+_register("_C", "silu_and_mul_pad", "(Tensor(a!) out, Tensor input, Tensor size) -> ()", _silu_and_mul_pad_impl)
+_register("_C", "dynamic_per_token_group_fp8_quant",
+          "(Tensor! out, Tensor! scale, Tensor input, int group_size) -> ()",
+          _dynamic_per_token_group_fp8_quant_impl)
+_register("_C", "dynamic_per_token_group_fp8_quant_with_size",
+          "(Tensor! out, Tensor! scale, Tensor input, Tensor real_size, int group_size) -> ()",
+          _dynamic_per_token_group_fp8_quant_with_size_impl)
+_register("_C", "silu_mul_per_token_group_quant",
+          "(Tensor! out, Tensor! scale, Tensor input, int group_size) -> ()", _silu_mul_per_token_group_quant_impl)
+_register("_C", "silu_mul_per_token_group_quant_with_size",
+          "(Tensor(a!) out, Tensor(a!) scale, Tensor input, Tensor size, int group_size) -> ()",
+          _silu_mul_per_token_group_quant_with_size_impl)
+_register("_C", "dynamic_per_token_scaled_fp8_quant",
+          "(Tensor! result, Tensor input, Tensor! scale, Tensor? scale_ub) -> ()",
+          _dynamic_per_token_scaled_fp8_quant_impl)
+_register("_C", "static_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor scale) -> ()",
+          _static_scaled_fp8_quant_impl)
+_register("_C", "silu_mul_static_fp8_quant",
+          "(Tensor(a!) out, Tensor input, Tensor scale, Tensor real_num_tokens) -> ()",
+          _silu_mul_static_fp8_quant_impl)
+_register("_moe_C", "moe_sum_pad", "(Tensor(a!) out, Tensor input, Tensor size, int dim, bool keepdim) -> ()",
+          _moe_sum_pad_impl)
+
+
+# 8bit (vllm_gcu/kernels/_custom_ops.py:298-317)
+def scaled_fp8_quant(input: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                     num_token_padding: Optional[int] = None, scale_ub: Optional[torch.Tensor] = None,
+                     use_per_token_if_dynamic: bool = False,
+                     output: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    if scale is None:
+        if use_per_token_if_dynamic:
+            output = torch.empty_like(input, dtype=torch.float8_e4m3fn)
+            shape = input.shape[:-1] + (1,)
+            scale = torch.empty(shape, device=input.device, dtype=torch.float32)
+            torch.ops._C.dynamic_per_token_scaled_fp8_quant(output, input, scale, scale_ub)
+        else:
+            raise NotImplementedError("dynamic_scaled_fp8_quant is not implemented for per tensor!")
+    else:
+        if output is None:
+            output = torch.empty_like(input, dtype=torch.float8_e4m3fn)
+        torch.ops._C.static_scaled_fp8_quant(output, input, scale)
+    return output, scale
+
+
+# vllm_gcu/kernels/_custom_ops.py:465-486
+def per_token_group_quant_fp8(x: torch.Tensor, group_size: int, eps: float = 1e-10,
+                              dtype: Optional[torch.dtype] = None, column_major_scales: bool = False,
+                              real_token_num: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    dtype = torch.float8_e4m3fn if dtype is None else dtype
+    x_q = torch.empty_like(x, device=x.device, dtype=dtype)
+    shape = x.shape[:-1] + (x.shape[-1] // group_size,)
+    x_s = torch.empty(shape, device=x.device, dtype=torch.float32)
+    if real_token_num is None:
+        torch.ops._C.dynamic_per_token_group_fp8_quant(x_q, x_s, x, group_size)
+    else:
+        torch.ops._C.dynamic_per_token_group_fp8_quant_with_size(x_q, x_s, x, real_token_num, group_size)
+    return x_q, x_s

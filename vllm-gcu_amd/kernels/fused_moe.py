@@ -1,0 +1,73 @@
+"""MoE host helpers: default tile configuration, token->expert alignment,
+the grouped-GEMM dispatcher and grouped top-k routing.
+
+Mirrors vllm_gcu/kernels/fused_moe.py (get_default_config :19-37,
+moe_align_block_size :40-108, invoke_fused_moe_kernel :111-231, grouped_topk
+:234-267) with the same names, arguments and operator calls.
+"""
+from typing import Any, Dict, List, Optional, Tuple
+
+import torch
+
+from . import _custom_ops as ops
+
+
+def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optional[str], is_marlin: bool,
+                       block_shape: Optional[List[int]] = None) -> Dict[str, int]:
+    """Only BLOCK_SIZE_M is consumed (as the align/GEMM block size).  The
+    reference hard-codes 64 for its hardware (fused_moe.py:29-36); on MI355X the
+    grouped GEMM runs 16-row MFMA tiles, so the block follows the expected rows
+    per expert: 16 for decode-sized batches up to 128 for prefill."""
+    per_expert = (M * topk) / max(E, 1)
+    if per_expert <= 16:
+        bm = 16
+    elif per_expert <= 32:
+        bm = 32
+    elif per_expert <= 96:
+        bm = 64
+    else:
+        bm = 128
+    return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int,
+                         expert_map: torch.Tensor = None,
+                         topk_ids_size=None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    max_num_tokens_padded = topk_ids.numel() + num_experts * (block_size - 1)
+    sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=topk_ids.device)
+    max_num_m_blocks = max_num_tokens_padded // block_size
+    expert_ids = torch.empty((max_num_m_blocks,), dtype=torch.int32, device=topk_ids.device)
+    num_tokens_post_pad = torch.empty((1), dtype=torch.int32, device=topk_ids.device)
+
+    if topk_ids_size is not None:
+        if expert_map is None:
+            ops.moe_align_block_size_pad(topk_ids, topk_ids_size, num_experts, block_size, sorted_ids,
+                                         expert_ids, num_tokens_post_pad)
+        else:
+            # the reference's VLLM_GCU_DEEPSEEK_FUSION path (fused_moe.py:72-82):
+            # the expert map is applied inside the operator
+            torch.ops._C.exts_moe_align_block_size(sorted_ids, expert_ids, num_tokens_post_pad, topk_ids,
+                                                   topk_ids_size, expert_map, num_experts, block_size)
+    else:
+        if num_experts >= 224:
+            ops.sgl_moe_align_block_size(topk_ids, num_experts, block_size, sorted_ids, expert_ids,
+                                         num_tokens_post_pad)
+        else:
+            ops.moe_align_block_size(topk_ids, num_experts, block_size, sorted_ids, expert_ids,
+                                     num_tokens_post_pad)
+        if expert_map is not None:
+            expert_ids = expert_map[expert_ids.long()].to(torch.int32)
+    return sorted_ids, expert_ids, num_tokens_post_pad
+
+
+def grouped_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int, renormalize: bool,
+                 num_expert_group: int = 0, topk_group: int = 0, scoring_func: str = "softmax",
+                 e_score_correction_bias: Optional[torch.Tensor] = None):
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    topk_weights = torch.empty((gating_output.shape[0], topk), device=gating_output.device, dtype=torch.float32)
+    topk_ids = torch.empty((gating_output.shape[0], topk), device=gating_output.device, dtype=torch.int32)
+    if hidden_states.numel() == 0:
+        return topk_weights, topk_ids
+    torch.ops._C.fused_grouped_topk(topk_weights, topk_ids, gating_output, topk, renormalize, num_expert_group,
+                                    topk_group, e_score_correction_bias, scoring_func)
+    return topk_weights, topk_ids
