@@ -170,6 +170,35 @@ int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, lon
 int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in_dtype, int out_dtype,
                    const int32_t* valid_rows, void* stream);
 
+/* ---- fused-MoE grouped GEMM and K-contiguous skinny GEMMs -------------------
+ * quant_mode: 0 = W4A16 (slab-layout int4 per expert [E, K/8, N], scales
+ * [E, K/g, N], zeros per zeros_kind), 1 = fp8-e4m3fn with 128x128 block scales
+ * (w [E, N, K], a_scale f32 [Ma, K/128], w_scale f32 [E, ceil(N/128), K/128]),
+ * 2 = int8 (a_scale f32 [Ma] or NULL, w_scale f32 [E, N]), 3 = unquantised
+ * f16/bf16 (w [E, N, K]), 4 = W8A16 (w int8 [E, N, K], w_scale [E, N] in the
+ * activation dtype).
+ *
+ * mi355q_moe_gemm replaces vllmInvokeFusedMoeNonGatherQuantKernel as called by
+ * fused_moe_quant_kernel / fused_moe_kernel (csrc/src/fused_moe_quant_kernel.cpp:30-200,
+ * fused_moe_kernel.cpp:27-68; shapes csrc/src/native_vllm.h:236-255): for every
+ * block b < num_tokens_post_pad / block_size with e = expert_ids[b] and every
+ * id t < numel in the block,  out[t, :] = a[t / topk, :] @ W[e]^T  (times
+ * topk_weights[t] when that pointer is given).  max_blocks = entries of
+ * expert_ids.  block_size in {16, 32, 64, 128}. */
+int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scale, const void* w_scale,
+                    const void* w_zeros, int zeros_kind, int quant_mode, int group_size,
+                    const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                    const int32_t* num_tokens_post_pad, int numel, int topk, int block_size,
+                    int max_blocks, int E, int K, int N, int act_dtype, int out_dtype, void* stream);
+/* Dense calls of the same kernels (quant_mode 1..4), replacing topsatenLinearQuant
+ * as called by linear_quant (csrc/src/linear_quant.cpp:16-95, fp8 block-scaled
+ * C = sum_kb (A_kb B_kb^T) As Bs) and by weight_only_quant
+ * (csrc/src/weight_only_quant.cpp:28-101, W8A16).  w is [N, K]; bias [N] in
+ * the output dtype or NULL. */
+int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_scale,
+                        const void* w_scale, const void* bias, int quant_mode, int group_size, int M,
+                        int K, int N, int act_dtype, int out_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

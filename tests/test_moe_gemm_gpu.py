@@ -1,0 +1,290 @@
+"""GPU parity of the fused-MoE grouped GEMMs and of the whole fused-experts
+sequence against the CPU oracle (naive per-(token, slot) loop over dense
+dequantised experts).  fp16/bf16 outputs within rtol 1e-2 / atol 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8 as of8
+from oracle import moe as om
+from oracle import w4 as ow4
+from oracle import w8a8 as o8
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from vllm_gcu_amd.kernels import _custom_ops
+    return _custom_ops
+
+
+@pytest.fixture(scope="module")
+def fmoe():
+    from vllm_gcu_amd.kernels import fused_moe
+    return fused_moe
+
+
+@pytest.fixture(scope="module")
+def rearrange():
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    return rearrange
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def f16(a):
+    return a.astype(np.float16).astype(np.float32)
+
+
+def bf16(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+
+
+def make_int4_experts(rng, E, K, N, g=128):
+    q = rng.integers(0, 16, size=(E, K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(E, K // g, N), dtype=np.uint8)
+    s = rng.uniform(0.001, 0.01, size=(E, K // g, N)).astype(np.float16)
+    return q, z, s
+
+
+def int4_to_device(rearrange, q, z):
+    qw = np.stack([ow4.gptq_pack_weight(q[e]) for e in range(q.shape[0])])
+    qz = np.stack([ow4.gptq_pack_zeros(z[e]) for e in range(z.shape[0])])
+    return rearrange.rearrange_uint4_int32_gptq(dev(qw), dev(qz))
+
+
+def run_grouped(fmoe, A, B, C, A_scale, B_scale, B_zp, tw, ids, E, block, mul, topk, **flags):
+    s, e, n = fmoe.moe_align_block_size(ids, block, E)
+    cfg = {"BLOCK_SIZE_M": block}
+    kw = dict(use_fp8_w8a8=False, use_int8_w8a8=False, use_int8_w8a16=False, use_int4_w4a16=False)
+    kw.update(flags)
+    fmoe.invoke_fused_moe_kernel(A, B, C, A_scale, B_scale, B_zp, tw, ids, s, e, n, mul, topk, cfg, **kw)
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("block", [16, 32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_grouped_w4a16_both_gemms(fmoe, rearrange, block, dtype):
+    print(f"case grouped w4a16 block={block} {dtype}", flush=True)
+    rng = np.random.default_rng(block)
+    M, E, T, K, N = 37, 4, 2, 256, 384
+    q, z, s = make_int4_experts(rng, E, K, N)
+    w, zp = int4_to_device(rearrange, q, z)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    sd = torch.from_numpy(s).to(dtype)
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    wf = lambda e: ow4.dequantize(q[e], z[e], sd[e].float().numpy(), 128)
+    # GEMM 1 form: A is [M, K], output row t reads A[t // topk], no routed weight
+    C = torch.full((M, T, N), 7.0, dtype=dtype, device="cuda")
+    run_grouped(fmoe, x.cuda(), w, C, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, False, T,
+                use_int4_w4a16=True, block_shape=[0, 128])
+    want = om.fused_moe_gemm(x.float().numpy(), wf, ids, T)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # GEMM 2 form: A is [M * topk, K], topk = 1, routed weights applied
+    x2 = torch.from_numpy(rng.standard_normal((M * T, K)).astype(np.float32)).to(dtype)
+    C2 = torch.empty((M, T, N), dtype=dtype, device="cuda")
+    run_grouped(fmoe, x2.cuda(), w, C2, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, True, 1,
+                use_int4_w4a16=True, block_shape=[0, 128])
+    want2 = om.fused_moe_gemm(x2.float().numpy(), wf, ids, 1, tw, True)
+    np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
+
+
+def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe):
+    # what the reference's moe_wna16 loader leaves on the layer: uint8 [E, N, K/2]
+    # half-group bytes (moe_wna16.py:464-466) and fp16 zeros = z * scales
+    rng = np.random.default_rng(5)
+    M, E, T, K, N = 20, 3, 2, 256, 256
+    q, z, s = make_int4_experts(rng, E, K, N)
+    rw = np.stack([np.ascontiguousarray(ow4.ref_halfgroup_pack(q[e]).T) for e in range(E)])
+    zs = (z.astype(np.float32) * s.astype(np.float32)).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    C = torch.empty((M, T, N), dtype=torch.float16, device="cuda")
+    run_grouped(fmoe, dev(x), dev(rw), C, None, dev(s), dev(zs), dev(tw), dev(ids), E, 64, False, T,
+                use_int4_w4a16=True, block_shape=[0, 128])
+    want = om.fused_moe_gemm(x.astype(np.float32), lambda e: ow4.dequantize_prescaled_zeros(q[e], zs[e], s[e], 128), ids, T)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("block", [16, 64, 128])
+def test_grouped_fp8_block(fmoe, ops, block):
+    print(f"case grouped fp8 block={block}", flush=True)
+    rng = np.random.default_rng(7 + block)
+    M, E, T, K, N = 50, 6, 3, 512, 384
+    wf32 = (rng.standard_normal((E, N, K)) * 0.02).astype(np.float32)
+    ws = rng.uniform(0.5, 2.0, size=(E, N // 128, K // 128)).astype(np.float32)
+    wq = np.stack([of8.to_e4m3fn(np.clip(wf32[e] * 100, -448, 448)) for e in range(E)])      # codes
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+    xq, xs = ops.per_token_group_quant_fp8(x.cuda(), 128)
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    C = torch.empty((M, T, N), dtype=torch.bfloat16, device="cuda")
+    run_grouped(fmoe, xq, dev(wq).view(torch.float8_e4m3fn), C, xs, dev(ws), None, dev(tw), dev(ids), E, block,
+                False, T, use_fp8_w8a8=True, block_shape=[128, 128])
+    xq_c, xs_c = xq.view(torch.uint8).cpu().numpy(), xs.cpu().numpy()
+    want = np.zeros((M * T, N), dtype=np.float32)
+    flat = ids.reshape(-1)
+    for t in range(M * T):
+        e = flat[t]
+        want[t] = of8.block_fp8_gemm(xq_c[t // T:t // T + 1], xs_c[t // T:t // T + 1], wq[e], ws[e])[0]
+    got = C.view(-1, N).float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL * np.abs(want).max())
+
+
+def test_grouped_int8_and_fp16_and_w8a16(fmoe, ops):
+    rng = np.random.default_rng(11)
+    M, E, T, K, N = 33, 4, 2, 256, 260
+    ids_w, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    # int8 per-token x per-channel
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    xq, xs = o8.dynamic_scaled_int8_quant(x)
+    wq = rng.integers(-127, 128, size=(E, N, K), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.02, size=(E, N, 1)).astype(np.float32)
+    C = torch.empty((M, T, N), dtype=torch.float16, device="cuda")
+    run_grouped(fmoe, dev(xq), dev(wq), C, dev(xs), dev(ws), None, dev(ids_w), dev(ids), E, 32, False, T,
+                use_int8_w8a8=True)
+    want = np.zeros((M * T, N), dtype=np.float32)
+    flat = ids.reshape(-1)
+    for t in range(M * T):
+        e = flat[t]
+        acc = o8.int8_gemm_i32(xq[t // T:t // T + 1], np.ascontiguousarray(wq[e].T))
+        want[t] = o8.scaled_mm_epilogue(acc, xs[t // T], ws[e, :, 0])[0]
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # unquantised fp16 experts (fused_moe_kernel), routed weight applied
+    wf = (rng.standard_normal((E, N, K)) * 0.05).astype(np.float16)
+    C = torch.empty((M, T, N), dtype=torch.float16, device="cuda")
+    run_grouped(fmoe, dev(x), dev(wf), C, None, None, None, dev(ids_w), dev(ids), E, 16, True, T)
+    want = om.fused_moe_gemm(x.astype(np.float32), lambda e: wf[e].astype(np.float32).T, ids, T, ids_w, True)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # W8A16 per channel
+    s16 = rng.uniform(0.001, 0.01, size=(E, N)).astype(np.float16)
+    C = torch.empty((M, T, N), dtype=torch.float16, device="cuda")
+    run_grouped(fmoe, dev(x), dev(wq), C, None, dev(s16), None, dev(ids_w), dev(ids), E, 64, False, T,
+                use_int8_w8a16=True, block_shape=[0, -1])
+    want = om.fused_moe_gemm(x.astype(np.float32),
+                             lambda e: (wq[e].astype(np.float32) * s16[e].astype(np.float32)[:, None]).T, ids, T)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_dense_block_fp8_and_w8a16(ops):
+    rng = np.random.default_rng(13)
+    M, K, N = 70, 512, 384
+    x = torch.from_numpy(rng.standard_normal((3, M, K)).astype(np.float32)).to(torch.bfloat16)
+    xq, xs = ops.per_token_group_quant_fp8(x.cuda(), 128)
+    wq = of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 2, -448, 448).astype(np.float32))
+    ws = rng.uniform(0.005, 0.02, size=(N // 128, K // 128)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    out = ops.w8a8_block_fp8_matmul(xq, dev(wq).view(torch.float8_e4m3fn), xs, dev(ws), [128, 128], torch.bfloat16,
+                                    torch.from_numpy(bias).to(torch.bfloat16).cuda())
+    assert out.shape == (3, M, N) and out.dtype == torch.bfloat16
+    want = of8.block_fp8_gemm(xq.view(torch.uint8).cpu().numpy().reshape(-1, K), xs.cpu().numpy().reshape(-1, K // 128),
+                              wq, ws, bias=bf16(bias))
+    np.testing.assert_allclose(out.float().cpu().numpy().reshape(-1, N), want, rtol=RTOL, atol=ATOL)
+    # GPTQ-8bit path: gptq_gemm_gcu(bit=8) -> weight_only_quant (_custom_ops.py:269-275)
+    w8 = rng.integers(-128, 128, size=(N, K), dtype=np.int8)
+    s16 = rng.uniform(0.001, 0.01, N).astype(np.float16)
+    xh = rng.standard_normal((M, K)).astype(np.float16)
+    out = ops.gptq_gemm_gcu(dev(xh), dev(w8), torch.empty(0, device="cuda"), dev(s16), torch.empty(0, device="cuda"), 8, None, -1)
+    want = o8.weight_only_int8(xh, w8, s16, -1)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+# ---------------------------------------------------- whole sequence ----
+def build_moe(mode):
+    from vllm_gcu_amd.kernels.modular_experts import TritonExpertsPad
+    from vllm_gcu_amd.kernels.modular_kernel import FusedMoEModularKernel
+    from vllm_gcu_amd.kernels.prepare_finalize import MoEPrepareAndFinalizeNoEP
+    if mode == "w4a16":
+        fe = TritonExpertsPad(use_int4_w4a16=True, block_shape=[0, 128])
+    else:
+        fe = TritonExpertsPad(use_fp8_w8a8=True, block_shape=[128, 128])
+    return FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), fe)
+
+
+@pytest.mark.parametrize("M,E,T,H,I", [(64, 8, 2, 512, 768), (5, 4, 2, 256, 256), (300, 8, 2, 512, 1024)])
+def test_fused_experts_w4a16_sequence(ops, rearrange, M, E, T, H, I):
+    print(f"case fused w4a16 M={M} E={E}", flush=True)
+    rng = np.random.default_rng(M)
+    q13, z13, s13 = make_int4_experts(rng, E, H, 2 * I)
+    q2, z2, s2 = make_int4_experts(rng, E, I, H)
+    w13, zp13 = int4_to_device(rearrange, q13, z13)
+    w2, zp2 = int4_to_device(rearrange, q2, z2)
+    x = rng.standard_normal((M, H)).astype(np.float16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    tw, ids = ops.fused_topk(None, dev(logits), T, True)
+    out = build_moe("w4a16")(dev(x), w13, w2, tw, ids, w1_scale=dev(s13), w2_scale=dev(s2), w1_zp=zp13, w2_zp=zp2)
+    two, ido, _ = om.topk_softmax(logits, T, True)
+    assert np.array_equal(ids.cpu().numpy(), ido)
+    want = om.fused_experts(x.astype(np.float32), lambda e: ow4.dequantize(q13[e], z13[e], s13[e], 128),
+                            lambda e: ow4.dequantize(q2[e], z2[e], s2[e], 128), two, ido, f16)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_fused_experts_fp8_block_sequence(ops, fmoe):
+    print("case fused fp8", flush=True)
+    rng = np.random.default_rng(3)
+    M, E, T, H, I = 48, 16, 4, 512, 256
+    w13 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, 2 * I, H)) * 0.5, -448, 448).astype(np.float32))
+    w2 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, H, I)) * 0.5, -448, 448).astype(np.float32))
+    s13 = rng.uniform(0.02, 0.1, size=(E, 2 * I // 128, H // 128)).astype(np.float32)
+    s2 = rng.uniform(0.02, 0.1, size=(E, H // 128, I // 128)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).to(torch.bfloat16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    tw, ids = fmoe.grouped_topk(x.cuda(), dev(logits), T, True, 4, 2, "sigmoid", None)
+    out = build_moe("fp8")(x.cuda(), dev(w13).view(torch.float8_e4m3fn), dev(w2).view(torch.float8_e4m3fn), tw, ids,
+                           w1_scale=dev(s13), w2_scale=dev(s2))
+    two, ido = om.grouped_topk(logits, T, True, 4, 2, "sigmoid", None)
+    assert np.array_equal(ids.cpu().numpy(), ido)
+
+    def deq(codes, sc):
+        return (of8.from_e4m3fn(codes) * np.repeat(np.repeat(sc, 128, 0), 128, 1)).T   # [K, N]
+
+    def qdq(a):                     # per-token-group fp8 round trip of an activation
+        qa, sa = of8.per_token_group_quant_fp8(a, 128)
+        return of8.from_e4m3fn(qa) * np.repeat(sa, 128, -1)
+
+    want = om.fused_experts(qdq(x.float().numpy()), lambda e: deq(w13[e], s13[e]), lambda e: deq(w2[e], s2[e]),
+                            two, ido, bf16, quant_a2=qdq)
+    got = out.float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+
+
+def test_config3_full_size_properties_and_sample(ops, rearrange):
+    # BASELINE config 3: 512 tokens, hidden 4096, 8 experts, intermediate 14336, top-2, int4 g=128
+    print("case config3", flush=True)
+    M, E, T, H, I = 512, 8, 2, 4096, 14336
+    g = torch.Generator().manual_seed(0)
+    w13 = torch.randint(-2**31, 2**31 - 1, (E, H // 8, 2 * I), dtype=torch.int32, generator=g)   # GPTQ words
+    w2 = torch.randint(-2**31, 2**31 - 1, (E, I // 8, H), dtype=torch.int32, generator=g)
+    z13 = torch.randint(-2**31, 2**31 - 1, (E, H // 128, 2 * I // 8), dtype=torch.int32, generator=g)
+    z2 = torch.randint(-2**31, 2**31 - 1, (E, I // 128, H // 8), dtype=torch.int32, generator=g)
+    s13 = (torch.rand(E, H // 128, 2 * I, generator=g) * 0.009 + 0.001).to(torch.float16)
+    s2 = (torch.rand(E, I // 128, H, generator=g) * 0.009 + 0.001).to(torch.float16)
+    x = torch.randn(M, H, generator=g).to(torch.float16)
+    logits = torch.randn(M, E, generator=g)
+    w13d, zp13 = rearrange.rearrange_uint4_int32_gptq(w13.cuda(), z13.cuda())
+    w2d, zp2 = rearrange.rearrange_uint4_int32_gptq(w2.cuda(), z2.cuda())
+    moe = build_moe("w4a16")
+    tw, ids = ops.fused_topk(None, logits.cuda(), T, True)
+    kw = dict(w1_scale=s13.cuda(), w2_scale=s2.cuda(), w1_zp=zp13, w2_zp=zp2)
+    out = moe(x.cuda(), w13d, w2d, tw, ids, **kw)
+    # permuting the tokens permutes the outputs bit for bit (rows are independent)
+    perm = torch.randperm(M, generator=g)
+    out_p = moe(x[perm].cuda(), w13d, w2d, tw[perm.cuda()], ids[perm.cuda()], **kw)
+    assert torch.equal(out_p, out[perm.cuda()])
+    # one token against the oracle (only its two experts are dequantised on the CPU)
+    tok = 17
+    e_tok = ids[tok].cpu().numpy()
+    two, ido, _ = om.topk_softmax(logits.numpy(), T, True)
+    assert np.array_equal(ids.cpu().numpy(), ido)
+
+    def expert(wq, zq, sc, e):
+        return ow4.dequantize(ow4.gptq_unpack_weight(wq[e].numpy()), ow4.gptq_unpack_zeros(zq[e].numpy()),
+                              sc[e].numpy(), 128)
+
+    want = om.fused_experts(x[tok:tok + 1].float().numpy(), lambda e: expert(w13, z13, s13, e),
+                            lambda e: expert(w2, z2, s2, e), two[tok:tok + 1], e_tok[None, :], f16)
+    np.testing.assert_allclose(out[tok:tok + 1].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)

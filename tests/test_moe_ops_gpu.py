@@ -168,6 +168,12 @@ def test_silu_and_mul_and_pad(ops, dtype):
     o2 = out2.view(-1, 256).float().cpu().numpy()
     np.testing.assert_allclose(o2[:20], want.reshape(-1, 256)[:20], rtol=RTOL, atol=ATOL)
     assert np.all(o2[20:] == 7.0)
+    # 3-D input: `size` counts tokens (leading dimension), not flattened rows
+    out3 = torch.full((37, 2, 256), 7.0, dtype=dtype, device="cuda")
+    torch.ops._C.silu_and_mul_pad(out3, x.cuda(), torch.tensor([20], dtype=torch.int32, device="cuda"))
+    o3 = out3.float().cpu().numpy()
+    np.testing.assert_allclose(o3[:20], want[:20], rtol=RTOL, atol=ATOL)
+    assert np.all(o3[20:] == 7.0)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

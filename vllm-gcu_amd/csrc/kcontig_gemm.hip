@@ -1,0 +1,428 @@
+// Skinny GEMMs whose weights are K-contiguous ([N, K] per expert): fp8-e4m3
+// with 128x128 block scales, int8 with per-token x per-channel scales, plain
+// fp16/bf16, and int8 weights with 16-bit activations (W8A16).  Used for the
+// fused-MoE grouped GEMM ("non-gather": rows are picked through
+// sorted_token_ids, weights through expert_ids) and for dense small-M calls.
+//
+// These shapes are bound by the HBM stream of the weights.  A workgroup (4
+// wavefronts) owns up to 64 rows and 256 columns; a wavefront owns 64 columns
+// (four 16-row MFMA "A" tiles of weights) and every row tile of activations,
+// so each weight byte is loaded once per workgroup and both operands go from
+// global memory straight into MFMA registers: lane (r = l % 16, q = l / 16)
+// holds the 32 consecutive k of row r that start at 128 kb + 32 q.  The next K
+// block is prefetched while the current one is multiplied.  Block scales are
+// applied to the fp32 partial sum of each 128-wide K block; the int8 mode
+// keeps exact int32 accumulators to the end.
+#include "common.h"
+
+namespace mi355q {
+namespace {
+
+enum { KC_FP8_BLOCK = 0, KC_INT8 = 1, KC_F16 = 2, KC_BF16 = 3, KC_W8A16_F16 = 4, KC_W8A16_BF16 = 5 };
+
+struct KcArgs {
+  void* out;                   // [rows_out, N] f16/bf16
+  const void* a;               // activations [Ma, K]
+  const void* w;               // weights [E, N, K]
+  const float* a_scale;        // fp8: [Ma, K/128]; int8: [Ma]
+  const void* w_scale;         // fp8: f32 [E, ceil(N/128), K/128]; int8: f32 [E, N]; W8A16: act dtype [E, N] or [E, K/g, N]
+  const void* bias;            // [N] in out dtype, dense mode only
+  int M, N, K;
+  int wgs;                     // W8A16 group size along K (K = per channel)
+  // grouped mode
+  const int* sorted_ids;
+  const int* expert_ids;
+  const int* npp;
+  const float* topk_weights;
+  int numel, topk, block_size;
+  long w_stride, ws_stride;    // per-expert strides (elements)
+};
+
+template <int MODE> struct Kc;
+template <> struct Kc<KC_FP8_BLOCK> {
+  static constexpr int ABYTES = 1, WBYTES = 1;
+  typedef f4 acc_t;
+};
+template <> struct Kc<KC_INT8> {
+  static constexpr int ABYTES = 1, WBYTES = 1;
+  typedef i4 acc_t;
+};
+template <> struct Kc<KC_F16> {
+  static constexpr int ABYTES = 2, WBYTES = 2;
+  typedef f4 acc_t;
+};
+template <> struct Kc<KC_BF16> {
+  static constexpr int ABYTES = 2, WBYTES = 2;
+  typedef f4 acc_t;
+};
+template <> struct Kc<KC_W8A16_F16> {
+  static constexpr int ABYTES = 2, WBYTES = 1;
+  typedef f4 acc_t;
+};
+template <> struct Kc<KC_W8A16_BF16> {
+  static constexpr int ABYTES = 2, WBYTES = 1;
+  typedef f4 acc_t;
+};
+
+// 16 signed bytes -> 16 halves / bfloat16 (exact)
+__device__ __forceinline__ void s8x16_to_f16(const u4& v, u4& lo, u4& hi) {
+  uint32_t o[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int w = (int)v[i];
+    _Float16 h0 = (_Float16)(float)(int8_t)(w & 0xff), h1 = (_Float16)(float)(int8_t)((w >> 8) & 0xff);
+    _Float16 h2 = (_Float16)(float)(int8_t)((w >> 16) & 0xff), h3 = (_Float16)(float)(int8_t)((w >> 24) & 0xff);
+    o[2 * i] = (uint32_t)bitcast<uint16_t>(h0) | ((uint32_t)bitcast<uint16_t>(h1) << 16);
+    o[2 * i + 1] = (uint32_t)bitcast<uint16_t>(h2) | ((uint32_t)bitcast<uint16_t>(h3) << 16);
+  }
+  lo = (u4){o[0], o[1], o[2], o[3]};
+  hi = (u4){o[4], o[5], o[6], o[7]};
+}
+__device__ __forceinline__ void s8x16_to_bf16(const u4& v, u4& lo, u4& hi) {
+  uint32_t o[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int w = (int)v[i];
+    uint32_t b0 = bitcast<uint32_t>((float)(int8_t)(w & 0xff)) >> 16, b1 = bitcast<uint32_t>((float)(int8_t)((w >> 8) & 0xff)) >> 16;
+    uint32_t b2 = bitcast<uint32_t>((float)(int8_t)((w >> 16) & 0xff)) >> 16, b3 = bitcast<uint32_t>((float)(int8_t)((w >> 24) & 0xff)) >> 16;
+    o[2 * i] = b0 | (b1 << 16);
+    o[2 * i + 1] = b2 | (b3 << 16);
+  }
+  lo = (u4){o[0], o[1], o[2], o[3]};
+  hi = (u4){o[4], o[5], o[6], o[7]};
+}
+
+template <int MODE, int ODT, int MT, bool GROUPED>
+__global__ void __launch_bounds__(256, 1)
+kcontig_gemm_kernel(KcArgs a) {
+  typedef Kc<MODE> T;
+  typedef typename T::acc_t acc_t;
+  constexpr int BM = 16 * MT;
+  constexpr int AV = T::ABYTES * 2;               // 16-byte vectors per lane per K block (activations)
+  constexpr int WV = T::WBYTES * 2;               // ... weights
+  __shared__ int tok[GROUPED ? BM : 1];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, q = lane >> 4;
+  const int N = a.N, K = a.K;
+  const int KB = K >> 7;
+  const int m0 = blockIdx.y * BM;
+  long expert = 0;
+  if (GROUPED) {
+    if (m0 >= *a.npp) return;
+    expert = a.expert_ids[m0 / a.block_size];
+    for (int r = tid; r < BM; r += 256) tok[r] = a.sorted_ids[m0 + r];
+    __syncthreads();
+  }
+  const int n0 = blockIdx.x * 256 + wave * 64;
+  if (n0 >= N) return;
+  const char* wbase = (const char*)a.w + expert * a.w_stride * T::WBYTES;
+
+  // per-lane row pointers
+  const char* wptr[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = min(n0 + 16 * i + r16, N - 1);
+    wptr[i] = wbase + ((size_t)n * K + 32 * q) * T::WBYTES;
+  }
+  const char* aptr[MT];
+  int arow[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    int row;
+    if (GROUPED) row = min(tok[16 * j + r16], a.numel - 1) / a.topk;
+    else row = min(m0 + 16 * j + r16, a.M - 1);
+    arow[j] = row;
+    aptr[j] = (const char*)a.a + ((size_t)row * K + 32 * q) * T::ABYTES;
+  }
+
+  acc_t acc[4][MT];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[i][j] = (acc_t){0, 0, 0, 0};
+
+  struct Blk {
+    u4 w[4][WV];
+    u4 x[MT][AV];
+    float as[MODE == KC_FP8_BLOCK ? MT : 1];
+    float ws;
+  };
+  const float* wsf = (const float*)a.w_scale + expert * a.ws_stride;
+  auto load_blk = [&](Blk& b, int kb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int v = 0; v < WV; ++v)
+        b.w[i][v] = __builtin_nontemporal_load((const u4*)(wptr[i] + (size_t)kb * 128 * T::WBYTES) + v);
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < AV; ++v) b.x[j][v] = *((const u4*)(aptr[j] + (size_t)kb * 128 * T::ABYTES) + v);
+    if (MODE == KC_FP8_BLOCK) {
+#pragma unroll
+      for (int j = 0; j < MT; ++j) b.as[j] = a.a_scale[(size_t)arow[j] * KB + kb];
+      b.ws = wsf[(size_t)(n0 >> 7) * KB + kb];
+    }
+  };
+
+  auto compute_blk = [&](const Blk& b, int kb) {
+    if (MODE == KC_FP8_BLOCK) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          f4 part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int v = 0; v < 2; ++v) {
+            const u4 wv = b.w[i][v], xv = b.x[j][v];
+            long w0 = (long)((unsigned long)wv[0] | ((unsigned long)wv[1] << 32));
+            long w1 = (long)((unsigned long)wv[2] | ((unsigned long)wv[3] << 32));
+            long x0 = (long)((unsigned long)xv[0] | ((unsigned long)xv[1] << 32));
+            long x1 = (long)((unsigned long)xv[2] | ((unsigned long)xv[3] << 32));
+            part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, x0, part, 0, 0, 0);
+            part = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, x1, part, 0, 0, 0);
+          }
+          const float sc = b.as[j] * b.ws;
+          acc[i][j] = bitcast<acc_t>(bitcast<f4>(acc[i][j]) + sc * part);
+        }
+    } else if (MODE == KC_INT8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+#pragma unroll
+          for (int v = 0; v < 2; ++v)
+            acc[i][j] = bitcast<acc_t>(__builtin_amdgcn_mfma_i32_16x16x64_i8(
+                bitcast<i4>(b.w[i][v]), bitcast<i4>(b.x[j][v]), bitcast<i4>(acc[i][j]), 0, 0, 0));
+    } else {
+      // 16-bit activations; weights 16-bit, or int8 converted on the fly
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        u4 wv[4];
+        if (MODE == KC_F16 || MODE == KC_BF16) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) wv[v] = b.w[i][v % WV];
+        } else if (MODE == KC_W8A16_F16) {
+          s8x16_to_f16(b.w[i][0], wv[0], wv[1]);
+          s8x16_to_f16(b.w[i][WV - 1], wv[2], wv[3]);
+        } else {
+          s8x16_to_bf16(b.w[i][0], wv[0], wv[1]);
+          s8x16_to_bf16(b.w[i][WV - 1], wv[2], wv[3]);
+        }
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            if (MODE == KC_F16 || MODE == KC_W8A16_F16)
+              acc[i][j] = bitcast<acc_t>(__builtin_amdgcn_mfma_f32_16x16x32_f16(
+                  bitcast<h8>(wv[v]), bitcast<h8>(b.x[j][v % AV]), bitcast<f4>(acc[i][j]), 0, 0, 0));
+            else
+              acc[i][j] = bitcast<acc_t>(__builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  bitcast<b8>(wv[v]), bitcast<b8>(b.x[j][v % AV]), bitcast<f4>(acc[i][j]), 0, 0, 0));
+          }
+      }
+    }
+    (void)kb;
+  };
+
+  {
+    Blk b0, b1;
+    load_blk(b0, 0);
+    int kb = 0;
+    while (true) {
+      load_blk(b1, min(kb + 1, KB - 1));
+      __builtin_amdgcn_sched_barrier(0);
+      compute_blk(b0, kb);
+      __builtin_amdgcn_sched_barrier(0);
+      if (++kb >= KB) break;
+      load_blk(b0, min(kb + 1, KB - 1));
+      __builtin_amdgcn_sched_barrier(0);
+      compute_blk(b1, kb);
+      __builtin_amdgcn_sched_barrier(0);
+      if (++kb >= KB) break;
+    }
+  }
+
+  // ---- epilogue: lane holds row (l % 16) of each row tile and columns
+  // n0 + 16 i + 4 q + {0..3}
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    int m;
+    bool ok;
+    float rw = 1.0f;
+    if (GROUPED) {
+      m = tok[16 * j + r16];
+      ok = m < a.numel;
+      if (ok && a.topk_weights) rw = a.topk_weights[m];
+    } else {
+      m = m0 + 16 * j + r16;
+      ok = m < a.M;
+    }
+    if (!ok) continue;
+    float xs = 1.0f;
+    if (MODE == KC_INT8 && a.a_scale) xs = a.a_scale[arow[j]];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 16 * i + 4 * q;
+      if (n >= N) continue;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (MODE == KC_INT8) {
+          const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + n + e];
+          v[e] = ((float)bitcast<i4>(acc[i][j])[e] * xs) * ws;
+        } else if (MODE == KC_W8A16_F16 || MODE == KC_W8A16_BF16) {
+          const uint16_t raw = ((const uint16_t*)a.w_scale)[expert * a.ws_stride + n + e];
+          const float ws = (MODE == KC_W8A16_F16) ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw);
+          v[e] = bitcast<f4>(acc[i][j])[e] * ws;
+        } else {
+          v[e] = bitcast<f4>(acc[i][j])[e];
+        }
+        v[e] *= rw;
+        if (!GROUPED && a.bias) v[e] += Elem<ODT>::to_f32(((const uint16_t*)a.bias)[n + e]);
+      }
+      u2 o;
+      o.x = (uint32_t)Elem<ODT>::from_f32(v[0]) | ((uint32_t)Elem<ODT>::from_f32(v[1]) << 16);
+      o.y = (uint32_t)Elem<ODT>::from_f32(v[2]) | ((uint32_t)Elem<ODT>::from_f32(v[3]) << 16);
+      *(u2*)((uint16_t*)a.out + (size_t)m * N + n) = o;
+    }
+  }
+}
+
+template <int MODE, int ODT, bool GROUPED>
+void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
+  dim3 grid((a.N + 255) / 256, row_blocks), block(256);
+  switch (mt) {
+    case 1: hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, GROUPED>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, GROUPED>), grid, block, 0, st, a); break;
+    default: hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, GROUPED>), grid, block, 0, st, a); break;
+  }
+}
+
+template <bool GROUPED>
+int launch_mode(const KcArgs& a, int mode, int odt, int mt, int row_blocks, hipStream_t st) {
+#define KC_CASE(M_, O_) \
+  if (mode == M_ && odt == O_) { launch_mt<M_, O_, GROUPED>(a, mt, row_blocks, st); return 0; }
+  KC_CASE(KC_FP8_BLOCK, MI355Q_BF16)
+  KC_CASE(KC_FP8_BLOCK, MI355Q_F16)
+  KC_CASE(KC_INT8, MI355Q_F16)
+  KC_CASE(KC_INT8, MI355Q_BF16)
+  KC_CASE(KC_F16, MI355Q_F16)
+  KC_CASE(KC_BF16, MI355Q_BF16)
+  KC_CASE(KC_W8A16_F16, MI355Q_F16)
+  KC_CASE(KC_W8A16_BF16, MI355Q_BF16)
+#undef KC_CASE
+  set_error("kcontig_gemm: unsupported mode %d with output dtype %d", mode, odt);
+  return 1;
+}
+
+int pick_mt(int rows) { return rows <= 16 ? 1 : (rows <= 32 ? 2 : 4); }
+
+}  // namespace
+
+int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                         const void* zeros, int zeros_kind, const float* topk_weights,
+                         const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
+                         int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
+                         int group_size, int dtype, hipStream_t st);
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+// quant_mode of the MoE / dense entry points
+//   0 = W4A16 (slab-layout int4), 1 = fp8 block-scaled, 2 = int8 per-token x per-channel,
+//   3 = unquantised 16-bit, 4 = W8A16 (int8 weights, per-channel scale in the activation dtype)
+extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scale,
+                               const void* w_scale, const void* w_zeros, int zeros_kind, int quant_mode,
+                               int group_size, const float* topk_weights, const int32_t* sorted_token_ids,
+                               const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int numel,
+                               int topk, int block_size, int max_blocks, int E, int K, int N, int act_dtype,
+                               int out_dtype, void* stream) {
+  MQ_REQUIRE(numel >= 0 && topk > 0 && E > 0 && K > 0 && N > 0, "moe_gemm: bad shape");
+  if (numel == 0 || max_blocks == 0) return 0;
+  MQ_REQUIRE(out && a && w && sorted_token_ids && expert_ids && num_tokens_post_pad, "moe_gemm: null pointer");
+  MQ_REQUIRE(block_size >= 16 && block_size % 16 == 0, "moe_gemm: block_size=%d must be a multiple of 16", block_size);
+  MQ_REQUIRE(K % 128 == 0, "moe_gemm: K=%d must be a multiple of 128", K);
+  hipStream_t st = as_stream(stream);
+  if (quant_mode == 0) {
+    MQ_REQUIRE(N % 128 == 0, "moe_gemm(w4a16): N=%d must be a multiple of 128", N);
+    MQ_REQUIRE(w_scale, "moe_gemm(w4a16): scales missing");
+    MQ_REQUIRE(out_dtype == act_dtype, "moe_gemm(w4a16): output dtype must equal the activation dtype");
+    return w4a16_grouped_launch(out, a, (const int32_t*)w, w_scale, w_zeros, zeros_kind, topk_weights,
+                                sorted_token_ids, expert_ids, num_tokens_post_pad, numel, topk, block_size,
+                                max_blocks, E, K, N, group_size <= 0 ? K : group_size, act_dtype, st);
+  }
+  MQ_REQUIRE(N % 4 == 0, "moe_gemm: N=%d must be a multiple of 4", N);
+  KcArgs g = {};
+  g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = nullptr;
+  g.M = numel; g.N = N; g.K = K; g.wgs = K;
+  g.sorted_ids = sorted_token_ids; g.expert_ids = expert_ids; g.npp = num_tokens_post_pad;
+  g.topk_weights = topk_weights; g.numel = numel; g.topk = topk; g.block_size = block_size;
+  g.w_stride = (long)N * K;
+  int mode;
+  if (quant_mode == 1) {
+    MQ_REQUIRE(a_scale && w_scale, "moe_gemm(fp8): scales missing");
+    MQ_REQUIRE(group_size == 128, "moe_gemm(fp8): only 128x128 block scales are supported, got %d", group_size);
+    mode = KC_FP8_BLOCK;
+    g.ws_stride = (long)((N + 127) / 128) * (K / 128);
+  } else if (quant_mode == 2) {
+    MQ_REQUIRE(w_scale, "moe_gemm(int8): weight scales missing");
+    mode = KC_INT8;
+    g.ws_stride = N;
+  } else if (quant_mode == 3) {
+    mode = act_dtype == MI355Q_F16 ? KC_F16 : KC_BF16;
+  } else if (quant_mode == 4) {
+    MQ_REQUIRE(w_scale, "moe_gemm(w8a16): weight scales missing");
+    MQ_REQUIRE(group_size <= 0 || group_size == K, "moe_gemm(w8a16): only per-channel scales are supported");
+    mode = act_dtype == MI355Q_F16 ? KC_W8A16_F16 : KC_W8A16_BF16;
+    g.ws_stride = N;
+  } else {
+    MQ_REQUIRE(false, "moe_gemm: unknown quant_mode %d", quant_mode);
+  }
+  // row tiles per workgroup: the align block, capped at 64 rows
+  const int rows_per_wg = block_size >= 64 ? 64 : block_size;
+  MQ_REQUIRE(block_size % rows_per_wg == 0 && (rows_per_wg == 16 || rows_per_wg == 32 || rows_per_wg == 64),
+             "moe_gemm: block_size=%d unsupported", block_size);
+  const int row_blocks = max_blocks * (block_size / rows_per_wg);
+  int rc = launch_mode<true>(g, mode, out_dtype, pick_mt(rows_per_wg), row_blocks, st);
+  if (rc) return rc;
+  MQ_LAUNCH_CHECK("moe_gemm");
+  return 0;
+}
+
+extern "C" int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_scale,
+                                   const void* w_scale, const void* bias, int quant_mode, int group_size,
+                                   int M, int K, int N, int act_dtype, int out_dtype, void* stream) {
+  MQ_REQUIRE(M >= 0 && K > 0 && N > 0, "kcontig_gemm: bad shape M=%d K=%d N=%d", M, K, N);
+  if (M == 0) return 0;
+  MQ_REQUIRE(out && a && w, "kcontig_gemm: null pointer");
+  MQ_REQUIRE(K % 128 == 0 && N % 4 == 0, "kcontig_gemm: K=%d must be a multiple of 128 and N=%d of 4", K, N);
+  KcArgs g = {};
+  g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = bias;
+  g.M = M; g.N = N; g.K = K; g.wgs = K;
+  g.numel = M; g.topk = 1; g.block_size = 64;
+  int mode;
+  if (quant_mode == 1) {
+    MQ_REQUIRE(a_scale && w_scale, "kcontig_gemm(fp8): scales missing");
+    MQ_REQUIRE(group_size == 128, "kcontig_gemm(fp8): only 128x128 block scales are supported, got %d", group_size);
+    mode = KC_FP8_BLOCK;
+  } else if (quant_mode == 2) {
+    MQ_REQUIRE(w_scale, "kcontig_gemm(int8): weight scales missing");
+    mode = KC_INT8;
+  } else if (quant_mode == 3) {
+    mode = act_dtype == MI355Q_F16 ? KC_F16 : KC_BF16;
+  } else if (quant_mode == 4) {
+    MQ_REQUIRE(w_scale, "kcontig_gemm(w8a16): weight scales missing");
+    MQ_REQUIRE(group_size <= 0 || group_size == K, "kcontig_gemm(w8a16): only per-channel scales are supported");
+    mode = act_dtype == MI355Q_F16 ? KC_W8A16_F16 : KC_W8A16_BF16;
+  } else {
+    MQ_REQUIRE(false, "kcontig_gemm: unknown quant_mode %d", quant_mode);
+  }
+  const int mt = pick_mt(M < 64 ? M : 64);
+  const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
+  int rc = launch_mode<false>(g, mode, out_dtype, mt, row_blocks, as_stream(stream));
+  if (rc) return rc;
+  MQ_LAUNCH_CHECK("kcontig_gemm");
+  return 0;
+}

@@ -41,10 +41,7 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
              "w4a16_gemm: unknown zeros_kind %d", zeros_kind);
   MQ_REQUIRE(zeros_kind == MI355Q_ZP_NONE || zeros, "w4a16_gemm: zeros pointer missing");
   MQ_REQUIRE(family >= 0 && family <= 2, "w4a16_gemm: unknown kernel family %d", family);
-  // bf16: the MFMA kernel rounds every dequantised weight to bf16 (8
-  // significant bits), which can exceed the 1e-2 parity bound on long dot
-  // products; bf16 therefore stays on the exact-integer streaming kernel
-  if (family == 0) family = (M <= 64 || group_size % 128 != 0 || dtype == MI355Q_BF16) ? 1 : 2;
+  if (family == 0) family = (M <= 64 || group_size % 128 != 0) ? 1 : 2;
   MQ_REQUIRE(family != 2 || group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   if (family == 1) {

@@ -4,9 +4,10 @@
 // wavefronts side by side along N: wave w owns 64 columns (four 16-column
 // tiles of one slab) for all 128 rows.  Because the slab layout already stores
 // each lane's MFMA B operand contiguously, a wavefront dequantises its own
-// columns straight into B operands in registers -- (q - z) * s rounded once to
-// the activation type -- and every operand is reused for the 8 row tiles, so no
-// weight is dequantised twice in a workgroup.  The activation tile is shared
+// columns straight into B operands in registers -- the exact integers (q - z),
+// the group scale is applied to the fp32 partial sum of each K block -- and
+// every operand is reused for the 8 row tiles, so no weight is dequantised
+// twice in a workgroup.  The activation tile is shared
 // by the 4 wavefronts through LDS (double buffered, rows padded by 16 B so
 // the 16-lane x 16 B operand reads are bank-conflict free).  fp32 accumulate.
 #include "common.h"
@@ -15,9 +16,8 @@ namespace mi355q {
 
 namespace {
 
-constexpr int BM = 128, BN = 256, BK = 128;
+constexpr int BN = 256, BK = 128;
 constexpr int A_ROW = BK * 2 + 16;                 // bytes per LDS row (padded)
-constexpr int A_BUF = BM * A_ROW;                  // bytes per buffer
 
 struct TileArgs {
   uint16_t* out;
@@ -27,30 +27,37 @@ struct TileArgs {
   const void* zeros;
   const uint16_t* bias;
   int M, K, N, gs;
+  // grouped (MoE) mode: rows come from sorted_ids, weights from expert_ids
+  const int* sorted_ids;      // [blocks * BM] flat (token, slot) ids, pad = numel
+  const int* expert_ids;      // [blocks]
+  const int* npp;             // device scalar: padded id count
+  const float* topk_weights;  // [numel] or null
+  int numel, topk;
+  long w_stride, s_stride, z_stride;   // per-expert strides in elements of the respective arrays
 };
 
+// B operands are the exact integers (q - z) in the activation type; the group
+// scale multiplies the fp32 partial sum of each 128-row K block instead of
+// every weight, so the only rounding left is that of the fp32 accumulation.
 template <int DT> struct TileMma;
 template <> struct TileMma<MI355Q_F16> {
   typedef h8 vec;
   static __device__ __forceinline__ f4 run(vec a, vec b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
-  // one packed word -> 8 weights (q - z) * s in fp16
-  //   zlo = (1024 + z) x2, zhi = (64 + z) x2, sc = s x2
-  static __device__ __forceinline__ vec dequant(uint32_t w, float z, float s) {
+  // one packed word -> 8 values (q - z); zlo = (1024 + z) x2, zhi = (64 + z) x2
+  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zlo, h2 zhi) {
     const uint32_t MAGIC = 0x64006400u;
     const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-    const _Float16 zl = (_Float16)(1024.0f + z), zh = (_Float16)(64.0f + z), sh = (_Float16)s;
-    const h2 zlo = {zl, zl}, zhi = {zh, zh}, sc = {sh, sh};
     uint32_t w8 = w >> 8;
-    h2 a0 = bitcast<h2>((w & 0x000f000fu) | MAGIC);
-    h2 a1 = bitcast<h2>((w & 0x00f000f0u) | MAGIC);
+    h2 a0 = bitcast<h2>((w & 0x000f000fu) | MAGIC);      // 1024 + q
+    h2 a1 = bitcast<h2>((w & 0x00f000f0u) | MAGIC);      // 1024 + 16 q
     h2 a2 = bitcast<h2>((w8 & 0x000f000fu) | MAGIC);
     h2 a3 = bitcast<h2>((w8 & 0x00f000f0u) | MAGIC);
-    h2 r0 = (a0 - zlo) * sc;
-    h2 r1 = __builtin_elementwise_fma(a1, sixteenth, -zhi) * sc;
-    h2 r2 = (a2 - zlo) * sc;
-    h2 r3 = __builtin_elementwise_fma(a3, sixteenth, -zhi) * sc;
+    h2 r0 = a0 - zlo;
+    h2 r1 = __builtin_elementwise_fma(a1, sixteenth, -zhi);
+    h2 r2 = a2 - zlo;
+    h2 r3 = __builtin_elementwise_fma(a3, sixteenth, -zhi);
     return (h8){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
   }
 };
@@ -59,31 +66,47 @@ template <> struct TileMma<MI355Q_BF16> {
   static __device__ __forceinline__ f4 run(vec a, vec b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+  // small integers held exactly in fp16 -> the same integers in bf16
+  static __device__ __forceinline__ uint32_t cvt(h2 r) {
+    uint32_t lo = bitcast<uint32_t>((float)r.x), hi = bitcast<uint32_t>((float)r.y);
+    return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
   }
-  static __device__ __forceinline__ vec dequant(uint32_t w, float z, float s) {
-    float v[8];
-#pragma unroll
-    for (int p = 0; p < 8; ++p) v[p] = ((float)((w >> (4 * p)) & 15u) - z) * s;
-    // nibble order {0,4,1,5,2,6,3,7} = k offsets 0..7
-    u4 r = {pack(v[0], v[4]), pack(v[1], v[5]), pack(v[2], v[6]), pack(v[3], v[7])};
+  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zlo, h2 zhi) {
+    h8 v = TileMma<MI355Q_F16>::dequant(w, zlo, zhi);
+    u4 r = {cvt((h2){v[0], v[1]}), cvt((h2){v[2], v[3]}), cvt((h2){v[4], v[5]}), cvt((h2){v[6], v[7]})};
     return bitcast<vec>(r);
   }
 };
 
-template <int DT, int ZK>
+// MT = row tiles of 16 per workgroup (block rows BM = 16 MT); GROUPED selects
+// the MoE row gather
+template <int DT, int ZK, int MT, bool GROUPED>
 __global__ void __launch_bounds__(256, 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
   typedef typename MM::vec vec;
+  constexpr int BM = 16 * MT;
+  constexpr int A_BUF = BM * A_ROW;
   extern __shared__ __align__(16) unsigned char lds[];
+  __shared__ int tok[GROUPED ? BM : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int c = lane & 15, kq = lane >> 4;
   const int N = a.N, K = a.K, M = a.M;
   const int G = K >> 7;
   const int m0 = blockIdx.y * BM;
+  const u4* qw = a.qw;
+  const uint16_t* scales = a.scales;
+  const char* zeros = (const char*)a.zeros;
+  if (GROUPED) {
+    if (m0 >= *a.npp) return;                       // block beyond the padded ids
+    const long e = a.expert_ids[blockIdx.y];
+    qw += e * a.w_stride;
+    scales += e * a.s_stride;
+    if (zeros) zeros += e * a.z_stride * (ZK == MI355Q_ZP_PACKED ? 4 : 2);
+    for (int r = tid; r < BM; r += 256) tok[r] = a.sorted_ids[m0 + r];
+    __syncthreads();
+  }
   // N may end in the middle of the 256-column tile: the two wavefronts of a
   // missing slab compute on the previous one and skip the epilogue
   const bool live = (blockIdx.x * 2 + (wave >> 1)) < (N >> 7);
@@ -91,30 +114,35 @@ w4a16_tile_kernel(TileArgs a) {
   const int t0 = (wave & 1) * 4;
   const int ncol = 128 * slab + 8 * c + t0;          // first of this lane's 4 columns
 
-  f4 acc[8][4];
+  f4 acc[MT][4];
 #pragma unroll
-  for (int mt = 0; mt < 8; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
 
   // global -> register staging of the next activation tile: thread tid loads
-  // 8 chunks of 16 B: row = pass * 16 + tid / 16, chunk = tid % 16
+  // MT chunks of 16 B: row = pass * 16 + tid / 16, chunk = tid % 16
   const int arow = tid >> 4, achunk = tid & 15;
-  u4 areg[8];
+  const uint16_t* aptr[MT];
+#pragma unroll
+  for (int p = 0; p < MT; ++p) {
+    int row;
+    if (GROUPED) row = min(tok[p * 16 + arow], a.numel - 1) / a.topk;   // pads read a valid row
+    else row = min(m0 + p * 16 + arow, M - 1);
+    aptr[p] = a.x + (size_t)row * K + 8 * achunk;
+  }
+  u4 areg[MT];
   auto load_a = [&](int g) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int row = min(m0 + p * 16 + arow, M - 1);
-      areg[p] = *(const u4*)(a.x + (size_t)row * K + 128 * g + 8 * achunk);
-    }
+    for (int p = 0; p < MT; ++p) areg[p] = *(const u4*)(aptr[p] + 128 * g);
   };
   auto store_a = [&](int buf) {
     unsigned char* base = lds + buf * A_BUF;
 #pragma unroll
-    for (int p = 0; p < 8; ++p) *(u4*)(base + (p * 16 + arow) * A_ROW + achunk * 16) = areg[p];
+    for (int p = 0; p < MT; ++p) *(u4*)(base + (p * 16 + arow) * A_ROW + achunk * 16) = areg[p];
   };
 
-  const u4* wbase = a.qw + ((size_t)slab * G * 8 + t0) * 64 + lane;
+  const u4* wbase = qw + ((size_t)slab * G * 8 + t0) * 64 + lane;
   u4 wreg[4];
   uint2 sreg;
   uint32_t zreg = 0x88888888u;
@@ -124,9 +152,9 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) wreg[t] = p[t * 64];
     const int qrow = (128 * g) / a.gs;
-    sreg = *(const uint2*)(a.scales + (size_t)qrow * N + ncol);
-    if (ZK == MI355Q_ZP_PACKED) zreg = ((const uint32_t*)a.zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)] >> (4 * t0);
-    if (ZK == MI355Q_ZP_PRESCALED) zsreg = *(const uint2*)((const uint16_t*)a.zeros + (size_t)qrow * N + ncol);
+    sreg = *(const uint2*)(scales + (size_t)qrow * N + ncol);
+    if (ZK == MI355Q_ZP_PACKED) zreg = ((const uint32_t*)zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)] >> (4 * t0);
+    if (ZK == MI355Q_ZP_PRESCALED) zsreg = *(const uint2*)((const uint16_t*)zeros + (size_t)qrow * N + ncol);
   };
 
   load_a(0);
@@ -140,35 +168,50 @@ w4a16_tile_kernel(TileArgs a) {
     u4 wcur[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) wcur[t] = wreg[t];
-    float sc[4], zf[4];
+    float sc[4];
+    h2 zlo[4], zhi[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const uint32_t sw = (t < 2) ? sreg.x : sreg.y;
       sc[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+      float zf;
       if (ZK == MI355Q_ZP_PRESCALED) {
         const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
-        // z * s was pre-multiplied by the loader; recover the real-valued zero-point
-        zf[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[t];
+        // the loader pre-multiplied an integer zero-point by the scale
+        // (z * s rounded to the activation type): recover the integer
+        zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[t]);
       } else {
-        zf[t] = (float)((zreg >> (4 * t)) & 15u);
+        zf = (float)((zreg >> (4 * t)) & 15u);
       }
+      const _Float16 zl = (_Float16)(1024.0f + zf), zh = (_Float16)(64.0f + zf);
+      zlo[t] = (h2){zl, zl};
+      zhi[t] = (h2){zh, zh};
     }
     const int gn = min(g + 1, G - 1);
     load_a(gn);
     load_b(gn);
 
+    // all 16 B operands of this K block (4 steps x 4 column tiles)
+    vec bv[4][4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zlo[t], zhi[t]);
+
     const unsigned char* abase = lds + buf * A_BUF + c * A_ROW + kq * 16;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      vec bv[4];
+    for (int mt = 0; mt < MT; ++mt) {
+      f4 part[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) bv[t] = MM::dequant(wcur[t][s], zf[t], sc[t]);
+      for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int mt = 0; mt < 8; ++mt) {
+      for (int s = 0; s < 4; ++s) {
         const vec av = bitcast<vec>(*(const u4*)(abase + mt * 16 * A_ROW + s * 64));
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[mt][t] = MM::run(av, bv[t], acc[mt][t]);
+        for (int t = 0; t < 4; ++t) part[t] = MM::run(av, bv[s][t], part[t]);
       }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[mt][t] += sc[t] * part[t];
     }
     // the other buffer was last read one iteration ago: every wavefront has
     // passed the barrier below since, so it can be overwritten now
@@ -184,37 +227,58 @@ w4a16_tile_kernel(TileArgs a) {
     for (int t = 0; t < 4; ++t) bs[t] = Elem<DT>::to_f32(a.bias[ncol + t]);
   }
 #pragma unroll
-  for (int mt = 0; mt < 8; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int m = m0 + mt * 16 + 4 * kq + i;
-      if (m < M) {
+      int m;
+      float rw = 1.0f;
+      bool ok;
+      if (GROUPED) {
+        m = tok[mt * 16 + 4 * kq + i];
+        ok = m < a.numel;
+        if (ok && a.topk_weights) rw = a.topk_weights[m];
+      } else {
+        m = m0 + mt * 16 + 4 * kq + i;
+        ok = m < M;
+      }
+      if (ok) {
         uint2 o;
-        o.x = (uint32_t)Elem<DT>::from_f32(acc[mt][0][i] + bs[0]) |
-              ((uint32_t)Elem<DT>::from_f32(acc[mt][1][i] + bs[1]) << 16);
-        o.y = (uint32_t)Elem<DT>::from_f32(acc[mt][2][i] + bs[2]) |
-              ((uint32_t)Elem<DT>::from_f32(acc[mt][3][i] + bs[3]) << 16);
+        o.x = (uint32_t)Elem<DT>::from_f32(acc[mt][0][i] * rw + bs[0]) |
+              ((uint32_t)Elem<DT>::from_f32(acc[mt][1][i] * rw + bs[1]) << 16);
+        o.y = (uint32_t)Elem<DT>::from_f32(acc[mt][2][i] * rw + bs[2]) |
+              ((uint32_t)Elem<DT>::from_f32(acc[mt][3][i] * rw + bs[3]) << 16);
         *(uint2*)(a.out + (size_t)m * N + ncol) = o;
       }
     }
 }
 
-template <int DT, int ZK>
-hipError_t launch_one(const TileArgs& a, hipStream_t st) {
-  dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM), block(256);
-  const size_t shmem = 2 * A_BUF;                  // 68 KiB: above the 64 KiB default
-  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK>,
+template <int DT, int ZK, int MT, bool GROUPED>
+hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
+  constexpr int BM = 16 * MT;
+  dim3 grid((a.N + BN - 1) / BN, row_blocks), block(256);
+  const size_t shmem = 2 * BM * A_ROW;             // up to 68 KiB: above the 64 KiB default
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   if (attr != hipSuccess) return attr;
-  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK>), grid, block, shmem, st, a);
+  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED>), grid, block, shmem, st, a);
   return hipSuccess;
 }
 
-template <int DT>
-hipError_t launch_zk(const TileArgs& a, int zk, hipStream_t st) {
-  if (zk == MI355Q_ZP_NONE) return launch_one<DT, MI355Q_ZP_NONE>(a, st);
-  if (zk == MI355Q_ZP_PACKED) return launch_one<DT, MI355Q_ZP_PACKED>(a, st);
-  return launch_one<DT, MI355Q_ZP_PRESCALED>(a, st);
+template <int DT, int MT, bool GROUPED>
+hipError_t launch_zk(const TileArgs& a, int zk, int row_blocks, hipStream_t st) {
+  if (zk == MI355Q_ZP_NONE) return launch_one<DT, MI355Q_ZP_NONE, MT, GROUPED>(a, row_blocks, st);
+  if (zk == MI355Q_ZP_PACKED) return launch_one<DT, MI355Q_ZP_PACKED, MT, GROUPED>(a, row_blocks, st);
+  return launch_one<DT, MI355Q_ZP_PRESCALED, MT, GROUPED>(a, row_blocks, st);
+}
+
+template <int DT, bool GROUPED>
+hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStream_t st) {
+  switch (mt) {
+    case 1: return launch_zk<DT, 1, GROUPED>(a, zk, row_blocks, st);
+    case 2: return launch_zk<DT, 2, GROUPED>(a, zk, row_blocks, st);
+    case 4: return launch_zk<DT, 4, GROUPED>(a, zk, row_blocks, st);
+    default: return launch_zk<DT, 8, GROUPED>(a, zk, row_blocks, st);
+  }
 }
 
 }  // namespace
@@ -224,7 +288,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                       int group_size, int dtype, hipStream_t st) {
   MQ_REQUIRE(group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
-  TileArgs a;
+  TileArgs a = {};
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;
   a.qw = (const u4*)qweight;
@@ -232,10 +296,42 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   a.zeros = zeros;
   a.bias = (const uint16_t*)bias;
   a.M = M; a.K = K; a.N = N; a.gs = group_size;
-  hipError_t e = (dtype == MI355Q_F16) ? launch_zk<MI355Q_F16>(a, zeros_kind, st)
-                                       : launch_zk<MI355Q_BF16>(a, zeros_kind, st);
+  // 128-row blocks once they fill the chip, 64-row blocks for mid-sized M
+  const int mt = ((long)((M + 127) / 128) * ((N + BN - 1) / BN) >= device_cu_count()) ? 8 : 4;
+  const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
+  hipError_t e = (dtype == MI355Q_F16) ? launch_mt<MI355Q_F16, false>(a, zeros_kind, mt, row_blocks, st)
+                                       : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
   MQ_REQUIRE(e == hipSuccess, "w4a16_gemm(tile): cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("w4a16_gemm(tile)");
+  return 0;
+}
+
+int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                         const void* zeros, int zeros_kind, const float* topk_weights,
+                         const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
+                         int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
+                         int group_size, int dtype, hipStream_t st) {
+  MQ_REQUIRE(group_size % 128 == 0, "moe_w4a16: group_size=%d must be a multiple of 128", group_size);
+  MQ_REQUIRE(block_size == 16 || block_size == 32 || block_size == 64 || block_size == 128,
+             "moe_w4a16: block_size=%d must be 16, 32, 64 or 128", block_size);
+  TileArgs a = {};
+  a.out = (uint16_t*)out;
+  a.x = (const uint16_t*)x;
+  a.qw = (const u4*)qweight;
+  a.scales = (const uint16_t*)scales;
+  a.zeros = zeros;
+  a.M = numel; a.K = K; a.N = N; a.gs = group_size;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
+  a.numel = numel; a.topk = topk;
+  a.w_stride = (long)(K / 8) * N / 4;              // u4 elements per expert
+  a.s_stride = (long)(K / group_size) * N;
+  a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
+  (void)E;
+  hipError_t e = (dtype == MI355Q_F16)
+                     ? launch_mt<MI355Q_F16, true>(a, zeros_kind, block_size / 16, max_blocks, st)
+                     : launch_mt<MI355Q_BF16, true>(a, zeros_kind, block_size / 16, max_blocks, st);
+  MQ_REQUIRE(e == hipSuccess, "moe_w4a16: cannot reserve LDS: %s", hipGetErrorString(e));
+  MQ_LAUNCH_CHECK("moe_w4a16");
   return 0;
 }
 

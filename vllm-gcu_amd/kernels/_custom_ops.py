@@ -507,8 +507,17 @@ def _silu_and_mul_impl(result, input):
     _silu_and_mul_common(result, input, None)
 
 
+def _leading_rows_to_flat(t: torch.Tensor, size: torch.Tensor) -> torch.Tensor:
+    """``size`` counts entries of the leading dimension (tokens); the kernels
+    work on rows flattened over every dimension but the last."""
+    size = size.to(torch.int32)
+    lead = t.shape[0]
+    inner = (t.numel() // t.shape[-1]) // max(lead, 1)
+    return size * inner if inner != 1 else size
+
+
 def _silu_and_mul_pad_impl(out, input, size):
-    _silu_and_mul_common(out, input, size.to(torch.int32) if size.dtype != torch.int32 else size)
+    _silu_and_mul_common(out, input, _leading_rows_to_flat(input, size))
 
 
 def _fp8_out_ok(out, shape):
@@ -538,7 +547,7 @@ def _dynamic_per_token_group_fp8_quant_impl(out, scale, input, group_size):
 
 
 def _dynamic_per_token_group_fp8_quant_with_size_impl(out, scale, input, real_size, group_size):
-    _group_quant_common(out, scale, input, real_size, group_size, False)
+    _group_quant_common(out, scale, input, _leading_rows_to_flat(input, real_size), group_size, False)
 
 
 def _silu_mul_per_token_group_quant_impl(out, scale, input, group_size):
@@ -546,12 +555,7 @@ def _silu_mul_per_token_group_quant_impl(out, scale, input, group_size):
 
 
 def _silu_mul_per_token_group_quant_with_size_impl(out, scale, input, size, group_size):
-    # `size` counts rows of the leading dimension; the kernel works on flattened rows
-    x = input
-    lead = x.shape[0]
-    inner = (x.numel() // x.shape[-1]) // max(lead, 1)
-    rows_valid = size.to(torch.int32) * inner if inner != 1 else size
-    _group_quant_common(out, scale, input, rows_valid, group_size, True)
+    _group_quant_common(out, scale, input, _leading_rows_to_flat(input, size), group_size, True)
 
 
 def _dynamic_per_token_scaled_fp8_quant_impl(result, input, scale, scale_ub):
@@ -588,10 +592,7 @@ def _static_scaled_fp8_quant_impl(result, input, scale):
 
 
 def _silu_mul_static_fp8_quant_impl(out, input, scale, real_num_tokens):
-    lead = input.shape[0]
-    inner = (input.numel() // input.shape[-1]) // max(lead, 1)
-    rows_valid = real_num_tokens.to(torch.int32) * inner if inner != 1 else real_num_tokens.to(torch.int32)
-    _static_fp8_common(out, input, scale, rows_valid, True)
+    _static_fp8_common(out, input, scale, _leading_rows_to_flat(input, real_num_tokens), True)
 
 
 def _moe_sum_pad_impl(out, input, size, dim, keepdim):
@@ -668,3 +669,169 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int, eps: float = 1e-
     else:
         torch.ops._C.dynamic_per_token_group_fp8_quant_with_size(x_q, x_s, x, real_token_num, group_size)
     return x_q, x_s
+
+
+# ---------------------------------------------------------------------------
+# fused-MoE grouped GEMM, block-fp8 and weight-only dense GEMMs
+# (csrc/torch_bindings.cpp:790-849, 1021-1027)
+# ---------------------------------------------------------------------------
+def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids, experts_ids,
+              num_tokens_post_pad, mul_routed_weight, topk, block_size, bias, real_token_num):
+    """``C.view(-1, N)[t] = A[t // topk] @ W[e(t)]^T (* topk_weights.flat[t])``
+    for every id ``t < numel`` listed in ``sorted_token_ids``.  The mode is read
+    off the arguments exactly as the reference's wrapper does
+    (fused_moe_quant_kernel.cpp:68-76, fused_moe.py:146-172)."""
+    rt.require_gpu(C, A, B, A_scale, B_scale, B_zp, topk_weights, topk_ids, sorted_token_ids, experts_ids,
+                   num_tokens_post_pad)
+    if bias is not None:
+        raise RuntimeError("fused_moe kernels take no bias (fused_moe_quant_kernel.cpp:77)")
+    numel = topk_ids.numel()
+    if numel == 0 or A.numel() == 0:
+        return
+    A = A.contiguous()
+    K = A.shape[-1]
+    N = C.shape[-1]
+    if not C.is_contiguous():
+        raise RuntimeError("fused_moe: C must be contiguous")
+    zk, zp, group = _lib.ZP_NONE, None, int(gs)
+    a_scale = w_scale = None
+    if A_scale is not None:
+        if A.dtype == torch.float8_e4m3fn:
+            mode = _lib.Q_FP8_BLOCK
+            a_scale = A_scale.to(torch.float32).contiguous()
+            w_scale = B_scale.to(torch.float32).contiguous()
+            w = B.contiguous()
+            if w.shape[-1] != K:
+                raise RuntimeError(f"fp8 expert weights must be [E, N, K]; got {tuple(w.shape)} for K={K}")
+        elif A.dtype == torch.int8:
+            mode = _lib.Q_INT8
+            a_scale = A_scale.to(torch.float32).reshape(-1).contiguous()
+            if a_scale.numel() not in (A.shape[0],):
+                raise RuntimeError("int8 MoE needs one activation scale per token")
+            w_scale = B_scale.to(torch.float32).reshape(B.shape[0], -1).contiguous()
+            w = B.contiguous()
+        else:
+            raise RuntimeError(f"A_scale given but activations are {A.dtype}")
+        act_code = _lib.F16
+    elif B.dtype == torch.int32 or (B.dtype in (torch.uint8, torch.int8) and B.shape[-1] * 2 == K):
+        mode = _lib.Q_W4A16
+        w = _slab_weight(B, transposed=True)
+        w_scale = B_scale.contiguous()
+        if w_scale.dtype != A.dtype:
+            w_scale = w_scale.to(A.dtype)
+        zp, zk = _zero_points(B_zp, A.dtype)
+        if zp is not None:
+            zp = zp.contiguous()
+        if group <= 0:
+            group = K
+        act_code = rt.dtype_code(A.dtype)
+    elif B.dtype == torch.int8:
+        mode = _lib.Q_W8A16
+        w = B.contiguous()
+        w_scale = B_scale.reshape(B.shape[0], -1).to(A.dtype).contiguous()
+        act_code = rt.dtype_code(A.dtype)
+    elif B.dtype == A.dtype and B_scale is None:
+        mode = _lib.Q_NONE
+        w = B.contiguous()
+        act_code = rt.dtype_code(A.dtype)
+    else:
+        raise RuntimeError(f"fused_moe: cannot infer the quantisation mode from A {A.dtype} / B {B.dtype}")
+    E = w.shape[0]
+    tw = None
+    if mul_routed_weight:
+        tw = topk_weights.to(torch.float32).contiguous()
+        if tw.numel() != numel:
+            raise RuntimeError("fused_moe: topk_weights must have one entry per (token, slot)")
+    for t in (sorted_token_ids, experts_ids, num_tokens_post_pad):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("fused_moe: sorted_token_ids / experts_ids / num_tokens_post_pad must be contiguous int32")
+    if sorted_token_ids.numel() < experts_ids.numel() * block_size:
+        raise RuntimeError("fused_moe: sorted_token_ids is shorter than experts_ids * block_size")
+    with torch.cuda.device(A.device):
+        _lib.call("mi355q_moe_gemm", C.data_ptr(), A.data_ptr(), w.data_ptr(), rt.ptr(a_scale), rt.ptr(w_scale),
+                  rt.ptr(zp), zk, mode, group, rt.ptr(tw), sorted_token_ids.data_ptr(), experts_ids.data_ptr(),
+                  num_tokens_post_pad.data_ptr(), numel, int(topk), int(block_size), experts_ids.numel(), E, K, N,
+                  act_code, rt.dtype_code(C.dtype), rt.stream_ptr())
+
+
+def _fused_moe_quant_kernel_impl(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids,
+                                 experts_ids, num_tokens_post_pad, mul_routed_weight, topk, block_size, bias,
+                                 real_token_num):
+    _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids, experts_ids,
+              num_tokens_post_pad, mul_routed_weight, topk, block_size, bias, real_token_num)
+
+
+def _fused_moe_kernel_impl(C, A, B, topk_weights, topk_ids, sorted_topk_ids, expert_ids, num_tokens_post_pad,
+                           mul_routed_weight, topk, block_size, bias):
+    _moe_gemm(C, A, B, None, None, 0, None, topk_weights, topk_ids, sorted_topk_ids, expert_ids,
+              num_tokens_post_pad, mul_routed_weight, topk, block_size, bias, None)
+
+
+def _kcontig(out, a, w, a_scale, w_scale, bias, mode, group):
+    rt.require_gpu(out, a, w, a_scale, w_scale, bias)
+    a2 = a.reshape(-1, a.shape[-1]).contiguous()
+    M, K = a2.shape
+    N = w.shape[0]
+    if w.shape[1] != K or not w.is_contiguous():
+        raise RuntimeError(f"weight must be contiguous [N, K]; got {tuple(w.shape)} for K={K}")
+    if not out.is_contiguous() or out.shape[-1] != N or out.numel() != M * N:
+        raise RuntimeError("output must be contiguous [.., N]")
+    if bias is not None:
+        bias = bias.to(out.dtype).contiguous()
+    act = _lib.F16 if a.dtype in (torch.float8_e4m3fn, torch.int8) else rt.dtype_code(a.dtype)
+    with torch.cuda.device(a.device):
+        _lib.call("mi355q_kcontig_gemm", out.data_ptr(), a2.data_ptr(), w.data_ptr(), rt.ptr(a_scale),
+                  rt.ptr(w_scale), rt.ptr(bias), mode, group, M, K, N, act, rt.dtype_code(out.dtype),
+                  rt.stream_ptr())
+
+
+def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
+    """fp8 block-scaled GEMM (linear_quant.cpp:16-95): lhs fp8 [.., K] with
+    scales [.., K/128]; rhs fp8 [N, K] with scales [N/128, K/128]."""
+    if lhs.numel() == 0:
+        return
+    if lhs.dtype != torch.float8_e4m3fn or rhs.dtype != torch.float8_e4m3fn:
+        raise RuntimeError("linear_quant: operands must be float8_e4m3fn")
+    _kcontig(out, lhs, rhs, lhs_scale.to(torch.float32).reshape(-1, lhs_scale.shape[-1]).contiguous(),
+             rhs_scale.to(torch.float32).contiguous(), bias, _lib.Q_FP8_BLOCK, 128)
+
+
+def _weight_only_quant_impl(output, input, qweight, bias, scale, group_size):
+    """W8A16 (weight_only_quant.cpp:28-101): qweight int8 [N, K], per-channel scale [N]."""
+    if input.numel() == 0:
+        return
+    if qweight.dtype != torch.int8:
+        raise RuntimeError("weight_only_quant: qweight must be int8 [N, K]")
+    if scale.numel() != qweight.shape[0]:
+        raise RuntimeError("weight_only_quant: only per-channel scales are supported")
+    _kcontig(output, input, qweight, None, scale.reshape(-1).to(input.dtype).contiguous(), bias, _lib.Q_W8A16, -1)
+
+
+# the three operators below are registered from C++ function pointers in the
+# reference (torch_bindings.cpp:793-817), so callers pass everything by position
+_register("_C", "fused_moe_quant_kernel",
+          "(Tensor(a!) C, Tensor A, Tensor B, Tensor? A_scale, Tensor? B_scale, int gs, Tensor? B_zp, "
+          "Tensor topk_weights, Tensor topk_ids, Tensor sorted_token_ids, Tensor experts_ids, "
+          "Tensor num_tokens_post_pad, bool mul_routed_weight, int topk, int block_size, Tensor? bias, "
+          "Tensor? real_token_num) -> ()", _fused_moe_quant_kernel_impl)
+_register("_C", "fused_moe_kernel",
+          "(Tensor(a!) C, Tensor A, Tensor B, Tensor topk_weights, Tensor topk_ids, Tensor sorted_topk_ids, "
+          "Tensor expert_ids, Tensor num_tokens_post_pad, bool mul_routed_weight, int topk, int block_size, "
+          "Tensor? bias) -> ()", _fused_moe_kernel_impl)
+_register("_C", "linear_quant",
+          "(Tensor! out, Tensor lhs, Tensor rhs, Tensor? bias, Tensor lhs_scale, Tensor rhs_scale) -> ()",
+          _linear_quant_impl)
+_register("_C", "weight_only_quant",
+          "(Tensor! output, Tensor input, Tensor qweight, Tensor? bias, Tensor scale, int group_size) -> ()",
+          _weight_only_quant_impl)
+
+
+# vllm_gcu/kernels/_custom_ops.py:564-579
+def w8a8_block_fp8_matmul(A: torch.Tensor, B: torch.Tensor, As: torch.Tensor, Bs: torch.Tensor,
+                          block_size: List[int], output_dtype: torch.dtype = torch.float16,
+                          bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    N, _ = B.shape
+    C_shape = A.shape[:-1] + (N,)
+    C = A.new_empty(C_shape, dtype=output_dtype)
+    torch.ops._C.linear_quant(C, A, B, bias, As, Bs)
+    return C

@@ -71,3 +71,52 @@ def grouped_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk:
     torch.ops._C.fused_grouped_topk(topk_weights, topk_ids, gating_output, topk, renormalize, num_expert_group,
                                     topk_group, e_score_correction_bias, scoring_func)
     return topk_weights, topk_ids
+
+
+def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A_scale: Optional[torch.Tensor],
+                            B_scale: Optional[torch.Tensor], B_zp: Optional[torch.Tensor],
+                            topk_weights: torch.Tensor, topk_ids: torch.Tensor, sorted_token_ids: torch.Tensor,
+                            expert_ids: torch.Tensor, num_tokens_post_padded: torch.Tensor,
+                            mul_routed_weight: bool, top_k: int, config: Dict[str, Any], use_fp8_w8a8: bool,
+                            use_int8_w8a8: bool, use_int8_w8a16: bool, use_int4_w4a16: bool,
+                            block_shape: Optional[List[int]] = None, real_token_num=None,
+                            per_channel_quant=False, bias=None, A_scale_rec=None) -> None:
+    """Same dispatch rules as fused_moe.py:111-231."""
+    assert topk_weights.stride(1) == 1
+    assert sorted_token_ids.stride(0) == 1
+    if use_fp8_w8a8 or use_int8_w8a8:
+        assert B_scale is not None
+    elif use_int8_w8a16 or use_int4_w4a16:
+        assert B_scale is not None
+        assert block_shape and block_shape[0] == 0
+        assert B_zp is None or B_zp.ndim == 3
+    else:
+        assert A_scale is None
+        assert B_scale is None
+    block_size = config["BLOCK_SIZE_M"]
+    if use_fp8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or use_int8_w8a8:
+        if use_fp8_w8a8:
+            B_zp = None
+            if B.dtype == torch.int8:
+                raise NotImplementedError("w4a8-fp8 experts (fused_moe_quant_kernel_ex) are not built")
+            group_size = block_shape[1]
+        elif use_int8_w8a8:
+            B_zp = None
+            group_size = 1
+            if B_scale is not None and B_scale.ndim == 3:
+                B_scale = B_scale.transpose(1, 2).contiguous()
+        elif use_int4_w4a16:
+            A_scale = None
+            group_size = block_shape[1]
+        else:
+            A_scale = None
+            group_size = -1
+            if B_scale.dim() == 3 and B_scale.shape[1] > 1:
+                raise NotImplementedError("group-wise w8a16 experts are not built (per-channel only)")
+        torch.ops._C.fused_moe_quant_kernel(C, A, B, A_scale, B_scale, group_size, B_zp, topk_weights, topk_ids,
+                                            sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                            mul_routed_weight, top_k, block_size, None, real_token_num)
+    else:
+        topk_weights = topk_weights.to(torch.float32)
+        torch.ops._C.fused_moe_kernel(C, A, B, topk_weights, topk_ids, sorted_token_ids, expert_ids,
+                                      num_tokens_post_padded, mul_routed_weight, top_k, block_size, bias)
