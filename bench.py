@@ -127,6 +127,7 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="also time every (shape, M) of the config")
     ap.add_argument("--split-k", type=int, default=0)
     ap.add_argument("--no-w8a8", action="store_true", help="skip the W8A8 int8 GEMM leg")
+    ap.add_argument("--moe", action="store_true", help="also time the two fused-MoE layers of the config")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); "
@@ -192,6 +193,11 @@ def main():
     }
     if not args.no_w8a8:
         out["w8a8_int8"] = w8a8_gemm_bench(ops, dev, stream)
+    if args.moe:
+        out["moe_w4a16"] = moe_bench(ops, dev, stream, "w4a16")
+        torch.cuda.empty_cache()
+        out["moe_fp8_block"] = moe_bench(ops, dev, stream, "fp8")
+        torch.cuda.empty_cache()
     if args.sweep:
         out["sweep"] = sweep(ops, dev, stream, args)
     if not args.no_cpu:
@@ -219,6 +225,69 @@ def w8a8_gemm_bench(ops, dev, stream, iters=20):
             "frac_int8_mfma_peak": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
             "dynamic_quant_us": round(tq * 1e6, 1),
             "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1)}
+
+
+def moe_bench(ops, dev, stream, which, iters=10):
+    """BASELINE configs[3] (Mixtral-8x7B layer, W4A16) and configs[4]
+    (DeepSeek-V3-style layer, fp8 block-scaled): routing + the whole
+    fused-experts sequence, one layer."""
+    import torch
+    from vllm_gcu_amd.kernels import fused_moe
+    from vllm_gcu_amd.kernels.modular_experts import TritonExpertsPad
+    from vllm_gcu_amd.kernels.modular_kernel import FusedMoEModularKernel
+    from vllm_gcu_amd.kernels.prepare_finalize import MoEPrepareAndFinalizeNoEP
+    g = torch.Generator(device="cpu").manual_seed(0)
+
+    def rnd_i32(*shape):
+        # random words filled on the device (the tensors are hundreds of MB)
+        return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device=dev)
+
+    if which == "w4a16":
+        M, H, E, I, T = 512, 4096, 8, 14336, 2
+        w13, w2 = rnd_i32(E, H // 8, 2 * I), rnd_i32(E, I // 8, H)
+        z13, z2 = rnd_i32(E, H // 128, 2 * I // 8), rnd_i32(E, I // 128, H // 8)
+        s13 = (torch.rand(E, H // 128, 2 * I, device=dev) * 0.009 + 0.001).half()
+        s2 = (torch.rand(E, I // 128, H, device=dev) * 0.009 + 0.001).half()
+        x = torch.randn(M, H, generator=g).half().to(dev)
+        logits = torch.randn(M, E, generator=g).to(dev)
+        moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad(use_int4_w4a16=True, block_shape=[0, 128]))
+        kw = dict(w1_scale=s13, w2_scale=s2, w1_zp=z13, w2_zp=z2)
+
+        def step():
+            tw, ids = ops.fused_topk(x, logits, T, True)
+            return moe(x, w13, w2, tw, ids, **kw)
+        flops = 2.0 * M * T * (H * 2 * I + I * H)
+        bytes_ = E * (H * 2 * I + I * H) // 2 + E * (H // 128 * 2 * I + I // 128 * H) * 2 \
+            + E * (H // 128 * 2 * I + I // 128 * H) // 2 + 2 * M * H * 2
+        name = "fused MoE W4A16, Mixtral-8x7B layer: 512 tok, hidden 4096, 8 experts, inter 14336, top-2"
+    else:
+        M, H, E, I, T = 256, 7168, 256, 2048, 8
+
+        def rnd_fp8(*shape):
+            b = torch.randint(0, 256, shape, dtype=torch.uint8, device=dev)
+            b[(b & 0x7f) == 0x7f] = 0                       # no NaN codes
+            return b.view(torch.float8_e4m3fn)
+        w13, w2 = rnd_fp8(E, 2 * I, H), rnd_fp8(E, H, I)
+        s13 = torch.rand(E, 2 * I // 128, H // 128, device=dev) * 1e-4 + 1e-5
+        s2 = torch.rand(E, H // 128, I // 128, device=dev) * 1e-4 + 1e-5
+        x = torch.randn(M, H, generator=g).to(torch.bfloat16).to(dev)
+        logits = torch.randn(M, E, generator=g).to(dev)
+        moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad(use_fp8_w8a8=True, block_shape=[128, 128]))
+        kw = dict(w1_scale=s13, w2_scale=s2)
+
+        def step():
+            tw, ids = fused_moe.grouped_topk(x, logits, T, True, 8, 4, "softmax", None)
+            return moe(x, w13, w2, tw, ids, **kw)
+        tw, ids = fused_moe.grouped_topk(x, logits, T, True, 8, 4, "softmax", None)
+        hit = int(torch.unique(ids).numel())
+        flops = 2.0 * M * T * (H * 2 * I + I * H)
+        bytes_ = hit * (2 * I * H + H * I + 4 * (2 * I // 128 * H // 128 + H // 128 * I // 128)) \
+            + M * H + M * H // 128 * 4 + M * H * 2
+        name = f"fused MoE fp8 block-scaled, DeepSeek-V3-style layer: 256 tok, hidden 7168, 256 experts ({hit} hit), inter 2048, top-8"
+    t = time_graph([step], iters, 2, stream) / iters
+    return {"workload": name, "us": round(t * 1e6, 1), "compulsory_bytes": int(bytes_),
+            "GBps": round(bytes_ / t / 1e9, 1), "frac_hbm": round(bytes_ / t / 1e9 / HBM_PEAK_GBPS, 4),
+            "TFLOPs": round(flops / t / 1e12, 1)}
 
 
 def sweep(ops, dev, stream, args):

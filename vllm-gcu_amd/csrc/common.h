@@ -79,6 +79,15 @@ template <> struct Elem<MI355Q_BF16> {
   static __device__ __forceinline__ uint16_t from_f32(float f) { return f32_to_bf16(f); }
 };
 
+// Kernels whose accumulators alone fill 128+ registers call this once: an
+// inline-asm AGPR operand makes the compiler keep MFMA accumulators in the
+// accumulation half of the register file (AGPR-form MFMA) instead of using it
+// only as a spill area for VGPR-form MFMAs.
+__device__ __forceinline__ void use_agpr_accumulators() {
+  int t = 0;
+  asm volatile("" : "+a"(t));
+}
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 int device_cu_count();

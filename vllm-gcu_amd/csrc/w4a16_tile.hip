@@ -8,8 +8,8 @@
 // the group scale is applied to the fp32 partial sum of each K block -- and
 // every operand is reused for the 8 row tiles, so no weight is dequantised
 // twice in a workgroup.  The activation tile is shared
-// by the 4 wavefronts through LDS (double buffered, rows padded by 16 B so
-// the 16-lane x 16 B operand reads are bank-conflict free).  fp32 accumulate.
+// by the 4 wavefronts through LDS (double buffered, rows padded by 32 B so
+// the operand reads are bank-conflict free).  fp32 accumulate.
 #include "common.h"
 
 namespace mi355q {
@@ -17,7 +17,10 @@ namespace mi355q {
 namespace {
 
 constexpr int BN = 256, BK = 128;
-constexpr int A_ROW = BK * 2 + 16;                 // bytes per LDS row (padded)
+// bytes per LDS row: 256 + 32 of padding.  Measured on MI355X, the MFMA operand
+// read (lane = row + 16 * chunk, 16 B each) runs at the full LDS rate with a
+// 288-byte pitch and at half of it with 272 or 264
+constexpr int A_ROW = BK * 2 + 32;
 
 struct TileArgs {
   uint16_t* out;
@@ -256,7 +259,7 @@ template <int DT, int ZK, int MT, bool GROUPED>
 hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
   constexpr int BM = 16 * MT;
   dim3 grid((a.N + BN - 1) / BN, row_blocks), block(256);
-  const size_t shmem = 2 * BM * A_ROW;             // up to 68 KiB: above the 64 KiB default
+  const size_t shmem = 2 * BM * A_ROW;             // up to 72 KiB: above the 64 KiB default
   static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   if (attr != hipSuccess) return attr;

@@ -4,21 +4,25 @@
 //
 // GEMM: out[M, N] = (xq[M, K] . wq[N, K]^T in int32) * x_scale[m] * w_scale[n].
 // Both operands are K-contiguous (that is what the MFMA lanes consume: 16
-// consecutive k per lane).  Workgroup tile 256 x 256, K step 128, four
-// wavefronts 2 x 2, each 128 x 128 = 8 x 8 MFMA tiles (256 int32 accumulator
-// registers).  Tiles are staged in LDS with a 16-byte-chunk XOR swizzle so the
-// 8-lane groups of a 128-bit LDS read hit 8 different bank groups; LDS is
-// double buffered and the next tile's global loads are issued before the
-// current tile's MFMAs.  The weights take the A operand slot so that each lane
+// consecutive k per lane).  Workgroup tile 256 x 256, K step 64, eight
+// wavefronts 2 (M) x 4 (N), each 128 rows x 64 columns = 8 x 4 MFMA tiles (128
+// int32 accumulator registers, two wavefronts per SIMD so one's LDS reads hide
+// behind the other's MFMAs).  Tiles go from global memory straight into LDS (global_load ...
+// lds, 16 B per lane, no staging registers) with a 16-byte-chunk XOR swizzle
+// so a 128-bit LDS operand read hits 16 different bank groups; LDS is a ring
+// of 4 K tiles of 64, three of them in flight while one feeds the MFMAs.  The weights take the A operand slot so that each lane
 // ends up with 4 consecutive output columns (one 8-byte store).
 #include "common.h"
 
 namespace mi355q {
 namespace {
 
-constexpr int TM = 256, TN = 256, TK = 128;
-constexpr int TILE_BYTES = 256 * TK;              // one operand tile (32 KiB)
+constexpr int TM = 256, TN = 256, TK = 64;
+constexpr int NSTAGE = 4;                         // LDS ring: 3 K tiles in flight behind the one in use
+constexpr int TILE_BYTES = 256 * TK;              // one operand tile (16 KiB)
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;       // x tile + w tile
+constexpr int CHUNKS = TK / 16;                   // 16-byte chunks per tile row
+constexpr int ROWS_PER_COPY = 64 / CHUNKS;        // tile rows moved by one wavefront copy
 
 struct I8Args {
   void* out;                // [M, N] f16 / bf16 / f32, row stride ldo elements
@@ -34,7 +38,11 @@ struct I8Args {
   int n_panels_swizzle;     // non-zero: XCD-aware tile order
 };
 
-__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ (row & 7); }
+// 16-byte chunk `chunk` of a 64-byte tile row lives in slot chunk ^ ((row >> 1) & 3).
+// Measured on MI355X with a 16-wavefront ds_read_b128 loop: the MFMA operand
+// read (lane = row + 16 * chunk) runs at the full 230 B/clk/CU with this
+// swizzle and at half that with none or with (row >> 2) & 3.
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 3); }
 
 template <int DT>
 __device__ __forceinline__ void store4(void* out, long idx, const float* v) {
@@ -56,18 +64,33 @@ __device__ __forceinline__ float load_bias(const void* bias, int bias_f32, int n
   return Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT>::to_f32(((const uint16_t*)bias)[n]);
 }
 
+// one wavefront instruction copies 64 x 16 B from global memory straight into
+// 1 KiB of LDS (lane l lands at base + 16 l); no registers, no LDS store
+__device__ __forceinline__ void dma16(const void* gptr, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+#ifndef MQ_I8_WAVES_N
+#define MQ_I8_WAVES_N 4
+#endif
+constexpr int WAVES_N = MQ_I8_WAVES_N;            // wavefronts along N (2 along M)
+constexpr int GEMM_THREADS = 128 * WAVES_N;
+constexpr int NI = 16 / WAVES_N, NJ = 8;          // MFMA tiles per wavefront: NI*16 columns x 128 rows
+
 template <int DT>
-__global__ void __launch_bounds__(256, 1)
+__global__ void __launch_bounds__(GEMM_THREADS, 1)
 w8a8_int8_gemm_kernel(I8Args a) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kq = lane >> 4;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  if (NI * NJ * 4 > 128) use_agpr_accumulators();
   const int M = a.M, N = a.N, K = a.K;
 
   // tile coordinates; with the swizzle, the workgroups that land on one XCD
   // (ids congruent mod 8) sweep all row tiles of the same weight panels
-  const int mtiles = (M + TM - 1) / TM, ntiles = (N + TN - 1) / TN;
+  const int mtiles = (M + TM - 1) / TM;
   int pid = blockIdx.x, tm, tn;
   if (a.n_panels_swizzle) {
     const int x = pid & 7, j = pid >> 3;
@@ -77,81 +100,139 @@ w8a8_int8_gemm_kernel(I8Args a) {
     tm = pid % mtiles;
     tn = pid / mtiles;
   }
-  (void)ntiles;
   const int m0 = tm * TM, n0 = tn * TN;
 
-  i4 acc[8][8];      // [n tile][m tile]: weights are the MFMA "A" operand
+  i4 acc[NI][NJ];    // [n tile][m tile]: weights are the MFMA "A" operand
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = (i4){0, 0, 0, 0};
+    for (int j = 0; j < NJ; ++j) acc[i][j] = (i4){0, 0, 0, 0};
 
-  // global -> LDS staging: each operand tile is 256 rows x 8 chunks of 16 B;
-  // thread t copies chunks t, t + 256, ... (8 per operand)
-  u4 xr[8], wr[8];
-  const int srow = tid >> 3, schunk = tid & 7;
-  auto gload = [&](int k0) {
+  // global -> LDS: an operand tile is 256 rows x TK bytes; one wavefront copy
+  // moves 1 KiB = ROWS_PER_COPY rows (lane = CHUNKS * row + slot); slot p of
+  // row r holds the 16-byte chunk swz(r, p) of that row, which makes the MFMA
+  // operand reads below bank-conflict free.
+  constexpr int COPIES = 256 / ROWS_PER_COPY / (2 * WAVES_N);   // per wavefront and operand
+  const int crow = lane / CHUNKS, cslot = lane % CHUNKS;
+  // 32-bit byte offsets from the tile's first row (rows past the matrix edge
+  // re-read the last row; their results are never stored)
+  uint32_t xo[COPIES], wo[COPIES];
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int r = p * 32 + srow;
-      const int xm = min(m0 + r, M - 1), wn_ = min(n0 + r, N - 1);
-      xr[p] = *(const u4*)(a.x + (long)xm * a.ldx + k0 + 16 * schunk);
-      wr[p] = *(const u4*)(a.w + (long)wn_ * a.ldw + k0 + 16 * schunk);
-    }
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* xs = lds + stage * STAGE_BYTES;
-    unsigned char* ws = xs + TILE_BYTES;
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int r = p * 32 + srow;
-      const int off = r * TK + swz(r, schunk) * 16;
-      *(u4*)(xs + off) = xr[p];
-      *(u4*)(ws + off) = wr[p];
-    }
-  };
-
-  gload(0);
-  lstore(0);
-  __syncthreads();
-
-  const int nk = K / TK;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int stage = kt & 1;
-    gload(min(kt + 1, nk - 1) * TK);
-    const unsigned char* xs = lds + stage * STAGE_BYTES;
-    const unsigned char* ws = xs + TILE_BYTES;
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      i4 bx[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int r = wm * 128 + j * 16 + l16;
-        bx[j] = *(const i4*)(xs + r * TK + swz(r, 4 * s + kq) * 16);
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int r = wn * 128 + i * 16 + l16;
-        const i4 aw = *(const i4*)(ws + r * TK + swz(r, 4 * s + kq) * 16);
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aw, bx[j], acc[i][j], 0, 0, 0);
-      }
-    }
-    lstore(stage ^ 1);
-    __syncthreads();
+  for (int p = 0; p < COPIES; ++p) {
+    const int r = (wave * COPIES + p) * ROWS_PER_COPY + crow;   // row of the tile, 0..255
+    const int chunk = swz(r, cslot);
+    xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * chunk);
+    wo[p] = (uint32_t)((min(n0 + r, N - 1) - n0) * a.ldw + 16 * chunk);
   }
+  const int8_t* xtile = a.x + (long)m0 * a.ldx;
+  const int8_t* wtile = a.w + (long)n0 * a.ldw;
+  auto issue = [&](int stage, int k0) {
+    unsigned char* xs = lds + stage * STAGE_BYTES + wave * COPIES * 1024;
+    unsigned char* ws = xs + TILE_BYTES;
+    const int8_t* xk = xtile + k0;
+    const int8_t* wk = wtile + k0;
+#pragma unroll
+    for (int p = 0; p < COPIES; ++p) {
+      dma16(xk + xo[p], xs + p * 1024);
+      dma16(wk + wo[p], ws + p * 1024);
+    }
+  };
+
+  // per-lane LDS read address: row l16 of a 16-row tile, logical chunk kq; the
+  // swizzle term only depends on the row modulo 16, so it is the same for
+  // every tile and tiles differ by a compile-time offset
+  const uint32_t lo = (uint32_t)(l16 * TK + swz(l16, kq) * 16);
+  const uint32_t xwave = wm * (16 * NJ) * TK, wwave = TILE_BYTES + wn * (16 * NI) * TK;
+
+  // Ring of NSTAGE K tiles in LDS and two register sets of MFMA operands.
+  // Iteration kt multiplies tile kt (already in registers) while it reads
+  // tile kt+1 from LDS into the other register set and starts the copy of
+  // tile kt+3; tile kt+2 is in flight.  The barrier at the top guarantees that
+  // everybody's copies of tile kt+1 have landed and that the buffer refilled
+  // next (tile kt-1's) is no longer read.  Every iteration issues exactly one
+  // tile (the tail re-reads the last one into a buffer nobody uses), so the
+  // wait counts below are constants.
+  static_assert(NSTAGE == 4 && (COPIES == 2 || COPIES == 4), "wait counts assume 2 * COPIES copy instructions per tile");
+  const int nk = K / TK;
+  struct Frag { i4 bx[NJ]; i4 aw[NI]; };
+  auto read_bx = [&](Frag& f, int tile) {
+    const unsigned char* xb = lds + (tile % NSTAGE) * STAGE_BYTES + xwave + lo;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) f.bx[j] = *(const i4*)(xb + j * 16 * TK);
+  };
+  auto read_aw = [&](Frag& f, int tile) {
+    const unsigned char* wb = lds + (tile % NSTAGE) * STAGE_BYTES + wwave + lo;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) f.aw[i] = *(const i4*)(wb + i * 16 * TK);
+  };
+  auto mma = [&](const Frag& f, int ib, int ie) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      if (i < ib || i >= ie) continue;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if (NI * NJ * 4 > 128) {
+          // 256 accumulator registers = the whole accumulation register file:
+          // the in-place AGPR form is spelled out so that no accumulator is
+          // ever copied (each one is next touched 64 MFMAs later)
+          asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(f.aw[i]), "v"(f.bx[j]));
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f.aw[i], f.bx[j], acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  };
+  // The LDS reads of the next tile are issued in two batches of at most 8,
+  // each followed by half of the current tile's MFMAs: the wait for the
+  // current operands can then leave the newer reads outstanding (the LDS
+  // counter only counts to 15).
+  auto step = [&](const Frag& cur, Frag& nxt, int kt) {
+    __builtin_amdgcn_s_waitcnt(COPIES == 2 ? 0x0f74 : 0x0f78);   // vmcnt(2 * COPIES): my copies of tile kt+1 landed
+    __builtin_amdgcn_s_barrier();                  // bare barrier: a fence would drain the ring
+    issue((kt + 3) % NSTAGE, min(kt + 3, nk - 1) * TK);
+    if (NI * NJ * 4 > 128) {
+      read_bx(nxt, kt + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(cur, 0, NI / 2);
+      __builtin_amdgcn_sched_barrier(0);
+      read_aw(nxt, kt + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(cur, NI / 2, NI);
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      // two wavefronts per SIMD: the instruction scheduler is free to mix the
+      // next tile's LDS reads into this tile's MFMAs
+      read_bx(nxt, kt + 1);
+      read_aw(nxt, kt + 1);
+      mma(cur, 0, NI);
+    }
+  };
+
+#pragma unroll
+  for (int p = 0; p < 3; ++p) issue(p, min(p, nk - 1) * TK);
+  Frag f0, f1;
+  __builtin_amdgcn_s_waitcnt(COPIES == 2 ? 0x0f78 : 0x4f70);    // vmcnt(4 * COPIES): tile 0 landed
+  __builtin_amdgcn_s_barrier();
+  read_bx(f0, 0);
+  read_aw(f0, 0);
+  for (int kt = 0; kt < nk; kt += 2) {             // nk is even (K % 128 == 0)
+    step(f0, f1, kt);
+    step(f1, f0, kt + 1);
+  }
+  // no copy may still be writing LDS when the workgroup retires
+  __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
+  if (NI * NJ * 4 > 128) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // last MFMA results settle before they are read
 
   // ---- epilogue: lane holds, per (n tile i, m tile j), output row
   // m = .. + l16 and columns n = .. + 4 kq + {0..3}
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int m = m0 + wm * 128 + j * 16 + l16;
+  for (int j = 0; j < NJ; ++j) {
+    const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
     if (m >= M) continue;
     const float xsc = a.x_scale ? a.x_scale[a.x_scale_per_row ? m : 0] : 1.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int n = n0 + wn * 128 + i * 16 + 4 * kq;
+    for (int i = 0; i < NI; ++i) {
+      const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
       if (n >= N) continue;                     // N is a multiple of 4
       if (a.acc_out) *(i4*)(a.acc_out + (long)m * N + n) = acc[i][j];
       float v[4];
@@ -218,12 +299,12 @@ int launch_gemm(const I8Args& a, hipStream_t st) {
   const int mtiles = (a.M + TM - 1) / TM, ntiles = (a.N + TN - 1) / TN;
   I8Args b = a;
   b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
-  const size_t shmem = 2 * STAGE_BYTES;          // 128 KiB
+  const size_t shmem = NSTAGE * STAGE_BYTES;     // 128 KiB
   static hipError_t attr = hipFuncSetAttribute((const void*)w8a8_int8_gemm_kernel<DT>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   MQ_REQUIRE(attr == hipSuccess, "w8a8_int8_gemm: cannot reserve %zu bytes of LDS: %s", shmem,
              hipGetErrorString(attr));
-  hipLaunchKernelGGL((w8a8_int8_gemm_kernel<DT>), dim3(mtiles * ntiles), dim3(256), shmem, st, b);
+  hipLaunchKernelGGL((w8a8_int8_gemm_kernel<DT>), dim3(mtiles * ntiles), dim3(GEMM_THREADS), shmem, st, b);
   MQ_LAUNCH_CHECK("w8a8_int8_gemm");
   return 0;
 }
@@ -240,7 +321,7 @@ extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* 
   MQ_REQUIRE(M >= 0 && N > 0 && K > 0, "w8a8_int8_gemm: bad shape M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
   MQ_REQUIRE(out && x && w, "w8a8_int8_gemm: null pointer");
-  MQ_REQUIRE(K % TK == 0, "w8a8_int8_gemm: K=%d must be a multiple of %d", K, TK);
+  MQ_REQUIRE(K % 128 == 0, "w8a8_int8_gemm: K=%d must be a multiple of 128", K);
   MQ_REQUIRE(N % 4 == 0, "w8a8_int8_gemm: N=%d must be a multiple of 4", N);
   MQ_REQUIRE(ldx % 16 == 0 && ldw % 16 == 0 && ldx >= K && ldw >= K,
              "w8a8_int8_gemm: operand row strides (%ld, %ld) must be >= K and multiples of 16", ldx, ldw);
