@@ -127,6 +127,8 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="also time every (shape, M) of the config")
     ap.add_argument("--split-k", type=int, default=0)
     ap.add_argument("--no-w8a8", action="store_true", help="skip the W8A8 int8 GEMM leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a 256 MiB device copy at the end (reference reading for rocprofv3 --pmc)")
     ap.add_argument("--moe", action="store_true", help="also time the two fused-MoE layers of the config")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -200,6 +202,15 @@ def main():
         torch.cuda.empty_cache()
     if args.sweep:
         out["sweep"] = sweep(ops, dev, stream, args)
+    if args.calibrate_copy:
+        # a plain copy of known size: its FETCH_SIZE / WRITE_SIZE readings scale
+        # the counters of the profiled kernels to bytes
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["calibration_copy_bytes"] = int(src.numel())
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_w4a16(M)
     print(json.dumps(out))

@@ -1,0 +1,273 @@
+"""The quantization method classes (create_weights -> load checkpoint tensors ->
+process_weights_after_loading -> apply) against the CPU oracle, the way a
+model layer drives them (gptq.py:105-296, awq.py:69-134, w8a8.py:88-171,
+fp8.py:49-205, moe_wna16.py:160-643 of the reference)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8 as of8
+from oracle import moe as om
+from oracle import w4 as ow4
+from oracle import w8a8 as o8
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def load(layer, name, value):
+    p = getattr(layer, name)
+    assert tuple(p.shape) == tuple(value.shape), (name, p.shape, value.shape)
+    p.data = value.to(p.dtype) if value.dtype != p.dtype else value
+
+
+def int4_case(rng, K, N, g):
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8)
+    s = rng.uniform(0.001, 0.01, size=(K // g, N)).astype(np.float16)
+    return q, z, s
+
+
+@pytest.mark.parametrize("M", [1, 16, 300])
+def test_gptq_linear_method(M):
+    from vllm_gcu_amd.kernels.quantization.gptq import GPTQGCUConfig
+    print(f"case gptq method M={M}", flush=True)
+    K, N, g = 1024, 768, 128
+    rng = np.random.default_rng(M)
+    q, z, s = int4_case(rng, K, N, g)
+    method = GPTQGCUConfig.from_config({"bits": 4, "group_size": g}).get_quant_method()
+    layer = torch.nn.Module()
+    method.create_weights(layer, K, [512, 256], K, N, torch.float16)
+    layer.cuda()
+    load(layer, "qweight", dev(ow4.gptq_pack_weight(q)))
+    load(layer, "qzeros", dev(ow4.gptq_pack_zeros(z)))
+    load(layer, "scales", dev(s))
+    method.process_weights_after_loading(layer)
+    x = rng.standard_normal((2, M, K)).astype(np.float16) if M == 16 else rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    out = method.apply(layer, dev(x), dev(bias))
+    want = ow4.w4a16_gemm(x.reshape(-1, K).astype(np.float32), q, z, s.astype(np.float32), g, bias.astype(np.float32))
+    assert out.shape == x.shape[:-1] + (N,)
+    np.testing.assert_allclose(out.float().cpu().numpy().reshape(-1, N), want, rtol=RTOL, atol=ATOL)
+    assert method.apply(layer, dev(x[:0])).shape[0] == 0
+
+
+def test_gptq_rejects_act_order_and_bad_group():
+    from vllm_gcu_amd.kernels.quantization.gptq import GPTQGCUConfig
+    method = GPTQGCUConfig(4, 128).get_quant_method()
+    layer = torch.nn.Module()
+    with pytest.raises(ValueError):
+        method.create_weights(layer, 192, [128], 192, 128, torch.float16)
+    method.create_weights(layer, 256, [128], 256, 128, torch.float16)
+    layer.cuda()
+    layer.g_idx.data = layer.g_idx.data.flip(0).contiguous()
+    with pytest.raises(ValueError):
+        method.process_weights_after_loading(layer)
+
+
+def test_gptq_8bit_symmetric():
+    from vllm_gcu_amd.kernels.quantization.gptq import GPTQGCUConfig
+    K, N = 512, 256
+    rng = np.random.default_rng(8)
+    w = rng.integers(0, 256, size=(K, N), dtype=np.uint8)                 # stored value, true weight = w - 128
+    s = rng.uniform(0.001, 0.01, size=(1, N)).astype(np.float16)
+    method = GPTQGCUConfig(8, -1).get_quant_method()
+    layer = torch.nn.Module()
+    method.create_weights(layer, K, [N], K, N, torch.float16)
+    layer.cuda()
+    packed = w.reshape(K // 4, 4, N).astype(np.uint32)
+    packed = (packed[:, 0] | (packed[:, 1] << 8) | (packed[:, 2] << 16) | (packed[:, 3] << 24)).view(np.int32)
+    load(layer, "qweight", dev(packed))
+    load(layer, "qzeros", dev(np.full((1, N // 4), 0x7f7f7f7f, dtype=np.int32)))
+    load(layer, "scales", dev(s))
+    method.process_weights_after_loading(layer)
+    x = rng.standard_normal((7, K)).astype(np.float16)
+    out = method.apply(layer, dev(x))
+    want = x.astype(np.float32) @ ((w.astype(np.float32) - 128) * s.astype(np.float32))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    layer.qzeros = None
+    layer2 = torch.nn.Module()
+    method.create_weights(layer2, K, [N], K, N, torch.float16)
+    layer2.cuda()
+    layer2.qzeros.data.zero_()
+    with pytest.raises(ValueError):
+        method.process_weights_after_loading(layer2)
+
+
+@pytest.mark.parametrize("M,dtype", [(4, torch.float16), (200, torch.bfloat16)])
+def test_awq_linear_method(M, dtype):
+    from vllm_gcu_amd.kernels.quantization.awq import AWQGCUConfig
+    print(f"case awq method M={M}", flush=True)
+    K, N, g = 512, 1024, 128
+    rng = np.random.default_rng(M)
+    q, z, s = int4_case(rng, K, N, g)
+    method = AWQGCUConfig.from_config({"w_bit": 4, "q_group_size": g, "zero_point": True}).get_quant_method()
+    layer = torch.nn.Module()
+    method.create_weights(layer, K, [N], K, N, dtype)
+    layer.cuda()
+    load(layer, "qweight", dev(ow4.awq_pack(q)))
+    load(layer, "qzeros", dev(ow4.awq_pack(z)))
+    sd = torch.from_numpy(s).to(dtype)
+    load(layer, "scales", sd.cuda())
+    method.process_weights_after_loading(layer)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    out = method.apply(layer, x.cuda())
+    want = ow4.w4a16_gemm(x.float().numpy(), q, z, sd.float().numpy(), g)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL * max(1.0, np.abs(want).max() / 8))
+
+
+def test_w8a8_linear_method_static_input_scales():
+    from vllm_gcu_amd.kernels.quantization.w8a8 import W8A8Config
+    print("case w8a8 method", flush=True)
+    M, K, N = 37, 512, 384
+    rng = np.random.default_rng(5)
+    w = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    in_scales = rng.uniform(0.01, 0.05, size=K).astype(np.float16)
+    out_scales = rng.uniform(1e-4, 1e-3, size=N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    method = W8A8Config().get_quant_method()
+    layer = torch.nn.Module()
+    method.create_weights(layer, K, [N], K, N, torch.float16)
+    layer.cuda()
+    load(layer, "weight", dev(w))
+    load(layer, "in_scales", dev(in_scales))
+    load(layer, "out_scales", dev(out_scales))
+    method.process_weights_after_loading(layer)
+    out = method.apply(layer, dev(x), dev(bias))
+    xq = o8.static_scaled_int8_quant(x, in_scales)
+    acc = o8.int8_gemm_i32(xq, np.ascontiguousarray(w.T))
+    want = o8.scaled_mm_epilogue(acc, 1.0, out_scales, bias.astype(np.float32))
+    assert out.dtype == torch.float16 and out.shape == (M, N)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_compressed_tensors_int8_kernel_dynamic():
+    from vllm_gcu_amd.kernels.quantization.w8a8 import CompressedTensorMMLinearKernel
+    M, K, N = 20, 256, 512
+    rng = np.random.default_rng(6)
+    w = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    ws = rng.uniform(1e-3, 1e-2, size=(N, 1)).astype(np.float32)
+    x = rng.standard_normal((2, M, K)).astype(np.float16)
+    layer = torch.nn.Module()
+    layer.weight = torch.nn.Parameter(dev(w), requires_grad=False)
+    layer.weight_scale = torch.nn.Parameter(dev(ws), requires_grad=False)
+    k = CompressedTensorMMLinearKernel()
+    k.process_weights_after_loading(layer)
+    out = k.apply_weights(layer, dev(x))
+    xq, xs = o8.dynamic_scaled_int8_quant(x.reshape(-1, K))
+    want = o8.scaled_mm_epilogue(o8.int8_gemm_i32(xq, np.ascontiguousarray(w.T)), xs, ws.reshape(-1))
+    assert out.shape == (2, M, N)
+    np.testing.assert_allclose(out.float().cpu().numpy().reshape(-1, N), want, rtol=RTOL, atol=ATOL)
+
+
+def test_fp8_linear_method_block_scaled():
+    from vllm_gcu_amd.kernels.quantization.fp8 import Fp8GCUConfig
+    print("case fp8 method", flush=True)
+    M, K, N = 33, 512, 768
+    rng = np.random.default_rng(7)
+    w = of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 0.5, -448, 448).astype(np.float32))
+    ws = rng.uniform(0.02, 0.1, size=(N // 128, K // 128)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.bfloat16)
+    layer = torch.nn.Module()
+    layer.weight = torch.nn.Parameter(dev(w).view(torch.float8_e4m3fn), requires_grad=False)
+    layer.weight_scale_inv = torch.nn.Parameter(dev(ws), requires_grad=False)
+    method = Fp8GCUConfig.from_config({"weight_block_size": [128, 128]}).get_quant_method()
+    out = method.apply(layer, x.cuda(), bias.cuda())
+    xq, xs = of8.per_token_group_quant_fp8(x.float().numpy(), 128)
+    want = of8.block_fp8_gemm(xq, xs, w, ws) + bias.float().numpy()
+    assert out.dtype == torch.bfloat16 and out.shape == (M, N)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+
+
+@pytest.mark.parametrize("fmt", ["gptq", "awq"])
+def test_moe_wna16_method(fmt):
+    from vllm_gcu_amd.kernels.quantization.moe_wna16 import MoeWNA16GCUConfig
+    print(f"case moe_wna16 method {fmt}", flush=True)
+    M, E, T, H, I, g = 40, 8, 2, 512, 384, 128
+    rng = np.random.default_rng(9)
+    q13 = rng.integers(0, 16, size=(E, H, 2 * I), dtype=np.uint8)
+    q2 = rng.integers(0, 16, size=(E, I, H), dtype=np.uint8)
+    z13 = rng.integers(0, 16, size=(E, H // g, 2 * I), dtype=np.uint8)
+    z2 = rng.integers(0, 16, size=(E, I // g, H), dtype=np.uint8)
+    s13 = rng.uniform(0.001, 0.01, size=(E, H // g, 2 * I)).astype(np.float16)
+    s2 = rng.uniform(0.001, 0.01, size=(E, I // g, H)).astype(np.float16)
+    pw = ow4.gptq_pack_weight if fmt == "gptq" else ow4.awq_pack
+    pz = ow4.gptq_pack_zeros if fmt == "gptq" else ow4.awq_pack
+    layer = torch.nn.Module()
+    for name, qq, zz, ss in (("w13", q13, z13, s13), ("w2", q2, z2, s2)):
+        setattr(layer, f"{name}_qweight", torch.nn.Parameter(dev(np.stack([pw(a) for a in qq])), requires_grad=False))
+        setattr(layer, f"{name}_qzeros", torch.nn.Parameter(dev(np.stack([pz(a) for a in zz])), requires_grad=False))
+        setattr(layer, f"{name}_scales", torch.nn.Parameter(dev(ss), requires_grad=False))
+    method = MoeWNA16GCUConfig(fmt, 4, g, True).get_quant_method()
+    method.process_weights_after_loading(layer)
+    x = rng.standard_normal((M, H)).astype(np.float16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    out = method.apply(layer, dev(x).clone(), dev(logits), top_k=T, renormalize=True)
+    two, ido, _ = om.topk_softmax(logits, T, True)
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)   # noqa: E731
+    want = om.fused_experts(x.astype(np.float32), lambda e: ow4.dequantize(q13[e], z13[e], s13[e].astype(np.float32), g),
+                            lambda e: ow4.dequantize(q2[e], z2[e], s2[e].astype(np.float32), g), two, ido, f16)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_fp8_and_int8_moe_methods_grouped_routing():
+    from vllm_gcu_amd.kernels.quantization.fp8 import Fp8GCUConfig
+    from vllm_gcu_amd.kernels.quantization.w8a8 import W8A8Config
+    print("case fp8/int8 moe methods", flush=True)
+    M, E, T, H, I = 24, 16, 4, 256, 256
+    rng = np.random.default_rng(10)
+    x = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).to(torch.bfloat16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    two, ido = om.grouped_topk(logits, T, True, 4, 2, "sigmoid", None)
+    bf16 = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).float().numpy()   # noqa: E731
+    route = dict(top_k=T, renormalize=True, use_grouped_topk=True, topk_group=2, num_expert_group=4,
+                 scoring_func="sigmoid")
+    # fp8 block-scaled experts
+    w13 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, 2 * I, H)) * 0.5, -448, 448).astype(np.float32))
+    w2 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, H, I)) * 0.5, -448, 448).astype(np.float32))
+    s13 = rng.uniform(0.02, 0.1, size=(E, 2 * I // 128, H // 128)).astype(np.float32)
+    s2 = rng.uniform(0.02, 0.1, size=(E, H // 128, I // 128)).astype(np.float32)
+    layer = torch.nn.Module()
+    layer.w13_weight = dev(w13).view(torch.float8_e4m3fn)
+    layer.w2_weight = dev(w2).view(torch.float8_e4m3fn)
+    layer.w13_weight_scale_inv, layer.w2_weight_scale_inv = dev(s13), dev(s2)
+    out = Fp8GCUConfig().get_quant_method(moe=True).apply(layer, x.cuda().clone(), dev(logits), **route)
+
+    def deq(codes, sc):
+        return (of8.from_e4m3fn(codes) * np.repeat(np.repeat(sc, 128, 0), 128, 1)).T
+
+    def qdq(a):
+        qa, sa = of8.per_token_group_quant_fp8(a, 128)
+        return of8.from_e4m3fn(qa) * np.repeat(sa, 128, -1)
+
+    want = om.fused_experts(qdq(x.float().numpy()), lambda e: deq(w13[e], s13[e]), lambda e: deq(w2[e], s2[e]),
+                            two, ido, bf16, quant_a2=qdq)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+
+    # int8 per-channel experts, per-token dynamic activations
+    w13i = rng.integers(-127, 128, size=(E, 2 * I, H), dtype=np.int8)
+    w2i = rng.integers(-127, 128, size=(E, H, I), dtype=np.int8)
+    c13 = rng.uniform(1e-3, 4e-3, size=(E, 2 * I)).astype(np.float32)
+    c2 = rng.uniform(1e-3, 4e-3, size=(E, H)).astype(np.float32)
+    m8 = W8A8Config().get_quant_method(moe=True)
+    layer8 = torch.nn.Module()
+    m8.create_weights(layer8, E, H, I, torch.bfloat16)
+    layer8.cuda()
+    load(layer8, "w13_weight", dev(w13i)); load(layer8, "w2_weight", dev(w2i))
+    load(layer8, "w13_out_scales", dev(c13)); load(layer8, "w2_out_scales", dev(c2))
+    out8 = m8.apply(layer8, x.cuda().clone(), dev(logits), **route)
+
+    def qdq8(a):
+        qa, sa = o8.dynamic_scaled_int8_quant(a)
+        return qa.astype(np.float32) * sa
+
+    want8 = om.fused_experts(qdq8(x.float().numpy()), lambda e: (w13i[e].astype(np.float32) * c13[e][:, None]).T,
+                             lambda e: (w2i[e].astype(np.float32) * c2[e][:, None]).T, two, ido, bf16, quant_a2=qdq8)
+    np.testing.assert_allclose(out8.float().cpu().numpy(), want8, rtol=2 * RTOL,
+                               atol=ATOL * max(1.0, np.abs(want8).max()))

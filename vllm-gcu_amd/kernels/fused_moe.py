@@ -73,6 +73,25 @@ def grouped_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk:
     return topk_weights, topk_ids
 
 
+def select_experts(hidden_states: torch.Tensor, router_logits: torch.Tensor, top_k: int, use_grouped_topk: bool,
+                   renormalize: bool, topk_group: Optional[int] = None, num_expert_group: Optional[int] = None,
+                   custom_routing_function=None, scoring_func: str = "softmax",
+                   e_score_correction_bias: Optional[torch.Tensor] = None):
+    """``FusedMoE.select_experts`` as the reference's MoE methods call it
+    (moe_wna16.py:612-623, w8a8.py:312-323, fp8.py:120-131): grouped top-k when
+    the model uses expert groups, a custom routing function if given, else
+    softmax top-k."""
+    from . import _custom_ops as ops
+    if use_grouped_topk:
+        assert topk_group is not None and num_expert_group is not None
+        return grouped_topk(hidden_states, router_logits, top_k, renormalize, num_expert_group, topk_group,
+                            scoring_func, e_score_correction_bias)
+    if custom_routing_function is not None:
+        return custom_routing_function(hidden_states=hidden_states, gating_output=router_logits, topk=top_k,
+                                       renormalize=renormalize)
+    return ops.fused_topk(hidden_states, router_logits, top_k, renormalize)
+
+
 def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A_scale: Optional[torch.Tensor],
                             B_scale: Optional[torch.Tensor], B_zp: Optional[torch.Tensor],
                             topk_weights: torch.Tensor, topk_ids: torch.Tensor, sorted_token_ids: torch.Tensor,

@@ -1,0 +1,95 @@
+"""fp8-e4m3fn block-scaled linear / MoE methods on MI355X.
+
+Mirrors ``Fp8GCULinearMethod`` / ``Fp8GCUMoEMethod`` and
+``apply_w8a8_block_fp8_linear`` (vllm_gcu/kernels/quantization/fp8.py:49-205).
+"""
+from typing import List, Optional
+
+import torch
+
+from .. import _custom_ops as ops
+from ..fused_moe import select_experts
+from ..modular_experts import TritonExpertsPad
+from ..modular_kernel import FusedMoEModularKernel
+from ..prepare_finalize import MoEPrepareAndFinalizeNoEP
+from .utils import register_gcu_quantization_config
+
+
+def apply_w8a8_block_fp8_linear(input: torch.Tensor, weight: torch.Tensor, block_size: List[int],
+                                weight_scale: torch.Tensor, input_scale: Optional[torch.Tensor] = None,
+                                bias: Optional[torch.Tensor] = None,
+                                cutlass_block_fp8_supported: bool = False) -> torch.Tensor:
+    output_dtype = input.dtype
+    if input_scale is None:
+        q_input, x_scale = ops.per_token_group_quant_fp8(input, block_size[1], dtype=torch.float8_e4m3fn,
+                                                         column_major_scales=False)
+    else:
+        # already quantised upstream (fp8.py:189-192); the 16-bit dtype cannot be
+        # recovered from the fp8 view, so the output defaults to bfloat16
+        q_input, x_scale = input.view(torch.float8_e4m3fn), input_scale
+        output_dtype = torch.bfloat16 if input.dtype == torch.float8_e4m3fn else input.dtype
+    output_shape = [*q_input.shape[:-1], weight.shape[0]]
+    output = ops.w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size,
+                                       output_dtype=output_dtype, bias=None)
+    if bias is not None:
+        output += bias
+    return output.to(dtype=output_dtype).view(*output_shape)
+
+
+@register_gcu_quantization_config("fp8_gcu")
+class Fp8GCUConfig:
+    def __init__(self, weight_block_size=(128, 128)):
+        self.weight_block_size = list(weight_block_size)
+
+    @classmethod
+    def get_name(cls) -> str:
+        return "fp8_gcu"
+
+    @classmethod
+    def from_config(cls, config):
+        return cls(config.get("weight_block_size", [128, 128]))
+
+    def get_quant_method(self, layer=None, prefix: str = "", moe: bool = False):
+        return Fp8GCUMoEMethod(self) if moe else Fp8GCULinearMethod(self)
+
+
+class Fp8GCULinearMethod:
+    """Weights ``weight`` fp8 [N, K] and ``weight_scale_inv`` f32 [N/128, K/128]."""
+
+    def __init__(self, quant_config: Fp8GCUConfig):
+        self.quant_config = quant_config
+        self.block_quant = quant_config.weight_block_size is not None
+
+    def apply(self, layer, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              x_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if not self.block_quant:
+            raise NotImplementedError("per-tensor fp8 linear is not built; block-quantised only")
+        return apply_w8a8_block_fp8_linear(input=x, weight=layer.weight,
+                                           block_size=self.quant_config.weight_block_size,
+                                           weight_scale=layer.weight_scale_inv,
+                                           input_scale=getattr(layer, "input_scale", None) if x_scale is None else x_scale,
+                                           bias=bias)
+
+
+class Fp8GCUMoEMethod:
+    """Experts ``w13_weight`` fp8 [E, 2I, H], ``w2_weight`` fp8 [E, H, I] with
+    ``*_weight_scale_inv`` f32 block scales (fp8.py:72-166)."""
+
+    def __init__(self, quant_config: Fp8GCUConfig):
+        self.quant_config = quant_config
+        self.fused_experts = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), self.select_gemm_impl())
+
+    def select_gemm_impl(self, prepare_finalize=None, moe=None):
+        return TritonExpertsPad(use_fp8_w8a8=True, block_shape=self.quant_config.weight_block_size)
+
+    def apply(self, layer, x, router_logits, top_k: int, renormalize: bool, use_grouped_topk: bool = False,
+              global_num_experts: int = -1, expert_map=None, topk_group=None, num_expert_group=None,
+              custom_routing_function=None, scoring_func: str = "softmax", e_score_correction_bias=None,
+              activation: str = "silu", apply_router_weight_on_input: bool = False):
+        topk_weights, topk_ids = select_experts(x, router_logits, top_k, use_grouped_topk, renormalize,
+                                                topk_group, num_expert_group, custom_routing_function,
+                                                scoring_func, e_score_correction_bias)
+        return self.fused_experts(x, layer.w13_weight, layer.w2_weight, topk_weights=topk_weights,
+                                  topk_ids=topk_ids, inplace=True, activation=activation,
+                                  global_num_experts=global_num_experts, expert_map=expert_map,
+                                  w1_scale=layer.w13_weight_scale_inv, w2_scale=layer.w2_weight_scale_inv)

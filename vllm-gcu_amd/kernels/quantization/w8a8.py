@@ -1,0 +1,122 @@
+"""W8A8 int8 linear methods on MI355X.
+
+``W8A8LinearMethod`` mirrors vllm_gcu/kernels/quantization/w8a8.py:88-171
+(static per-channel input scales, single fused output scale, ``dot_bias_quant``).
+``CompressedTensorMMLinearKernel`` mirrors compressed_tensor.py:14-41 (dynamic
+per-token activation scales, ``cutlass_scaled_mm``).  The reference transposes
+the weight to ``[K, N]`` at load time for its hardware; the int8 MFMA consumes
+K-contiguous operands, so the checkpoint's ``[N, K]`` tensor is kept and the
+operator is handed its ``.t()`` view.
+"""
+from typing import Optional
+
+import torch
+from torch.nn import Parameter
+
+from .. import _custom_ops as ops
+from ..fused_moe import select_experts
+from ..modular_experts import TritonExpertsPad
+from ..modular_kernel import FusedMoEModularKernel
+from ..prepare_finalize import MoEPrepareAndFinalizeNoEP
+from .utils import register_gcu_quantization_config
+
+
+@register_gcu_quantization_config("w8a8_gcu")
+class W8A8Config:
+    @classmethod
+    def get_name(cls) -> str:
+        return "w8a8_gcu"
+
+    @classmethod
+    def get_supported_act_dtypes(cls):
+        return [torch.half, torch.bfloat16]
+
+    @classmethod
+    def from_config(cls, config):
+        return cls()
+
+    def get_quant_method(self, layer=None, prefix: str = "", moe: bool = False):
+        return FusedW8A8MoEMethod(self) if moe else W8A8LinearMethod(self)
+
+
+class W8A8LinearMethod:
+    def __init__(self, quant_config: W8A8Config):
+        self.quant_config = quant_config
+
+    def create_weights(self, layer, input_size_per_partition, output_partition_sizes, input_size,
+                       output_size, params_dtype, **extra_weight_attrs):
+        layer.out_dtype = params_dtype
+        out = sum(output_partition_sizes)
+        layer.register_parameter("weight", Parameter(torch.empty(out, input_size_per_partition, dtype=torch.int8),
+                                                     requires_grad=False))          # (N, K)
+        layer.register_parameter("out_scales", Parameter(torch.ones(out, dtype=torch.float32),
+                                                         requires_grad=False))      # (N)
+        layer.register_parameter("in_scales", Parameter(torch.ones(input_size_per_partition, dtype=params_dtype),
+                                                        requires_grad=False))       # (K)
+
+    def process_weights_after_loading(self, layer) -> None:
+        # keep [N, K] storage; the operator sees the [K, N] view
+        layer.weight = Parameter(layer.weight.data.contiguous(), requires_grad=False)
+
+    def apply(self, layer, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if x.dtype in self.quant_config.get_supported_act_dtypes():
+            x = ops.scaled_int8_quant(x, layer.in_scales)[0]
+        assert x.dtype == torch.int8
+        shape = list(x.shape)
+        shape[-1] = int(layer.weight.shape[0])
+        output = torch.empty(shape, dtype=layer.out_dtype, device=x.device)
+        ops.dot_bias_quant(output, x, layer.weight.t(), layer.out_scales, bias)
+        return output
+
+
+class CompressedTensorMMLinearKernel:
+    """Dynamic per-token int8 activations x per-channel int8 weights."""
+
+    def process_weights_after_loading(self, layer) -> None:
+        layer.weight = Parameter(layer.weight.data.contiguous(), requires_grad=False)   # [N, K]
+
+    def apply_weights(self, layer, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        x_q, x_s, _ = ops.scaled_int8_quant(x.contiguous(), getattr(layer, "input_scale", None))
+        x_2d = x_q.reshape(-1, x_q.shape[-1])
+        out = ops.cutlass_scaled_mm(x_2d, layer.weight.t(), x_s, layer.weight_scale, x.dtype, bias)
+        return out.reshape(x.shape[:-1] + (layer.weight.shape[0],))
+
+
+class FusedW8A8MoEMethod:
+    """int8 experts ``w13_weight [E, 2I, H]`` / ``w2_weight [E, H, I]`` with
+    per-channel ``*_out_scales`` (w8a8.py:174-345).  Activations are quantised
+    per token on the fly; ``*_in_scales`` of the checkpoint (static per-channel
+    smoothing scales) are forwarded when the layer carries them."""
+
+    def __init__(self, quant_config: W8A8Config):
+        self.quant_config = quant_config
+        self.fused_experts = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), self.select_gemm_impl())
+
+    def select_gemm_impl(self, prepare_finalize=None, moe=None):
+        return TritonExpertsPad(use_int8_w8a8=True, per_channel_quant=True, per_act_token_quant=True)
+
+    def create_weights(self, layer, num_experts, hidden_size, intermediate_size_per_partition, params_dtype,
+                       **extra_weight_attrs):
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+
+        def reg(name, t):
+            layer.register_parameter(name, Parameter(t, requires_grad=False))
+        reg("w13_weight", torch.empty(E, 2 * I, H, dtype=torch.int8))
+        reg("w2_weight", torch.empty(E, H, I, dtype=torch.int8))
+        reg("w13_out_scales", torch.zeros(E, 2 * I, dtype=torch.float32))
+        reg("w2_out_scales", torch.zeros(E, H, dtype=torch.float32))
+
+    def apply(self, layer, x, router_logits, top_k: int, renormalize: bool, use_grouped_topk: bool = False,
+              global_num_experts: int = -1, expert_map=None, topk_group=None, num_expert_group=None,
+              custom_routing_function=None, scoring_func: str = "softmax", e_score_correction_bias=None,
+              activation: str = "silu", apply_router_weight_on_input: bool = False):
+        topk_weights, topk_ids = select_experts(x, router_logits, top_k, use_grouped_topk, renormalize,
+                                                topk_group, num_expert_group, custom_routing_function,
+                                                scoring_func, e_score_correction_bias)
+        return self.fused_experts(x, layer.w13_weight, layer.w2_weight, topk_weights=topk_weights,
+                                  topk_ids=topk_ids, inplace=True, activation=activation,
+                                  global_num_experts=global_num_experts, expert_map=expert_map,
+                                  w1_scale=layer.w13_out_scales, w2_scale=layer.w2_out_scales,
+                                  a1_scale=getattr(layer, "w13_in_scales", None),
+                                  a2_scale=getattr(layer, "w2_in_scales", None),
+                                  apply_router_weight_on_input=apply_router_weight_on_input)
