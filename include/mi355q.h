@@ -80,8 +80,10 @@ int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight,
                       const void* bias, int M, int K, int N, int group_size,
                       int dtype, void* workspace, size_t workspace_bytes,
                       void* stream);
-/* tuning hook used by the benchmark: force the split-K factor (0 = auto) and
- * the kernel family (0 = auto, 1 = streaming, 2 = LDS/MFMA) */
+/* tuning hook used by the benchmark.  split_k: bits 0..7 force the split-K
+ * factor, bits 8..15 the tiles (of 16 columns) per workgroup of the streaming
+ * kernel (1, 2, 4 or 8); 0 in a field = automatic.  family: 0 = auto,
+ * 1 = streaming, 2 = LDS/MFMA. */
 int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          const void* scales, const void* zeros, int zeros_kind,
                          const void* bias, int M, int K, int N, int group_size,
@@ -198,6 +200,14 @@ int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scal
 int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_scale,
                         const void* w_scale, const void* bias, int quant_mode, int group_size, int M,
                         int K, int N, int act_dtype, int out_dtype, void* stream);
+
+/* ---- measurement probe -------------------------------------------------------
+ * No counterpart in the reference.  Streams `bytes` of device memory through
+ * `workgroups` workgroups of 256 threads with 16-byte loads and no arithmetic:
+ * the time of this read of a kernel's weight bytes is the floor the benchmark
+ * quotes next to the weight-streaming kernels.  bytes must be a multiple of
+ * workgroups * 32 KiB; sink is 16 writable bytes (never written in practice). */
+int mi355q_probe_stream_read(const void* src, size_t bytes, int workgroups, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -47,6 +47,7 @@ SIGNATURES = {
     "mi355q_moe_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
+    "mi355q_probe_stream_read": (c_int, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
     "mi355q_kcontig_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_int, c_void_p]),
 }

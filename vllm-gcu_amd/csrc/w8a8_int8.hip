@@ -4,25 +4,26 @@
 //
 // GEMM: out[M, N] = (xq[M, K] . wq[N, K]^T in int32) * x_scale[m] * w_scale[n].
 // Both operands are K-contiguous (that is what the MFMA lanes consume: 16
-// consecutive k per lane).  Workgroup tile 256 x 256, K step 64, eight
-// wavefronts 2 (M) x 4 (N), each 128 rows x 64 columns = 8 x 4 MFMA tiles (128
-// int32 accumulator registers, two wavefronts per SIMD so one's LDS reads hide
-// behind the other's MFMAs).  Tiles go from global memory straight into LDS (global_load ...
-// lds, 16 B per lane, no staging registers) with a 16-byte-chunk XOR swizzle
-// so a 128-bit LDS operand read hits 16 different bank groups; LDS is a ring
-// of 4 K tiles of 64, three of them in flight while one feeds the MFMAs.  The weights take the A operand slot so that each lane
-// ends up with 4 consecutive output columns (one 8-byte store).
+// consecutive k per lane).  A workgroup of eight wavefronts owns a 256 x TN
+// output tile, TN = 256 (2 x 4 wavefronts of 128 x 64) or 224 (4 x 2 wavefronts
+// of 64 x 112; 28672 = 128 x 224, so the Llama-3-70B MLP shape makes exactly
+// four full rounds of 256 workgroups).  K advances in LDS tiles of 128 bytes
+// per row: a whole 128-byte line per row and request, which halves the L2
+// request count of a 64-byte tile (the L2 was the busiest unit).  Tiles go
+// from global memory straight into LDS (global_load ... lds, 16 B per lane, no
+// staging registers) with a 16-byte-chunk XOR swizzle that keeps the 128-bit
+// operand reads bank-conflict free.  Two LDS stages and two register sets of
+// operands: while half a tile (k = 64) is multiplied, the next half's operands
+// are read from LDS, and the copy of the tile after next is in flight.  The
+// weights take the A operand slot so that each lane ends up with 4 consecutive
+// output columns (one 8-byte store).
 #include "common.h"
 
 namespace mi355q {
 namespace {
 
-constexpr int TM = 256, TN = 256, TK = 64;
-constexpr int NSTAGE = 4;                         // LDS ring: 3 K tiles in flight behind the one in use
-constexpr int TILE_BYTES = 256 * TK;              // one operand tile (16 KiB)
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;       // x tile + w tile
-constexpr int CHUNKS = TK / 16;                   // 16-byte chunks per tile row
-constexpr int ROWS_PER_COPY = 64 / CHUNKS;        // tile rows moved by one wavefront copy
+constexpr int TM = 256, TKB = 128;                // tile rows of x, bytes of K per LDS tile row
+constexpr int GEMM_THREADS = 512;
 
 struct I8Args {
   void* out;                // [M, N] f16 / bf16 / f32, row stride ldo elements
@@ -37,12 +38,6 @@ struct I8Args {
   int x_scale_per_row, w_scale_per_col, bias_f32;
   int n_panels_swizzle;     // non-zero: XCD-aware tile order
 };
-
-// 16-byte chunk `chunk` of a 64-byte tile row lives in slot chunk ^ ((row >> 1) & 3).
-// Measured on MI355X with a 16-wavefront ds_read_b128 loop: the MFMA operand
-// read (lane = row + 16 * chunk) runs at the full 230 B/clk/CU with this
-// swizzle and at half that with none or with (row >> 2) & 3.
-__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 3); }
 
 template <int DT>
 __device__ __forceinline__ void store4(void* out, long idx, const float* v) {
@@ -71,180 +66,257 @@ __device__ __forceinline__ void dma16(const void* gptr, void* lds_wave_base) {
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
-#ifndef MQ_I8_WAVES_N
-#define MQ_I8_WAVES_N 4
-#endif
-constexpr int WAVES_N = MQ_I8_WAVES_N;            // wavefronts along N (2 along M)
-constexpr int GEMM_THREADS = 128 * WAVES_N;
-constexpr int NI = 16 / WAVES_N, NJ = 8;          // MFMA tiles per wavefront: NI*16 columns x 128 rows
-
-template <int DT>
+// WM x WN wavefronts, each NJ x NI MFMA tiles of 16 x 16 (rows of x by rows of w)
+template <int DT, int WM, int WN, int NI, int NJ>
 __global__ void __launch_bounds__(GEMM_THREADS, 1)
 w8a8_int8_gemm_kernel(I8Args a) {
+  static_assert(WM * WN == 8 && WM * NJ * 16 == TM, "eight wavefronts cover 256 rows of x");
+  constexpr int TN = WN * NI * 16;
+  constexpr int X_BYTES = TM * TKB, W_BYTES = TN * TKB, STAGE_BYTES = X_BYTES + W_BYTES;
+  constexpr int XCOPIES = TM / 8 / 8;                   // 1 KiB copies (8 rows) per wavefront, x tile
+  constexpr int WGROUPS = TN / 8;                       // 8-row groups of the w tile
+  constexpr int WCOPIES = (WGROUPS + 7) / 8;
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kq = lane >> 4;
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  if (NI * NJ * 4 > 128) use_agpr_accumulators();
+  const int wm = wave / WN, wn = wave % WN;
   const int M = a.M, N = a.N, K = a.K;
 
-  // tile coordinates; with the swizzle, the workgroups that land on one XCD
-  // (ids congruent mod 8) sweep all row tiles of the same weight panels
+  // Persistent workgroups: workgroup w takes output tiles w, w + grid, ...
+  // Tile coordinates: with the swizzle, the tiles whose id is congruent mod 8
+  // (they run on one XCD, the grid being a multiple of 8) sweep all row tiles
+  // of the same weight panels.
   const int mtiles = (M + TM - 1) / TM;
-  int pid = blockIdx.x, tm, tn;
-  if (a.n_panels_swizzle) {
-    const int x = pid & 7, j = pid >> 3;
-    tm = j % mtiles;
-    tn = (j / mtiles) * 8 + x;
-  } else {
-    tm = pid % mtiles;
-    tn = pid / mtiles;
-  }
-  const int m0 = tm * TM, n0 = tn * TN;
+  const int total_tiles = mtiles * ((N + TN - 1) / TN);
+  auto tile_origin = [&](int tile, int& m0, int& n0) {
+    int tm, tn;
+    if (a.n_panels_swizzle) {
+      const int x = tile & 7, j = tile >> 3;
+      tm = j % mtiles;
+      tn = (j / mtiles) * 8 + x;
+    } else {
+      tm = tile % mtiles;
+      tn = tile / mtiles;
+    }
+    m0 = tm * TM;
+    n0 = tn * TN;
+  };
 
   i4 acc[NI][NJ];    // [n tile][m tile]: weights are the MFMA "A" operand
-#pragma unroll
-  for (int i = 0; i < NI; ++i)
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) acc[i][j] = (i4){0, 0, 0, 0};
 
-  // global -> LDS: an operand tile is 256 rows x TK bytes; one wavefront copy
-  // moves 1 KiB = ROWS_PER_COPY rows (lane = CHUNKS * row + slot); slot p of
-  // row r holds the 16-byte chunk swz(r, p) of that row, which makes the MFMA
-  // operand reads below bank-conflict free.
-  constexpr int COPIES = 256 / ROWS_PER_COPY / (2 * WAVES_N);   // per wavefront and operand
-  const int crow = lane / CHUNKS, cslot = lane % CHUNKS;
-  // 32-bit byte offsets from the tile's first row (rows past the matrix edge
-  // re-read the last row; their results are never stored)
-  uint32_t xo[COPIES], wo[COPIES];
+  // global -> LDS.  One copy moves 8 tile rows of 128 bytes: lane = 8 * row +
+  // slot, and slot p of row r receives the row's 16-byte chunk p ^ (r & 7), so
+  // that the operand reads below (16 rows x 4 chunks per instruction) spread
+  // over all banks.  8 consecutive lanes fetch one whole 128-byte line.
+  // Wavefront v copies row groups v, v + 8, ...; rows past the matrix edge
+  // re-read the last row (their results are never stored).
+  const int crow = lane >> 3, cchunk = (lane & 7) ^ (crow & 7);
+  uint32_t xo[XCOPIES], wo[WCOPIES];
+  const int8_t *xtile, *wtile;
+  auto set_copy_tile = [&](int tile) {         // the output tile whose operands the copies fetch
+    int m0, n0;
+    tile_origin(tile, m0, n0);
 #pragma unroll
-  for (int p = 0; p < COPIES; ++p) {
-    const int r = (wave * COPIES + p) * ROWS_PER_COPY + crow;   // row of the tile, 0..255
-    const int chunk = swz(r, cslot);
-    xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * chunk);
-    wo[p] = (uint32_t)((min(n0 + r, N - 1) - n0) * a.ldw + 16 * chunk);
-  }
-  const int8_t* xtile = a.x + (long)m0 * a.ldx;
-  const int8_t* wtile = a.w + (long)n0 * a.ldw;
-  auto issue = [&](int stage, int k0) {
-    unsigned char* xs = lds + stage * STAGE_BYTES + wave * COPIES * 1024;
-    unsigned char* ws = xs + TILE_BYTES;
-    const int8_t* xk = xtile + k0;
-    const int8_t* wk = wtile + k0;
+    for (int p = 0; p < XCOPIES; ++p) {
+      const int r = (wave + 8 * p) * 8 + crow;
+      xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * cchunk);
+    }
 #pragma unroll
-    for (int p = 0; p < COPIES; ++p) {
-      dma16(xk + xo[p], xs + p * 1024);
-      dma16(wk + wo[p], ws + p * 1024);
+    for (int p = 0; p < WCOPIES; ++p) {
+      const int r = (wave + 8 * p) * 8 + crow;
+      wo[p] = (uint32_t)((min(n0 + r, N - 1) - n0) * a.ldw + 16 * cchunk);
+    }
+    xtile = a.x + (long)m0 * a.ldx;
+    wtile = a.w + (long)n0 * a.ldw;
+  };
+  // copy slot s of this wavefront: slots 0 .. XCOPIES-1 are its x row groups,
+  // the rest its w row groups (the last one only exists for some wavefronts)
+  constexpr int NSLOT = XCOPIES + WCOPIES;
+  auto copy_slot = [&](int s, int stage, int k0) {
+    unsigned char* xs = lds + stage * STAGE_BYTES;
+    if (s < XCOPIES) {
+      dma16(xtile + k0 + xo[s], xs + (wave + 8 * s) * 1024);
+    } else {
+      const int p = s - XCOPIES;
+      if (wave + 8 * p < WGROUPS) dma16(wtile + k0 + wo[p < WCOPIES ? p : 0], xs + X_BYTES + (wave + 8 * p) * 1024);
     }
   };
+  auto issue = [&](int stage, int k0) {
+#pragma unroll
+    for (int s = 0; s < NSLOT; ++s) copy_slot(s, stage, k0);
+  };
 
-  // per-lane LDS read address: row l16 of a 16-row tile, logical chunk kq; the
-  // swizzle term only depends on the row modulo 16, so it is the same for
-  // every tile and tiles differ by a compile-time offset
-  const uint32_t lo = (uint32_t)(l16 * TK + swz(l16, kq) * 16);
-  const uint32_t xwave = wm * (16 * NJ) * TK, wwave = TILE_BYTES + wn * (16 * NI) * TK;
-
-  // Ring of NSTAGE K tiles in LDS and two register sets of MFMA operands.
-  // Iteration kt multiplies tile kt (already in registers) while it reads
-  // tile kt+1 from LDS into the other register set and starts the copy of
-  // tile kt+3; tile kt+2 is in flight.  The barrier at the top guarantees that
-  // everybody's copies of tile kt+1 have landed and that the buffer refilled
-  // next (tile kt-1's) is no longer read.  Every iteration issues exactly one
-  // tile (the tail re-reads the last one into a buffer nobody uses), so the
-  // wait counts below are constants.
-  static_assert(NSTAGE == 4 && (COPIES == 2 || COPIES == 4), "wait counts assume 2 * COPIES copy instructions per tile");
-  const int nk = K / TK;
+  // Operand reads: lane (l16, kq) of half h takes chunk 4 h + kq of row l16 of
+  // each 16-row MFMA tile.  They are written in assembly and waited for by
+  // hand: with a direct-to-LDS copy in flight the compiler turns every wait it
+  // inserts itself into "wait for everything", which would serialise the
+  // reads of the next operands with the MFMAs of the current ones; reads it
+  // cannot see need no wait of its own.  lds_wait ties the registers to the
+  // wait so that their first use cannot move above it.
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
+  uint32_t lo[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) lo[h] = lds_base + (uint32_t)(l16 * TKB + (((4 * h + kq) ^ (l16 & 7)) * 16));
+  const uint32_t xwave = wm * (16 * NJ) * TKB, wwave = X_BYTES + wn * (16 * NI) * TKB;
   struct Frag { i4 bx[NJ]; i4 aw[NI]; };
-  auto read_bx = [&](Frag& f, int tile) {
-    const unsigned char* xb = lds + (tile % NSTAGE) * STAGE_BYTES + xwave + lo;
+  // read r of an operand set: r < NJ is x tile r, the rest are w tiles
+  auto read_one = [&](Frag& f, int r, uint32_t xb, uint32_t wb) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) f.bx[j] = *(const i4*)(xb + j * 16 * TK);
+    for (int j = 0; j < NJ; ++j)
+      if (r == j) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.bx[j]) : "v"(xb), "n"(j * 16 * TKB));
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      if (r == NJ + i) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.aw[i]) : "v"(wb), "n"(i * 16 * TKB));
   };
-  auto read_aw = [&](Frag& f, int tile) {
-    const unsigned char* wb = lds + (tile % NSTAGE) * STAGE_BYTES + wwave + lo;
+  auto read_frag = [&](Frag& f, int stage, int h) {
+    const uint32_t xb = lo[h] + (uint32_t)(stage * STAGE_BYTES) + xwave;
+    const uint32_t wb = lo[h] + (uint32_t)(stage * STAGE_BYTES) + wwave;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) f.aw[i] = *(const i4*)(wb + i * 16 * TK);
+    for (int r = 0; r < NJ + NI; ++r) read_one(f, r, xb, wb);
   };
-  auto mma = [&](const Frag& f, int ib, int ie) {
+  auto lds_wait = [&](Frag& f) {
+    // "s_waitcnt lgkmcnt(0)" with every operand register as an in/out operand
+    // (each register exactly once: a duplicate would come back as a stale copy)
+    static_assert((NJ == 8 && NI == 4) || (NJ == 4 && NI == 7), "operand lists are written out");
+    if constexpr (NJ == 8) {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(f.bx[0]), "+v"(f.bx[1]), "+v"(f.bx[2]), "+v"(f.bx[3]), "+v"(f.bx[4]), "+v"(f.bx[5]),
+                     "+v"(f.bx[6]), "+v"(f.bx[7]), "+v"(f.aw[0]), "+v"(f.aw[1]), "+v"(f.aw[2]), "+v"(f.aw[3]));
+    } else {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(f.bx[0]), "+v"(f.bx[1]), "+v"(f.bx[2]), "+v"(f.bx[3]), "+v"(f.aw[0]), "+v"(f.aw[1]),
+                     "+v"(f.aw[2]), "+v"(f.aw[3]), "+v"(f.aw[4]), "+v"(f.aw[5]), "+v"(f.aw[6]));
+    }
+  };
+  // One half: the MFMAs of `cur`, and between them (a) the LDS reads of the
+  // next operand set `nxt`, one after each of the first MFMAs, and (b) copy
+  // slots SB .. SE-1 of a later tile, the first after MFMA C0 and then one
+  // every CE MFMAs.  Everything a wavefront has to issue besides MFMAs is
+  // spread out like this on purpose: the eight wavefronts run in lockstep
+  // behind the workgroup barrier, so a phase of reads or copies of its own
+  // would idle the matrix pipes of the whole CU (a burst of copies also blocks
+  // every wavefront in the address unit, 64 B/clk per CU).
+#ifndef MQ_I8_RE
+#define MQ_I8_RE 2
+#endif
+  constexpr int RE = MQ_I8_RE;                      // one LDS read every RE MFMAs
+  auto half = [&](const Frag& cur, Frag& nxt, int rstage, int rh, int SB, int SE, int C0, int CE,
+                  int cstage, int k0) {
+    const uint32_t xb = lo[rh] + (uint32_t)(rstage * STAGE_BYTES) + xwave;
+    const uint32_t wb = lo[rh] + (uint32_t)(rstage * STAGE_BYTES) + wwave;
+    int n = 0;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      if (i < ib || i >= ie) continue;
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        if (NI * NJ * 4 > 128) {
-          // 256 accumulator registers = the whole accumulation register file:
-          // the in-place AGPR form is spelled out so that no accumulator is
-          // ever copied (each one is next touched 64 MFMAs later)
-          asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(f.aw[i]), "v"(f.bx[j]));
-        } else {
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f.aw[i], f.bx[j], acc[i][j], 0, 0, 0);
-        }
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.aw[i], cur.bx[j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (n % RE == 0 && n / RE < NJ + NI) read_one(nxt, n / RE, xb, wb);
+        if (n >= C0 && (n - C0) % CE == 0 && SB + (n - C0) / CE < SE) copy_slot(SB + (n - C0) / CE, cstage, k0);
+        __builtin_amdgcn_sched_barrier(0);
+        ++n;
+      }
+  };
+  constexpr int NM = NI * NJ;
+  static_assert(NM > 3 + 3 * (NSLOT - 1) && NM >= RE * (NJ + NI), "not enough MFMAs to spread the copies and reads");
+
+  // The K tiles of all the output tiles of this workgroup form one stream;
+  // stream element g lives in LDS stage g % 2.  Half 0 of element g multiplies
+  // (g, 0) while it reads (g, 1); half 1 multiplies (g, 1) while it reads
+  // (g + 1, 0) and issues the copy of element g + 2 into g's stage.  The
+  // barrier between the halves means: everybody's copies of element g + 1 have
+  // landed, and everybody has finished reading element g.  The stream runs
+  // across output tiles, so the first K tiles of the next output tile arrive
+  // while the epilogue of this one runs; past the last output tile the copies
+  // re-read its last K tile into a stage nobody reads.
+  const int nt = K / TKB;
+  int tile = blockIdx.x;
+  set_copy_tile(tile);
+  issue(0, 0);
+  issue(1, min(1, nt - 1) * TKB);
+  int copy_tile = tile;
+  if (nt == 1 && tile + (int)gridDim.x < total_tiles) {      // element 1 already belongs to the next output tile
+    copy_tile = tile + gridDim.x;
+    set_copy_tile(copy_tile);
+    issue(1, 0);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  Frag f0, f1;
+  read_frag(f0, 0, 0);
+  lds_wait(f0);
+  int g = 0;                                       // stream position of the current K tile
+  for (; tile < total_tiles; tile += gridDim.x) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) acc[i][j] = (i4){0, 0, 0, 0};
+    for (int T = 0; T < nt; ++T, ++g) {
+      const int st = g & 1;
+      half(f0, f1, st, 1, 0, 0, 0, 1, st, 0);
+      lds_wait(f1);
+      __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): my copies of element g + 1 landed
+      __builtin_amdgcn_s_barrier();                // bare barrier: the waits are explicit, no fence needed
+      // element g + 2: K tile (T + 2) % nt of output tile number (T + 2) / nt after this one
+      int kt = T + 2, ahead = 0;
+      while (kt >= nt) { kt -= nt; ++ahead; }
+      const int want = tile + ahead * (int)gridDim.x;
+      if (want >= total_tiles) kt = nt - 1;        // past the end: harmless re-read, never consumed
+      else if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
+      half(f1, f0, st ^ 1, 0, 0, NSLOT, 3, 3, st, kt * TKB);
+      lds_wait(f0);
+    }
+
+    // ---- epilogue: lane holds, per (n tile i, m tile j), output row
+    // m = .. + l16 and columns n = .. + 4 kq + {0..3}.  Every scale and bias
+    // value the lane needs is loaded before the first store: the compiler must
+    // assume the output may alias them, so loads placed between the stores
+    // would each wait out a full memory round trip.
+    int m0, n0;
+    tile_origin(tile, m0, n0);
+    float xsc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int m = min(m0 + wm * (16 * NJ) + j * 16 + l16, M - 1);
+      xsc[j] = a.x_scale ? a.x_scale[a.x_scale_per_row ? m : 0] : 1.0f;
+    }
+    float wsc[NI][4], bia[NI][4];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = min(n0 + wn * (16 * NI) + i * 16 + 4 * kq, N - 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        wsc[i][e] = a.w_scale ? a.w_scale[a.w_scale_per_col ? n + e : 0] : 1.0f;
+        bia[i][e] = a.bias ? load_bias<DT>(a.bias, a.bias_f32, n + e) : 0.0f;
       }
     }
-  };
-  // The LDS reads of the next tile are issued in two batches of at most 8,
-  // each followed by half of the current tile's MFMAs: the wait for the
-  // current operands can then leave the newer reads outstanding (the LDS
-  // counter only counts to 15).
-  auto step = [&](const Frag& cur, Frag& nxt, int kt) {
-    __builtin_amdgcn_s_waitcnt(COPIES == 2 ? 0x0f74 : 0x0f78);   // vmcnt(2 * COPIES): my copies of tile kt+1 landed
-    __builtin_amdgcn_s_barrier();                  // bare barrier: a fence would drain the ring
-    issue((kt + 3) % NSTAGE, min(kt + 3, nk - 1) * TK);
-    if (NI * NJ * 4 > 128) {
-      read_bx(nxt, kt + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      mma(cur, 0, NI / 2);
-      __builtin_amdgcn_sched_barrier(0);
-      read_aw(nxt, kt + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      mma(cur, NI / 2, NI);
-      __builtin_amdgcn_sched_barrier(0);
-    } else {
-      // two wavefronts per SIMD: the instruction scheduler is free to mix the
-      // next tile's LDS reads into this tile's MFMAs
-      read_bx(nxt, kt + 1);
-      read_aw(nxt, kt + 1);
-      mma(cur, 0, NI);
-    }
-  };
-
 #pragma unroll
-  for (int p = 0; p < 3; ++p) issue(p, min(p, nk - 1) * TK);
-  Frag f0, f1;
-  __builtin_amdgcn_s_waitcnt(COPIES == 2 ? 0x0f78 : 0x4f70);    // vmcnt(4 * COPIES): tile 0 landed
-  __builtin_amdgcn_s_barrier();
-  read_bx(f0, 0);
-  read_aw(f0, 0);
-  for (int kt = 0; kt < nk; kt += 2) {             // nk is even (K % 128 == 0)
-    step(f0, f1, kt);
-    step(f1, f0, kt + 1);
+    for (int j = 0; j < NJ; ++j) {
+      const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
+      if (m >= M) continue;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+        if (n >= N) continue;                     // N is a multiple of 4
+        if (a.acc_out) *(i4*)(a.acc_out + (long)m * N + n) = acc[i][j];
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = ((float)acc[i][j][e] * xsc[j]) * wsc[i][e];
+          if (a.bias) v[e] += bia[i][e];
+        }
+        store4<DT>(a.out, (long)m * a.ldo + n, v);
+      }
+    }
+    // The operands of the next output tile's first half are read again here
+    // rather than kept from the last half above: that frees their registers
+    // for the epilogue (the copy has landed: it was waited for at the last
+    // barrier of the K loop).
+    read_frag(f0, g & 1, 0);
+    lds_wait(f0);
   }
   // no copy may still be writing LDS when the workgroup retires
   __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
-  if (NI * NJ * 4 > 128) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // last MFMA results settle before they are read
-
-  // ---- epilogue: lane holds, per (n tile i, m tile j), output row
-  // m = .. + l16 and columns n = .. + 4 kq + {0..3}
-#pragma unroll
-  for (int j = 0; j < NJ; ++j) {
-    const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
-    if (m >= M) continue;
-    const float xsc = a.x_scale ? a.x_scale[a.x_scale_per_row ? m : 0] : 1.0f;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
-      if (n >= N) continue;                     // N is a multiple of 4
-      if (a.acc_out) *(i4*)(a.acc_out + (long)m * N + n) = acc[i][j];
-      float v[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float wsc = a.w_scale ? a.w_scale[a.w_scale_per_col ? n + e : 0] : 1.0f;
-        v[e] = ((float)acc[i][j][e] * xsc) * wsc;
-        if (a.bias) v[e] += load_bias<DT>(a.bias, a.bias_f32, n + e);
-      }
-      store4<DT>(a.out, (long)m * a.ldo + n, v);
-    }
-  }
 }
 
 // ---- activation quantisers -------------------------------------------------
@@ -294,19 +366,34 @@ static_int8_quant_kernel(int8_t* out, const void* x, const float* scale, int per
   out[i] = sat_rne_s8(ld_act<DT>(x, i) * inv);
 }
 
-template <int DT>
-int launch_gemm(const I8Args& a, hipStream_t st) {
+template <int DT, int WM, int WN, int NI, int NJ>
+int launch_tile(const I8Args& a, hipStream_t st) {
+  constexpr int TN = WN * NI * 16;
   const int mtiles = (a.M + TM - 1) / TM, ntiles = (a.N + TN - 1) / TN;
   I8Args b = a;
   b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
-  const size_t shmem = NSTAGE * STAGE_BYTES;     // 128 KiB
-  static hipError_t attr = hipFuncSetAttribute((const void*)w8a8_int8_gemm_kernel<DT>,
+  const size_t shmem = 2 * (size_t)(TM + TN) * TKB;      // two stages, 120 or 128 KiB
+  static hipError_t attr = hipFuncSetAttribute((const void*)w8a8_int8_gemm_kernel<DT, WM, WN, NI, NJ>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   MQ_REQUIRE(attr == hipSuccess, "w8a8_int8_gemm: cannot reserve %zu bytes of LDS: %s", shmem,
              hipGetErrorString(attr));
-  hipLaunchKernelGGL((w8a8_int8_gemm_kernel<DT>), dim3(mtiles * ntiles), dim3(GEMM_THREADS), shmem, st, b);
+  // one workgroup per CU (a multiple of 8, so tile id mod 8 stays the XCD)
+  int grid = mtiles * ntiles, cus = device_cu_count() / 8 * 8;
+  if (cus >= 8 && grid > cus) grid = cus;
+  hipLaunchKernelGGL((w8a8_int8_gemm_kernel<DT, WM, WN, NI, NJ>), dim3(grid), dim3(GEMM_THREADS), shmem, st, b);
   MQ_LAUNCH_CHECK("w8a8_int8_gemm");
   return 0;
+}
+
+// Tile width: the one that wastes fewer tile slots in the last round of
+// workgroups over the CUs (time ~ rounds x tile width).
+template <int DT>
+int launch_gemm(const I8Args& a, hipStream_t st) {
+  const long cus = device_cu_count(), mtiles = (a.M + TM - 1) / TM;
+  const long t256 = mtiles * ((a.N + 255) / 256), t224 = mtiles * ((a.N + 223) / 224);
+  const long cost256 = (t256 + cus - 1) / cus * 256, cost224 = (t224 + cus - 1) / cus * 224;
+  if (cost224 < cost256) return launch_tile<DT, 4, 2, 7, 4>(a, st);
+  return launch_tile<DT, 2, 4, 4, 8>(a, st);
 }
 
 }  // namespace
