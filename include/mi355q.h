@@ -71,7 +71,8 @@ int mi355q_w4_unpack(const int32_t* packed, uint8_t* dst, int batch, int K, int 
  * x, out, scales, bias share `dtype` (F16 or BF16); qweight is the slab
  * layout; scales [K/g, N]; group_size a multiple of 32 dividing K (or -1 for
  * one group).  M <= 64 runs the split-K streaming kernel, larger M the
- * LDS-staged MFMA kernel.  `workspace` must hold
+ * LDS-staged MFMA kernel (which splits K over two kernels when its grid would
+ * leave most of the chip idle).  `workspace` must hold
  * mi355q_w4a16_workspace_bytes() bytes, be zero-filled once before first use,
  * and must not be shared by launches that may overlap in time. */
 size_t mi355q_w4a16_workspace_bytes(int M, int K, int N);

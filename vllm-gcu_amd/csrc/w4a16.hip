@@ -10,15 +10,22 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
 size_t w4a16_stream_workspace_bytes(int M, int N);
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
-                      int group_size, int dtype, hipStream_t st);
+                      int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
+size_t w4a16_tile_workspace_bytes(int M, int K, int N);
 }  // namespace mi355q
 
 using namespace mi355q;
 
+static constexpr size_t TILE_WS_OFFSET = (size_t)1 << 20;
+
 extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
-  (void)K;
-  if (M <= 0 || N <= 0) return 0;
-  return w4a16_stream_workspace_bytes(M > 64 ? 64 : M, N);
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const size_t s = w4a16_stream_workspace_bytes(M > 64 ? 64 : M, N);
+  // the split-K partials of the MFMA kernel live behind the first MiB, which
+  // holds the streaming kernel's arrival counters (they must stay zero)
+  const size_t t = M > 64 ? w4a16_tile_workspace_bytes(M, K, N) : 0;
+  const size_t tt = t ? t + TILE_WS_OFFSET : 0;
+  return s > tt ? s : tt;
 }
 
 extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
@@ -57,8 +64,10 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
     }
     return 0;
   }
+  const bool ws_ok = workspace && workspace_bytes > TILE_WS_OFFSET;
   return w4a16_tile_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
-                           as_stream(stream));
+                           ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,
+                           ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, as_stream(stream));
 }
 
 extern "C" int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight, const void* scales,

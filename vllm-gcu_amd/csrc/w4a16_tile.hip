@@ -36,6 +36,10 @@ struct TileArgs {
   const int* npp;             // device scalar: padded id count
   const float* topk_weights;  // [numel] or null
   int numel, topk;
+  // dense split-K: blockIdx.z takes K blocks [z * kper, (z + 1) * kper) and writes an fp32
+  // partial tile to partial[z][M][N]; a second kernel adds the partials up
+  int kper;                   // K blocks per split (G when there is no split)
+  float* partial;             // null: write the output directly
   long w_stride, s_stride, z_stride;   // per-expert strides in elements of the respective arrays
 };
 
@@ -82,18 +86,24 @@ template <> struct TileMma<MI355Q_BF16> {
 };
 
 // MT = row tiles of 16 per workgroup (block rows BM = 16 MT); GROUPED selects
-// the MoE row gather
-template <int DT, int ZK, int MT, bool GROUPED>
-__global__ void __launch_bounds__(256, 1)
+// the MoE row gather.  WM = 1: four wavefronts, each all BM rows of its 64
+// columns.  WM = 2: eight wavefronts, the upper four take the upper half of
+// the rows (both halves dequantise the same weights, but two wavefronts per
+// SIMD keep the matrix pipe fed while one of them waits or dequantises).
+template <int DT, int ZK, int MT, bool GROUPED, int WM>
+__global__ void __launch_bounds__(256 * WM, 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
   typedef typename MM::vec vec;
+  static_assert(MT % WM == 0, "row tiles split evenly over the wavefront rows");
   constexpr int BM = 16 * MT;
+  constexpr int MTW = MT / WM;                    // row tiles per wavefront
+  constexpr int NTHR = 256 * WM;
   constexpr int A_BUF = BM * A_ROW;
   extern __shared__ __align__(16) unsigned char lds[];
   __shared__ int tok[GROUPED ? BM : 1];
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = (tid >> 6) & 3, wmh = tid >> 8;
   const int c = lane & 15, kq = lane >> 4;
   const int N = a.N, K = a.K, M = a.M;
   const int G = K >> 7;
@@ -107,7 +117,7 @@ w4a16_tile_kernel(TileArgs a) {
     qw += e * a.w_stride;
     scales += e * a.s_stride;
     if (zeros) zeros += e * a.z_stride * (ZK == MI355Q_ZP_PACKED ? 4 : 2);
-    for (int r = tid; r < BM; r += 256) tok[r] = a.sorted_ids[m0 + r];
+    for (int r = tid; r < BM; r += NTHR) tok[r] = a.sorted_ids[m0 + r];
     __syncthreads();
   }
   // N may end in the middle of the 256-column tile: the two wavefronts of a
@@ -117,32 +127,32 @@ w4a16_tile_kernel(TileArgs a) {
   const int t0 = (wave & 1) * 4;
   const int ncol = 128 * slab + 8 * c + t0;          // first of this lane's 4 columns
 
-  f4 acc[MT][4];
+  f4 acc[MTW][4];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
 
   // global -> register staging of the next activation tile: thread tid loads
-  // MT chunks of 16 B: row = pass * 16 + tid / 16, chunk = tid % 16
+  // MTW chunks of 16 B: row = pass * 16 WM + tid / 16, chunk = tid % 16
   const int arow = tid >> 4, achunk = tid & 15;
-  const uint16_t* aptr[MT];
+  const uint16_t* aptr[MTW];
 #pragma unroll
-  for (int p = 0; p < MT; ++p) {
+  for (int p = 0; p < MTW; ++p) {
     int row;
-    if (GROUPED) row = min(tok[p * 16 + arow], a.numel - 1) / a.topk;   // pads read a valid row
-    else row = min(m0 + p * 16 + arow, M - 1);
+    if (GROUPED) row = min(tok[p * 16 * WM + arow], a.numel - 1) / a.topk;   // pads read a valid row
+    else row = min(m0 + p * 16 * WM + arow, M - 1);
     aptr[p] = a.x + (size_t)row * K + 8 * achunk;
   }
-  u4 areg[MT];
+  u4 areg[MTW];
   auto load_a = [&](int g) {
 #pragma unroll
-    for (int p = 0; p < MT; ++p) areg[p] = *(const u4*)(aptr[p] + 128 * g);
+    for (int p = 0; p < MTW; ++p) areg[p] = *(const u4*)(aptr[p] + 128 * g);
   };
   auto store_a = [&](int buf) {
     unsigned char* base = lds + buf * A_BUF;
 #pragma unroll
-    for (int p = 0; p < MT; ++p) *(u4*)(base + (p * 16 + arow) * A_ROW + achunk * 16) = areg[p];
+    for (int p = 0; p < MTW; ++p) *(u4*)(base + (p * 16 * WM + arow) * A_ROW + achunk * 16) = areg[p];
   };
 
   const u4* wbase = qw + ((size_t)slab * G * 8 + t0) * 64 + lane;
@@ -160,13 +170,14 @@ w4a16_tile_kernel(TileArgs a) {
     if (ZK == MI355Q_ZP_PRESCALED) zsreg = *(const uint2*)((const uint16_t*)zeros + (size_t)qrow * N + ncol);
   };
 
-  load_a(0);
-  load_b(0);
+  const int gb = GROUPED ? 0 : (int)blockIdx.z * a.kper, ge = GROUPED ? G : min(G, gb + a.kper);
+  load_a(gb);
+  load_b(gb);
   store_a(0);
   __syncthreads();
 
-  for (int g = 0; g < G; ++g) {
-    const int buf = g & 1;
+  for (int g = gb; g < ge; ++g) {
+    const int buf = (g - gb) & 1;
     // operands of this K block, then start the next block's loads
     u4 wcur[4];
 #pragma unroll
@@ -190,7 +201,7 @@ w4a16_tile_kernel(TileArgs a) {
       zlo[t] = (h2){zl, zl};
       zhi[t] = (h2){zh, zh};
     }
-    const int gn = min(g + 1, G - 1);
+    const int gn = min(g + 1, ge - 1);
     load_a(gn);
     load_b(gn);
 
@@ -201,9 +212,9 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zlo[t], zhi[t]);
 
-    const unsigned char* abase = lds + buf * A_BUF + c * A_ROW + kq * 16;
+    const unsigned char* abase = lds + buf * A_BUF + (wmh * MTW * 16 + c) * A_ROW + kq * 16;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int mt = 0; mt < MTW; ++mt) {
       f4 part[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
@@ -230,21 +241,26 @@ w4a16_tile_kernel(TileArgs a) {
     for (int t = 0; t < 4; ++t) bs[t] = Elem<DT>::to_f32(a.bias[ncol + t]);
   }
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int m;
       float rw = 1.0f;
       bool ok;
       if (GROUPED) {
-        m = tok[mt * 16 + 4 * kq + i];
+        m = tok[(wmh * MTW + mt) * 16 + 4 * kq + i];
         ok = m < a.numel;
         if (ok && a.topk_weights) rw = a.topk_weights[m];
       } else {
-        m = m0 + mt * 16 + 4 * kq + i;
+        m = m0 + (wmh * MTW + mt) * 16 + 4 * kq + i;
         ok = m < M;
       }
-      if (ok) {
+      if (!GROUPED && a.partial) {
+        if (ok) {
+          float* pp = a.partial + ((size_t)blockIdx.z * M + m) * N + ncol;
+          *(f4*)pp = (f4){acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]};
+        }
+      } else if (ok) {
         uint2 o;
         o.x = (uint32_t)Elem<DT>::from_f32(acc[mt][0][i] * rw + bs[0]) |
               ((uint32_t)Elem<DT>::from_f32(acc[mt][1][i] * rw + bs[1]) << 16);
@@ -255,15 +271,36 @@ w4a16_tile_kernel(TileArgs a) {
     }
 }
 
+// out[m, n] = sum over splits of partial[s][m][n] (+ bias[n]), added in split order
+template <int DT>
+__global__ void __launch_bounds__(256)
+w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* bias, long MN, int N, int splits) {
+  const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= MN) return;
+  f4 v = *(const f4*)(partial + i);
+  for (int s = 1; s < splits; ++s) v += *(const f4*)(partial + (size_t)s * MN + i);
+  if (bias) {
+    const int n = (int)(i % N);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] += Elem<DT>::to_f32(bias[n + e]);
+  }
+  uint2 o;
+  o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
+  o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);
+  *(uint2*)(out + i) = o;
+}
+
 template <int DT, int ZK, int MT, bool GROUPED>
 hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
   constexpr int BM = 16 * MT;
-  dim3 grid((a.N + BN - 1) / BN, row_blocks), block(256);
-  const size_t shmem = 2 * BM * A_ROW;             // up to 72 KiB: above the 64 KiB default
-  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED>,
+  constexpr int WM = MT >= 4 ? 2 : 1;              // eight wavefronts once there are rows to split
+  const int G = a.K >> 7;
+  dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
+  const size_t shmem = 2 * BM * A_ROW;             // up to 144 KiB: above the 64 KiB default
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   if (attr != hipSuccess) return attr;
-  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED>), grid, block, shmem, st, a);
+  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>), grid, block, shmem, st, a);
   return hipSuccess;
 }
 
@@ -286,9 +323,32 @@ hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStrea
 
 }  // namespace
 
+// split-K plan for grids that leave most of the chip idle: as many splits as
+// bring the grid to about one workgroup per CU, at least 4 K blocks each, and
+// partial tiles of at most TILE_SPLITK_BYTES in total
+constexpr size_t TILE_SPLITK_BYTES = (size_t)64 << 20;
+static int tile_rows_mt(int M, int N) {
+  // 128-row blocks once they fill the chip, 64-row blocks for mid-sized M
+  return ((long)((M + 127) / 128) * ((N + BN - 1) / BN) >= device_cu_count()) ? 8 : 4;
+}
+static int tile_splits(int M, int K, int N) {
+  const int mt = tile_rows_mt(M, N), G = K / 128;
+  const long wgs = (long)((M + 16 * mt - 1) / (16 * mt)) * ((N + BN - 1) / BN);
+  const long cus = device_cu_count();
+  if (wgs * 2 > cus) return 1;
+  long s = (cus + wgs / 2) / wgs;
+  if (s > G / 4) s = G / 4;
+  while (s > 1 && (size_t)s * M * N * sizeof(float) > TILE_SPLITK_BYTES) --s;
+  return s < 1 ? 1 : (int)s;
+}
+size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
+  const int s = tile_splits(M, K, N);
+  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
-                      int group_size, int dtype, hipStream_t st) {
+                      int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
   MQ_REQUIRE(group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   TileArgs a = {};
@@ -299,13 +359,29 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   a.zeros = zeros;
   a.bias = (const uint16_t*)bias;
   a.M = M; a.K = K; a.N = N; a.gs = group_size;
-  // 128-row blocks once they fill the chip, 64-row blocks for mid-sized M
-  const int mt = ((long)((M + 127) / 128) * ((N + BN - 1) / BN) >= device_cu_count()) ? 8 : 4;
+  const int mt = tile_rows_mt(M, N);
   const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
+  const int G = K / 128;
+  int splits = tile_splits(M, K, N);
+  if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * M * N * sizeof(float))) splits = 1;
+  a.kper = (G + splits - 1) / splits;
+  splits = (G + a.kper - 1) / a.kper;                // no empty splits
+  a.partial = splits > 1 ? (float*)workspace : nullptr;
   hipError_t e = (dtype == MI355Q_F16) ? launch_mt<MI355Q_F16, false>(a, zeros_kind, mt, row_blocks, st)
                                        : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
   MQ_REQUIRE(e == hipSuccess, "w4a16_gemm(tile): cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("w4a16_gemm(tile)");
+  if (splits > 1) {
+    const long MN = (long)M * N;
+    const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
+    if (dtype == MI355Q_F16)
+      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
+                         (const float*)workspace, (const uint16_t*)bias, MN, N, splits);
+    else
+      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
+                         (const float*)workspace, (const uint16_t*)bias, MN, N, splits);
+    MQ_LAUNCH_CHECK("w4a16_gemm(split-K reduce)");
+  }
   return 0;
 }
 
@@ -326,6 +402,7 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   a.M = numel; a.K = K; a.N = N; a.gs = group_size;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
   a.numel = numel; a.topk = topk;
+  a.kper = K / 128; a.partial = nullptr;
   a.w_stride = (long)(K / 8) * N / 4;              // u4 elements per expert
   a.s_stride = (long)(K / group_size) * N;
   a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
