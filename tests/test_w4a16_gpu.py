@@ -212,6 +212,25 @@ def test_tile_gemm_exact_and_agrees_with_stream(ops, rearrange):
     assert torch.equal(a.cpu(), want) and torch.equal(b.cpu(), want)
 
 
+@pytest.mark.parametrize("M,K,N", [(128, 4096, 512), (96, 2048, 256), (130, 1536, 384)])
+def test_tile_gemm_split_k_small_grid(ops, rearrange, M, K, N):
+    # few output tiles and a long K: the MFMA kernel splits K over workgroups
+    # and a second kernel adds the fp32 partial tiles (and the bias) in order
+    print(f"case tile split-K M={M} K={K} N={N}", flush=True)
+    g = 128
+    q, z, s, x = make_case(M + N, M, K, N, g)
+    bias = np.random.default_rng(2).standard_normal(N).astype(np.float32)
+    a = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=2)
+    b = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=2)
+    assert torch.equal(a, b)                               # run-to-run identical
+    want = oracle(q, z, s, x, g, torch.float16, bias=bias)
+    np.testing.assert_allclose(a.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # exact inputs: any split must reproduce the oracle bit for bit
+    q, z, s, x = make_case(5, M, K, N, g, exact=True)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=2)
+    assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16))
+
+
 def test_tile_gemm_zero_kinds_and_group_256(ops, rearrange):
     M, K, N, g = 130, 512, 256, 256
     q, z, s, x = make_case(77, M, K, N, g)
