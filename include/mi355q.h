@@ -118,6 +118,13 @@ int mi355q_dynamic_int8_quant(int8_t* out, float* scales, const void* x, int M, 
 int mi355q_static_int8_quant(int8_t* out, const void* x, const float* scale, int per_channel, int M,
                              int K, int dtype, void* stream);
 
+/* Replaces topsvllmSiluMulQuant as called by silu_mul_static_int8_quant
+ * (csrc/src/silu_mul_static_int8_quant.cpp:11-28): x is [rows, 2d];
+ * q = sat_s8(rne((silu(x[:, :d]) * x[:, d:]) * (1/scale))), the activation and the
+ * reciprocal both rounded to the input dtype; scale is one value or [d]. */
+int mi355q_silu_mul_static_int8_quant(int8_t* out, const void* x, const float* scale, int per_channel,
+                                      long rows, int d, int dtype, void* stream);
+
 /* ---- MoE routing ------------------------------------------------------------
  * Replaces topsvllm's topk_softmax (csrc/src/topk_softmax.cpp:27-34):
  * softmax over E experts in fp32, top-k descending (ties to the lower index);
@@ -165,8 +172,10 @@ int mi355q_fp8_group_quant(uint8_t* out, float* scales, const void* x, long rows
 /* dynamic_per_token_scaled_fp8_quant (csrc/src/dynamic_per_token_scaled_fp8_quant.cpp): one scale per row */
 int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x, int rows, int K, int dtype,
                            const int32_t* valid_rows, void* stream);
-/* static_scaled_fp8_quant and silu_mul_static_fp8_quant (csrc/torch_bindings.cpp:291, 714):
- * q = e4m3fn(clamp(x / scale)) with one fp32 scale */
+/* static_scaled_fp8_quant, silu_mul_static_fp8_quant and mul_static_fp8_quant
+ * (csrc/torch_bindings.cpp:714, 291, 301; csrc/src/mul_static_fp8_quant.cpp:11-22):
+ * q = e4m3fn(clamp(v / scale)) with one fp32 scale; fuse_silu_mul 0: v = x [rows, K];
+ * 1: v = silu(x[:, :K]) * x[:, K:] of x [rows, 2K]; 2: v = x[:, :K] * x[:, K:] */
 int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, long rows, int K,
                             int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream);
 /* moe_sum_pad (csrc/src/moe_sum.cpp:64-131): out[m, :] = sum_t in[m, t, :], fp32 accumulate */

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from oracle import fp8 as of8
+from oracle import w8a8 as o8
 from oracle import moe as om
 
 pytestmark = pytest.mark.gpu
@@ -232,6 +233,36 @@ def test_per_token_and_static_fp8_quant(ops):
     q, _ = ops.scaled_fp8_quant(x.cuda(), sc.cuda())
     y = np.clip(x.float().numpy() / np.float32(0.02), -448, 448).astype(np.float32)
     assert np.array_equal(q.view(torch.uint8).cpu().numpy(), of8.to_e4m3fn(y))
+
+
+def test_mul_and_silu_mul_static_quant_equal_unfused_sequences(ops):
+    # mul_static_fp8_quant == (left * right rounded to the input dtype) then static_scaled_fp8_quant;
+    # silu_mul_static_int8_quant == silu_and_mul then static_scaled_int8_quant
+    # (the fusion tables of vllm_gcu/compilation/fusion.py:129-152)
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(37, 2, 512, generator=g).to(torch.bfloat16).cuda()
+    sc = torch.tensor([0.05], dtype=torch.float32, device="cuda")
+    n = torch.tensor([30], dtype=torch.int32, device="cuda")
+    got = torch.zeros(37, 2, 256, dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
+    torch.ops._C.mul_static_fp8_quant(got, x, sc, n)
+    mid = (x[..., :256].float() * x[..., 256:].float()).to(torch.bfloat16)
+    ref = torch.empty(37, 2, 256, dtype=torch.float8_e4m3fn, device="cuda")
+    torch.ops._C.static_scaled_fp8_quant(ref, mid, sc)
+    assert torch.equal(got[:30].view(torch.uint8), ref[:30].view(torch.uint8))
+    assert torch.all(got[30:].view(torch.uint8) == 0)
+    want = of8.to_e4m3fn(np.clip(mid[:30].float().cpu().numpy() / np.float32(0.05), -448, 448).astype(np.float32))
+    assert np.array_equal(got[:30].view(torch.uint8).cpu().numpy(), want)
+
+    for scale in (torch.tensor(0.02, dtype=torch.float32), torch.rand(256, generator=g) * 0.05 + 0.01):
+        xs = torch.randn(19, 512, generator=g).to(torch.float16).cuda()
+        q = torch.empty(19, 256, dtype=torch.int8, device="cuda")
+        ops.silu_mul_quant(q, xs, scale.cuda())
+        mid = torch.empty(19, 256, dtype=torch.float16, device="cuda")
+        torch.ops._C.silu_and_mul(mid, xs)
+        ref, _, _ = ops.scaled_int8_quant(mid, scale.cuda())
+        assert torch.equal(q, ref)
+        # and the CPU oracle on the same rounded activation
+        assert np.array_equal(q.cpu().numpy(), o8.static_scaled_int8_quant(mid.cpu().numpy(), scale.numpy()))
 
 
 @pytest.mark.parametrize("dtype,odtype", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),

@@ -138,7 +138,8 @@ token_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, int K, co
   }
 }
 
-template <int DT, bool SILU>
+// FUSE: 0 = quantise x; 1 = silu(x[:, :K]) * x[:, K:] first; 2 = x[:, :K] * x[:, K:] first
+template <int DT, int FUSE>
 __global__ void __launch_bounds__(256)
 static_fp8_quant_kernel(uint8_t* out, const uint16_t* x, const float* scale, long rows, int K,
                         const int* valid_rows) {
@@ -147,10 +148,11 @@ static_fp8_quant_kernel(uint8_t* out, const uint16_t* x, const float* scale, lon
   const float s = *scale;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     float v;
-    if (SILU) {
+    if (FUSE) {
       const long r = i / K;
       const int c = (int)(i - r * K);
-      v = round_act<DT>(silu_mul(Elem<DT>::to_f32(x[r * 2 * K + c]), Elem<DT>::to_f32(x[r * 2 * K + K + c])));
+      const float l = Elem<DT>::to_f32(x[r * 2 * K + c]), g = Elem<DT>::to_f32(x[r * 2 * K + K + c]);
+      v = round_act<DT>(FUSE == 1 ? silu_mul(l, g) : l * g);
     } else {
       v = Elem<DT>::to_f32(x[i]);
     }
@@ -268,15 +270,21 @@ extern "C" int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float*
   MQ_REQUIRE(out && scale && x, "fp8_static_quant: null pointer");
   hipStream_t st = as_stream(stream);
   unsigned g = grid_for(rows * K);
-  if (fuse_silu_mul) {
+  MQ_REQUIRE(fuse_silu_mul >= 0 && fuse_silu_mul <= 2, "fp8_static_quant: unknown fusion %d", fuse_silu_mul);
+  if (fuse_silu_mul == 1) {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, true>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, true>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 1>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 1>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      "fp8_static_quant");
+  } else if (fuse_silu_mul == 2) {
+    MQ_DISPATCH_16(dtype,
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 2>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 2>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
       "fp8_static_quant");
   } else {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, false>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, false>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 0>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 0>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
       "fp8_static_quant");
   }
   MQ_LAUNCH_CHECK("fp8_static_quant");

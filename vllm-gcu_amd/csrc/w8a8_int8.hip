@@ -366,6 +366,22 @@ static_int8_quant_kernel(int8_t* out, const void* x, const float* scale, int per
   out[i] = sat_rne_s8(ld_act<DT>(x, i) * inv);
 }
 
+// silu(x[:, :d]) * x[:, d:] rounded to the input dtype, then quantised like
+// static_int8_quant (reciprocal of the scale rounded to the input dtype)
+template <int DT>
+__global__ void __launch_bounds__(256)
+silu_mul_static_int8_quant_kernel(int8_t* out, const uint16_t* x, const float* scale, int per_channel, long total, int d) {
+  long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const long r = i / d;
+  const int c = (int)(i - r * d);
+  float inv = 1.0f / scale[per_channel ? c : 0];
+  inv = Elem<DT>::to_f32(Elem<DT>::from_f32(inv));
+  const float l = Elem<DT>::to_f32(x[r * 2 * d + c]), g = Elem<DT>::to_f32(x[r * 2 * d + d + c]);
+  const float act = Elem<DT>::to_f32(Elem<DT>::from_f32(l * (1.0f / (1.0f + expf(-l))) * g));
+  out[i] = sat_rne_s8(act * inv);
+}
+
 template <int DT, int WM, int WN, int NI, int NJ>
 int launch_tile(const I8Args& a, hipStream_t st) {
   constexpr int TN = WN * NI * 16;
@@ -459,5 +475,24 @@ extern "C" int mi355q_static_int8_quant(int8_t* out, const void* x, const float*
   else
     MQ_REQUIRE(false, "static_int8_quant: bad dtype %d", dtype);
   MQ_LAUNCH_CHECK("static_int8_quant");
+  return 0;
+}
+
+extern "C" int mi355q_silu_mul_static_int8_quant(int8_t* out, const void* x, const float* scale, int per_channel,
+                                                 long rows, int d, int dtype, void* stream) {
+  MQ_REQUIRE(rows >= 0 && d > 0, "silu_mul_static_int8_quant: bad shape rows=%ld d=%d", rows, d);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && scale && x, "silu_mul_static_int8_quant: null pointer");
+  MQ_REQUIRE(dtype == MI355Q_F16 || dtype == MI355Q_BF16, "silu_mul_static_int8_quant: dtype %d must be f16 or bf16", dtype);
+  const long total = rows * d;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t st = as_stream(stream);
+  if (dtype == MI355Q_F16)
+    hipLaunchKernelGGL((silu_mul_static_int8_quant_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, out,
+                       (const uint16_t*)x, scale, per_channel, total, d);
+  else
+    hipLaunchKernelGGL((silu_mul_static_int8_quant_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, out,
+                       (const uint16_t*)x, scale, per_channel, total, d);
+  MQ_LAUNCH_CHECK("silu_mul_static_int8_quant");
   return 0;
 }

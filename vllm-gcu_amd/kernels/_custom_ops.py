@@ -463,6 +463,11 @@ def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: i
     return topk_weights, topk_ids
 
 
+def silu_mul_quant(out: torch.Tensor, input: torch.Tensor, scaling: torch.Tensor) -> None:
+    """vllm_gcu/kernels/_custom_ops.py:397-400."""
+    torch.ops._C.silu_mul_static_int8_quant(out, input, scaling)
+
+
 # fused moe (vllm_gcu/kernels/_custom_ops.py:490-543)
 def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
                          num_tokens_post_pad) -> None:
@@ -588,11 +593,34 @@ def _static_fp8_common(out, input, scale, real_rows, fuse):
 
 
 def _static_scaled_fp8_quant_impl(result, input, scale):
-    _static_fp8_common(result, input, scale, None, False)
+    _static_fp8_common(result, input, scale, None, 0)
 
 
 def _silu_mul_static_fp8_quant_impl(out, input, scale, real_num_tokens):
-    _static_fp8_common(out, input, scale, _leading_rows_to_flat(input, real_num_tokens), True)
+    _static_fp8_common(out, input, scale, _leading_rows_to_flat(input, real_num_tokens), 1)
+
+
+def _mul_static_fp8_quant_impl(out, input, scale, real_num_tokens):
+    _static_fp8_common(out, input, scale, _leading_rows_to_flat(input, real_num_tokens), 2)
+
+
+def _silu_mul_static_int8_quant_impl(result, input, scale):
+    # csrc/src/silu_mul_static_int8_quant.cpp:11-28: a 0-d scale is per tensor,
+    # anything else per channel of the gated half
+    rt.require_gpu(result, input, scale)
+    if input.numel() == 0:
+        return
+    x = input.contiguous()
+    rows, kin = _rows_last(x)
+    d = kin // 2
+    if result.dtype != torch.int8 or tuple(result.shape) != tuple(x.shape[:-1]) + (d,) or not result.is_contiguous():
+        raise RuntimeError(f"silu_mul_static_int8_quant: result must be contiguous int8 {tuple(x.shape[:-1]) + (d,)}")
+    sc = scale.to(torch.float32).reshape(-1).contiguous()
+    if sc.numel() not in (1, d):
+        raise RuntimeError(f"silu_mul_static_int8_quant: scale must have 1 or {d} entries, got {sc.numel()}")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_silu_mul_static_int8_quant", result.data_ptr(), x.data_ptr(), sc.data_ptr(),
+                  int(sc.numel() > 1), rows, d, rt.dtype_code(x.dtype), rt.stream_ptr())
 
 
 def _moe_sum_pad_impl(out, input, size, dim, keepdim):
@@ -629,6 +657,10 @@ _register("_C", "dynamic_per_token_scaled_fp8_quant",
           _dynamic_per_token_scaled_fp8_quant_impl)
 _register("_C", "static_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor scale) -> ()",
           _static_scaled_fp8_quant_impl)
+_register("_C", "mul_static_fp8_quant",
+          "(Tensor(a!) out, Tensor input, Tensor scale, Tensor real_num_tokens) -> ()", _mul_static_fp8_quant_impl)
+_register("_C", "silu_mul_static_int8_quant", "(Tensor(a!) result, Tensor input, Tensor scale) -> ()",
+          _silu_mul_static_int8_quant_impl)
 _register("_C", "silu_mul_static_fp8_quant",
           "(Tensor(a!) out, Tensor input, Tensor scale, Tensor real_num_tokens) -> ()",
           _silu_mul_static_fp8_quant_impl)
