@@ -33,7 +33,7 @@ INT8_PEAK_TOPS = 5000.0
 # then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy of --calibrate-copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per
 # unit).  Keyed by (M, --split-k); other settings were not profiled.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 36314399}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 35800368}
 
 
 def w4a16_bytes(M, K, N, g=GROUP):
@@ -95,33 +95,35 @@ def time_graph(fn_list, steps, warmup, stream):
     return e0.elapsed_time(e1) * 1e-3
 
 
-def cpu_baseline_w4a16(M, budget_s=20.0):
+def cpu_baseline_w4a16(M, target_s=12.0):
     """The CPU oracle (dequantize + torch.matmul, fp32) on the same four
-    shapes, all host threads.  Returns GB/s of the same algorithmic bytes."""
+    shapes, all host threads: whole passes over the four layers are repeated
+    until about target_s seconds of CPU work are done.  Returns GB/s of the
+    same algorithmic bytes."""
     import numpy as np
     import torch
     from oracle import w4 as ow4
     torch.set_num_threads(os.cpu_count() or 1)
     rng = np.random.default_rng(0)
-    tot_b, tot_t, done = 0, 0.0, []
-    t_start = time.time()
+    cases = []
     for name, K, N in LLAMA3_8B:
         q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
         z = rng.integers(0, 16, size=(K // GROUP, N), dtype=np.uint8)
         s = rng.uniform(0.001, 0.01, size=(K // GROUP, N)).astype(np.float16)
         x = rng.standard_normal((M, K)).astype(np.float16)
-        t0 = time.time()
-        ow4.w4a16_gemm(x, q, z, s, GROUP)
-        dt = time.time() - t0
-        tot_b += w4a16_bytes(M, K, N)
-        tot_t += dt
-        done.append(name)
-        if time.time() - t_start > budget_s:
-            break
+        cases.append((K, N, q, z, s, x))
+    tot_b, tot_t, passes = 0, 0.0, 0
+    while tot_t < target_s and passes < 200:
+        for K, N, q, z, s, x in cases:
+            t0 = time.time()
+            ow4.w4a16_gemm(x, q, z, s, GROUP)
+            tot_t += time.time() - t0
+            tot_b += w4a16_bytes(M, K, N)
+        passes += 1
     return {"value": round(tot_b / tot_t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"one pass of oracle.w4.w4a16_gemm (numpy dequantize + torch fp32 matmul) over "
-                      f"layers {','.join(done)} at M={M}; {tot_t:.2f} s"}
+            "sample": f"{passes} passes of oracle.w4.w4a16_gemm (numpy dequantize + torch fp32 matmul) over the "
+                      f"four layers at M={M}; {tot_t:.1f} s of CPU work"}
 
 
 def main():
