@@ -166,7 +166,8 @@ __global__ void __launch_bounds__(256, MT == 1 ? 2 : 1)
 w4a16_stream_kernel(StreamArgs a) {
   typedef Mma<DT> MM;
   typedef typename MM::vec vec;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // the wavefront index is made visibly uniform: K-block indices and loop control then live in scalar registers
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, kq = lane >> 4;
   constexpr int TG = 8 / NT;                          // tile groups per slab
   constexpr int HW = NT >= 2 ? NT / 2 : 1;            // packed 16-bit pairs per lane
@@ -288,33 +289,49 @@ w4a16_stream_kernel(StreamArgs a) {
   };
 
   {
-    Block b0, b1;
+    // Two block buffers: the next K block of this wavefront is in flight while
+    // one is consumed (deeper rings were measured and are slower).  The
+    // prefetch is unconditional (past the end it re-reads a block of this
+    // wavefront) and every step leaves the loop through a plain break, so the
+    // body is straight-line code and the compiler waits for exactly the block
+    // being consumed.
+    //
+    // K order: the wavefront's nb blocks are visited starting at a
+    // workgroup-dependent position.  All workgroups read the same activation
+    // rows, and a K block of them (16 rows x 256 B at a pitch of 2 K bytes)
+    // sits in very few L2 channels: in a common order every workgroup of an XCD
+    // would hammer those channels at the same moment.  (The order is fixed per
+    // workgroup, so results stay run-to-run identical.)
+    Block ring[2];
     Acts xa;
-    int g = gb + wave;
-    if (g < ge) {
-      // the prefetch is unconditional (the last one re-reads this wave's own
-      // final block) so the loop body is straight-line code and the compiler
-      // can wait for exactly the block being consumed
-      const int glast = g + ((ge - 1 - g) & ~3);
-      load_block(b0, g);
+    const int g0 = gb + wave;
+    const int nb = (ge - g0 + 3) >> 2;               // K blocks of this wavefront
+    if (nb > 0) {
+      const int rot = (int)((blockIdx.x >> 3) * 5u % (unsigned)nb);
+      auto blk = [&](int i) {                        // i-th block in this workgroup's order
+        int j = i + rot;
+        if (j >= nb) j -= nb;
+        if (j >= nb) j -= nb;                        // i may run one past the end
+        return g0 + 4 * j;
+      };
+      load_block(ring[0], blk(0));
+      int i = 0;
       while (true) {
         // sched_barrier: keep the prefetch ahead of the arithmetic, the
         // instruction scheduler would otherwise sink the loads next to
         // their first use one iteration later
-        load_acts(xa, g);
-        load_block(b1, min(g + 4, glast));
+        load_acts(xa, blk(i));
+        load_block(ring[1], blk(i + 1));
         __builtin_amdgcn_sched_barrier(0);
-        compute_block(b0, xa);
+        compute_block(ring[0], xa);
         __builtin_amdgcn_sched_barrier(0);
-        g += 4;
-        if (g >= ge) break;
-        load_acts(xa, g);
-        load_block(b0, min(g + 4, glast));
+        if (++i >= nb) break;
+        load_acts(xa, blk(i));
+        load_block(ring[0], blk(i + 1));
         __builtin_amdgcn_sched_barrier(0);
-        compute_block(b1, xa);
+        compute_block(ring[1], xa);
         __builtin_amdgcn_sched_barrier(0);
-        g += 4;
-        if (g >= ge) break;
+        if (++i >= nb) break;
       }
     }
   }
