@@ -201,7 +201,8 @@ int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scal
                     const void* w_zeros, int zeros_kind, int quant_mode, int group_size,
                     const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                     const int32_t* num_tokens_post_pad, int numel, int topk, int block_size,
-                    int max_blocks, int E, int K, int N, int act_dtype, int out_dtype, void* stream);
+                    int max_blocks, int E, int K, int N, int act_dtype, int out_dtype, int w_layout,
+                    void* stream);
 /* Dense calls of the same kernels (quant_mode 1..4), replacing topsatenLinearQuant
  * as called by linear_quant (csrc/src/linear_quant.cpp:16-95, fp8 block-scaled
  * C = sum_kb (A_kb B_kb^T) As Bs) and by weight_only_quant
@@ -209,7 +210,15 @@ int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scal
  * the output dtype or NULL. */
 int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_scale,
                         const void* w_scale, const void* bias, int quant_mode, int group_size, int M,
-                        int K, int N, int act_dtype, int out_dtype, void* stream);
+                        int K, int N, int act_dtype, int out_dtype, int w_layout, void* stream);
+/* Weight layout of quant_mode 1..4 (w_layout above).  0: row-major [E, N, K], the checkpoint's
+ * and the reference's (vllm_gcu/kernels/quantization/fp8.py:72-166 keeps it).  1: "kslab",
+ * this library's streaming order of the same bytes, N % 64 == 0:
+ * [E][N/64][K/128][4 tiles of 16 rows][2*elem_bytes vectors][64 lanes][16 B], where lane l of
+ * vector v of tile i holds bytes (128 kb + 32 (l/16)) * elem_bytes + 16 v .. +16 of row
+ * 64 ng + 16 i + l%16 -- each wavefront load reads one contiguous KiB.  No counterpart in
+ * the reference (load-time conversion, like its int4 rearrange). */
+int mi355q_kslab_repack(const void* src, void* dst, int batch, int N, int K, int elem_bytes, void* stream);
 
 /* ---- measurement probe -------------------------------------------------------
  * No counterpart in the reference.  Streams `bytes` of device memory through

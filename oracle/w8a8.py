@@ -97,3 +97,43 @@ def weight_only_int8(x: np.ndarray, w_nk: np.ndarray, scale: np.ndarray,
     if bias is not None:
         out = out + bias.astype(np.float32)[None, :]
     return out
+
+
+# ----------------------------------------------------------------------------
+# This build's streaming order for K-contiguous weights ("kslab")
+# ----------------------------------------------------------------------------
+def kslab_pack(w: np.ndarray) -> np.ndarray:
+    """[.., N, K] of 1- or 2-byte elements -> same shape/dtype, bytes in the
+    order ``[N/64][K/128][4 tiles][2*elem_bytes vectors][64 lanes][16 B]``: lane
+    ``l`` of vector ``v`` of tile ``i`` in (row group G, K block kb) holds the 16
+    bytes at byte offset ``(128 kb + 32 (l // 16)) * elem_bytes + 16 v`` of row
+    ``64 G + 16 i + l % 16``.  No counterpart in the reference (its fp8 / int8
+    weights stay row-major, vllm_gcu/kernels/quantization/fp8.py:72-166);
+    pinned by :func:`kslab_unpack`, a scalar walk of the same definition."""
+    wb = w.dtype.itemsize
+    N, K = w.shape[-2:]
+    assert wb in (1, 2) and N % 64 == 0 and K % 128 == 0
+    lead = w.shape[:-2]
+    b = np.ascontiguousarray(w).view(np.uint8).reshape(-1, N // 64, 4, 16, K // 128, 4, 2 * wb, 16)
+    #                          axes:  e, G, i, r, kb, q, v, byte  ->  e, G, kb, i, v, q, r, byte
+    out = np.ascontiguousarray(b.transpose(0, 1, 4, 2, 6, 5, 3, 7))
+    return out.reshape(-1).view(w.dtype).reshape(*lead, N, K)
+
+
+def kslab_unpack(p: np.ndarray) -> np.ndarray:
+    """Inverse of :func:`kslab_pack` for one matrix, as a scalar index walk."""
+    wb = p.dtype.itemsize
+    N, K = p.shape
+    flat = np.ascontiguousarray(p).view(np.uint8).reshape(-1)
+    rows = np.zeros((N, K * wb), dtype=np.uint8)
+    idx = 0
+    for G in range(N // 64):
+        for kb in range(K // 128):
+            for i in range(4):
+                for v in range(2 * wb):
+                    for lane in range(64):
+                        n = 64 * G + 16 * i + lane % 16
+                        off = (128 * kb + 32 * (lane // 16)) * wb + 16 * v
+                        rows[n, off:off + 16] = flat[idx:idx + 16]
+                        idx += 16
+    return rows.reshape(-1).view(p.dtype).reshape(N, K)

@@ -192,6 +192,60 @@ def test_dense_block_fp8_and_w8a16(ops):
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("dtype,shape", [(np.uint8, (3, 128, 256)), (np.uint16, (2, 64, 384)), (np.uint8, (192, 128))])
+def test_kslab_repack_bit_exact(rearrange, dtype, shape):
+    print(f"case kslab repack {dtype.__name__} {shape}", flush=True)
+    rng = np.random.default_rng(17)
+    w = rng.integers(0, np.iinfo(dtype).max, size=shape, dtype=dtype)
+    tdt = torch.int8 if dtype == np.uint8 else torch.float16
+    got = rearrange.to_kslab(dev(w).view(tdt))
+    assert rearrange.is_kslab(got) and got.shape == tuple(shape) and got.dtype == tdt
+    want = o8.kslab_pack(w)
+    assert np.array_equal(got.view(torch.uint8).cpu().numpy().reshape(-1), want.view(np.uint8).reshape(-1))
+    assert rearrange.to_kslab(got) is got
+    with pytest.raises(RuntimeError):
+        rearrange.to_kslab(torch.zeros((100, 128), dtype=torch.int8, device="cuda"))
+
+
+def test_kslab_and_row_major_weights_give_identical_results(fmoe, ops, rearrange, monkeypatch):
+    """Same kernel arithmetic in either weight order: outputs must be bit-identical,
+    for weights converted by the caller, converted implicitly, and left row-major."""
+    rng = np.random.default_rng(19)
+    M, E, T, K, N = 45, 5, 2, 384, 320
+    wq = np.stack([of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 3, -448, 448).astype(np.float32))
+                   for _ in range(E)])
+    ws = rng.uniform(0.5, 2.0, size=(E, (N + 127) // 128, K // 128)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+    xq, xs = ops.per_token_group_quant_fp8(x.cuda(), 128)
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    outs = []
+    for how in ("row-major", "implicit", "explicit"):
+        print(f"case kslab equivalence grouped fp8 {how}", flush=True)
+        monkeypatch.setattr(ops, "_AUTO_KSLAB", how != "row-major")
+        w = dev(wq).view(torch.float8_e4m3fn)
+        if how == "explicit":
+            w = rearrange.to_kslab(w)
+        C = torch.empty((M, T, N), dtype=torch.bfloat16, device="cuda")
+        run_grouped(fmoe, xq, w, C, xs, dev(ws), None, dev(tw), dev(ids), E, 16, False, T, use_fp8_w8a8=True,
+                    block_shape=[128, 128])
+        outs.append(C.view(torch.int16).cpu().numpy())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    # dense W8A16 (2-byte activations, 1-byte weights) and dense 16-bit weights through linear_quant's kernel
+    w8 = rng.integers(-128, 128, size=(N, K), dtype=np.int8)
+    s16 = rng.uniform(0.001, 0.01, N).astype(np.float16)
+    xh = dev(rng.standard_normal((M, K)).astype(np.float16))
+    outs = []
+    for auto in (False, True):
+        print(f"case kslab equivalence dense w8a16 auto={auto}", flush=True)
+        monkeypatch.setattr(ops, "_AUTO_KSLAB", auto)
+        o = ops.gptq_gemm_gcu(xh, dev(w8), torch.empty(0, device="cuda"), dev(s16), torch.empty(0, device="cuda"),
+                              8, None, -1)
+        outs.append(o.view(torch.int16).cpu().numpy())
+    assert np.array_equal(outs[0], outs[1])
+    want = o8.weight_only_int8(xh.cpu().numpy(), w8, s16, -1)
+    np.testing.assert_allclose(o.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
 # ---------------------------------------------------- whole sequence ----
 def build_moe(mode):
     from vllm_gcu_amd.kernels.modular_experts import TritonExpertsPad

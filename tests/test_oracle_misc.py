@@ -231,3 +231,23 @@ def test_silu_sum_and_fused_experts_identity():
             a = h[:I] / (1 + np.exp(-h[:I])) * h[I:]
             want[m] += tw[m, t] * (a @ w2[e].astype(np.float64))
     np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.uint16])
+def test_kslab_pack_is_inverted_by_scalar_walk_and_keeps_kib_runs(dtype):
+    rng = np.random.default_rng(5)
+    N, K = 128, 256
+    w = rng.integers(0, np.iinfo(dtype).max, size=(N, K), dtype=dtype)
+    p = w8a8.kslab_pack(w)
+    assert p.shape == w.shape and p.dtype == w.dtype
+    assert np.array_equal(w8a8.kslab_unpack(p), w)
+    # batched input packs each matrix on its own
+    both = w8a8.kslab_pack(np.stack([w, w[::-1]]))
+    assert np.array_equal(both[0], p) and np.array_equal(w8a8.kslab_unpack(both[1]), w[::-1])
+    # first KiB = vector 0 of tile 0 of block (0, 0): lane l holds 16 bytes of row l % 16 at byte 32*wb*(l//16)
+    wb = w.dtype.itemsize
+    kib = p.view(np.uint8).reshape(-1)[:1024].reshape(64, 16)
+    rows = w.view(np.uint8).reshape(N, K * wb)
+    for lane in (0, 1, 15, 16, 37, 63):
+        off = 32 * wb * (lane // 16)
+        assert np.array_equal(kib[lane], rows[lane % 16, off:off + 16])

@@ -178,7 +178,11 @@ def test_fp8_linear_method_block_scaled():
     layer.weight = torch.nn.Parameter(dev(w).view(torch.float8_e4m3fn), requires_grad=False)
     layer.weight_scale_inv = torch.nn.Parameter(dev(ws), requires_grad=False)
     method = Fp8GCUConfig.from_config({"weight_block_size": [128, 128]}).get_quant_method()
+    before = method.apply(layer, x.cuda(), bias.cuda())
+    method.process_weights_after_loading(layer)
+    assert getattr(layer.weight, "_mi355q_kslab", False)          # re-ordered in place at load time
     out = method.apply(layer, x.cuda(), bias.cuda())
+    assert torch.equal(before, out)
     xq, xs = of8.per_token_group_quant_fp8(x.float().numpy(), 128)
     want = of8.block_fp8_gemm(xq, xs, w, ws) + bias.float().numpy()
     assert out.dtype == torch.bfloat16 and out.shape == (M, N)
@@ -237,7 +241,10 @@ def test_fp8_and_int8_moe_methods_grouped_routing():
     layer.w13_weight = dev(w13).view(torch.float8_e4m3fn)
     layer.w2_weight = dev(w2).view(torch.float8_e4m3fn)
     layer.w13_weight_scale_inv, layer.w2_weight_scale_inv = dev(s13), dev(s2)
-    out = Fp8GCUConfig().get_quant_method(moe=True).apply(layer, x.cuda().clone(), dev(logits), **route)
+    method = Fp8GCUConfig().get_quant_method(moe=True)
+    method.process_weights_after_loading(layer)
+    assert layer.w13_weight._mi355q_kslab and layer.w2_weight._mi355q_kslab
+    out = method.apply(layer, x.cuda().clone(), dev(logits), **route)
 
     def deq(codes, sc):
         return (of8.from_e4m3fn(codes) * np.repeat(np.repeat(sc, 128, 0), 128, 1)).T
@@ -261,6 +268,8 @@ def test_fp8_and_int8_moe_methods_grouped_routing():
     layer8.cuda()
     load(layer8, "w13_weight", dev(w13i)); load(layer8, "w2_weight", dev(w2i))
     load(layer8, "w13_out_scales", dev(c13)); load(layer8, "w2_out_scales", dev(c2))
+    m8.process_weights_after_loading(layer8)
+    assert layer8.w13_weight._mi355q_kslab and layer8.w2_weight._mi355q_kslab
     out8 = m8.apply(layer8, x.cuda().clone(), dev(logits), **route)
 
     def qdq8(a):

@@ -4,6 +4,14 @@
 // fused-MoE grouped GEMM ("non-gather": rows are picked through
 // sorted_token_ids, weights through expert_ids) and for dense small-M calls.
 //
+// Weight layouts.  Row-major [N, K] (the checkpoint's) works, but a wavefront
+// load instruction then touches 16 rows and uses half of each 128-byte line
+// (measured: 4.4 TB/s on the DeepSeek-style fp8 layer).  The "kslab" layout
+// stores every 64-column x 128-k block of a wavefront in the order its lanes
+// consume it -- [N/64][K/128][4 tiles][vector][64 lanes][16 B] -- so that each
+// load instruction reads one contiguous KiB and a wavefront walks one
+// contiguous stream (5.9 TB/s on the same layer); mi355q_kslab_repack converts.
+//
 // These shapes are bound by the HBM stream of the weights.  A workgroup (4
 // wavefronts) owns up to 64 rows and 256 columns; a wavefront owns 64 columns
 // (four 16-row MFMA "A" tiles of weights) and every row tile of activations,
@@ -28,7 +36,7 @@ struct KcArgs {
   const void* w_scale;         // fp8: f32 [E, ceil(N/128), K/128]; int8: f32 [E, N]; W8A16: act dtype [E, N] or [E, K/g, N]
   const void* bias;            // [N] in out dtype, dense mode only
   int M, N, K;
-  int wgs;                     // W8A16 group size along K (K = per channel)
+  int kslab;                   // weights are in the kslab layout (N % 64 == 0)
   // grouped mode
   const int* sorted_ids;
   const int* expert_ids;
@@ -119,10 +127,17 @@ kcontig_gemm_kernel(KcArgs a) {
 
   // per-lane row pointers
   const char* wptr[4];
+  // byte strides between K blocks and between the 16-byte vectors of a lane
+  const long kstride = a.kslab ? 4 * 2048 * T::WBYTES : 128 * T::WBYTES;
+  const int vstride = a.kslab ? 1024 : 16;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int n = min(n0 + 16 * i + r16, N - 1);
-    wptr[i] = wbase + ((size_t)n * K + 32 * q) * T::WBYTES;
+    if (a.kslab) {
+      wptr[i] = wbase + (((size_t)(n0 >> 6) * KB) * 4 + i) * (2048 * T::WBYTES) + lane * 16;
+    } else {
+      const int n = min(n0 + 16 * i + r16, N - 1);
+      wptr[i] = wbase + ((size_t)n * K + 32 * q) * T::WBYTES;
+    }
   }
   const char* aptr[MT];
   int arow[MT];
@@ -153,7 +168,7 @@ kcontig_gemm_kernel(KcArgs a) {
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int v = 0; v < WV; ++v)
-        b.w[i][v] = __builtin_nontemporal_load((const u4*)(wptr[i] + (size_t)kb * 128 * T::WBYTES) + v);
+        b.w[i][v] = __builtin_nontemporal_load((const u4*)(wptr[i] + (size_t)kb * kstride + v * vstride));
 #pragma unroll
     for (int j = 0; j < MT; ++j)
 #pragma unroll
@@ -289,6 +304,25 @@ kcontig_gemm_kernel(KcArgs a) {
   }
 }
 
+// row-major [batch, N, K] -> kslab: one 16-byte chunk per thread
+__global__ void __launch_bounds__(256)
+kslab_repack_kernel(const u4* src, u4* dst, long chunks, int N, int K, int wb) {
+  const long c = (long)blockIdx.x * 256 + threadIdx.x;
+  if (c >= chunks) return;
+  const int wv = 2 * wb, KB = K >> 7;
+  const long per_mat = (long)N * K * wb / 16;
+  const long e = c / per_mat;
+  long r = c - e * per_mat;
+  const int lane = (int)(r & 63); r >>= 6;
+  const int v = (int)(r % wv); r /= wv;
+  const int i = (int)(r & 3); r >>= 2;
+  const int kb = (int)(r % KB);
+  const long ng = r / KB;
+  const long n = ng * 64 + i * 16 + (lane & 15);
+  const long byte = ((long)kb * 128 + 32 * (lane >> 4)) * wb + 16 * v;
+  dst[c] = src[e * per_mat + (n * K * wb + byte) / 16];
+}
+
 template <int MODE, int ODT, bool GROUPED>
 void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
   dim3 grid((a.N + 255) / 256, row_blocks), block(256);
@@ -338,7 +372,7 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
                                int group_size, const float* topk_weights, const int32_t* sorted_token_ids,
                                const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int numel,
                                int topk, int block_size, int max_blocks, int E, int K, int N, int act_dtype,
-                               int out_dtype, void* stream) {
+                               int out_dtype, int w_layout, void* stream) {
   MQ_REQUIRE(numel >= 0 && topk > 0 && E > 0 && K > 0 && N > 0, "moe_gemm: bad shape");
   if (numel == 0 || max_blocks == 0) return 0;
   MQ_REQUIRE(out && a && w && sorted_token_ids && expert_ids && num_tokens_post_pad, "moe_gemm: null pointer");
@@ -354,9 +388,10 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
                                 max_blocks, E, K, N, group_size <= 0 ? K : group_size, act_dtype, st);
   }
   MQ_REQUIRE(N % 4 == 0, "moe_gemm: N=%d must be a multiple of 4", N);
+  MQ_REQUIRE(w_layout == 0 || (w_layout == 1 && N % 64 == 0), "moe_gemm: weight layout %d needs N=%d %% 64 == 0", w_layout, N);
   KcArgs g = {};
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = nullptr;
-  g.M = numel; g.N = N; g.K = K; g.wgs = K;
+  g.M = numel; g.N = N; g.K = K; g.kslab = w_layout;
   g.sorted_ids = sorted_token_ids; g.expert_ids = expert_ids; g.npp = num_tokens_post_pad;
   g.topk_weights = topk_weights; g.numel = numel; g.topk = topk; g.block_size = block_size;
   g.w_stride = (long)N * K;
@@ -393,14 +428,15 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
 
 extern "C" int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_scale,
                                    const void* w_scale, const void* bias, int quant_mode, int group_size,
-                                   int M, int K, int N, int act_dtype, int out_dtype, void* stream) {
+                                   int M, int K, int N, int act_dtype, int out_dtype, int w_layout, void* stream) {
   MQ_REQUIRE(M >= 0 && K > 0 && N > 0, "kcontig_gemm: bad shape M=%d K=%d N=%d", M, K, N);
   if (M == 0) return 0;
   MQ_REQUIRE(out && a && w, "kcontig_gemm: null pointer");
   MQ_REQUIRE(K % 128 == 0 && N % 4 == 0, "kcontig_gemm: K=%d must be a multiple of 128 and N=%d of 4", K, N);
+  MQ_REQUIRE(w_layout == 0 || (w_layout == 1 && N % 64 == 0), "kcontig_gemm: weight layout %d needs N=%d %% 64 == 0", w_layout, N);
   KcArgs g = {};
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = bias;
-  g.M = M; g.N = N; g.K = K; g.wgs = K;
+  g.M = M; g.N = N; g.K = K; g.kslab = w_layout;
   g.numel = M; g.topk = 1; g.block_size = 64;
   int mode;
   if (quant_mode == 1) {
@@ -424,5 +460,18 @@ extern "C" int mi355q_kcontig_gemm(void* out, const void* a, const void* w, cons
   int rc = launch_mode<false>(g, mode, out_dtype, mt, row_blocks, as_stream(stream));
   if (rc) return rc;
   MQ_LAUNCH_CHECK("kcontig_gemm");
+  return 0;
+}
+
+extern "C" int mi355q_kslab_repack(const void* src, void* dst, int batch, int N, int K, int elem_bytes,
+                                   void* stream) {
+  MQ_REQUIRE(batch > 0 && N > 0 && K > 0, "kslab_repack: bad shape batch=%d N=%d K=%d", batch, N, K);
+  MQ_REQUIRE(src && dst && src != dst, "kslab_repack: needs distinct source and destination");
+  MQ_REQUIRE(N % 64 == 0 && K % 128 == 0, "kslab_repack: N=%d must be a multiple of 64 and K=%d of 128", N, K);
+  MQ_REQUIRE(elem_bytes == 1 || elem_bytes == 2, "kslab_repack: element size %d must be 1 or 2", elem_bytes);
+  const long chunks = (long)batch * N * K * elem_bytes / 16;
+  hipLaunchKernelGGL(kslab_repack_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     (const u4*)src, (u4*)dst, chunks, N, K, elem_bytes);
+  MQ_LAUNCH_CHECK("kslab_repack");
   return 0;
 }

@@ -11,6 +11,8 @@ converts tensors to raw pointers and calls the C ABI of ``libmi355q.so``.
 """
 from typing import List, Optional, Tuple
 
+import os
+
 import torch
 
 from .. import _lib
@@ -707,6 +709,24 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int, eps: float = 1e-
 # fused-MoE grouped GEMM, block-fp8 and weight-only dense GEMMs
 # (csrc/torch_bindings.cpp:790-849, 1021-1027)
 # ---------------------------------------------------------------------------
+_AUTO_KSLAB = os.environ.get("MI355Q_AUTO_KSLAB", "1") != "0"
+
+
+def _kcontig_weight(w: torch.Tensor):
+    """-> (weight tensor, layout code).  K-contiguous weights stream about a
+    third faster in the kslab order; a row-major tensor that qualifies is
+    converted on first use and the copy cached on it (twice the memory -- the
+    method classes convert in place at load time instead; MI355Q_AUTO_KSLAB=0
+    turns the implicit conversion off)."""
+    from .quantization import rearrange
+    if rearrange.is_kslab(w):
+        return w, 1
+    w = w.contiguous()
+    if _AUTO_KSLAB and rearrange.kslab_eligible(w):
+        return _converted(w, rearrange.to_kslab), 1
+    return w, 0
+
+
 def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids, experts_ids,
               num_tokens_post_pad, mul_routed_weight, topk, block_size, bias, real_token_num):
     """``C.view(-1, N)[t] = A[t // topk] @ W[e(t)]^T (* topk_weights.flat[t])``
@@ -768,6 +788,9 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
         act_code = rt.dtype_code(A.dtype)
     else:
         raise RuntimeError(f"fused_moe: cannot infer the quantisation mode from A {A.dtype} / B {B.dtype}")
+    layout = 0
+    if mode != _lib.Q_W4A16:
+        w, layout = _kcontig_weight(w)
     E = w.shape[0]
     tw = None
     if mul_routed_weight:
@@ -783,7 +806,7 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
         _lib.call("mi355q_moe_gemm", C.data_ptr(), A.data_ptr(), w.data_ptr(), rt.ptr(a_scale), rt.ptr(w_scale),
                   rt.ptr(zp), zk, mode, group, rt.ptr(tw), sorted_token_ids.data_ptr(), experts_ids.data_ptr(),
                   num_tokens_post_pad.data_ptr(), numel, int(topk), int(block_size), experts_ids.numel(), E, K, N,
-                  act_code, rt.dtype_code(C.dtype), rt.stream_ptr())
+                  act_code, rt.dtype_code(C.dtype), layout, rt.stream_ptr())
 
 
 def _fused_moe_quant_kernel_impl(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids,
@@ -811,10 +834,11 @@ def _kcontig(out, a, w, a_scale, w_scale, bias, mode, group):
     if bias is not None:
         bias = bias.to(out.dtype).contiguous()
     act = _lib.F16 if a.dtype in (torch.float8_e4m3fn, torch.int8) else rt.dtype_code(a.dtype)
+    w, layout = _kcontig_weight(w)
     with torch.cuda.device(a.device):
         _lib.call("mi355q_kcontig_gemm", out.data_ptr(), a2.data_ptr(), w.data_ptr(), rt.ptr(a_scale),
                   rt.ptr(w_scale), rt.ptr(bias), mode, group, M, K, N, act, rt.dtype_code(out.dtype),
-                  rt.stream_ptr())
+                  layout, rt.stream_ptr())
 
 
 def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):

@@ -12,6 +12,7 @@ from ..fused_moe import select_experts
 from ..modular_experts import TritonExpertsPad
 from ..modular_kernel import FusedMoEModularKernel
 from ..prepare_finalize import MoEPrepareAndFinalizeNoEP
+from . import rearrange
 from .utils import register_gcu_quantization_config
 
 
@@ -60,6 +61,11 @@ class Fp8GCULinearMethod:
         self.quant_config = quant_config
         self.block_quant = quant_config.weight_block_size is not None
 
+    def process_weights_after_loading(self, layer) -> None:
+        # the reference keeps the checkpoint tensors as they are (fp8.py:72-166);
+        # here the weight bytes are re-ordered once for contiguous wavefront loads
+        rearrange.kslab_parameters_(layer, ("weight",))
+
     def apply(self, layer, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
               x_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
         if not self.block_quant:
@@ -81,6 +87,9 @@ class Fp8GCUMoEMethod:
 
     def select_gemm_impl(self, prepare_finalize=None, moe=None):
         return TritonExpertsPad(use_fp8_w8a8=True, block_shape=self.quant_config.weight_block_size)
+
+    def process_weights_after_loading(self, layer) -> None:
+        rearrange.kslab_parameters_(layer, ("w13_weight", "w2_weight"))
 
     def apply(self, layer, x, router_logits, top_k: int, renormalize: bool, use_grouped_topk: bool = False,
               global_num_experts: int = -1, expert_map=None, topk_group=None, num_expert_group=None,

@@ -105,3 +105,51 @@ def unpack_slab(packed: torch.Tensor) -> torch.Tensor:
         _lib.call("mi355q_w4_unpack", packed.contiguous().data_ptr(), dst.data_ptr(),
                   1 if batch is None else batch, K, N, rt.stream_ptr())
     return dst
+
+
+def is_kslab(w: torch.Tensor) -> bool:
+    return bool(getattr(w, "_mi355q_kslab", False))
+
+
+def kslab_eligible(w: torch.Tensor) -> bool:
+    return (w.dim() in (2, 3) and w.element_size() in (1, 2) and w.shape[-2] % 64 == 0
+            and w.shape[-1] % 128 == 0 and w.is_contiguous())
+
+
+def to_kslab(w: torch.Tensor) -> torch.Tensor:
+    """K-contiguous weights ``[N, K]`` / ``[E, N, K]`` (fp8, int8 or 16-bit) ->
+    the same bytes in the streaming "kslab" order (see include/mi355q.h); the
+    result keeps shape and dtype and carries the attribute ``_mi355q_kslab``.
+    The reference keeps these weights row-major (fp8.py:72-166, w8a8.py:240-262);
+    this is a load-time conversion of this build, like its int4 rearrange."""
+    rt.require_gpu(w)
+    if is_kslab(w):
+        return w
+    if not kslab_eligible(w):
+        raise RuntimeError(f"to_kslab: need contiguous [.., N % 64 == 0, K % 128 == 0] 1- or 2-byte weights, "
+                           f"got {w.dtype} {tuple(w.shape)}")
+    batch = 1 if w.dim() == 2 else w.shape[0]
+    dst = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        _lib.call("mi355q_kslab_repack", w.data_ptr(), dst.data_ptr(), batch, w.shape[-2], w.shape[-1],
+                  w.element_size(), rt.stream_ptr())
+    dst._mi355q_kslab = True
+    return dst
+
+
+def mark_kslab(p: torch.Tensor) -> torch.Tensor:
+    """Re-attach the layout flag after wrapping a kslab tensor (e.g. in a Parameter)."""
+    p._mi355q_kslab = True
+    return p
+
+
+def kslab_parameters_(layer, names) -> None:
+    """Load-time, in place: replace each named parameter of ``layer`` that
+    qualifies by its kslab-ordered copy (the row-major tensor is dropped, so no
+    weight is resident twice)."""
+    for name in names:
+        w = getattr(layer, name, None)
+        if w is None or is_kslab(w) or not w.is_cuda or not kslab_eligible(w.data):
+            continue
+        packed = torch.nn.Parameter(to_kslab(w.data), requires_grad=False)
+        setattr(layer, name, mark_kslab(packed))

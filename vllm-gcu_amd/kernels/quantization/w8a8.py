@@ -18,6 +18,7 @@ from ..fused_moe import select_experts
 from ..modular_experts import TritonExpertsPad
 from ..modular_kernel import FusedMoEModularKernel
 from ..prepare_finalize import MoEPrepareAndFinalizeNoEP
+from . import rearrange
 from .utils import register_gcu_quantization_config
 
 
@@ -94,6 +95,11 @@ class FusedW8A8MoEMethod:
 
     def select_gemm_impl(self, prepare_finalize=None, moe=None):
         return TritonExpertsPad(use_int8_w8a8=True, per_channel_quant=True, per_act_token_quant=True)
+
+    def process_weights_after_loading(self, layer) -> None:
+        # experts stay [E, N, K] as loaded (w8a8.py:240-262 transposes nothing either);
+        # their bytes are re-ordered once for contiguous wavefront loads
+        rearrange.kslab_parameters_(layer, ("w13_weight", "w2_weight"))
 
     def create_weights(self, layer, num_experts, hidden_size, intermediate_size_per_partition, params_dtype,
                        **extra_weight_attrs):
