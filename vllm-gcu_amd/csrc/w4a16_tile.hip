@@ -6,10 +6,11 @@
 // each lane's MFMA B operand contiguously, a wavefront dequantises its own
 // columns straight into B operands in registers -- the exact integers (q - z),
 // the group scale is applied to the fp32 partial sum of each K block -- and
-// every operand is reused for the 8 row tiles, so no weight is dequantised
-// twice in a workgroup.  The activation tile is shared
-// by the 4 wavefronts through LDS (double buffered, rows padded by 32 B so
-// the operand reads are bank-conflict free).  fp32 accumulate.
+// every operand is reused for all row tiles of the wavefront.  The activation
+// tile is shared by the wavefronts through LDS (double buffered, rows padded by
+// 32 B so the operand reads are bank-conflict free).  fp32 accumulate.  The
+// fp16 128-row variant runs a hand-pipelined K loop (see PIPE below), the
+// others a plain one.
 #include "common.h"
 
 namespace mi355q {
@@ -52,8 +53,9 @@ template <> struct TileMma<MI355Q_F16> {
   static __device__ __forceinline__ f4 run(vec a, vec b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
-  // one packed word -> 8 values (q - z); zlo = (1024 + z) x2, zhi = (64 + z) x2
-  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zlo, h2 zhi) {
+  // one packed word -> 8 values (q - z); zz = {1024 + z, 64 + z}
+  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz) {
+    const h2 zlo = {zz.x, zz.x}, zhi = {zz.y, zz.y};
     const uint32_t MAGIC = 0x64006400u;
     const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
     uint32_t w8 = w >> 8;
@@ -78,8 +80,8 @@ template <> struct TileMma<MI355Q_BF16> {
     uint32_t lo = bitcast<uint32_t>((float)r.x), hi = bitcast<uint32_t>((float)r.y);
     return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
   }
-  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zlo, h2 zhi) {
-    h8 v = TileMma<MI355Q_F16>::dequant(w, zlo, zhi);
+  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz) {
+    h8 v = TileMma<MI355Q_F16>::dequant(w, zz);
     u4 r = {cvt((h2){v[0], v[1]}), cvt((h2){v[2], v[3]}), cvt((h2){v[4], v[5]}), cvt((h2){v[6], v[7]})};
     return bitcast<vec>(r);
   }
@@ -136,34 +138,36 @@ w4a16_tile_kernel(TileArgs a) {
   // global -> register staging of the next activation tile: thread tid loads
   // MTW chunks of 16 B: row = pass * 16 WM + tid / 16, chunk = tid % 16
   const int arow = tid >> 4, achunk = tid & 15;
-  const uint16_t* aptr[MTW];
+  // byte offsets from a.x (32-bit: the host checks that the activation matrix is below 4 GiB)
+  uint32_t aofs[MTW];
 #pragma unroll
   for (int p = 0; p < MTW; ++p) {
     int row;
     if (GROUPED) row = min(tok[p * 16 * WM + arow], a.numel - 1) / a.topk;   // pads read a valid row
     else row = min(m0 + p * 16 * WM + arow, M - 1);
-    aptr[p] = a.x + (size_t)row * K + 8 * achunk;
+    aofs[p] = ((uint32_t)row * (uint32_t)K + 8u * achunk) * 2u;
   }
   u4 areg[MTW];
   auto load_a = [&](int g) {
 #pragma unroll
-    for (int p = 0; p < MTW; ++p) areg[p] = *(const u4*)(aptr[p] + 128 * g);
+    for (int p = 0; p < MTW; ++p) areg[p] = *(const u4*)((const char*)a.x + (aofs[p] + 256u * (uint32_t)g));
   };
-  auto store_a = [&](int buf) {
-    unsigned char* base = lds + buf * A_BUF;
+  auto store_a = [&](unsigned buf_off) {
+    unsigned char* base = lds + buf_off;
 #pragma unroll
     for (int p = 0; p < MTW; ++p) *(u4*)(base + (p * 16 * WM + arow) * A_ROW + achunk * 16) = areg[p];
   };
 
   const u4* wbase = qw + ((size_t)slab * G * 8 + t0) * 64 + lane;
-  u4 wreg[4];
   uint2 sreg;
   uint32_t zreg = 0x88888888u;
   uint2 zsreg = {0u, 0u};
-  auto load_b = [&](int g) {
+  auto load_w = [&](u4 (&w)[4], int g) {
     const u4* p = wbase + (size_t)g * 512;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) wreg[t] = p[t * 64];
+    for (int t = 0; t < 4; ++t) w[t] = p[t * 64];
+  };
+  auto load_sz = [&](int g) {
     const int qrow = (128 * g) / a.gs;
     sreg = *(const uint2*)(scales + (size_t)qrow * N + ncol);
     if (ZK == MI355Q_ZP_PACKED) zreg = ((const uint32_t*)zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)] >> (4 * t0);
@@ -171,66 +175,185 @@ w4a16_tile_kernel(TileArgs a) {
   };
 
   const int gb = GROUPED ? 0 : (int)blockIdx.z * a.kper, ge = GROUPED ? G : min(G, gb + a.kper);
-  load_a(gb);
-  load_b(gb);
-  store_a(0);
-  __syncthreads();
-
-  for (int g = gb; g < ge; ++g) {
-    const int buf = (g - gb) & 1;
-    // operands of this K block, then start the next block's loads
-    u4 wcur[4];
+  // The pipelined loop needs nearly the whole register file; it is used where it fits
+  // (fp16, 128-row tiles), the plain loop elsewhere.
+  constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED;
+  if constexpr (PIPE) {
+    // Software pipeline, written out because the compiler otherwise sinks every
+    // load next to its use.  Activations: global loads at the top of the K block
+    // before their use, stored into the other LDS buffer near its end.  Weights:
+    // two register sets that swap roles every K block; a set is re-requested as
+    // soon as its last word has been dequantised.  B operands of K step s + 1 are dequantised while the matrix
+    // instructions of step s run, one column tile per matrix group; A operands
+    // come from LDS two matrix groups ahead.  Each K block accumulates into its
+    // own partial tile, scaled into the running sum as its rows finish.  The one
+    // barrier per K block sits just before the first read of the other buffer:
+    // all reads of the current buffer have been issued by then (and the barrier
+    // waits for them), so two buffers are enough.
+    // scales stay packed as loaded (two per register) and are widened where they are used
+    uint2 sc, scp;
+    auto scale_of = [&](uint2 sv, int t) {
+      const uint32_t sw = (t < 2) ? sv.x : sv.y;
+      return Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+    };
+    h2 zz[4];
+    auto prep = [&]() {
+      sc = sreg;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) wcur[t] = wreg[t];
-    float sc[4];
-    h2 zlo[4], zhi[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const uint32_t sw = (t < 2) ? sreg.x : sreg.y;
-      sc[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
-      float zf;
-      if (ZK == MI355Q_ZP_PRESCALED) {
-        const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
-        // the loader pre-multiplied an integer zero-point by the scale
-        // (z * s rounded to the activation type): recover the integer
-        zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[t]);
-      } else {
-        zf = (float)((zreg >> (4 * t)) & 15u);
+      for (int t = 0; t < 4; ++t) {
+        if (ZK == MI355Q_ZP_PRESCALED) {
+          const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
+          // the loader pre-multiplied an integer zero-point by the scale
+          // (z * s rounded to the activation type): recover the integer
+          const float zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / scale_of(sc, t));
+          zz[t] = (h2){(_Float16)(1024.0f + zf), (_Float16)(64.0f + zf)};
+        } else {
+          // fp16 bit patterns directly: 1024 + z = 0x6400 | z, 64 + z = 0x5400 | z << 4
+          const uint32_t z = (zreg >> (4 * t)) & 15u;
+          zz[t] = bitcast<h2>(0x54006400u | z | (z << 20));
+        }
       }
-      const _Float16 zl = (_Float16)(1024.0f + zf), zh = (_Float16)(64.0f + zf);
-      zlo[t] = (h2){zl, zl};
-      zhi[t] = (h2){zh, zh};
-    }
-    const int gn = min(g + 1, ge - 1);
-    load_a(gn);
-    load_b(gn);
+    };
+    const unsigned aoff = (wmh * MTW * 16 + c) * A_ROW + kq * 16;
+    auto lds_a = [&](unsigned buf_off, int mt, int st) {
+      return bitcast<vec>(*(const u4*)(lds + buf_off + aoff + mt * 16 * A_ROW + st * 64));
+    };
 
-    // all 16 B operands of this K block (4 steps x 4 column tiles)
-    vec bv[4][4];
+    u4 w0[4], w1[4];
+    load_a(gb);
+    load_w(w0, gb);
+    load_sz(gb);
+    store_a(0);
+    prep();
+    vec bv[4];
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-#pragma unroll
-      for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zlo[t], zhi[t]);
-
-    const unsigned char* abase = lds + buf * A_BUF + (wmh * MTW * 16 + c) * A_ROW + kq * 16;
-#pragma unroll
-    for (int mt = 0; mt < MTW; ++mt) {
-      f4 part[4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const vec av = bitcast<vec>(*(const u4*)(abase + mt * 16 * A_ROW + s * 64));
-#pragma unroll
-        for (int t = 0; t < 4; ++t) part[t] = MM::run(av, bv[s][t], part[t]);
-      }
-#pragma unroll
-      for (int t = 0; t < 4; ++t) acc[mt][t] += sc[t] * part[t];
-    }
-    // the other buffer was last read one iteration ago: every wavefront has
-    // passed the barrier below since, so it can be overwritten now
-    store_a(buf ^ 1);
+    for (int t = 0; t < 4; ++t) bv[t] = MM::dequant(w0[t][0], zz[t]);
+    load_w(w1, min(gb + 1, ge - 1));
+    load_sz(min(gb + 1, ge - 1));
+    f4 part[MTW][4];
     __syncthreads();
+    constexpr int NJ = 4 * MTW;                      // matrix groups (K step x row tile) per K block
+    constexpr int TPG = 4 / MTW > 0 ? 4 / MTW : 1;   // column tiles dequantised per group
+    static_assert(MTW == 1 || MTW == 2 || MTW == 4, "row tiles per wavefront");
+      constexpr int PF = 2;                          // LDS prefetch distance in matrix groups
+    vec avr[4];
+#pragma unroll
+    for (int j = 0; j < PF; ++j) avr[j] = lds_a(0, j % MTW, j / MTW);
+    unsigned cur = 0, nxt = A_BUF;
+
+    auto kblock = [&](int g, u4 (&wc)[4], u4 (&wn)[4]) {
+      load_a(min(g + 1, ge - 1));
+      __builtin_amdgcn_sched_barrier(0);
+      vec bn[4];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int st = j / MTW, mt = j % MTW;
+        if (j == (NJ >= 8 ? NJ - 4 : 0)) store_a(nxt);   // block g + 1, requested at the top
+        if (j == NJ - PF) __syncthreads();
+        {
+          const int jj = j + PF;
+          avr[jj % 4] = jj < NJ ? lds_a(cur, jj % MTW, jj / MTW) : lds_a(nxt, (jj - NJ) % MTW, (jj - NJ) / MTW);
+        }
+        if (st == 3 && mt == 0) {
+          // operands of the next K block from here on; its words arrived during this one
+          scp = sc;
+          prep();
+          load_sz(min(g + 2, ge - 1));
+        }
+#pragma unroll
+        for (int t = mt * TPG; t < (mt + 1) * TPG; ++t)
+          bn[t] = MM::dequant(st < 3 ? wc[t][st + 1] : wn[t][0], zz[t]);
+        if (st == 2 && mt == MTW - 1) load_w(wc, min(g + 2, ge - 1));   // last word of wc just went
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          part[mt][t] = MM::run(avr[j % 4], bv[t], st == 0 ? (f4){0.f, 0.f, 0.f, 0.f} : part[mt][t]);
+        if (st == 3 && mt > 0) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[mt - 1][t] += scale_of(scp, t) * part[mt - 1][t];
+        }
+        if (mt == MTW - 1) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) bv[t] = bn[t];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[MTW - 1][t] += scale_of(scp, t) * part[MTW - 1][t];
+      const unsigned o = cur;
+      cur = nxt;
+      nxt = o;
+    };
+    for (int g = gb;; g += 2) {
+      kblock(g, w0, w1);
+      if (g + 1 >= ge) break;
+      kblock(g + 1, w1, w0);
+      if (g + 2 >= ge) break;
+    }
+  } else {
+    // Plain loop: operands of the whole K block dequantised up front, the next block's loads
+    // pinned at the top, one partial tile per row tile.  Two wavefronts per SIMD cover each
+    // other's dequantisation bursts.
+    u4 wreg[4];
+    load_a(gb);
+    load_w(wreg, gb);
+    load_sz(gb);
+    store_a(0);
+    __syncthreads();
+    for (int g = gb; g < ge; ++g) {
+      const unsigned buf = ((g - gb) & 1) * A_BUF;
+      u4 wcur[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) wcur[t] = wreg[t];
+      float sc[4];
+      h2 zz[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t sw = (t < 2) ? sreg.x : sreg.y;
+        sc[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+        float zf;
+        if (ZK == MI355Q_ZP_PRESCALED) {
+          const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
+          // the loader pre-multiplied an integer zero-point by the scale
+          // (z * s rounded to the activation type): recover the integer
+          zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[t]);
+        } else {
+          zf = (float)((zreg >> (4 * t)) & 15u);
+        }
+        zz[t] = (h2){(_Float16)(1024.0f + zf), (_Float16)(64.0f + zf)};
+      }
+      const int gn = min(g + 1, ge - 1);
+      load_a(gn);
+      load_w(wreg, gn);
+      load_sz(gn);
+      __builtin_amdgcn_sched_barrier(0);     // keep the prefetch at the top: a full K block to land
+
+      // all 16 B operands of this K block (4 steps x 4 column tiles)
+      vec bv[4][4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zz[t]);
+
+      const unsigned char* abase = lds + buf + (wmh * MTW * 16 + c) * A_ROW + kq * 16;
+#pragma unroll
+      for (int mt = 0; mt < MTW; ++mt) {
+        f4 part[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const vec av = bitcast<vec>(*(const u4*)(abase + mt * 16 * A_ROW + s * 64));
+#pragma unroll
+          for (int t = 0; t < 4; ++t) part[t] = MM::run(av, bv[s][t], part[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[mt][t] += sc[t] * part[t];
+      }
+      // the other buffer was last read one iteration ago: every wavefront has
+      // passed the barrier below since, so it can be overwritten now
+      store_a(A_BUF - buf);
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: 4 adjacent columns per (row tile, i) ----
@@ -292,16 +415,18 @@ w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* 
 
 template <int DT, int ZK, int MT, bool GROUPED>
 hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
-  constexpr int BM = 16 * MT;
-  constexpr int WM = MT >= 4 ? 2 : 1;              // eight wavefronts once there are rows to split
-  const int G = a.K >> 7;
-  dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
-  const size_t shmem = 2 * BM * A_ROW;             // up to 144 KiB: above the 64 KiB default
-  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-  if (attr != hipSuccess) return attr;
-  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>), grid, block, shmem, st, a);
-  return hipSuccess;
+  {
+    constexpr int BM = 16 * MT;
+    constexpr int WM = MT >= 4 ? 2 : 1;            // eight wavefronts once there are rows to split
+    const int G = a.K >> 7;
+    dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
+    const size_t shmem = 2 * BM * A_ROW;           // up to 72 KiB: above the 64 KiB default
+    static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>), grid, block, shmem, st, a);
+    return hipSuccess;
+  }
 }
 
 template <int DT, int MT, bool GROUPED>
@@ -328,8 +453,10 @@ hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStrea
 // partial tiles of at most TILE_SPLITK_BYTES in total
 constexpr size_t TILE_SPLITK_BYTES = (size_t)64 << 20;
 static int tile_rows_mt(int M, int N) {
-  // 128-row blocks once they fill the chip, 64-row blocks for mid-sized M
-  return ((long)((M + 127) / 128) * ((N + BN - 1) / BN) >= device_cu_count()) ? 8 : 4;
+  // 128-row blocks as soon as there are more than 64 rows (measured faster from M = 96 up,
+  // split-K filling the chip where the grid alone does not), 64-row blocks below
+  (void)N;
+  return M > 64 ? 8 : 4;
 }
 static int tile_splits(int M, int K, int N) {
   const int mt = tile_rows_mt(M, N), G = K / 128;
@@ -351,6 +478,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                       int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
   MQ_REQUIRE(group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
+  MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
   TileArgs a = {};
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;
@@ -391,6 +519,8 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                          int group_size, int dtype, hipStream_t st) {
   MQ_REQUIRE(group_size % 128 == 0, "moe_w4a16: group_size=%d must be a multiple of 128", group_size);
+  MQ_REQUIRE((size_t)(numel / (topk > 0 ? topk : 1)) * K * 2 < ((size_t)1 << 32),
+             "moe_w4a16: activation matrix of %d rows x %d is 4 GiB or more", numel / (topk > 0 ? topk : 1), K);
   MQ_REQUIRE(block_size == 16 || block_size == 32 || block_size == 64 || block_size == 128,
              "moe_w4a16: block_size=%d must be 16, 32, 64 or 128", block_size);
   TileArgs a = {};
