@@ -38,7 +38,10 @@ enum {
   MI355Q_W4_SRC_GPTQ = 0,      /* int32 [K/8, N], nibble i of row r = k 8r+i (rearrange.py:13-21)     */
   MI355Q_W4_SRC_AWQ = 1,       /* int32 [K, N/8], AWQ interleave (rearrange.py:66-95)                 */
   MI355Q_W4_SRC_REF_KN = 2,    /* uint8 [K/2, N] reference half-group layout (rearrange.py:36-56)     */
-  MI355Q_W4_SRC_REF_NK = 3     /* uint8 [N, K/2] the same, stored transposed for MoE experts          */
+  MI355Q_W4_SRC_REF_NK = 3,    /* uint8 [N, K/2] the same, stored transposed for MoE experts          */
+  MI355Q_W4_SRC_REF_KN_G64S = 4 /* int8 [K/2, N], half-groups of 32 rows, nibbles hold w - 8 (the w4a8
+                                  experts: rearrange.py:61-133 with use_w4a8, rearrange_group 64, as
+                                  vllm_gcu/kernels/quantization/w4a8.py:134-220 stores them)          */
                                /* (vllm_gcu/kernels/quantization/moe_wna16.py:464-466)                */
 };
 
@@ -178,6 +181,21 @@ int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x, int rows,
  * 1: v = silu(x[:, :K]) * x[:, K:] of x [rows, 2K]; 2: v = x[:, :K] * x[:, K:] */
 int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, long rows, int K,
                             int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream);
+/* rms_norm / fused_add_rms_norm and their fusions with the activation quantisers
+ * (csrc/torch_bindings.cpp:254-272 rms_norm, fused_add_rms_norm; :277-317 *_static_fp8_quant;
+ * :852-871 *_static_int8_quant; :1124-1143 *_per_token_group_quant_fp8; equivalences
+ * vllm_gcu/compilation/fusion.py:104-127, 183-330).  Rows of K elements (K % 8 == 0):
+ * z = x (+ residual; residual := z when given), o = act(act(z * rsqrt(mean z^2 + eps)) * weight)
+ * with act() = rounding to `dtype`; quant_mode 0: out = o; 1: out = e4m3fn(o / *scale);
+ * 2: out = e4m3fn per group of group_size with out_scales f32 [rows, K/group_size];
+ * 3: out = int8 rne(o * act(1 / *scale)).  out may alias x when quant_mode is 0. */
+int mi355q_rms_norm(void* out, float* out_scales, const void* x, void* residual, const void* weight,
+                    const float* scale, float eps, long rows, int K, int quant_mode, int group_size,
+                    int dtype, void* stream);
+/* fp8-e4m3fn -> f16 / bf16, exact; n a multiple of 4.  Feeds fp8 activations to the int4 expert
+ * GEMM of fused_moe_quant_kernel_ex (csrc/src/fused_moe_quant_kernel_ex.cpp:13-45), which the
+ * reference's vendor kernel consumes directly. */
+int mi355q_fp8_to_half(void* out, const uint8_t* in, long n, int out_dtype, void* stream);
 /* moe_sum_pad (csrc/src/moe_sum.cpp:64-131): out[m, :] = sum_t in[m, t, :], fp32 accumulate */
 int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in_dtype, int out_dtype,
                    const int32_t* valid_rows, void* stream);
@@ -187,8 +205,14 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
  * [E, K/g, N], zeros per zeros_kind), 1 = fp8-e4m3fn with 128x128 block scales
  * (w [E, N, K], a_scale f32 [Ma, K/128], w_scale f32 [E, ceil(N/128), K/128]),
  * 2 = int8 (a_scale f32 [Ma] or NULL, w_scale f32 [E, N]), 3 = unquantised
- * f16/bf16 (w [E, N, K]), 4 = W8A16 (w int8 [E, N, K], w_scale [E, N] in the
- * activation dtype).
+ * f16/bf16 (w [E, N, K]), 4 = W8A16 (w int8 [E, N, K], w_scale in the activation
+ * dtype: [E, N] per channel with group_size <= 0 or K, [E, K/g, N] with
+ * group_size g = 64 or 128, as weight_only_quant and the w8a16 experts take them,
+ * csrc/src/weight_only_quant.cpp:28-101, vllm_gcu/kernels/fused_moe.py:163-169), 5 = symmetric int4 experts as in mode 0 but with fp32 group
+ * scales w_scale [E, K/g, N] and a_scale = one fp32 value multiplied into every
+ * output (the w4a8-fp8 experts of fused_moe_quant_kernel_ex,
+ * csrc/src/fused_moe_quant_kernel_ex.cpp:13-45: a holds the fp8 activations
+ * widened by mi355q_fp8_to_half, a_scale their dequantisation scale).
  *
  * mi355q_moe_gemm replaces vllmInvokeFusedMoeNonGatherQuantKernel as called by
  * fused_moe_quant_kernel / fused_moe_kernel (csrc/src/fused_moe_quant_kernel.cpp:30-200,

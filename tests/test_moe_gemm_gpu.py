@@ -246,6 +246,88 @@ def test_kslab_and_row_major_weights_give_identical_results(fmoe, ops, rearrange
     np.testing.assert_allclose(o.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("g", [64, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_w8a16_group_scales_dense_and_grouped(fmoe, ops, g, dtype):
+    """weight_only_quant / w8a16 experts with scales [K/g, N] (weight_only_quant.cpp:28-101,
+    fused_moe.py:163-169)."""
+    print(f"case w8a16 group={g} {dtype}", flush=True)
+    rng = np.random.default_rng(37 + g)
+    M, E, T, K, N = 35, 3, 2, 384, 320
+    rnd = bf16 if dtype == torch.bfloat16 else f16
+    xh = rnd(rng.standard_normal((M, K)).astype(np.float32))
+    w8 = rng.integers(-128, 128, size=(E, N, K), dtype=np.int8)
+    sg = rnd(rng.uniform(0.001, 0.01, size=(E, K // g, N)).astype(np.float32))
+    xd = torch.from_numpy(xh).to(dtype).cuda()
+    # dense, through the 8-bit GPTQ entry (the group scales are what it forwards)
+    out = ops.gptq_gemm_gcu(xd, dev(w8[0]), torch.empty(0, device="cuda"), torch.from_numpy(sg[0]).to(dtype).cuda(),
+                            torch.empty(0, device="cuda"), 8, None, g)
+    want = o8.weight_only_int8(xh, w8[0], sg[0], g)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # grouped
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    C = torch.empty((M, T, N), dtype=dtype, device="cuda")
+    run_grouped(fmoe, xd, dev(w8), C, None, torch.from_numpy(sg).to(dtype).cuda(), None, dev(tw), dev(ids), E, 32,
+                True, T, use_int8_w8a16=True, block_shape=[0, g])
+
+    def wf(e):
+        return (w8[e].astype(np.float32).reshape(N, K // g, g) * sg[e].T.reshape(N, K // g, 1)).reshape(N, K).T
+
+    want = om.fused_moe_gemm(xh, wf, ids, T, tw, True)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def make_w4a8_experts(rng, E, K, N):
+    """Logical unsigned weights, their reference-layout int8 tensor [E, N, K/2]
+    (memory [E, K/2, N], w4a8.py:199-220) and the AWQ checkpoint tensor."""
+    wl = rng.integers(0, 16, size=(E, K, N), dtype=np.uint8)
+    s = rng.uniform(0.002, 0.02, size=(E, K // 128, N)).astype(np.float32)
+    awq = np.stack([ow4.awq_pack(wl[e]) for e in range(E)])
+    ref = np.stack([ow4.rearrange_awq(awq[e], None, s[e], rearrange_group=64, zeros_in_int8=True, use_w4a8=True)[0]
+                    for e in range(E)])                      # int8 [E, K/2, N]
+    return wl, s, awq, ref
+
+
+def test_w4a8_reference_layout_and_checkpoint_repack_bit_exact(rearrange):
+    print("case w4a8 repack", flush=True)
+    rng = np.random.default_rng(23)
+    E, K, N = 3, 256, 384
+    wl, s, awq, ref = make_w4a8_experts(rng, E, K, N)
+    want = np.stack([ow4.native_pack(wl[e]) for e in range(E)])
+    got_ref = rearrange.from_reference_w4a8(dev(ref).view(E, N, K // 2))
+    got_awq, _ = rearrange.rearrange_uint4_int32_awq(dev(awq), None)
+    assert np.array_equal(got_ref.cpu().numpy(), want)
+    assert np.array_equal(got_awq.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("dtype,block,mul", [(torch.bfloat16, 16, False), (torch.float16, 64, True),
+                                            (torch.bfloat16, 128, True)])
+def test_fused_moe_quant_kernel_ex_w4a8(fmoe, rearrange, dtype, block, mul):
+    """fp8 activations x symmetric int4 experts with fp32 group scales, divided by the
+    reciprocal input scale: out[t] = (deq(A)[t / T] @ ((w - 8) s)[e]) / A_scale_rec."""
+    print(f"case w4a8 grouped {dtype} block={block} mul={mul}", flush=True)
+    rng = np.random.default_rng(29 + block)
+    M, E, T, K, N = 41, 4, 2, 256, 384
+    wl, s, awq, ref = make_w4a8_experts(rng, E, K, N)
+    a_scale = np.float32(0.037)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    xq = of8.to_e4m3fn(np.clip(x / a_scale, -448, 448))                    # codes
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    rec = torch.tensor([1.0 / a_scale], dtype=torch.float32, device="cuda")
+    sort, eids, npp = fmoe.moe_align_block_size(dev(ids), block, E)
+    a_deq = of8.from_e4m3fn(xq)
+    want = om.fused_moe_gemm(a_deq, lambda e: (wl[e].astype(np.float32) - 8.0) * np.repeat(s[e], 128, 0), ids, T,
+                             tw if mul else None, mul) * a_scale
+    for how in ("reference layout", "slab"):
+        B = dev(ref).view(E, N, K // 2) if how == "reference layout" else rearrange.rearrange_uint4_int32_awq(dev(awq), None)[0]
+        C = torch.full((M, T, N), float("nan"), dtype=dtype, device="cuda")
+        torch.ops._C.fused_moe_quant_kernel_ex(C, dev(xq).view(torch.float8_e4m3fn), B, rec, dev(s), None, None,
+                                               dev(tw), dev(ids), sort, eids, npp, None, mul, T, block, 128, -1)
+        torch.cuda.synchronize()
+        got = C.view(-1, N).float().cpu().numpy()
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL * max(1.0, np.abs(want).max()), err_msg=how)
+
+
 # ---------------------------------------------------- whole sequence ----
 def build_moe(mode):
     from vllm_gcu_amd.kernels.modular_experts import TritonExpertsPad

@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from oracle import fp8, moe, w8a8
+from oracle import fp8, moe, norm, w8a8
 
 
 # ---------------------------------------------------------------- int8 ----
@@ -251,3 +251,36 @@ def test_kslab_pack_is_inverted_by_scalar_walk_and_keeps_kib_runs(dtype):
     for lane in (0, 1, 15, 16, 37, 63):
         off = 32 * wb * (lane // 16)
         assert np.array_equal(kib[lane], rows[lane % 16, off:off + 16])
+
+
+def _f16(a):
+    return np.asarray(a, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def test_rms_norm_closed_forms_and_invariants():
+    rng = np.random.default_rng(41)
+    K = 256
+    w = _f16(rng.uniform(0.5, 1.5, K))
+    # constant row: z / rms(z) = sign -> out = sign * w (eps = 0)
+    for c in (3.0, -0.25):
+        out = norm.rms_norm(np.full((1, K), c, np.float32), w, 0.0, _f16)
+        assert np.array_equal(out[0], np.sign(c) * w)
+    # power-of-two scale invariance is exact without eps
+    x = _f16(rng.standard_normal((5, K)))
+    assert np.array_equal(norm.rms_norm(x, w, 0.0, _f16), norm.rms_norm(4.0 * x, w, 0.0, _f16))
+    # float64 evaluation within the rounding of two fp16 roundings
+    ref = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-5) * w
+    np.testing.assert_allclose(norm.rms_norm(x, w, 1e-5, _f16), ref, rtol=2e-3, atol=1e-4)
+    # a huge eps shrinks the output towards zero: rsqrt(var + eps) ~ eps^-1/2
+    big = norm.rms_norm(x, w, 1e6, _f16)
+    np.testing.assert_allclose(big, _f16(_f16(x * np.float32(1e-3)) * w), rtol=2e-3, atol=1e-6)
+
+
+def test_fused_add_rms_norm_is_add_then_norm():
+    rng = np.random.default_rng(43)
+    K = 128
+    x, r = _f16(rng.standard_normal((4, K))), _f16(rng.standard_normal((4, K)) * 3)
+    w = _f16(rng.uniform(0.5, 1.5, K))
+    out, z = norm.fused_add_rms_norm(x, r, w, 1e-6, _f16)
+    assert np.array_equal(z, _f16(x + r))
+    assert np.array_equal(out, norm.rms_norm(z, w, 1e-6, _f16))

@@ -131,6 +131,26 @@ def test_rearrange_awq_restatement():
     assert np.array_equal(got, ((q.astype(np.int8) - 8) & 15))
 
 
+def test_rearrange_awq_w4a8_branch_scalar_walk():
+    """use_w4a8 (rearrange.py:104-106): nibbles hold w - 8 in two's complement, zeros dropped;
+    with rearrange_group 64 the low nibble of byte row 32 G + i is k = 64 G + i, the high
+    nibble k = 64 G + 32 + i -- checked element by element."""
+    rng = np.random.default_rng(21)
+    K, N = 128, 16
+    wl = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    scales = rng.uniform(0.01, 0.02, size=(K // 64, N)).astype(np.float32)
+    rw, z = w4.rearrange_awq(w4.awq_pack(wl), None, scales, rearrange_group=64, zeros_in_int8=True, use_w4a8=True)
+    assert z is None and rw.dtype == np.int8 and rw.shape == (K // 2, N)
+    b = rw.view(np.uint8)
+    for k in range(K):
+        G, i = divmod(k, 64)
+        for n in range(N):
+            byte = int(b[32 * G + (i & 31), n])
+            nib = (byte >> 4) if i >= 32 else (byte & 15)
+            signed = nib - 16 if nib >= 8 else nib
+            assert signed == int(wl[k, n]) - 8
+
+
 def test_native_layout_inverse_and_spot_checks():
     rng = np.random.default_rng(7)
     K, N = 256, 256

@@ -280,3 +280,65 @@ def test_fp8_and_int8_moe_methods_grouped_routing():
                              lambda e: (w2i[e].astype(np.float32) * c2[e][:, None]).T, two, ido, bf16, quant_a2=qdq8)
     np.testing.assert_allclose(out8.float().cpu().numpy(), want8, rtol=2 * RTOL,
                                atol=ATOL * max(1.0, np.abs(want8).max()))
+
+    # the same experts under the compressed-tensors parameter names
+    from vllm_gcu_amd.kernels.quantization.w8a8 import GCUCompressedTensorsW8A8Int8MoEMethod
+    mc = GCUCompressedTensorsW8A8Int8MoEMethod()
+    layerc = torch.nn.Module()
+    mc.create_weights(layerc, E, H, I, torch.bfloat16)
+    layerc.cuda()
+    load(layerc, "w13_weight", dev(w13i)); load(layerc, "w2_weight", dev(w2i))
+    load(layerc, "w13_weight_scale", dev(c13[:, :, None])); load(layerc, "w2_weight_scale", dev(c2[:, :, None]))
+    mc.process_weights_after_loading(layerc)
+    outc = mc.apply(layerc, x.cuda().clone(), dev(logits), **route)
+    assert torch.equal(outc, out8)
+
+
+@pytest.mark.parametrize("rearranged", [False, True])
+def test_moe_w4a8_method(rearranged):
+    """W4A8Config -> MoeW4A8Method: create_weights / load / process / apply against the float
+    layer evaluated on the same quantised operands (fp8 activations with the static scales,
+    symmetric int4 experts with fp32 group scales)."""
+    from vllm_gcu_amd.kernels.quantization import QUANTIZATION_METHODS
+    print(f"case w4a8 moe method rearranged={rearranged}", flush=True)
+    M, E, T, H, I = 37, 8, 2, 256, 384
+    rng = np.random.default_rng(31)
+    cfg = QUANTIZATION_METHODS["w4a8_gcu"].from_config(
+        {"quant_method": "w4a8", "bits": 4, "group_size": 128, "zero_point": False, "rearranged": rearranged})
+    method = cfg.get_quant_method(moe=True)
+    w13 = rng.integers(0, 16, size=(E, H, 2 * I), dtype=np.uint8)
+    w2 = rng.integers(0, 16, size=(E, I, H), dtype=np.uint8)
+    s13 = rng.uniform(0.002, 0.01, size=(E, H // 128, 2 * I)).astype(np.float32)
+    s2 = rng.uniform(0.002, 0.01, size=(E, I // 128, H)).astype(np.float32)
+    a1, a2 = np.float32(0.02), np.float32(0.05)            # activation scales; the checkpoint holds 1 / scale
+
+    def ckpt(w, s):
+        if not rearranged:
+            return np.stack([ow4.awq_pack(w[e]) for e in range(E)])
+        return np.stack([ow4.rearrange_awq(ow4.awq_pack(w[e]), None, s[e], rearrange_group=64, zeros_in_int8=True,
+                                           use_w4a8=True)[0] for e in range(E)])
+
+    layer = torch.nn.Module()
+    method.create_weights(layer, E, H, I, torch.bfloat16)
+    layer.cuda()
+    load(layer, "w13_qweight", dev(ckpt(w13, s13))); load(layer, "w2_qweight", dev(ckpt(w2, s2)))
+    load(layer, "w13_scales", dev(s13)); load(layer, "w2_scales", dev(s2))
+    method.load_input_scale(layer.w13_input_scale, torch.tensor([1.0 / a1], device="cuda"))
+    method.load_input_scale(layer.w2_input_scale, torch.tensor([1.0 / a2], device="cuda"))
+    method.process_weights_after_loading(layer)
+    assert layer.w13_qweight.dtype == torch.int32 and tuple(layer.w13_qweight.shape) == (E, H // 8, 2 * I)
+    x = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).to(torch.bfloat16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    out = method.apply(layer, x.cuda(), dev(logits), top_k=T, renormalize=True)
+    assert out.dtype == torch.bfloat16 and out.shape == (M, H)
+
+    def fake_quant(v, sc):
+        return of8.from_e4m3fn(of8.to_e4m3fn(np.clip(v / sc, -448, 448).astype(np.float32))) * sc
+
+    bf16 = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).float().numpy()   # noqa: E731
+    two, ido, _ = om.topk_softmax(logits, T, True)
+    want = om.fused_experts(fake_quant(x.float().numpy(), a1),
+                            lambda e: (w13[e].astype(np.float32) - 8) * np.repeat(s13[e], 128, 0),
+                            lambda e: (w2[e].astype(np.float32) - 8) * np.repeat(s2[e], 128, 0),
+                            two, ido, bf16, quant_a2=lambda v: fake_quant(v, a2))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))

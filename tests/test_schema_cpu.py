@@ -4,8 +4,9 @@ reference's (tests/golden/op_schemas.txt), argument by argument.
 Allowed differences, each a widening the reference itself relies on (it passes
 Python ``None`` for these plain ``Tensor`` arguments and tests ``.defined()``,
 fused_moe.py:256-266, modular_experts.py:246): ``Tensor`` -> ``Tensor?`` for
-``azp``, ``e_score_correction_bias``, ``expert_map``, ``real_token_num`` and
-``B_scale`` (absent for unquantised experts).  ``(a!)`` and ``!`` both mean
+``azp``, ``e_score_correction_bias``, ``expert_map``, ``real_token_num``,
+``B_scale`` (absent for unquantised experts) and ``B_zero`` (fused_moe.py:182
+passes None).  ``(a!)`` and ``!`` both mean
 "written in place" and compare equal.
 """
 import os
@@ -16,7 +17,7 @@ import torch
 from vllm_gcu_amd.kernels import _custom_ops  # noqa: F401  (registers the ops)
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "op_schemas.txt")
-WIDENED = {"azp", "e_score_correction_bias", "expert_map", "real_token_num", "B_scale"}
+WIDENED = {"azp", "e_score_correction_bias", "expert_map", "real_token_num", "B_scale", "B_zero"}
 
 
 def golden_rows():

@@ -5,15 +5,15 @@ fails, an exception is raised.
 """
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_long, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi355q.so")
 
 F16, BF16, F32 = 0, 1, 2
 ZP_NONE, ZP_PACKED, ZP_PRESCALED = 0, 1, 2
-W4_SRC_GPTQ, W4_SRC_AWQ, W4_SRC_REF_KN, W4_SRC_REF_NK = 0, 1, 2, 3
-Q_W4A16, Q_FP8_BLOCK, Q_INT8, Q_NONE, Q_W8A16 = 0, 1, 2, 3, 4
+W4_SRC_GPTQ, W4_SRC_AWQ, W4_SRC_REF_KN, W4_SRC_REF_NK, W4_SRC_REF_KN_G64S = 0, 1, 2, 3, 4
+Q_W4A16, Q_FP8_BLOCK, Q_INT8, Q_NONE, Q_W8A16, Q_W4_F32SCALE = 0, 1, 2, 3, 4, 5
 
 # name -> (restype, argtypes); must list every symbol include/mi355q.h declares
 SIGNATURES = {
@@ -44,6 +44,9 @@ SIGNATURES = {
                                        c_void_p]),
     "mi355q_fp8_token_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_fp8_static_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_long, c_int,
+                                c_int, c_int, c_int, c_void_p]),
+    "mi355q_fp8_to_half": (c_int, [c_void_p, c_void_p, c_long, c_int, c_void_p]),
     "mi355q_moe_sum": (c_int, [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_moe_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,

@@ -189,6 +189,102 @@ moe_sum_kernel(void* out, const uint16_t* in, long rows, int T, int K, const int
   }
 }
 
+// ---- RMS norm (+ residual add) (+ quantisation of the normalised row) -------
+// One workgroup per row, two passes over it (the second one hits the L2):
+//   z = x (+ residual, rounded to the activation type and written back to residual)
+//   n = act(z * rsqrt(mean(z^2) + eps)),  o = act(n * weight)
+// then QM 0: o; 1: e4m3fn(clamp(o / scale)); 2: e4m3fn per group of gs with its own scale
+// absmax / 448; 3: int8 rne(o * act(1 / scale)) -- each exactly what the separate
+// quantisation operator makes of the stored o.
+template <int DT, bool ADD, int QM>
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* residual, const uint16_t* weight,
+                const float* scale, float eps, int K, int gs) {
+  const long row = blockIdx.x;
+  const int chunks = K / 8;
+  const uint16_t* xr = x + row * K;
+  uint16_t* rr = ADD ? residual + row * K : nullptr;
+  __shared__ float red[4];
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < chunks; c += 256) {
+    float v[8];
+    unpack8<DT>(*(const u4*)(xr + 8 * c), v);
+    if (ADD) {
+      float r[8];
+      unpack8<DT>(*(const u4*)(rr + 8 * c), r);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = round_act<DT>(v[e] + r[e]);
+      *(u4*)(rr + 8 * c) = pack8<DT>(v);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = (red[0] + red[1]) + (red[2] + red[3]);
+  const float rs = rsqrtf(ss / (float)K + eps);
+  float qs = 1.f;
+  if (QM == 1) qs = *scale;
+  if (QM == 3) qs = round_act<DT>(1.0f / *scale);
+  const int lpg = QM == 2 ? gs / 8 : 1;
+  const int padded = (chunks + 255) / 256 * 256;       // every lane stays in the loop for the group shuffles
+  for (int c0 = threadIdx.x; c0 < padded; c0 += 256) {
+    const bool live = c0 < chunks;
+    const int c = live ? c0 : 0;
+    float v[8], w[8];
+    // a thread re-reads only what it wrote itself in the first pass
+    unpack8<DT>(*(const u4*)((ADD ? (const uint16_t*)rr : xr) + 8 * c), v);
+    unpack8<DT>(*(const u4*)(weight + 8 * c), w);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = round_act<DT>(round_act<DT>(v[e] * rs) * w[e]);
+    if (QM == 0) {
+      if (live) *(u4*)((uint16_t*)out + row * K + 8 * c) = pack8<DT>(v);
+    } else if (QM == 1) {
+      float q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(v[e] / qs);
+      if (live) *(u2*)((uint8_t*)out + row * K + 8 * c) = to_fp8x8(q);
+    } else if (QM == 2) {
+      float mx = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
+      if (!live) mx = 0.f;
+      for (int o = 1; o < lpg; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      const float sg = fmaxf(mx, 1e-10f) / FP8_MAX;
+      float q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(v[e] / sg);
+      if (live) {
+        *(u2*)((uint8_t*)out + row * K + 8 * c) = to_fp8x8(q);
+        if ((c % lpg) == 0) out_scales[row * (K / gs) + c / lpg] = sg;
+      }
+    } else {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float a = fminf(fmaxf(__builtin_rintf(v[e] * qs), -128.f), 127.f);
+        float b = fminf(fmaxf(__builtin_rintf(v[4 + e] * qs), -128.f), 127.f);
+        lo |= ((uint32_t)(int)a & 0xffu) << (8 * e);
+        hi |= ((uint32_t)(int)b & 0xffu) << (8 * e);
+      }
+      if (live) *(u2*)((uint8_t*)out + row * K + 8 * c) = (u2){lo, hi};
+    }
+  }
+}
+
+template <int DT, bool ADD>
+void launch_rms(int qm, dim3 grid, hipStream_t st, void* out, float* out_scales, const uint16_t* x,
+                uint16_t* residual, const uint16_t* weight, const float* scale, float eps, int K, int gs) {
+  switch (qm) {
+    case 0: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 0>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+    case 1: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 1>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+    case 2: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 2>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+    default: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 3>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+  }
+}
+
 inline unsigned grid_for(long items) {
   long b = (items + 255) / 256;
   long cap = (long)device_cu_count() * 16;
@@ -310,5 +406,65 @@ extern "C" int mi355q_moe_sum(void* out, const void* in, long rows, int topk, in
   else
     hipLaunchKernelGGL((moe_sum_kernel<MI355Q_BF16, MI355Q_F32>), dim3(g), dim3(256), 0, st, out, p, rows, topk, K, valid_rows);
   MQ_LAUNCH_CHECK("moe_sum");
+  return 0;
+}
+
+// ---- fp8-e4m3fn -> f16 / bf16, exact (every e4m3fn value is representable in both) ----
+template <int DT>
+__global__ void __launch_bounds__(256)
+fp8_to_half_kernel(uint16_t* out, const uint32_t* in, long words) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < words; i += (long)gridDim.x * 256) {
+    const int w = (int)in[i];
+    const f2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+    uint2 o;
+    o.x = (uint32_t)Elem<DT>::from_f32(lo.x) | ((uint32_t)Elem<DT>::from_f32(lo.y) << 16);
+    o.y = (uint32_t)Elem<DT>::from_f32(hi.x) | ((uint32_t)Elem<DT>::from_f32(hi.y) << 16);
+    *(uint2*)(out + 4 * i) = o;
+  }
+}
+
+extern "C" int mi355q_fp8_to_half(void* out, const uint8_t* in, long n, int out_dtype, void* stream) {
+  MQ_REQUIRE(n >= 0 && n % 4 == 0, "fp8_to_half: element count %ld must be a multiple of 4", n);
+  if (n == 0) return 0;
+  MQ_REQUIRE(out && in, "fp8_to_half: null pointer");
+  MQ_REQUIRE(out_dtype == MI355Q_F16 || out_dtype == MI355Q_BF16, "fp8_to_half: output dtype %d must be f16 or bf16", out_dtype);
+  hipStream_t st = as_stream(stream);
+  const unsigned g = grid_for(n / 4);
+  if (out_dtype == MI355Q_F16)
+    hipLaunchKernelGGL((fp8_to_half_kernel<MI355Q_F16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint32_t*)in, n / 4);
+  else
+    hipLaunchKernelGGL((fp8_to_half_kernel<MI355Q_BF16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint32_t*)in, n / 4);
+  MQ_LAUNCH_CHECK("fp8_to_half");
+  return 0;
+}
+
+extern "C" int mi355q_rms_norm(void* out, float* out_scales, const void* x, void* residual, const void* weight,
+                               const float* scale, float eps, long rows, int K, int quant_mode, int group_size,
+                               int dtype, void* stream) {
+  MQ_REQUIRE(rows >= 0 && K > 0 && K % 8 == 0, "rms_norm: bad shape rows=%ld K=%d (K %% 8 == 0)", rows, K);
+  if (rows == 0) return 0;
+  MQ_REQUIRE(out && x && weight, "rms_norm: null pointer");
+  MQ_REQUIRE(rows <= 0x7fffffffL, "rms_norm: too many rows");
+  MQ_REQUIRE(quant_mode >= 0 && quant_mode <= 3, "rms_norm: quant_mode %d must be 0..3", quant_mode);
+  MQ_REQUIRE(dtype == MI355Q_F16 || dtype == MI355Q_BF16, "rms_norm: dtype %d must be f16 or bf16", dtype);
+  if (quant_mode == 1 || quant_mode == 3) MQ_REQUIRE(scale, "rms_norm: static scale missing");
+  if (quant_mode == 2) {
+    MQ_REQUIRE(out_scales, "rms_norm: group scales output missing");
+    MQ_REQUIRE((group_size == 64 || group_size == 128 || group_size == 256 || group_size == 512) && K % group_size == 0,
+               "rms_norm: group_size %d must be 64..512 (a power of two) and divide K=%d", group_size, K);
+  }
+  hipStream_t st = as_stream(stream);
+  const dim3 grid((unsigned)rows);
+  const uint16_t* xp = (const uint16_t*)x;
+  uint16_t* rp = (uint16_t*)residual;
+  const uint16_t* wp = (const uint16_t*)weight;
+  if (dtype == MI355Q_F16) {
+    if (residual) launch_rms<MI355Q_F16, true>(quant_mode, grid, st, out, out_scales, xp, rp, wp, scale, eps, K, group_size);
+    else launch_rms<MI355Q_F16, false>(quant_mode, grid, st, out, out_scales, xp, rp, wp, scale, eps, K, group_size);
+  } else {
+    if (residual) launch_rms<MI355Q_BF16, true>(quant_mode, grid, st, out, out_scales, xp, rp, wp, scale, eps, K, group_size);
+    else launch_rms<MI355Q_BF16, false>(quant_mode, grid, st, out, out_scales, xp, rp, wp, scale, eps, K, group_size);
+  }
+  MQ_LAUNCH_CHECK("rms_norm");
   return 0;
 }

@@ -26,7 +26,8 @@
 namespace mi355q {
 namespace {
 
-enum { KC_FP8_BLOCK = 0, KC_INT8 = 1, KC_F16 = 2, KC_BF16 = 3, KC_W8A16_F16 = 4, KC_W8A16_BF16 = 5 };
+enum { KC_FP8_BLOCK = 0, KC_INT8 = 1, KC_F16 = 2, KC_BF16 = 3, KC_W8A16_F16 = 4, KC_W8A16_BF16 = 5,
+       KC_W8A16G_F16 = 6, KC_W8A16G_BF16 = 7 };   // G: group-wise scales [E, K/g, N], g = 64 or 128
 
 struct KcArgs {
   void* out;                   // [rows_out, N] f16/bf16
@@ -37,6 +38,7 @@ struct KcArgs {
   const void* bias;            // [N] in out dtype, dense mode only
   int M, N, K;
   int kslab;                   // weights are in the kslab layout (N % 64 == 0)
+  int wgroup;                  // W8A16 group-wise modes: 64 or 128
   // grouped mode
   const int* sorted_ids;
   const int* expert_ids;
@@ -71,6 +73,8 @@ template <> struct Kc<KC_W8A16_BF16> {
   static constexpr int ABYTES = 2, WBYTES = 1;
   typedef f4 acc_t;
 };
+template <> struct Kc<KC_W8A16G_F16> : Kc<KC_W8A16_F16> {};
+template <> struct Kc<KC_W8A16G_BF16> : Kc<KC_W8A16_BF16> {};
 
 // 16 signed bytes -> 16 halves / bfloat16 (exact)
 __device__ __forceinline__ void s8x16_to_f16(const u4& v, u4& lo, u4& hi) {
@@ -106,6 +110,9 @@ kcontig_gemm_kernel(KcArgs a) {
   typedef Kc<MODE> T;
   typedef typename T::acc_t acc_t;
   constexpr int BM = 16 * MT;
+  constexpr bool W8H = MODE == KC_W8A16_F16 || MODE == KC_W8A16G_F16;     // int8 weights, f16 activations
+  constexpr bool W8B = MODE == KC_W8A16_BF16 || MODE == KC_W8A16G_BF16;   // ... bf16 activations
+  constexpr bool GW = MODE == KC_W8A16G_F16 || MODE == KC_W8A16G_BF16;    // group-wise weight scales
   constexpr int AV = T::ABYTES * 2;               // 16-byte vectors per lane per K block (activations)
   constexpr int WV = T::WBYTES * 2;               // ... weights
   __shared__ int tok[GROUPED ? BM : 1];
@@ -161,7 +168,10 @@ kcontig_gemm_kernel(KcArgs a) {
     u4 x[MT][AV];
     float as[MODE == KC_FP8_BLOCK ? MT : 1];
     float ws;
+    uint2 gs[GW ? 4 : 1][2];   // group-wise scales of this lane's 4 columns per row tile, per 64-wide half
   };
+  const uint16_t* ws16 = (const uint16_t*)a.w_scale + expert * a.ws_stride;
+  const int gper = GW ? 128 / a.wgroup : 1;        // scale groups per K block
   const float* wsf = (const float*)a.w_scale + expert * a.ws_stride;
   auto load_blk = [&](Blk& b, int kb) {
 #pragma unroll
@@ -177,6 +187,15 @@ kcontig_gemm_kernel(KcArgs a) {
 #pragma unroll
       for (int j = 0; j < MT; ++j) b.as[j] = a.a_scale[(size_t)arow[j] * KB + kb];
       b.ws = wsf[(size_t)(n0 >> 7) * KB + kb];
+    }
+    if (GW) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = min(n0 + 16 * i + 4 * q, N - 4);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          b.gs[i][h] = *(const uint2*)(ws16 + (size_t)(kb * gper + min(h, gper - 1)) * N + n);
+      }
     }
   };
 
@@ -217,7 +236,7 @@ kcontig_gemm_kernel(KcArgs a) {
         if (MODE == KC_F16 || MODE == KC_BF16) {
 #pragma unroll
           for (int v = 0; v < 4; ++v) wv[v] = b.w[i][v % WV];
-        } else if (MODE == KC_W8A16_F16) {
+        } else if (W8H) {
           s8x16_to_f16(b.w[i][0], wv[0], wv[1]);
           s8x16_to_f16(b.w[i][WV - 1], wv[2], wv[3]);
         } else {
@@ -225,16 +244,40 @@ kcontig_gemm_kernel(KcArgs a) {
           s8x16_to_bf16(b.w[i][WV - 1], wv[2], wv[3]);
         }
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
+        for (int j = 0; j < MT; ++j) {
+          auto mma = [&](const u4& wop, int v, f4 c) {
+            if (MODE == KC_F16 || W8H)
+              return __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<h8>(wop), bitcast<h8>(b.x[j][v % AV]), c, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(wop), bitcast<b8>(b.x[j][v % AV]), c, 0, 0, 0);
+          };
+          if (!GW) {
+            f4 sum = bitcast<f4>(acc[i][j]);
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            if (MODE == KC_F16 || MODE == KC_W8A16_F16)
-              acc[i][j] = bitcast<acc_t>(__builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  bitcast<h8>(wv[v]), bitcast<h8>(b.x[j][v % AV]), bitcast<f4>(acc[i][j]), 0, 0, 0));
-            else
-              acc[i][j] = bitcast<acc_t>(__builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  bitcast<b8>(wv[v]), bitcast<b8>(b.x[j][v % AV]), bitcast<f4>(acc[i][j]), 0, 0, 0));
+            for (int v = 0; v < 4; ++v) sum = mma(wv[v], v, sum);
+            acc[i][j] = bitcast<acc_t>(sum);
+          } else {
+            // A lane holds 32 consecutive k (32 q ..), so a 64-wide scale group is a pair of
+            // lane quarters, not a pair of steps: with two groups per K block each one is
+            // multiplied on its own with the other quarters' weights zeroed.
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              if (h >= gper) break;
+              const bool mine = gper == 1 || (q >> 1) == h;
+              f4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+              for (int v = 0; v < 4; ++v) sum = mma(mine ? wv[v] : (u4){0u, 0u, 0u, 0u}, v, sum);
+              const uint2 sv = b.gs[i][h];
+              f4 t = bitcast<f4>(acc[i][j]);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const uint32_t sw = e < 2 ? sv.x : sv.y;
+                const uint16_t raw = (uint16_t)((e & 1) ? (sw >> 16) : (sw & 0xffffu));
+                t[e] += sum[e] * (W8H ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw));
+              }
+              acc[i][j] = bitcast<acc_t>(t);
+            }
           }
+        }
       }
     }
     (void)kb;
@@ -286,9 +329,9 @@ kcontig_gemm_kernel(KcArgs a) {
         if (MODE == KC_INT8) {
           const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + n + e];
           v[e] = ((float)bitcast<i4>(acc[i][j])[e] * xs) * ws;
-        } else if (MODE == KC_W8A16_F16 || MODE == KC_W8A16_BF16) {
+        } else if ((W8H || W8B) && !GW) {
           const uint16_t raw = ((const uint16_t*)a.w_scale)[expert * a.ws_stride + n + e];
-          const float ws = (MODE == KC_W8A16_F16) ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw);
+          const float ws = W8H ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw);
           v[e] = bitcast<f4>(acc[i][j])[e] * ws;
         } else {
           v[e] = bitcast<f4>(acc[i][j])[e];
@@ -345,6 +388,8 @@ int launch_mode(const KcArgs& a, int mode, int odt, int mt, int row_blocks, hipS
   KC_CASE(KC_BF16, MI355Q_BF16)
   KC_CASE(KC_W8A16_F16, MI355Q_F16)
   KC_CASE(KC_W8A16_BF16, MI355Q_BF16)
+  KC_CASE(KC_W8A16G_F16, MI355Q_F16)
+  KC_CASE(KC_W8A16G_BF16, MI355Q_BF16)
 #undef KC_CASE
   set_error("kcontig_gemm: unsupported mode %d with output dtype %d", mode, odt);
   return 1;
@@ -355,6 +400,7 @@ int pick_mt(int rows) { return rows <= 16 ? 1 : (rows <= 32 ? 2 : 4); }
 }  // namespace
 
 int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                         const float* scales_f32, const float* out_scale,
                          const void* zeros, int zeros_kind, const float* topk_weights,
                          const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
@@ -383,9 +429,19 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
     MQ_REQUIRE(N % 128 == 0, "moe_gemm(w4a16): N=%d must be a multiple of 128", N);
     MQ_REQUIRE(w_scale, "moe_gemm(w4a16): scales missing");
     MQ_REQUIRE(out_dtype == act_dtype, "moe_gemm(w4a16): output dtype must equal the activation dtype");
-    return w4a16_grouped_launch(out, a, (const int32_t*)w, w_scale, w_zeros, zeros_kind, topk_weights,
-                                sorted_token_ids, expert_ids, num_tokens_post_pad, numel, topk, block_size,
-                                max_blocks, E, K, N, group_size <= 0 ? K : group_size, act_dtype, st);
+    return w4a16_grouped_launch(out, a, (const int32_t*)w, w_scale, nullptr, nullptr, w_zeros, zeros_kind,
+                                topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, numel, topk,
+                                block_size, max_blocks, E, K, N, group_size <= 0 ? K : group_size, act_dtype, st);
+  }
+  if (quant_mode == 5) {
+    MQ_REQUIRE(N % 128 == 0, "moe_gemm(w4, fp32 scales): N=%d must be a multiple of 128", N);
+    MQ_REQUIRE(w_scale, "moe_gemm(w4, fp32 scales): scales missing");
+    MQ_REQUIRE(out_dtype == act_dtype, "moe_gemm(w4, fp32 scales): output dtype must equal the activation dtype");
+    MQ_REQUIRE(!w_zeros && zeros_kind == MI355Q_ZP_NONE, "moe_gemm(w4, fp32 scales): symmetric weights only");
+    return w4a16_grouped_launch(out, a, (const int32_t*)w, nullptr, (const float*)w_scale, a_scale, nullptr,
+                                MI355Q_ZP_NONE, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad,
+                                numel, topk, block_size, max_blocks, E, K, N, group_size <= 0 ? K : group_size,
+                                act_dtype, st);
   }
   MQ_REQUIRE(N % 4 == 0, "moe_gemm: N=%d must be a multiple of 4", N);
   MQ_REQUIRE(w_layout == 0 || (w_layout == 1 && N % 64 == 0), "moe_gemm: weight layout %d needs N=%d %% 64 == 0", w_layout, N);
@@ -409,9 +465,15 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
     mode = act_dtype == MI355Q_F16 ? KC_F16 : KC_BF16;
   } else if (quant_mode == 4) {
     MQ_REQUIRE(w_scale, "moe_gemm(w8a16): weight scales missing");
-    MQ_REQUIRE(group_size <= 0 || group_size == K, "moe_gemm(w8a16): only per-channel scales are supported");
-    mode = act_dtype == MI355Q_F16 ? KC_W8A16_F16 : KC_W8A16_BF16;
-    g.ws_stride = N;
+    if (group_size <= 0 || group_size == K) {
+      mode = act_dtype == MI355Q_F16 ? KC_W8A16_F16 : KC_W8A16_BF16;
+      g.ws_stride = N;
+    } else {
+      MQ_REQUIRE(group_size == 64 || group_size == 128, "moe_gemm(w8a16): group size %d must be 64, 128 or per channel", group_size);
+      mode = act_dtype == MI355Q_F16 ? KC_W8A16G_F16 : KC_W8A16G_BF16;
+      g.wgroup = group_size;
+      g.ws_stride = (long)(K / group_size) * N;
+    }
   } else {
     MQ_REQUIRE(false, "moe_gemm: unknown quant_mode %d", quant_mode);
   }
@@ -450,8 +512,13 @@ extern "C" int mi355q_kcontig_gemm(void* out, const void* a, const void* w, cons
     mode = act_dtype == MI355Q_F16 ? KC_F16 : KC_BF16;
   } else if (quant_mode == 4) {
     MQ_REQUIRE(w_scale, "kcontig_gemm(w8a16): weight scales missing");
-    MQ_REQUIRE(group_size <= 0 || group_size == K, "kcontig_gemm(w8a16): only per-channel scales are supported");
-    mode = act_dtype == MI355Q_F16 ? KC_W8A16_F16 : KC_W8A16_BF16;
+    if (group_size <= 0 || group_size == K) {
+      mode = act_dtype == MI355Q_F16 ? KC_W8A16_F16 : KC_W8A16_BF16;
+    } else {
+      MQ_REQUIRE(group_size == 64 || group_size == 128, "kcontig_gemm(w8a16): group size %d must be 64, 128 or per channel", group_size);
+      mode = act_dtype == MI355Q_F16 ? KC_W8A16G_F16 : KC_W8A16G_BF16;
+      g.wgroup = group_size;
+    }
   } else {
     MQ_REQUIRE(false, "kcontig_gemm: unknown quant_mode %d", quant_mode);
   }

@@ -45,6 +45,18 @@ w4_repack_kernel(const void* __restrict__ src, int fmt, uint32_t* __restrict__ d
       uint32_t v = q[(long)(k0 + j) * (N >> 3) + (n >> 3)];
       out |= ((v >> sh) & 15u) << (4 * nib_of_j(j));
     }
+  } else if (fmt == MI355Q_W4_SRC_REF_KN_G64S) {
+    // half-groups of 32 rows, signed nibbles (w - 8 in two's complement): group-of-64-local
+    // row i < 32 in the low nibble, i >= 32 in the high nibble of byte row 32 G64 + (i & 31)
+    const uint8_t* q = (const uint8_t*)src + b * ((long)(K >> 1) * N);
+    const int k = k0 & 63, hi = k >= 32;
+    const long row0 = 32 * (long)(k0 >> 6) + (k & 31);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint8_t v = q[(row0 + j) * N + n];
+      const uint32_t nib = ((hi ? (v >> 4) : (v & 15u)) ^ 8u) & 15u;
+      out |= nib << (4 * nib_of_j(j));
+    }
   } else {
     // reference half-group bytes: group-local row i < 64 in the low nibble,
     // i >= 64 in the high nibble of byte row 64g + (i & 63)
@@ -114,7 +126,7 @@ using namespace mi355q;
 extern "C" int mi355q_w4_repack(const void* src, int src_format, int32_t* dst, int batch, int K,
                                 int N, void* stream) {
   MQ_REQUIRE(src && dst, "w4_repack: null pointer");
-  MQ_REQUIRE(src_format >= MI355Q_W4_SRC_GPTQ && src_format <= MI355Q_W4_SRC_REF_NK,
+  MQ_REQUIRE(src_format >= MI355Q_W4_SRC_GPTQ && src_format <= MI355Q_W4_SRC_REF_KN_G64S,
              "w4_repack: unknown source format %d", src_format);
   MQ_REQUIRE(batch >= 0 && K > 0 && N > 0 && K % 128 == 0 && N % 128 == 0,
              "w4_repack: K=%d and N=%d must be positive multiples of 128", K, N);

@@ -27,7 +27,9 @@ struct TileArgs {
   uint16_t* out;
   const uint16_t* x;
   const u4* qw;
-  const uint16_t* scales;
+  const uint16_t* scales;       // group scales in the activation type, or
+  const float* scales_f32;      // ... in fp32 (SF32 kernels; the other pointer is unused)
+  const float* out_scale;       // optional device scalar multiplied into every output
   const void* zeros;
   const uint16_t* bias;
   int M, K, N, gs;
@@ -92,7 +94,7 @@ template <> struct TileMma<MI355Q_BF16> {
 // columns.  WM = 2: eight wavefronts, the upper four take the upper half of
 // the rows (both halves dequantise the same weights, but two wavefronts per
 // SIMD keep the matrix pipe fed while one of them waits or dequantises).
-template <int DT, int ZK, int MT, bool GROUPED, int WM>
+template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false>
 __global__ void __launch_bounds__(256 * WM, 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
@@ -112,12 +114,14 @@ w4a16_tile_kernel(TileArgs a) {
   const int m0 = blockIdx.y * BM;
   const u4* qw = a.qw;
   const uint16_t* scales = a.scales;
+  const float* scales32 = a.scales_f32;
   const char* zeros = (const char*)a.zeros;
   if (GROUPED) {
     if (m0 >= *a.npp) return;                       // block beyond the padded ids
     const long e = a.expert_ids[blockIdx.y];
     qw += e * a.w_stride;
-    scales += e * a.s_stride;
+    if (SF32) scales32 += e * a.s_stride;
+    else scales += e * a.s_stride;
     if (zeros) zeros += e * a.z_stride * (ZK == MI355Q_ZP_PACKED ? 4 : 2);
     for (int r = tid; r < BM; r += NTHR) tok[r] = a.sorted_ids[m0 + r];
     __syncthreads();
@@ -160,6 +164,7 @@ w4a16_tile_kernel(TileArgs a) {
 
   const u4* wbase = qw + ((size_t)slab * G * 8 + t0) * 64 + lane;
   uint2 sreg;
+  f4 sreg32;
   uint32_t zreg = 0x88888888u;
   uint2 zsreg = {0u, 0u};
   auto load_w = [&](u4 (&w)[4], int g) {
@@ -169,7 +174,8 @@ w4a16_tile_kernel(TileArgs a) {
   };
   auto load_sz = [&](int g) {
     const int qrow = (128 * g) / a.gs;
-    sreg = *(const uint2*)(scales + (size_t)qrow * N + ncol);
+    if (SF32) sreg32 = *(const f4*)(scales32 + (size_t)qrow * N + ncol);
+    else sreg = *(const uint2*)(scales + (size_t)qrow * N + ncol);
     if (ZK == MI355Q_ZP_PACKED) zreg = ((const uint32_t*)zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)] >> (4 * t0);
     if (ZK == MI355Q_ZP_PRESCALED) zsreg = *(const uint2*)((const uint16_t*)zeros + (size_t)qrow * N + ncol);
   };
@@ -177,7 +183,7 @@ w4a16_tile_kernel(TileArgs a) {
   const int gb = GROUPED ? 0 : (int)blockIdx.z * a.kper, ge = GROUPED ? G : min(G, gb + a.kper);
   // The pipelined loop needs nearly the whole register file; it is used where it fits
   // (fp16, 128-row tiles), the plain loop elsewhere.
-  constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED;
+  constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED && !SF32;
   if constexpr (PIPE) {
     // Software pipeline, written out because the compiler otherwise sinks every
     // load next to its use.  Activations: global loads at the top of the K block
@@ -309,7 +315,7 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const uint32_t sw = (t < 2) ? sreg.x : sreg.y;
-        sc[t] = Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+        sc[t] = SF32 ? sreg32[t] : Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
         float zf;
         if (ZK == MI355Q_ZP_PRESCALED) {
           const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
@@ -358,6 +364,7 @@ w4a16_tile_kernel(TileArgs a) {
 
   // ---- epilogue: 4 adjacent columns per (row tile, i) ----
   if (!live) return;
+  const float oscale = a.out_scale ? *a.out_scale : 1.0f;
   float bs[4] = {0.f, 0.f, 0.f, 0.f};
   if (a.bias) {
 #pragma unroll
@@ -368,12 +375,12 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int m;
-      float rw = 1.0f;
+      float rw = oscale;
       bool ok;
       if (GROUPED) {
         m = tok[(wmh * MTW + mt) * 16 + 4 * kq + i];
         ok = m < a.numel;
-        if (ok && a.topk_weights) rw = a.topk_weights[m];
+        if (ok && a.topk_weights) rw *= a.topk_weights[m];
       } else {
         m = m0 + (wmh * MTW + mt) * 16 + 4 * kq + i;
         ok = m < M;
@@ -413,7 +420,7 @@ w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* 
   *(uint2*)(out + i) = o;
 }
 
-template <int DT, int ZK, int MT, bool GROUPED>
+template <int DT, int ZK, int MT, bool GROUPED, bool SF32 = false>
 hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
   {
     constexpr int BM = 16 * MT;
@@ -421,16 +428,20 @@ hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
     const int G = a.K >> 7;
     dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
     const size_t shmem = 2 * BM * A_ROW;           // up to 72 KiB: above the 64 KiB default
-    static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>,
+    static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM>), grid, block, shmem, st, a);
+    hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>), grid, block, shmem, st, a);
     return hipSuccess;
   }
 }
 
 template <int DT, int MT, bool GROUPED>
 hipError_t launch_zk(const TileArgs& a, int zk, int row_blocks, hipStream_t st) {
+  if constexpr (GROUPED) {
+    // fp32 group scales: symmetric int4 experts only
+    if (a.scales_f32) return launch_one<DT, MI355Q_ZP_NONE, MT, true, true>(a, row_blocks, st);
+  }
   if (zk == MI355Q_ZP_NONE) return launch_one<DT, MI355Q_ZP_NONE, MT, GROUPED>(a, row_blocks, st);
   if (zk == MI355Q_ZP_PACKED) return launch_one<DT, MI355Q_ZP_PACKED, MT, GROUPED>(a, row_blocks, st);
   return launch_one<DT, MI355Q_ZP_PRESCALED, MT, GROUPED>(a, row_blocks, st);
@@ -514,6 +525,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
 }
 
 int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                         const float* scales_f32, const float* out_scale,
                          const void* zeros, int zeros_kind, const float* topk_weights,
                          const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
@@ -528,6 +540,10 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   a.x = (const uint16_t*)x;
   a.qw = (const u4*)qweight;
   a.scales = (const uint16_t*)scales;
+  a.scales_f32 = scales_f32;
+  a.out_scale = out_scale;
+  MQ_REQUIRE(!scales_f32 || (zeros_kind == MI355Q_ZP_NONE && !zeros),
+             "moe_w4a16: fp32 group scales go with symmetric weights only");
   a.zeros = zeros;
   a.M = numel; a.K = K; a.N = N; a.gs = group_size;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;

@@ -670,6 +670,101 @@ _register("_moe_C", "moe_sum_pad", "(Tensor(a!) out, Tensor input, Tensor size, 
           _moe_sum_pad_impl)
 
 
+# ---------------------------------------------------------------------------
+# RMS norm and its fusions with the activation quantisers
+# (csrc/torch_bindings.cpp:254-317, 852-871, 1124-1143; the fused operators are
+# what vllm_gcu/compilation/fusion.py:104-127 substitutes for norm -> quantiser)
+# ---------------------------------------------------------------------------
+def _rms_common(out, out_scales, input, residual, weight, scale, epsilon, quant_mode, group_size=0):
+    rt.require_gpu(out, out_scales, input, residual, weight, scale)
+    if input.numel() == 0:
+        return
+    if input.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"rms_norm: input must be f16/bf16, got {input.dtype}")
+    if not input.is_contiguous() or not out.is_contiguous():
+        raise RuntimeError("rms_norm: input and output must be contiguous")
+    rows, K = _rows_last(input)
+    if weight.numel() != K:
+        raise RuntimeError(f"rms_norm: weight has {weight.numel()} elements for rows of {K}")
+    if tuple(out.shape) != tuple(input.shape):
+        raise RuntimeError(f"rms_norm: output shape {tuple(out.shape)} != input shape {tuple(input.shape)}")
+    want = {0: input.dtype, 1: torch.float8_e4m3fn, 2: torch.float8_e4m3fn, 3: torch.int8}[quant_mode]
+    if out.dtype != want:
+        raise RuntimeError(f"rms_norm: output must be {want}, got {out.dtype}")
+    if residual is not None and (residual.dtype != input.dtype or tuple(residual.shape) != tuple(input.shape)
+                                 or not residual.is_contiguous()):
+        raise RuntimeError("rms_norm: residual must match the input (dtype, shape, contiguous)")
+    w = weight.to(input.dtype).contiguous()
+    sc = None
+    if quant_mode in (1, 3):
+        sc = scale.to(torch.float32).reshape(-1)
+        if sc.numel() != 1:
+            raise RuntimeError("rms_norm + static quant takes a single scale")
+    if quant_mode == 2:
+        if out_scales.dtype != torch.float32 or not out_scales.is_contiguous() or \
+                out_scales.numel() != rows * (K // group_size):
+            raise RuntimeError("rms_norm + group quant: scales must be contiguous f32 [.., K / group_size]")
+    with torch.cuda.device(input.device):
+        _lib.call("mi355q_rms_norm", out.data_ptr(), rt.ptr(out_scales), input.data_ptr(), rt.ptr(residual),
+                  w.data_ptr(), rt.ptr(sc), float(epsilon), rows, K, quant_mode, int(group_size),
+                  rt.dtype_code(input.dtype), rt.stream_ptr())
+
+
+def _rms_norm_impl(result, input, weight, epsilon):
+    _rms_common(result, None, input, None, weight, None, epsilon, 0)
+
+
+def _fused_add_rms_norm_impl(input, residual, weight, epsilon):
+    _rms_common(input, None, input, residual, weight, None, epsilon, 0)
+
+
+def _rms_norm_static_fp8_quant_impl(result, input, weight, scale, epsilon):
+    _rms_common(result, None, input, None, weight, scale, epsilon, 1)
+
+
+def _fused_add_rms_norm_static_fp8_quant_impl(result, input, residual, weight, scale, epsilon):
+    _rms_common(result, None, input, residual, weight, scale, epsilon, 1)
+
+
+def _rms_norm_per_token_group_quant_fp8_impl(out, scale, input, weight, epsilon, group_size):
+    _rms_common(out, scale, input, None, weight, None, epsilon, 2, group_size)
+
+
+def _fused_add_rms_norm_per_token_group_quant_fp8_impl(out, residual, scale, input, weight, epsilon, group_size):
+    _rms_common(out, scale, input, residual, weight, None, epsilon, 2, group_size)
+
+
+def _rms_norm_static_int8_quant_impl(result, input, weight, scale, epsilon):
+    _rms_common(result, None, input, None, weight, scale, epsilon, 3)
+
+
+def _fused_add_rms_norm_static_int8_quant_impl(result, input, residual, weight, epsilon, scale):
+    _rms_common(result, None, input, residual, weight, scale, epsilon, 3)
+
+
+_register("_C", "rms_norm", "(Tensor! result, Tensor input, Tensor weight, float epsilon) -> ()", _rms_norm_impl)
+_register("_C", "fused_add_rms_norm", "(Tensor! input, Tensor! residual, Tensor weight, float epsilon) -> ()",
+          _fused_add_rms_norm_impl)
+_register("_C", "rms_norm_static_fp8_quant",
+          "(Tensor! result, Tensor input, Tensor weight, Tensor scale, float epsilon) -> ()",
+          _rms_norm_static_fp8_quant_impl)
+_register("_C", "fused_add_rms_norm_static_fp8_quant",
+          "(Tensor! result, Tensor input, Tensor! residual, Tensor weight, Tensor scale, float epsilon) -> ()",
+          _fused_add_rms_norm_static_fp8_quant_impl)
+_register("_C", "rms_norm_per_token_group_quant_fp8",
+          "(Tensor! out, Tensor! scale, Tensor input, Tensor weight, float epsilon, int group_size) -> ()",
+          _rms_norm_per_token_group_quant_fp8_impl)
+_register("_C", "fused_add_rms_norm_per_token_group_quant_fp8",
+          "(Tensor! out, Tensor! residual, Tensor! scale, Tensor input, Tensor weight, float epsilon, "
+          "int group_size) -> ()", _fused_add_rms_norm_per_token_group_quant_fp8_impl)
+_register("_C", "rms_norm_static_int8_quant",
+          "(Tensor(a!) result, Tensor input, Tensor weight, Tensor scale, float epsilon) -> ()",
+          _rms_norm_static_int8_quant_impl)
+_register("_C", "fused_add_rms_norm_static_int8_quant",
+          "(Tensor(a!) result, Tensor input, Tensor(a!) residual, Tensor weight, float epsilon, Tensor scale) -> ()",
+          _fused_add_rms_norm_static_int8_quant_impl)
+
+
 # 8bit (vllm_gcu/kernels/_custom_ops.py:298-317)
 def scaled_fp8_quant(input: torch.Tensor, scale: Optional[torch.Tensor] = None,
                      num_token_padding: Optional[int] = None, scale_ub: Optional[torch.Tensor] = None,
@@ -780,7 +875,13 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
     elif B.dtype == torch.int8:
         mode = _lib.Q_W8A16
         w = B.contiguous()
-        w_scale = B_scale.reshape(B.shape[0], -1).to(A.dtype).contiguous()
+        if group in (64, 128) and B_scale.dim() == 3 and B_scale.shape[1] == K // group:
+            w_scale = B_scale.to(A.dtype).contiguous()                    # [E, K/g, N]
+        else:
+            w_scale = B_scale.reshape(B.shape[0], -1).to(A.dtype).contiguous()
+            if w_scale.shape[1] != N:
+                raise RuntimeError(f"w8a16 experts: scales {tuple(B_scale.shape)} fit neither [E, N] nor [E, K/g, N]")
+            group = -1
         act_code = rt.dtype_code(A.dtype)
     elif B.dtype == A.dtype and B_scale is None:
         mode = _lib.Q_NONE
@@ -814,6 +915,71 @@ def _fused_moe_quant_kernel_impl(C, A, B, A_scale, B_scale, gs, B_zp, topk_weigh
                                  real_token_num):
     _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids, experts_ids,
               num_tokens_post_pad, mul_routed_weight, topk, block_size, bias, real_token_num)
+
+
+def _fused_moe_quant_kernel_ex_impl(C, A, B, A_scale, B_scale, B_zero, bias, topk_weights, topk_ids,
+                                    sorted_token_ids, experts_ids, num_tokens_post_pad, real_token_num,
+                                    mul_routed_weight, topk, block_size, group_k, group_n):
+    """w4a8-fp8 experts (fused_moe_quant_kernel_ex.cpp:13-45, called from
+    fused_moe.py:173-195): fp8 activations with one static scale, symmetric int4
+    weights with fp32 group scales ``[E, K/group_k, N]``.
+
+    ``A_scale`` is what the reference passes there: the *reciprocal* of the
+    scale the activations were quantised with (``layer.w13_input_scale_rec``,
+    w4a8.py:222-235).  The vendor kernel's arithmetic is not part of the
+    reference; with ``static_scaled_fp8_quant`` dividing by its scale, the only
+    reading under which quantise -> GEMM reproduces the float layer is
+    ``C = (A @ dequant(B)) / A_scale``, which is what runs here.  fp8 values
+    are widened exactly to C's dtype and multiplied on the fp16/bf16 matrix
+    pipe with fp32 accumulation."""
+    rt.require_gpu(C, A, B, A_scale, B_scale, topk_weights, topk_ids, sorted_token_ids, experts_ids,
+                   num_tokens_post_pad)
+    if bias is not None:
+        raise RuntimeError("fused_moe_quant_kernel_ex takes no bias")
+    if B_zero is not None and B_zero.numel():
+        raise RuntimeError("fused_moe_quant_kernel_ex: w4a8 experts are symmetric (w4a8.py:143 passes no zeros)")
+    if group_n not in (-1, 1):
+        raise RuntimeError(f"fused_moe_quant_kernel_ex: group_n={group_n}: scales are per output channel")
+    numel = topk_ids.numel()
+    if numel == 0 or A.numel() == 0:
+        return
+    if A.dtype != torch.float8_e4m3fn:
+        raise RuntimeError(f"fused_moe_quant_kernel_ex: activations must be float8_e4m3fn, got {A.dtype}")
+    if not C.is_contiguous() or C.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("fused_moe_quant_kernel_ex: C must be contiguous f16/bf16")
+    A = A.contiguous()
+    K, N = A.shape[-1], C.shape[-1]
+    if B.dtype == torch.int32:
+        w = B                                           # slab tensor from this build's loader
+    elif B.dtype in (torch.int8, torch.uint8) and B.shape[-1] * 2 == K:
+        w = _converted(B, rearrange.from_reference_w4a8)
+    else:
+        raise RuntimeError(f"fused_moe_quant_kernel_ex: int4 experts expected, got {B.dtype} {tuple(B.shape)}")
+    if w.shape[-2] * 8 != K or w.shape[-1] != N:
+        raise RuntimeError(f"fused_moe_quant_kernel_ex: weights {tuple(w.shape)} do not match K={K}, N={N}")
+    E = w.shape[0]
+    w_scale = B_scale.to(torch.float32).contiguous()
+    if tuple(w_scale.shape) != (E, K // group_k, N):
+        raise RuntimeError(f"fused_moe_quant_kernel_ex: scales {tuple(w_scale.shape)} != {(E, K // group_k, N)}")
+    out_scale = _converted(A_scale, lambda t: (1.0 / t.detach().to(torch.float32)).reshape(-1)[:1].contiguous())
+    a16 = torch.empty(A.shape, dtype=C.dtype, device=A.device)
+    tw = None
+    if mul_routed_weight:
+        tw = topk_weights.to(torch.float32).contiguous()
+        if tw.numel() != numel:
+            raise RuntimeError("fused_moe: topk_weights must have one entry per (token, slot)")
+    for t in (sorted_token_ids, experts_ids, num_tokens_post_pad):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("fused_moe: sorted_token_ids / experts_ids / num_tokens_post_pad must be contiguous int32")
+    if sorted_token_ids.numel() < experts_ids.numel() * block_size:
+        raise RuntimeError("fused_moe: sorted_token_ids is shorter than experts_ids * block_size")
+    code = rt.dtype_code(C.dtype)
+    with torch.cuda.device(A.device):
+        _lib.call("mi355q_fp8_to_half", a16.data_ptr(), A.data_ptr(), A.numel(), code, rt.stream_ptr())
+        _lib.call("mi355q_moe_gemm", C.data_ptr(), a16.data_ptr(), w.data_ptr(), out_scale.data_ptr(),
+                  w_scale.data_ptr(), 0, _lib.ZP_NONE, _lib.Q_W4_F32SCALE, int(group_k), rt.ptr(tw),
+                  sorted_token_ids.data_ptr(), experts_ids.data_ptr(), num_tokens_post_pad.data_ptr(), numel,
+                  int(topk), int(block_size), experts_ids.numel(), E, K, N, code, code, 0, rt.stream_ptr())
 
 
 def _fused_moe_kernel_impl(C, A, B, topk_weights, topk_ids, sorted_topk_ids, expert_ids, num_tokens_post_pad,
@@ -853,14 +1019,22 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
 
 
 def _weight_only_quant_impl(output, input, qweight, bias, scale, group_size):
-    """W8A16 (weight_only_quant.cpp:28-101): qweight int8 [N, K], per-channel scale [N]."""
+    """W8A16 (weight_only_quant.cpp:28-101): qweight int8 [N, K]; scale [N] per
+    channel (group_size -1) or [K/g, N] for groups of 64 / 128 along K, the
+    shapes GPTQGCULinearMethod leaves behind for 8-bit checkpoints (gptq.py:262-270)."""
     if input.numel() == 0:
         return
     if qweight.dtype != torch.int8:
         raise RuntimeError("weight_only_quant: qweight must be int8 [N, K]")
-    if scale.numel() != qweight.shape[0]:
-        raise RuntimeError("weight_only_quant: only per-channel scales are supported")
-    _kcontig(output, input, qweight, None, scale.reshape(-1).to(input.dtype).contiguous(), bias, _lib.Q_W8A16, -1)
+    N, K = qweight.shape
+    if scale.numel() == N:
+        _kcontig(output, input, qweight, None, scale.reshape(-1).to(input.dtype).contiguous(), bias, _lib.Q_W8A16, -1)
+        return
+    g = int(group_size)
+    if g not in (64, 128) or tuple(scale.shape) != (K // g, N):
+        raise RuntimeError(f"weight_only_quant: scales {tuple(scale.shape)} with group_size {group_size}: expected "
+                           f"[N] or [K/g, N] with g = 64 or 128")
+    _kcontig(output, input, qweight, None, scale.to(input.dtype).contiguous(), bias, _lib.Q_W8A16, g)
 
 
 # the three operators below are registered from C++ function pointers in the
@@ -870,6 +1044,11 @@ _register("_C", "fused_moe_quant_kernel",
           "Tensor topk_weights, Tensor topk_ids, Tensor sorted_token_ids, Tensor experts_ids, "
           "Tensor num_tokens_post_pad, bool mul_routed_weight, int topk, int block_size, Tensor? bias, "
           "Tensor? real_token_num) -> ()", _fused_moe_quant_kernel_impl)
+_register("_C", "fused_moe_quant_kernel_ex",
+          "(Tensor(a!) C, Tensor A, Tensor B, Tensor A_scale, Tensor B_scale, Tensor? B_zero, Tensor? bias, "
+          "Tensor topk_weights, Tensor topk_ids, Tensor sorted_token_ids, Tensor experts_ids, "
+          "Tensor num_tokens_post_pad, Tensor? real_token_num, bool mul_routed_weight, int topk, "
+          "int block_size, int group_k, int group_n) -> ()", _fused_moe_quant_kernel_ex_impl)
 _register("_C", "fused_moe_kernel",
           "(Tensor(a!) C, Tensor A, Tensor B, Tensor topk_weights, Tensor topk_ids, Tensor sorted_topk_ids, "
           "Tensor expert_ids, Tensor num_tokens_post_pad, bool mul_routed_weight, int topk, int block_size, "

@@ -114,11 +114,11 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A
         assert B_scale is None
     block_size = config["BLOCK_SIZE_M"]
     if use_fp8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or use_int8_w8a8:
+        w4a8 = use_fp8_w8a8 and B.dtype in (torch.int8, torch.int32)   # int4 experts, fp8 activations
         if use_fp8_w8a8:
             B_zp = None
-            if B.dtype == torch.int8:
-                raise NotImplementedError("w4a8-fp8 experts (fused_moe_quant_kernel_ex) are not built")
-            group_size = block_shape[1]
+            if not w4a8:
+                group_size = block_shape[1]
         elif use_int8_w8a8:
             B_zp = None
             group_size = 1
@@ -131,10 +131,20 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, A
             A_scale = None
             group_size = -1
             if B_scale.dim() == 3 and B_scale.shape[1] > 1:
-                raise NotImplementedError("group-wise w8a16 experts are not built (per-channel only)")
-        torch.ops._C.fused_moe_quant_kernel(C, A, B, A_scale, B_scale, group_size, B_zp, topk_weights, topk_ids,
-                                            sorted_token_ids, expert_ids, num_tokens_post_padded,
-                                            mul_routed_weight, top_k, block_size, None, real_token_num)
+                group_size = B.shape[2] // B_scale.shape[1]
+                assert group_size in [64, 128], \
+                    f"Unsupported shape, B: {B.shape}, B_scale: {B_scale.shape} for w8a16(int8)."
+        if w4a8:
+            # fused_moe.py:173-195: the reciprocal input scale goes where the kernel expects A_scale
+            assert A_scale_rec is not None
+            torch.ops._C.fused_moe_quant_kernel_ex(C, A, B, A_scale_rec, B_scale, B_zp, None, topk_weights,
+                                                   topk_ids, sorted_token_ids, expert_ids,
+                                                   num_tokens_post_padded, real_token_num, mul_routed_weight,
+                                                   top_k, block_size, 128, -1)
+        else:
+            torch.ops._C.fused_moe_quant_kernel(C, A, B, A_scale, B_scale, group_size, B_zp, topk_weights,
+                                                topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                                mul_routed_weight, top_k, block_size, None, real_token_num)
     else:
         topk_weights = topk_weights.to(torch.float32)
         torch.ops._C.fused_moe_kernel(C, A, B, topk_weights, topk_ids, sorted_token_ids, expert_ids,

@@ -33,8 +33,8 @@ def moe_problem_size(a1: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_
     """(E, M, N, K, topk) with N = 2 * intermediate; handles the int4 layouts."""
     E = w1.shape[0]
     M, K = a1.shape
-    if int4 and w1.dtype == torch.int32:
-        N = w1.shape[2]                      # slab tensor [E, K/8, N]
+    if w1.dtype == torch.int32:
+        N = w1.shape[2]                      # slab tensor [E, K/8, N] (w4a16 and w4a8 experts)
     else:
         N = w1.shape[1]                      # [E, N, K] (or reference int4 [E, N, K/2])
     return E, M, N, K, topk_ids.shape[1]
@@ -100,11 +100,17 @@ class TritonExpertsPad:
                                 use_fp8_w8a8=self.use_fp8_w8a8, use_int8_w8a8=self.use_int8_w8a8,
                                 use_int8_w8a16=self.use_int8_w8a16, use_int4_w4a16=self.use_int4_w4a16,
                                 per_channel_quant=self.per_act_token_quant, block_shape=self.block_shape,
-                                real_token_num=expert_num_tokens if static_shape else None)
+                                real_token_num=expert_num_tokens if static_shape else None,
+                                A_scale_rec=a1q_scale_rec)
 
         if activation != "silu":
             raise ValueError(f"Unsupported FusedMoe activation: {activation}")
-        if self.use_fp8_w8a8:
+        if self.use_fp8_w8a8 and w1.dtype in (torch.int8, torch.int32):
+            # w4a8 experts: one static scale for the second GEMM's activations (modular_experts.py:197-211)
+            assert a2_scale is not None
+            torch.ops._C.silu_mul_static_fp8_quant(cache2.view(-1, top_k_num, N // 2), cache1, a2_scale,
+                                                   expert_num_tokens)
+        elif self.use_fp8_w8a8:
             group_size = self.block_shape[1]
             a2_scale = torch.empty((num_tokens * top_k_num, N // 2 // group_size), dtype=torch.float32,
                                    device=cache1.device)
@@ -129,6 +135,7 @@ class TritonExpertsPad:
                                 use_fp8_w8a8=self.use_fp8_w8a8, use_int8_w8a8=self.use_int8_w8a8,
                                 use_int8_w8a16=self.use_int8_w8a16, use_int4_w4a16=self.use_int4_w4a16,
                                 per_channel_quant=self.per_act_token_quant, block_shape=self.block_shape,
-                                real_token_num=expert_num_tokens if static_shape else None)
+                                real_token_num=expert_num_tokens if static_shape else None,
+                                A_scale_rec=a2_scale_rec)
 
         torch.ops._moe_C.moe_sum_pad(output, cache3, expert_num_tokens, 1, False)

@@ -83,6 +83,20 @@ def from_reference_layout(rweight: torch.Tensor, transposed: bool = False) -> to
     return _repack(rweight, fmt, batch, K, N)
 
 
+def from_reference_w4a8(rweight: torch.Tensor) -> torch.Tensor:
+    """The reference's w4a8 expert tensor -> slab layout int32 [E, K/8, N].
+
+    ``rweight`` is int8 with shape [E, N, K/2] whose memory is [E, K/2, N]
+    (w4a8.py:199-220 permutes, makes contiguous and then only *views* the
+    transposed shape; fused_moe_quant_kernel_ex.cpp:37 views it back), bytes in
+    half-groups of 32 rows holding ``w - 8`` as signed nibbles (rearrange.py:
+    61-133 with ``use_w4a8``, ``rearrange_group=64``).  The slab tensor holds the
+    unsigned ``w`` with the implicit zero-point 8."""
+    assert rweight.dtype in (torch.int8, torch.uint8) and rweight.dim() == 3
+    E, N, K2 = rweight.shape
+    return _repack(rweight, _lib.W4_SRC_REF_KN_G64S, E, 2 * K2, N)
+
+
 def pack_int8_zeros(z: torch.Tensor) -> torch.Tensor:
     """int8/uint8 zero-points [..., G, N] (the AWQ ``zeros_in_int8`` form,
     awq.py:80-106) -> packed int32 [..., G, N/8]."""

@@ -126,3 +126,50 @@ class FusedW8A8MoEMethod:
                                   a1_scale=getattr(layer, "w13_in_scales", None),
                                   a2_scale=getattr(layer, "w2_in_scales", None),
                                   apply_router_weight_on_input=apply_router_weight_on_input)
+
+
+class GCUCompressedTensorsW8A8Int8MoEMethod(FusedW8A8MoEMethod):
+    """compressed-tensors int8 experts (vllm_gcu/patch/patch_0_9_2/compressed_tensor.py:12-89,
+    over upstream ``CompressedTensorsW8A8Int8MoEMethod``): the same kernels as
+    ``FusedW8A8MoEMethod`` under the compressed-tensors parameter names --
+    ``w13_weight [E, 2I, H]`` / ``w2_weight [E, H, I]`` int8, per-channel
+    ``*_weight_scale [E, N, 1]`` fp32, ``*_input_scale`` None for per-token
+    dynamic activations (``per_act_token=True``) or one static scale each."""
+
+    def __init__(self, quant_config: Optional[W8A8Config] = None, per_act_token: bool = True):
+        self.per_act_token = per_act_token
+        super().__init__(quant_config or W8A8Config())
+
+    def select_gemm_impl(self, prepare_finalize=None, moe=None):
+        return TritonExpertsPad(use_int8_w8a8=True, per_channel_quant=True,
+                                per_act_token_quant=self.per_act_token)
+
+    def create_weights(self, layer, num_experts, hidden_size, intermediate_size_per_partition, params_dtype,
+                       **extra_weight_attrs):
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+
+        def reg(name, t):
+            layer.register_parameter(name, Parameter(t, requires_grad=False))
+        reg("w13_weight", torch.empty(E, 2 * I, H, dtype=torch.int8))
+        reg("w2_weight", torch.empty(E, H, I, dtype=torch.int8))
+        reg("w13_weight_scale", torch.ones(E, 2 * I, 1, dtype=torch.float32))
+        reg("w2_weight_scale", torch.ones(E, H, 1, dtype=torch.float32))
+        layer.w13_input_scale = None
+        layer.w2_input_scale = None
+
+    def apply(self, layer, x, router_logits, top_k: int, renormalize: bool, use_grouped_topk: bool = False,
+              topk_group=None, num_expert_group=None, global_num_experts: int = -1, expert_map=None,
+              custom_routing_function=None, scoring_func: str = "softmax", routed_scaling_factor: float = 1.0,
+              e_score_correction_bias=None, apply_router_weight_on_input: bool = False, activation: str = "silu",
+              enable_eplb: bool = False):
+        if enable_eplb:
+            raise NotImplementedError("EPLB not supported for `CompressedTensorsW8A8Int8MoEMethod` yet.")
+        topk_weights, topk_ids = select_experts(x, router_logits, top_k, use_grouped_topk, renormalize,
+                                                topk_group, num_expert_group, custom_routing_function,
+                                                scoring_func, e_score_correction_bias)
+        return self.fused_experts(x, layer.w13_weight, layer.w2_weight, topk_weights=topk_weights,
+                                  topk_ids=topk_ids, inplace=True, activation=activation,
+                                  global_num_experts=global_num_experts, expert_map=expert_map,
+                                  w1_scale=layer.w13_weight_scale, w2_scale=layer.w2_weight_scale,
+                                  a1_scale=layer.w13_input_scale, a2_scale=layer.w2_input_scale,
+                                  apply_router_weight_on_input=apply_router_weight_on_input)
