@@ -33,7 +33,7 @@ INT8_PEAK_TOPS = 5000.0
 # then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy of --calibrate-copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per
 # unit).  Keyed by (M, --split-k); other settings were not profiled.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 35800368}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 35169011}
 
 
 def w4a16_bytes(M, K, N, g=GROUP):
@@ -213,6 +213,14 @@ def main():
                 "avg_launch_us": round(launch_us, 3), "algorithmic_bytes_per_launch": step_bytes // launches,
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic}
+    if M > 64:
+        # --m above the decode range: the launches are the MFMA tile kernel and the bound is the fp16 matrix peak
+        step_flops = sum(2.0 * M * K * N for _, K, N in LLAMA3_8B)
+        tf = step_flops / launches / (launch_us * 1e-6) / 1e12
+        roofline = {"bound": "mfma", "kernel": "w4a16_tile_kernel", "launches_per_step": launches,
+                    "avg_launch_us": round(launch_us, 3), "algorithmic_flops_per_launch": step_flops / launches,
+                    "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4),
+                    "traffic": None}
 
     out = {
         "metric": "W4A16 GEMM HBM GB/s (algorithmic bytes / time), Llama-3-8B linear shapes",
@@ -236,6 +244,9 @@ def main():
         torch.cuda.empty_cache()
         out["moe_fp8_block"] = moe_bench(ops, dev, stream, "fp8")
         torch.cuda.empty_cache()
+        out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")
+        torch.cuda.empty_cache()
+        out["norm_quant"] = glue_bench(ops, dev, stream)
     if args.sweep:
         out["sweep"] = sweep(ops, dev, stream, args)
     if args.calibrate_copy:
@@ -309,6 +320,25 @@ def moe_bench(ops, dev, stream, which, iters=10):
         bytes_ = E * (H * 2 * I + I * H) // 2 + E * (H // 128 * 2 * I + I // 128 * H) * 2 \
             + E * (H // 128 * 2 * I + I // 128 * H) // 2 + 2 * M * H * 2
         name = "fused MoE W4A16, Mixtral-8x7B layer: 512 tok, hidden 4096, 8 experts, inter 14336, top-2"
+    elif which == "w4a8":
+        # the Mixtral-8x7B layer of configs[3] with w4a8-fp8 experts: fp8 activations with one
+        # static scale per GEMM, symmetric int4 weights, fp32 group scales
+        M, H, E, I, T = 512, 4096, 8, 14336, 2
+        w13, w2 = rnd_i32(E, H // 8, 2 * I), rnd_i32(E, I // 8, H)
+        s13 = torch.rand(E, H // 128, 2 * I, device=dev) * 0.009 + 0.001
+        s2 = torch.rand(E, I // 128, H, device=dev) * 0.009 + 0.001
+        a1, a2 = torch.tensor([0.02], device=dev), torch.tensor([0.5], device=dev)
+        x = torch.randn(M, H, generator=g).half().to(dev)
+        logits = torch.randn(M, E, generator=g).to(dev)
+        moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad(use_fp8_w8a8=True, block_shape=None))
+        kw = dict(w1_scale=s13, w2_scale=s2, a1_scale=a1, a2_scale=a2, a1_scale_rec=1.0 / a1, a2_scale_rec=1.0 / a2)
+
+        def step():
+            tw, ids = ops.fused_topk(x, logits, T, True)
+            return moe(x, w13, w2, tw, ids, **kw)
+        flops = 2.0 * M * T * (H * 2 * I + I * H)
+        bytes_ = E * (H * 2 * I + I * H) // 2 + E * (H // 128 * 2 * I + I // 128 * H) * 4 + 2 * M * H * 2
+        name = "fused MoE w4a8-fp8, Mixtral-8x7B layer shape: 512 tok, hidden 4096, 8 experts, inter 14336, top-2"
     else:
         M, H, E, I, T = 256, 7168, 256, 2048, 8
 
@@ -337,6 +367,30 @@ def moe_bench(ops, dev, stream, which, iters=10):
     return {"workload": name, "us": round(t * 1e6, 1), "compulsory_bytes": int(bytes_),
             "GBps": round(bytes_ / t / 1e9, 1), "frac_hbm": round(bytes_ / t / 1e9 / HBM_PEAK_GBPS, 4),
             "TFLOPs": round(flops / t / 1e12, 1)}
+
+
+def glue_bench(ops, dev, stream, iters=50):
+    """The norm + quantise prologue of a block-fp8 layer: 2048 tokens of hidden 7168, bf16 ->
+    fp8 with one scale per 128 values, with and without the residual add.  HBM-bound."""
+    import torch
+    rows, K = 2048, 7168
+    x = torch.randn(rows, K, device=dev).to(torch.bfloat16)
+    r = torch.randn(rows, K, device=dev).to(torch.bfloat16)
+    w = torch.ones(K, device=dev, dtype=torch.bfloat16)
+    q = torch.empty((rows, K), dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.empty((rows, K // 128), dtype=torch.float32, device=dev)
+    out = {}
+    for name, fn, nbytes in (
+            ("rms_norm_per_token_group_quant_fp8",
+             lambda: torch.ops._C.rms_norm_per_token_group_quant_fp8(q, s, x, w, 1e-6, 128),
+             rows * K * 3 + rows * K // 128 * 4),
+            ("fused_add_rms_norm_per_token_group_quant_fp8",
+             lambda: torch.ops._C.fused_add_rms_norm_per_token_group_quant_fp8(q, r, s, x, w, 1e-6, 128),
+             rows * K * 7 + rows * K // 128 * 4)):
+        t = time_graph([fn], iters, 5, stream) / iters
+        out[name] = {"shape": [rows, K], "us": round(t * 1e6, 2), "GBps": round(nbytes / t / 1e9, 1),
+                     "frac_hbm": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4)}
+    return out
 
 
 def sweep(ops, dev, stream, args):

@@ -275,8 +275,9 @@ rms_norm_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* resid
 }
 
 template <int DT, bool ADD>
-void launch_rms(int qm, dim3 grid, hipStream_t st, void* out, float* out_scales, const uint16_t* x,
+void launch_rms(int qm, long rows, hipStream_t st, void* out, float* out_scales, const uint16_t* x,
                 uint16_t* residual, const uint16_t* weight, const float* scale, float eps, int K, int gs) {
+  const dim3 grid((unsigned)rows);
   switch (qm) {
     case 0: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 0>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
     case 1: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 1>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
@@ -454,7 +455,7 @@ extern "C" int mi355q_rms_norm(void* out, float* out_scales, const void* x, void
                "rms_norm: group_size %d must be 64..512 (a power of two) and divide K=%d", group_size, K);
   }
   hipStream_t st = as_stream(stream);
-  const dim3 grid((unsigned)rows);
+  const long grid = rows;
   const uint16_t* xp = (const uint16_t*)x;
   uint16_t* rp = (uint16_t*)residual;
   const uint16_t* wp = (const uint16_t*)weight;
