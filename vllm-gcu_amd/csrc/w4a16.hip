@@ -23,7 +23,7 @@ extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
   const size_t s = w4a16_stream_workspace_bytes(M > 64 ? 64 : M, N);
   // the split-K partials of the MFMA kernel live behind the first MiB, which
   // holds the streaming kernel's arrival counters (they must stay zero)
-  const size_t t = M > 64 ? w4a16_tile_workspace_bytes(M, K, N) : 0;
+  const size_t t = M > 32 ? w4a16_tile_workspace_bytes(M, K, N) : 0;
   const size_t tt = t ? t + TILE_WS_OFFSET : 0;
   return s > tt ? s : tt;
 }
@@ -48,7 +48,12 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
              "w4a16_gemm: unknown zeros_kind %d", zeros_kind);
   MQ_REQUIRE(zeros_kind == MI355Q_ZP_NONE || zeros, "w4a16_gemm: zeros pointer missing");
   MQ_REQUIRE(family >= 0 && family <= 2, "w4a16_gemm: unknown kernel family %d", family);
-  if (family == 0) family = (M <= 64 || group_size % 128 != 0) ? 1 : 2;
+  if (family == 0) {
+    // streaming kernel up to 32 rows; 33..64 rows: the MFMA kernel where its pipelined loop exists
+    // (fp16, integer zero-points; measured equal or up to 22 % faster there), else streaming again
+    const bool piped = dtype == MI355Q_F16 && zeros_kind != MI355Q_ZP_PRESCALED;
+    family = (group_size % 128 != 0 || M <= 32 || (M <= 64 && !piped)) ? 1 : 2;
+  }
   MQ_REQUIRE(family != 2 || group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   if (family == 1) {

@@ -95,7 +95,7 @@ template <> struct TileMma<MI355Q_BF16> {
 // the rows (both halves dequantise the same weights, but two wavefronts per
 // SIMD keep the matrix pipe fed while one of them waits or dequantises).
 template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false>
-__global__ void __launch_bounds__(256 * WM, 1)
+__global__ void __launch_bounds__(256 * WM, WM == 1 ? 2 : 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
   typedef typename MM::vec vec;
@@ -424,7 +424,9 @@ template <int DT, int ZK, int MT, bool GROUPED, bool SF32 = false>
 hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
   {
     constexpr int BM = 16 * MT;
-    constexpr int WM = MT >= 4 ? 2 : 1;            // eight wavefronts once there are rows to split
+    // eight wavefronts once there are rows to split -- except dense 64-row tiles (M <= 64), which
+    // are bound by memory latency: four wavefronts on the pipelined loop, two workgroups per CU
+    constexpr int WM = (MT >= 8 || (MT == 4 && GROUPED)) ? 2 : 1;
     const int G = a.K >> 7;
     dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
     const size_t shmem = 2 * BM * A_ROW;           // up to 72 KiB: above the 64 KiB default
@@ -472,9 +474,12 @@ static int tile_rows_mt(int M, int N) {
 static int tile_splits(int M, int K, int N) {
   const int mt = tile_rows_mt(M, N), G = K / 128;
   const long wgs = (long)((M + 16 * mt - 1) / (16 * mt)) * ((N + BN - 1) / BN);
-  const long cus = device_cu_count();
-  if (wgs * 2 > cus) return 1;
-  long s = (cus + wgs / 2) / wgs;
+  // 64-row tiles run two workgroups per CU
+  const long target = (long)device_cu_count() * (mt == 4 ? 2 : 1);
+  if (wgs * 2 > target) return 1;
+  // 128-row tiles: the nearest count; 64-row tiles must all be resident at once (a second
+  // round of a few workgroups would double the time), so never above the target
+  long s = mt == 4 ? target / wgs : (target + wgs / 2) / wgs;
   if (s > G / 4) s = G / 4;
   while (s > 1 && (size_t)s * M * N * sizeof(float) > TILE_SPLITK_BYTES) --s;
   return s < 1 ? 1 : (int)s;
