@@ -49,6 +49,19 @@ struct TileArgs {
 // B operands are the exact integers (q - z) in the activation type; the group
 // scale multiplies the fp32 partial sum of each 128-row K block instead of
 // every weight, so the only rounding left is that of the fp32 accumulation.
+// (a & mask) | orv in one v_and_or_b32: the kernels keep the mask in a scalar and the magic in a
+// vector register (an opaque asm) -- as literals the compiler has to emit an and + or pair.
+struct DqConst {
+  uint32_t magic, mlo, mhi;
+};
+__device__ __forceinline__ DqConst dq_consts() {
+  DqConst k = {0x64006400u, 0x000f000fu, 0x00f000f0u};
+  asm volatile("" : "+v"(k.magic));
+  asm volatile("" : "+s"(k.mlo));
+  asm volatile("" : "+s"(k.mhi));
+  return k;
+}
+
 template <int DT> struct TileMma;
 template <> struct TileMma<MI355Q_F16> {
   typedef h8 vec;
@@ -56,15 +69,14 @@ template <> struct TileMma<MI355Q_F16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
   // one packed word -> 8 values (q - z); zz = {1024 + z, 64 + z}
-  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz) {
+  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz, const DqConst& k) {
     const h2 zlo = {zz.x, zz.x}, zhi = {zz.y, zz.y};
-    const uint32_t MAGIC = 0x64006400u;
     const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
     uint32_t w8 = w >> 8;
-    h2 a0 = bitcast<h2>((w & 0x000f000fu) | MAGIC);      // 1024 + q
-    h2 a1 = bitcast<h2>((w & 0x00f000f0u) | MAGIC);      // 1024 + 16 q
-    h2 a2 = bitcast<h2>((w8 & 0x000f000fu) | MAGIC);
-    h2 a3 = bitcast<h2>((w8 & 0x00f000f0u) | MAGIC);
+    h2 a0 = bitcast<h2>((w & k.mlo) | k.magic);       // 1024 + q
+    h2 a1 = bitcast<h2>((w & k.mhi) | k.magic);       // 1024 + 16 q
+    h2 a2 = bitcast<h2>((w8 & k.mlo) | k.magic);
+    h2 a3 = bitcast<h2>((w8 & k.mhi) | k.magic);
     h2 r0 = a0 - zlo;
     h2 r1 = __builtin_elementwise_fma(a1, sixteenth, -zhi);
     h2 r2 = a2 - zlo;
@@ -82,8 +94,8 @@ template <> struct TileMma<MI355Q_BF16> {
     uint32_t lo = bitcast<uint32_t>((float)r.x), hi = bitcast<uint32_t>((float)r.y);
     return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
   }
-  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz) {
-    h8 v = TileMma<MI355Q_F16>::dequant(w, zz);
+  static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz, const DqConst& k) {
+    h8 v = TileMma<MI355Q_F16>::dequant(w, zz, k);
     u4 r = {cvt((h2){v[0], v[1]}), cvt((h2){v[2], v[3]}), cvt((h2){v[4], v[5]}), cvt((h2){v[6], v[7]})};
     return bitcast<vec>(r);
   }
@@ -138,6 +150,8 @@ w4a16_tile_kernel(TileArgs a) {
   for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  const DqConst dqk = dq_consts();
 
   // global -> register staging of the next activation tile: thread tid loads
   // MTW chunks of 16 B: row = pass * 16 WM + tid / 16, chunk = tid % 16
@@ -233,7 +247,7 @@ w4a16_tile_kernel(TileArgs a) {
     prep();
     vec bv[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) bv[t] = MM::dequant(w0[t][0], zz[t]);
+    for (int t = 0; t < 4; ++t) bv[t] = MM::dequant(w0[t][0], zz[t], dqk);
     load_w(w1, min(gb + 1, ge - 1));
     load_sz(min(gb + 1, ge - 1));
     f4 part[MTW][4];
@@ -268,7 +282,7 @@ w4a16_tile_kernel(TileArgs a) {
         }
 #pragma unroll
         for (int t = mt * TPG; t < (mt + 1) * TPG; ++t)
-          bn[t] = MM::dequant(st < 3 ? wc[t][st + 1] : wn[t][0], zz[t]);
+          bn[t] = MM::dequant(st < 3 ? wc[t][st + 1] : wn[t][0], zz[t], dqk);
         if (st == 2 && mt == MTW - 1) load_w(wc, min(g + 2, ge - 1));   // last word of wc just went
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -338,7 +352,7 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
       for (int s = 0; s < 4; ++s)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zz[t]);
+        for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zz[t], dqk);
 
       const unsigned char* abase = lds + buf + (wmh * MTW * 16 + c) * A_ROW + kq * 16;
 #pragma unroll
