@@ -194,12 +194,14 @@ w4a16_stream_kernel(StreamArgs a) {
   // ahead, so the only memory wait inside the compute phase is for the block
   // being consumed while the next block's loads stay in flight (the wait
   // counter retires in order: a late load would drain the prefetch too).
+  // activations ride along one block ahead up to 32 rows (16 for the small-group variant, which has no registers to spare)
+  constexpr bool XA = MT == 1 || (MT == 2 && SPF == 4);
   struct Block {
     u4 w[NT];
     uint32_t sraw[4 / SPF][HW];
     uint32_t zraw[ZK == MI355Q_ZP_PRESCALED ? 4 / SPF : 1][HW];
     uint32_t zword[4 / SPF];
-    u4 xr[MT <= 2 ? 4 * MT : 1];    // activations ride along one block ahead up to 32 rows
+    u4 xr[XA ? 4 * MT : 1];
   };
   auto load_block = [&](Block& b, int g) {
     const u4* p = wbase + (size_t)g * 512;
@@ -213,22 +215,22 @@ w4a16_stream_kernel(StreamArgs a) {
       if (ZK == MI355Q_ZP_PACKED) b.zword[f] = ((const uint32_t*)a.zeros)[(size_t)qrow * (N >> 3) + (ncol8 >> 3)];
       if (ZK == MI355Q_ZP_PRESCALED) load_halves<NT>((const uint16_t*)a.zeros + (size_t)qrow * N + ncol, b.zraw[f]);
     }
-    if (MT <= 2) {
+    if (XA) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
           // rows past M repeat the last row: output rows are independent and
           // rows >= M are never stored, so no predicated load is needed
-          b.xr[MT <= 2 ? 4 * mt + s : 0] =
+          b.xr[XA ? 4 * mt + s : 0] =
               *(const u4*)(a.x + (size_t)min(16 * mt + c, a.M - 1) * K + 128 * g + 32 * s + 8 * kq);
         }
     }
   };
   // activations of block g for 64-row launches (too many registers to carry a block ahead)
-  struct Acts { u4 xr[MT <= 2 ? 1 : MT][4]; };
+  struct Acts { u4 xr[XA ? 1 : MT][4]; };
   auto load_acts = [&](Acts& x, int g) {
-    if (MT <= 2) return;
+    if (XA) return;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -252,7 +254,7 @@ w4a16_stream_kernel(StreamArgs a) {
         corr[mt] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < SPF; ++s) {
-          const u4 raw = (MT <= 2) ? b.xr[MT <= 2 ? 4 * mt + SPF * f + s : 0] : xa.xr[MT <= 2 ? 0 : mt][SPF * f + s];
+          const u4 raw = XA ? b.xr[XA ? 4 * mt + SPF * f + s : 0] : xa.xr[XA ? 0 : mt][SPF * f + s];
           av[mt][s] = MM::prep_a(raw);
           xs[mt] = MM::run(bitcast<vec>(raw), MM::splat(1.0f), xs[mt]);
           if (MM::kScaledA) corr[mt] = MM::run(av[mt][s], MM::splat(MM::kBase), corr[mt]);
