@@ -287,7 +287,7 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40):
             "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1)}
 
 
-def moe_bench(ops, dev, stream, which, iters=10):
+def moe_bench(ops, dev, stream, which, iters=10, tokens=None):
     """BASELINE configs[3] (Mixtral-8x7B layer, W4A16) and configs[4]
     (DeepSeek-V3-style layer, fp8 block-scaled): routing + the whole
     fused-experts sequence, one layer."""
@@ -303,7 +303,7 @@ def moe_bench(ops, dev, stream, which, iters=10):
         return torch.randint(-2**31, 2**31 - 1, shape, dtype=torch.int32, device=dev)
 
     if which == "w4a16":
-        M, H, E, I, T = 512, 4096, 8, 14336, 2
+        M, H, E, I, T = tokens or 512, 4096, 8, 14336, 2
         w13, w2 = rnd_i32(E, H // 8, 2 * I), rnd_i32(E, I // 8, H)
         z13, z2 = rnd_i32(E, H // 128, 2 * I // 8), rnd_i32(E, I // 128, H // 8)
         s13 = (torch.rand(E, H // 128, 2 * I, device=dev) * 0.009 + 0.001).half()
@@ -319,7 +319,7 @@ def moe_bench(ops, dev, stream, which, iters=10):
         flops = 2.0 * M * T * (H * 2 * I + I * H)
         bytes_ = E * (H * 2 * I + I * H) // 2 + E * (H // 128 * 2 * I + I // 128 * H) * 2 \
             + E * (H // 128 * 2 * I + I // 128 * H) // 2 + 2 * M * H * 2
-        name = "fused MoE W4A16, Mixtral-8x7B layer: 512 tok, hidden 4096, 8 experts, inter 14336, top-2"
+        name = f"fused MoE W4A16, Mixtral-8x7B layer: {M} tok, hidden 4096, 8 experts, inter 14336, top-2"
     elif which == "w4a8":
         # the Mixtral-8x7B layer of configs[3] with w4a8-fp8 experts: fp8 activations with one
         # static scale per GEMM, symmetric int4 weights, fp32 group scales

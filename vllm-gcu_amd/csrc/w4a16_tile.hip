@@ -434,22 +434,25 @@ w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* 
   *(uint2*)(out + i) = o;
 }
 
+template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32>
+hipError_t launch_wm(const TileArgs& a, int row_blocks, hipStream_t st) {
+  constexpr int BM = 16 * MT;
+  const int G = a.K >> 7;
+  dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
+  const size_t shmem = 2 * BM * A_ROW;             // up to 72 KiB: above the 64 KiB default
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  if (attr != hipSuccess) return attr;
+  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>), grid, block, shmem, st, a);
+  return hipSuccess;
+}
+
 template <int DT, int ZK, int MT, bool GROUPED, bool SF32 = false>
 hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
-  {
-    constexpr int BM = 16 * MT;
-    // eight wavefronts once there are rows to split -- except dense 64-row tiles (M <= 64), which
-    // are bound by memory latency: four wavefronts on the pipelined loop, two workgroups per CU
-    constexpr int WM = (MT >= 8 || (MT == 4 && GROUPED)) ? 2 : 1;
-    const int G = a.K >> 7;
-    dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
-    const size_t shmem = 2 * BM * A_ROW;           // up to 72 KiB: above the 64 KiB default
-    static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-    if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>), grid, block, shmem, st, a);
-    return hipSuccess;
-  }
+  // up to 64 rows: four wavefronts, each all rows of its 64 columns, two workgroups per CU;
+  // 128-row tiles (MoE blocks of 128 only): eight wavefronts, 2 (M) x 4 (N)
+  constexpr int WM = MT >= 8 ? 2 : 1;
+  return launch_wm<DT, ZK, MT, GROUPED, WM, SF32>(a, row_blocks, st);
 }
 
 template <int DT, int MT, bool GROUPED>
@@ -480,10 +483,12 @@ hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStrea
 // partial tiles of at most TILE_SPLITK_BYTES in total
 constexpr size_t TILE_SPLITK_BYTES = (size_t)64 << 20;
 static int tile_rows_mt(int M, int N) {
-  // 128-row blocks as soon as there are more than 64 rows (measured faster from M = 96 up,
-  // split-K filling the chip where the grid alone does not), 64-row blocks below
+  // 64-row tiles for every dense shape: four wavefronts on the pipelined loop, two workgroups
+  // per CU -- measured equal or faster than 128-row tiles of eight wavefronts from M = 65 to
+  // 8192 (M = 2048: qkv 134 -> 112 us, gate_up 461 -> 449 us), fp16 and bf16
+  (void)M;
   (void)N;
-  return M > 64 ? 8 : 4;
+  return 4;
 }
 static int tile_splits(int M, int K, int N) {
   const int mt = tile_rows_mt(M, N), G = K / 128;
