@@ -326,6 +326,11 @@ __device__ __forceinline__ float ld_act(const void* p, long i) {
   return Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT>::to_f32(((const uint16_t*)p)[i]);
 }
 
+template <int DT>
+__device__ __forceinline__ float ld_half(uint16_t raw) {
+  return Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT>::to_f32(raw);
+}
+
 __device__ __forceinline__ int8_t sat_rne_s8(float y) {
   y = __builtin_rintf(y);                       // round half to even
   y = fminf(fmaxf(y, -128.0f), 127.0f);
@@ -340,7 +345,21 @@ dynamic_int8_quant_kernel(int8_t* out, float* scales, const void* x, int K, cons
   if (valid_rows && row >= *valid_rows) return;
   __shared__ float red[4];
   float mx = 0.f;
-  for (int k = threadIdx.x; k < K; k += 256) mx = fmaxf(mx, fabsf(ld_act<DT>(x, (long)row * K + k)));
+  // 16-bit inputs with K % 8 == 0: 16-byte loads, 8-byte stores (8 elements per lane and step)
+  const bool vec8 = DT != MI355Q_F32 && (K & 7) == 0;
+  const uint16_t* xr = (const uint16_t*)x + (long)row * K;
+  if (vec8) {
+    for (int c = threadIdx.x; c < (K >> 3); c += 256) {
+      const u4 v = *(const u4*)(xr + 8 * c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mx = fmaxf(mx, fabsf(ld_half<DT>((uint16_t)(v[i] & 0xffffu))));
+        mx = fmaxf(mx, fabsf(ld_half<DT>((uint16_t)(v[i] >> 16))));
+      }
+    }
+  } else {
+    for (int k = threadIdx.x; k < K; k += 256) mx = fmaxf(mx, fabsf(ld_act<DT>(x, (long)row * K + k)));
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
@@ -348,6 +367,21 @@ dynamic_int8_quant_kernel(int8_t* out, float* scales, const void* x, int K, cons
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   if (threadIdx.x == 0) scales[row] = mx / 127.0f;
   const float inv = 127.0f / mx;                // inf for an all-zero row
+  if (vec8) {
+    for (int c = threadIdx.x; c < (K >> 3); c += 256) {
+      const u4 v = *(const u4*)(xr + 8 * c);    // the row was just read: an L2 hit
+      uint32_t q[2] = {0u, 0u};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t w = v[e >> 1];
+        float y = ld_half<DT>((uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu))) * inv;
+        if (y != y) y = 0.f;                    // 0 * inf
+        q[e >> 2] |= ((uint32_t)(uint8_t)sat_rne_s8(y)) << (8 * (e & 3));
+      }
+      *(u2*)(out + (long)row * K + 8 * c) = (u2){q[0], q[1]};
+    }
+    return;
+  }
   for (int k = threadIdx.x; k < K; k += 256) {
     float y = ld_act<DT>(x, (long)row * K + k) * inv;
     if (y != y) y = 0.f;                        // 0 * inf
