@@ -209,16 +209,49 @@ moe_align_kernel(const IdT* __restrict__ topk_ids, int numel, int top, const int
     estart[e + 1] = (run + B - 1) / B * B;       // padded count, scanned below
   }
   __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    estart[0] = 0;
-    for (int e = 0; e < E; ++e) {
-      int c = estart[e + 1];
-      estart[e] = run;
-      run += c;
+  // exclusive scan of the padded counts by the first wavefront: each lane sums a run of
+  // consecutive experts, the lane totals are scanned with shuffles
+  if (wv == 0) {
+    const int per = (E + 63) / 64;
+    const int e0 = min(E, lane * per), e1 = min(E, e0 + per);
+    int sum = 0;
+    for (int e = e0; e < e1; ++e) sum += estart[e + 1];
+    int incl = sum;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o);
+      if (lane >= o) incl += up;
     }
-    estart[E] = run;
-    *npp = run;
+    int run = incl - sum;                          // exclusive prefix of this lane's run
+    const int total = __shfl(incl, 63);
+    // estart[e] must not be overwritten before the lane that reads estart[e + 1] = old count
+    // of expert e has consumed it: every lane first reads its own run, then all write
+    int vals[16];
+    const bool small = per <= 16;
+    if (small) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) vals[k] = (e0 + k < e1) ? estart[e0 + k + 1] : 0;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (small) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k)
+        if (e0 + k < e1) {
+          estart[e0 + k] = run;
+          run += vals[k];
+        }
+      if (lane == 63) estart[E] = total;
+    } else if (lane == 0) {
+      // more than 1024 experts: plain serial scan
+      int r = 0;
+      for (int e = 0; e < E; ++e) {
+        const int c = estart[e + 1];
+        estart[e] = r;
+        r += c;
+      }
+      estart[E] = r;
+    }
+    if (lane == 0) *npp = total;
   }
   __syncthreads();
   // block -> expert table (unused blocks get expert 0)
