@@ -110,6 +110,20 @@ def test_stream_gemm_parity(ops, rearrange, M, dtype):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("M", [33, 48, 64])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("family", [1, 2])
+def test_33_to_64_rows_either_kernel_family(ops, rearrange, M, dtype, family):
+    """The dispatcher picks the family by dtype in this range; both must hold the tolerance for both."""
+    K, N, g = 2048, 512, 128
+    print(f"case family={family} M={M} {dtype}", flush=True)
+    q, z, s, x = make_case(100 + M, M, K, N, g)
+    bias = np.random.default_rng(M).standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias, family=family).float().cpu().numpy()
+    want = oracle(q, z, s, x, g, dtype, bias=bias)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("split_k", [1, 2, 3, 8])
 def test_stream_gemm_exact_and_split_invariant(ops, rearrange, split_k):
     # power-of-two scales + small integer activations: every product and every
