@@ -280,11 +280,21 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40):
     t = time_graph([lambda: torch.ops._C.cutlass_scaled_mm(out, xq, wt, xs, ws, None)], iters, warmup, stream) / iters
     tq = time_graph([lambda: ops.scaled_int8_quant(x)], iters, 3, stream) / iters
     ops_ = 2.0 * M * K * N
+    # decode: 16 tokens against the same layer, weights as the linear method keeps them after
+    # loading (kslab order); three weight copies in turn so that none is served from a cache
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    Md = 16
+    ksl = [rearrange.to_kslab(w_nk if i == 0 else w_nk.roll(i, 0)) for i in range(3)]
+    outd = torch.empty(Md, N, dtype=torch.float16, device=dev)
+    fns = [(lambda w=w: torch.ops._C.cutlass_scaled_mm(outd, xq[:Md], w.t(), xs[:Md], ws, None)) for w in ksl]
+    td = time_graph(fns, iters, 3, stream) / iters
     return {"workload": "W8A8 int8 GEMM M=2048 K=8192 N=28672, fused per-token x per-channel scales, fp16 out",
             "gemm_us": round(t * 1e6, 1), "TOPs": round(ops_ / t / 1e12, 1),
             "frac_int8_mfma_peak": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
             "dynamic_quant_us": round(tq * 1e6, 1),
-            "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1)}
+            "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1),
+            "decode_m16_us": round(td * 1e6, 1),
+            "decode_m16_GBps": round((N * K + Md * K + 2 * Md * N) / td / 1e9, 1)}
 
 
 def moe_bench(ops, dev, stream, which, iters=10, tokens=None):

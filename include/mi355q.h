@@ -101,7 +101,9 @@ int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
  *   out[m, n] = (sum_k x[m, k] * w[n, k]  in int32) * x_scale[m or 0] * w_scale[n or 0] (+ bias[n])
  * x is [M, K] int8 with row stride ldx bytes; w is [N, K] int8 (K contiguous)
  * with row stride ldw bytes -- the physical layout of a checkpoint's [N, K]
- * weight, i.e. the `weight.t()` view the compressed-tensors path passes.
+ * weight, i.e. the `weight.t()` view the compressed-tensors path passes; ldw = 0
+ * says that w is in the kslab order instead (see mi355q_kslab_repack; N % 64 == 0),
+ * the layout mi355q_kcontig_gemm streams fastest at decode-sized M.
  * Scale pointers may be NULL (= 1.0); *_per_row / *_per_col select a vector
  * or a single value.  bias is in the output dtype, or fp32 when bias_f32.
  * acc_out (optional) receives the raw int32 accumulators [M, N] for parity

@@ -77,6 +77,32 @@ def test_int8_gemm_accumulators_bit_exact_both_layouts(ops, M, K, N):
     assert np.array_equal(acc2.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("M,K,N", [(1, 128, 64), (33, 384, 320), (300, 1024, 448), (513, 2048, 1024)])
+def test_int8_gemm_kslab_weights(ops, M, K, N):
+    """Weights re-ordered by rearrange.to_kslab: the MFMA tile kernel reads them in place (raw
+    accumulators bit-exact), and up to 48 rows the operator switches to the weight-streaming kernel,
+    whose outputs must equal the tile kernel's on row-major weights bit for bit."""
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print(f"case i8 kslab {M}x{K}x{N}", flush=True)
+    rng = np.random.default_rng(M * 7 + K + N)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    wk = rearrange.to_kslab(dev(w_nk))
+    assert rearrange.is_kslab(wk.t())                      # the flag survives the view the operators receive
+    want = o8.int8_gemm_i32(x, np.ascontiguousarray(w_nk.T))
+    acc = ops.int8_gemm_accumulators(dev(x), wk.t())
+    assert np.array_equal(acc.cpu().numpy(), want)
+    xs = rng.uniform(0.001, 0.01, size=(M, 1)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.float16).cuda()
+    for b in (None, bias):
+        a = ops.cutlass_scaled_mm(dev(x), wk.t(), dev(xs), dev(ws), torch.float16, b)
+        r = ops.cutlass_scaled_mm(dev(x), dev(w_nk).t(), dev(xs), dev(ws), torch.float16, b)
+        assert torch.equal(a, r)
+        wantf = o8.scaled_mm_epilogue(want, xs, ws, None if b is None else b.float().cpu().numpy())
+        np.testing.assert_allclose(a.float().cpu().numpy(), wantf, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_cutlass_scaled_mm_epilogue(ops, dtype):
     rng = np.random.default_rng(3)

@@ -37,6 +37,7 @@ struct I8Args {
   long ldx, ldw, ldo;
   int x_scale_per_row, w_scale_per_col, bias_f32;
   int n_panels_swizzle;     // non-zero: XCD-aware tile order
+  int w_kslab;              // w is in the kslab order (see include/mi355q.h) instead of row-major
 };
 
 template <int DT>
@@ -124,10 +125,21 @@ w8a8_int8_gemm_kernel(I8Args a) {
 #pragma unroll
     for (int p = 0; p < WCOPIES; ++p) {
       const int r = (wave + 8 * p) * 8 + crow;
-      wo[p] = (uint32_t)((min(n0 + r, N - 1) - n0) * a.ldw + 16 * cchunk);
+      if (a.w_kslab) {
+        // kslab: [N/64][K/128][4 tiles of 16 rows][2 vectors][64 lanes = 16 rows x 4 segments][16 B].
+        // One chunk of 8 consecutive rows is 128 contiguous bytes there, so lane = 8 * position +
+        // row: 8 consecutive lanes again fetch one whole line, and LDS holds the group chunk-major,
+        // position p of an odd group holding chunk p ^ 1 (see the operand reads).
+        const uint32_t n = (uint32_t)min(n0 + (wave + 8 * p) * 8 + (lane & 7), N - 1);
+        const uint32_t c = (uint32_t)((lane >> 3) ^ (wave & 1));
+        wo[p] = ((n >> 6) * (uint32_t)(K >> 7) * 4u + ((n & 63u) >> 4)) * 2048u + (c & 1u) * 1024u +
+                ((c >> 1) * 16u + (n & 15u)) * 16u;
+      } else {
+        wo[p] = (uint32_t)((min(n0 + r, N - 1) - n0) * a.ldw + 16 * cchunk);
+      }
     }
     xtile = a.x + (long)m0 * a.ldx;
-    wtile = a.w + (long)n0 * a.ldw;
+    wtile = a.w_kslab ? a.w : a.w + (long)n0 * a.ldw;
   };
   // copy slot s of this wavefront: slots 0 .. XCOPIES-1 are its x row groups,
   // the rest its w row groups (the last one only exists for some wavefronts)
@@ -138,7 +150,9 @@ w8a8_int8_gemm_kernel(I8Args a) {
       dma16(xtile + k0 + xo[s], xs + (wave + 8 * s) * 1024);
     } else {
       const int p = s - XCOPIES;
-      if (wave + 8 * p < WGROUPS) dma16(wtile + k0 + wo[p < WCOPIES ? p : 0], xs + X_BYTES + (wave + 8 * p) * 1024);
+      // a K tile of 128 bytes per row is 8 KiB further on in the kslab order
+      if (wave + 8 * p < WGROUPS)
+        dma16(wtile + (a.w_kslab ? (long)k0 * 64 : (long)k0) + wo[p < WCOPIES ? p : 0], xs + X_BYTES + (wave + 8 * p) * 1024);
     }
   };
   auto issue = [&](int stage, int k0) {
@@ -157,6 +171,13 @@ w8a8_int8_gemm_kernel(I8Args a) {
   uint32_t lo[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) lo[h] = lds_base + (uint32_t)(l16 * TKB + (((4 * h + kq) ^ (l16 & 7)) * 16));
+  // kslab weights lie chunk-major in LDS: 8-row group, then chunk position (chunk ^ 1 in odd
+  // groups, so that the two groups of a 16-row tile fall on different banks), then row
+  uint32_t wlo[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    wlo[h] = a.w_kslab ? lds_base + (uint32_t)((l16 >> 3) * 1024 + (((4 * h + kq) ^ (l16 >> 3)) * 128) + (l16 & 7) * 16)
+                       : lo[h];
   const uint32_t xwave = wm * (16 * NJ) * TKB, wwave = X_BYTES + wn * (16 * NI) * TKB;
   struct Frag { i4 bx[NJ]; i4 aw[NI]; };
   // read r of an operand set: r < NJ is x tile r, the rest are w tiles
@@ -170,7 +191,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   };
   auto read_frag = [&](Frag& f, int stage, int h) {
     const uint32_t xb = lo[h] + (uint32_t)(stage * STAGE_BYTES) + xwave;
-    const uint32_t wb = lo[h] + (uint32_t)(stage * STAGE_BYTES) + wwave;
+    const uint32_t wb = wlo[h] + (uint32_t)(stage * STAGE_BYTES) + wwave;
 #pragma unroll
     for (int r = 0; r < NJ + NI; ++r) read_one(f, r, xb, wb);
   };
@@ -203,7 +224,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   auto half = [&](const Frag& cur, Frag& nxt, int rstage, int rh, int SB, int SE, int C0, int CE,
                   int cstage, int k0) {
     const uint32_t xb = lo[rh] + (uint32_t)(rstage * STAGE_BYTES) + xwave;
-    const uint32_t wb = lo[rh] + (uint32_t)(rstage * STAGE_BYTES) + wwave;
+    const uint32_t wb = wlo[rh] + (uint32_t)(rstage * STAGE_BYTES) + wwave;
     int n = 0;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -460,8 +481,11 @@ extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* 
   MQ_REQUIRE(out && x && w, "w8a8_int8_gemm: null pointer");
   MQ_REQUIRE(K % 128 == 0, "w8a8_int8_gemm: K=%d must be a multiple of 128", K);
   MQ_REQUIRE(N % 4 == 0, "w8a8_int8_gemm: N=%d must be a multiple of 4", N);
-  MQ_REQUIRE(ldx % 16 == 0 && ldw % 16 == 0 && ldx >= K && ldw >= K,
+  const bool kslab = ldw == 0;
+  MQ_REQUIRE(ldx % 16 == 0 && ldx >= K && (kslab || (ldw % 16 == 0 && ldw >= K)),
              "w8a8_int8_gemm: operand row strides (%ld, %ld) must be >= K and multiples of 16", ldx, ldw);
+  MQ_REQUIRE(!kslab || (N % 64 == 0 && (size_t)N * K < ((size_t)1 << 32)),
+             "w8a8_int8_gemm: kslab weights need N=%d %% 64 == 0 and fewer than 4 Gi elements", N);
   MQ_REQUIRE(ldo >= N && ldo % 4 == 0, "w8a8_int8_gemm: output row stride %ld must be >= N and a multiple of 4", ldo);
   MQ_REQUIRE(out_dtype >= MI355Q_F16 && out_dtype <= MI355Q_F32, "w8a8_int8_gemm: bad out dtype %d", out_dtype);
   I8Args a;
@@ -469,6 +493,7 @@ extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* 
   a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;
   a.x_scale_per_row = x_scale_per_row; a.w_scale_per_col = w_scale_per_col; a.bias_f32 = bias_f32;
   a.n_panels_swizzle = 0;
+  a.w_kslab = kslab ? 1 : 0;
   if (out_dtype == MI355Q_F16) return launch_gemm<MI355Q_F16>(a, as_stream(stream));
   if (out_dtype == MI355Q_BF16) return launch_gemm<MI355Q_BF16>(a, as_stream(stream));
   return launch_gemm<MI355Q_F32>(a, as_stream(stream));

@@ -187,6 +187,9 @@ def _gptq_gemm_gcu_fake(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bi
 # ---------------------------------------------------------------------------
 # W8A8 int8 (csrc/torch_bindings.cpp:734-766, 1002-1019)
 # ---------------------------------------------------------------------------
+_INT8_STREAM_MAX_M = 48      # measured on MI355X (K 8192, N 28672): 49-67 us against 94 us up to M = 32, equal at 64
+
+
 def _int8_weight_nk(weight: torch.Tensor):
     """-> (tensor whose memory is [N, K] K-contiguous, row stride in bytes).
 
@@ -198,6 +201,9 @@ def _int8_weight_nk(weight: torch.Tensor):
     """
     if weight.dim() != 2 or weight.dtype != torch.int8:
         raise RuntimeError(f"int8 weight must be a 2-D int8 tensor, got {weight.dtype} {tuple(weight.shape)}")
+    if rearrange.is_kslab(weight):
+        # bytes re-ordered at load time (rearrange.to_kslab): row stride 0 tells the library so
+        return weight, 0
     if weight.stride(0) == 1 and weight.stride(1) >= weight.shape[0] and weight.stride(1) % 16 == 0:
         return weight, weight.stride(1)
     wt = _converted(weight, lambda t: t.t().contiguous())
@@ -240,6 +246,15 @@ def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
             bias = bias.to(torch.float32)
             bias_f32 = 1
         bias = bias.contiguous()
+    if ldw == 0 and M <= _INT8_STREAM_MAX_M and acc_out is None and ws_col and (xs is None or xs_row or M == 1) \
+            and not bias_f32 and out.dtype in (torch.float16, torch.bfloat16) and x2.is_contiguous() \
+            and out2.stride(0) == N:
+        # decode-sized M on kslab weights: the weight-streaming kernel (same int32 sums, same
+        # epilogue order: bit-identical results) reads them about twice as fast
+        with torch.cuda.device(x.device):
+            _lib.call("mi355q_kcontig_gemm", out2.data_ptr(), x2.data_ptr(), w.data_ptr(), rt.ptr(xs), ws.data_ptr(),
+                      rt.ptr(bias), _lib.Q_INT8, 0, M, K, N, _lib.F16, rt.dtype_code(out.dtype), 1, rt.stream_ptr())
+        return
     with torch.cuda.device(x.device):
         _lib.call("mi355q_w8a8_int8_gemm", out2.data_ptr(), rt.ptr(acc_out), x2.data_ptr(), w.data_ptr(),
                   rt.ptr(xs), xs_row, rt.ptr(ws), ws_col, rt.ptr(bias), bias_f32, M, N, K,
@@ -251,9 +266,10 @@ def _cutlass_scaled_mm_impl(out, x, weight, x_scale, w_scale, bias):
 
 
 def _dot_bias_quant_impl(out, lhs, rhs, scale, bias):
-    # single scale[N]: the activation scale is pre-folded (w8a8.py:157-171);
-    # bias is promoted to fp32 (dot_bias_quant.cpp:19-21)
-    _scaled_int8_mm(out, lhs, rhs, None, scale, None if bias is None else bias.to(torch.float32))
+    # single scale[N]: the activation scale is pre-folded (w8a8.py:157-171).  The reference
+    # promotes the bias to fp32 before adding it (dot_bias_quant.cpp:19-21); the kernels read a
+    # bias of the output type and widen each element, which is the same sum
+    _scaled_int8_mm(out, lhs, rhs, None, scale, bias)
 
 
 def _dynamic_scaled_int8_quant_impl(output, input, scales, azp):

@@ -7,6 +7,8 @@ the reference layout) are converted by HIP kernels into the MI355X slab layout
 the W4A16 kernels stream (see include/mi355q.h), and zero-points are kept as
 packed int4 instead of being pre-multiplied by the scales.
 """
+import weakref
+
 import torch
 
 from .. import _runtime as rt
@@ -121,8 +123,37 @@ def unpack_slab(packed: torch.Tensor) -> torch.Tensor:
     return dst
 
 
+# kslab allocations by (device index, address) -> byte size: the flag has to survive views
+# (``weight.t()`` is what the int8 operators receive), which drop Python attributes
+_KSLAB_ALLOCS = {}           # (device, address) -> [bytes, live tensor objects that carry the flag]
+
+
+def _unregister_kslab(key) -> None:
+    ent = _KSLAB_ALLOCS.get(key)
+    if ent is not None:
+        ent[1] -= 1
+        if ent[1] <= 0:
+            del _KSLAB_ALLOCS[key]
+
+
+def _register_kslab(t: torch.Tensor) -> None:
+    """Entries live as long as a flagged tensor object on that memory does (the tensor made by
+    to_kslab, a Parameter wrapped around it and marked with mark_kslab, ...)."""
+    key = (t.device.index, t.data_ptr())
+    ent = _KSLAB_ALLOCS.setdefault(key, [t.numel() * t.element_size(), 0])
+    ent[0] = t.numel() * t.element_size()
+    ent[1] += 1
+    weakref.finalize(t, _unregister_kslab, key)
+
+
 def is_kslab(w: torch.Tensor) -> bool:
-    return bool(getattr(w, "_mi355q_kslab", False))
+    """True for a tensor made by :func:`to_kslab`, for a Parameter / view marked with
+    :func:`mark_kslab`, and for any view that starts at the address of such an allocation and
+    covers all of it (e.g. ``w.t()``)."""
+    if getattr(w, "_mi355q_kslab", False):
+        return True
+    ent = _KSLAB_ALLOCS.get((w.device.index, w.data_ptr())) if w.is_cuda else None
+    return ent is not None and ent[0] == w.numel() * w.element_size()
 
 
 def kslab_eligible(w: torch.Tensor) -> bool:
@@ -148,12 +179,14 @@ def to_kslab(w: torch.Tensor) -> torch.Tensor:
         _lib.call("mi355q_kslab_repack", w.data_ptr(), dst.data_ptr(), batch, w.shape[-2], w.shape[-1],
                   w.element_size(), rt.stream_ptr())
     dst._mi355q_kslab = True
+    _register_kslab(dst)
     return dst
 
 
 def mark_kslab(p: torch.Tensor) -> torch.Tensor:
     """Re-attach the layout flag after wrapping a kslab tensor (e.g. in a Parameter)."""
     p._mi355q_kslab = True
+    _register_kslab(p)
     return p
 
 
