@@ -57,11 +57,13 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
   MQ_REQUIRE(family != 2 || group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   if (family == 1) {
-    // the streaming kernel covers 64 rows per launch; taller inputs (only
-    // reached with group sizes below 128) go through it in row chunks
+    // the streaming kernel covers 64 rows per launch (32 with group sizes
+    // below 128, whose four scale rows per K block leave no registers for
+    // more); taller inputs go through it in row chunks
     const size_t esz = 2;
-    for (int m0 = 0; m0 < M; m0 += 64) {
-      const int mc = M - m0 < 64 ? M - m0 : 64;
+    const int chunk = group_size % 128 == 0 ? 64 : 32;
+    for (int m0 = 0; m0 < M; m0 += chunk) {
+      const int mc = M - m0 < chunk ? M - m0 : chunk;
       int rc = w4a16_stream_launch((char*)out + (size_t)m0 * N * esz, (const char*)x + (size_t)m0 * K * esz,
                                    qweight, scales, zeros, zeros_kind, bias, mc, K, N, group_size, dtype,
                                    workspace, workspace_bytes, split_k, as_stream(stream));

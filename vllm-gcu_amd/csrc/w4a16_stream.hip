@@ -26,6 +26,7 @@ struct StreamArgs {
   const uint16_t* bias;
   int M, K, N;
   int gs;            // quantisation group size (rows of K per scale row)
+  uint32_t gs_magic; // ceil(2^32 / gs): k / gs == umulhi(k, gs_magic) for every k < K
   int splits;
   float* partial;    // [splits][16*MT][N]
   int* counters;     // one per blockIdx.x (<= N/16), zero between launches
@@ -161,6 +162,28 @@ __device__ __forceinline__ void load_halves(const uint16_t* p, uint32_t* dst) {
   else dst[0] = *p;
 }
 
+// Buffer loads: an offset at or past the descriptor's size reads as zero
+// without touching memory, which makes "no such K block" a branch-free case
+// (callers add 2^31 to the lane offset; every buffer here is below 2 GiB).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u4 buf_load16(rsrc_t r, uint32_t off) {
+  return bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
+}
+// streamed once: non-temporal
+__device__ __forceinline__ u4 buf_load16_nt(rsrc_t r, uint32_t off) {
+  return bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 2));
+}
+template <int NT>
+__device__ __forceinline__ void buf_load_halves(rsrc_t r, uint32_t off, uint32_t* dst) {
+  if (NT == 8) { u4 v = buf_load16(r, off); dst[0] = v[0]; dst[NT > 2 ? 1 : 0] = v[1]; dst[NT > 4 ? 2 : 0] = v[2]; dst[NT > 6 ? 3 : 0] = v[3]; }
+  else if (NT == 4) { u2 v = bitcast<u2>(__builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0)); dst[0] = v[0]; dst[NT > 2 ? 1 : 0] = v[1]; }
+  else if (NT == 2) dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
+  else dst[0] = __builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0);
+}
+
 template <int DT, int MT, int ZK, int SPF, int NT>
 __global__ void __launch_bounds__(256, (MT == 1 || (MT == 2 && NT <= 4)) ? 2 : 1)
 w4a16_stream_kernel(StreamArgs a) {
@@ -184,7 +207,6 @@ w4a16_stream_kernel(StreamArgs a) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
 
-  const u4* wbase = a.qw + (size_t)slab * G * 512 + t0 * 64 + lane;
   const int ncol8 = 128 * slab + 8 * c;              // first of this lane's 8 slab columns
   const int ncol = ncol8 + t0;                       // first of the NT columns this workgroup owns
   const uint32_t magic = launder_vgpr(MM::magic());
@@ -203,41 +225,63 @@ w4a16_stream_kernel(StreamArgs a) {
     uint32_t zword[4 / SPF];
     u4 xr[XA ? 4 * MT : 1];
   };
-  auto load_block = [&](Block& b, int g) {
-    const u4* p = wbase + (size_t)g * 512;
+  constexpr int W = 4;                                // wavefronts per workgroup (eight were measured: not faster)
+  // K blocks of this wavefront: gb + wave, + W, ...; visited from a
+  // workgroup-dependent start (see the loop below)
+  const int g0 = gb + wave;
+  const int nb = (ge - g0 + W - 1) / W;
+  const int rot = nb > 0 ? (int)((blockIdx.x >> 3) * 5u % (unsigned)nb) : 0;
+  auto blk = [&](int i) {                            // i-th block in this workgroup's order, i < nb
+    int j = i + rot;
+    if (j >= nb) j -= nb;
+    return g0 + W * j;
+  };
+  const rsrc_t wres = make_rsrc(a.qw + (size_t)slab * G * 512, (uint32_t)G * 8192u);
+  const rsrc_t sres = make_rsrc(a.scales, (uint32_t)(K / a.gs) * N * 2u);
+  const rsrc_t zres = make_rsrc(a.zeros, ZK == MI355Q_ZP_PACKED ? (uint32_t)(K / a.gs) * (N >> 3) * 4u
+                                                                 : (uint32_t)(K / a.gs) * N * 2u);
+  const rsrc_t xres = make_rsrc(a.x, (uint32_t)a.M * K * 2u);
+  const uint32_t wlane = (uint32_t)(t0 * 64 + lane) * 16u;
+  uint32_t xlane[MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) b.w[t] = __builtin_nontemporal_load(p + t * 64);
+  for (int mt = 0; mt < MT; ++mt)
+    // rows past M repeat the last row: output rows are independent and rows >= M are never stored
+    xlane[mt] = ((uint32_t)min(16 * mt + c, a.M - 1) * K + 8 * kq) * 2u;
+  // block i of this wavefront's order; i >= nb loads nothing (zeros, no memory traffic)
+  auto load_block = [&](Block& b, int i) {
+    const bool have = i < nb;
+    const uint32_t oob = have ? 0u : 0x80000000u;
+    const int g = have ? blk(i) : g0;
+    const uint32_t wo = wlane + (uint32_t)g * 8192u + oob;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) b.w[t] = buf_load16_nt(wres, wo + t * 1024);
 #pragma unroll
     for (int f = 0; f < 4 / SPF; ++f) {
-      const int qrow = (128 * g + 32 * SPF * f) / a.gs;
-      load_halves<NT>(a.scales + (size_t)qrow * N + ncol, b.sraw[f]);
+      const uint32_t krow = 128 * g + 32 * SPF * f;
+      const uint32_t qrow = __umulhi(krow, a.gs_magic);
+      buf_load_halves<NT>(sres, (qrow * N + ncol) * 2u + oob, b.sraw[f]);
       b.zword[f] = 0x88888888u;
-      if (ZK == MI355Q_ZP_PACKED) b.zword[f] = ((const uint32_t*)a.zeros)[(size_t)qrow * (N >> 3) + (ncol8 >> 3)];
-      if (ZK == MI355Q_ZP_PRESCALED) load_halves<NT>((const uint16_t*)a.zeros + (size_t)qrow * N + ncol, b.zraw[f]);
+      if (ZK == MI355Q_ZP_PACKED)
+        b.zword[f] = __builtin_amdgcn_raw_buffer_load_b32(zres, (int)((qrow * (N >> 3) + (ncol8 >> 3)) * 4u + oob), 0, 0);
+      if (ZK == MI355Q_ZP_PRESCALED) buf_load_halves<NT>(zres, (qrow * N + ncol) * 2u + oob, b.zraw[f]);
     }
     if (XA) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          // rows past M repeat the last row: output rows are independent and
-          // rows >= M are never stored, so no predicated load is needed
-          b.xr[XA ? 4 * mt + s : 0] =
-              *(const u4*)(a.x + (size_t)min(16 * mt + c, a.M - 1) * K + 128 * g + 32 * s + 8 * kq);
-        }
+        for (int s = 0; s < 4; ++s)
+          b.xr[XA ? 4 * mt + s : 0] = buf_load16(xres, xlane[mt] + (uint32_t)(128 * g + 32 * s) * 2u + oob);
     }
   };
-  // activations of block g for 64-row launches (too many registers to carry a block ahead)
+  // activations of block i for launches that cannot carry them a block ahead (no registers to spare)
   struct Acts { u4 xr[XA ? 1 : MT][4]; };
-  auto load_acts = [&](Acts& x, int g) {
+  auto load_acts = [&](Acts& x, int i) {
     if (XA) return;
+    const int g = blk(i);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int row = min(16 * mt + c, a.M - 1);
-        x.xr[mt][s] = *(const u4*)(a.x + (size_t)row * K + 128 * g + 32 * s + 8 * kq);
-      }
+      for (int s = 0; s < 4; ++s) x.xr[mt][s] = buf_load16(xres, xlane[mt] + (uint32_t)(128 * g + 32 * s) * 2u);
   };
 
   auto compute_block = [&](const Block& b, const Acts& xa) {
@@ -295,11 +339,11 @@ w4a16_stream_kernel(StreamArgs a) {
 
   {
     // Two block buffers: the next K block of this wavefront is in flight while
-    // one is consumed (deeper rings were measured and are slower).  The
-    // prefetch is unconditional (past the end it re-reads a block of this
-    // wavefront) and every step leaves the loop through a plain break, so the
-    // body is straight-line code and the compiler waits for exactly the block
-    // being consumed.
+    // one is consumed (deeper rings were measured and are not faster).  The
+    // prefetch is unconditional (past the end it is a descriptor-range miss:
+    // zeros, no traffic) and every step leaves the loop through a plain break,
+    // so the body is straight-line code and the compiler waits for exactly
+    // the block being consumed.
     //
     // K order: the wavefront's nb blocks are visited starting at a
     // workgroup-dependent position.  All workgroups read the same activation
@@ -309,30 +353,21 @@ w4a16_stream_kernel(StreamArgs a) {
     // workgroup, so results stay run-to-run identical.)
     Block ring[2];
     Acts xa;
-    const int g0 = gb + wave;
-    const int nb = (ge - g0 + 3) >> 2;               // K blocks of this wavefront
     if (nb > 0) {
-      const int rot = (int)((blockIdx.x >> 3) * 5u % (unsigned)nb);
-      auto blk = [&](int i) {                        // i-th block in this workgroup's order
-        int j = i + rot;
-        if (j >= nb) j -= nb;
-        if (j >= nb) j -= nb;                        // i may run one past the end
-        return g0 + 4 * j;
-      };
-      load_block(ring[0], blk(0));
+      load_block(ring[0], 0);
       int i = 0;
       while (true) {
         // sched_barrier: keep the prefetch ahead of the arithmetic, the
         // instruction scheduler would otherwise sink the loads next to
         // their first use one iteration later
-        load_acts(xa, blk(i));
-        load_block(ring[1], blk(i + 1));
+        load_acts(xa, i);
+        load_block(ring[1], i + 1);
         __builtin_amdgcn_sched_barrier(0);
         compute_block(ring[0], xa);
         __builtin_amdgcn_sched_barrier(0);
         if (++i >= nb) break;
-        load_acts(xa, blk(i));
-        load_block(ring[0], blk(i + 1));
+        load_acts(xa, i);
+        load_block(ring[0], i + 1);
         __builtin_amdgcn_sched_barrier(0);
         compute_block(ring[1], xa);
         __builtin_amdgcn_sched_barrier(0);
@@ -341,10 +376,15 @@ w4a16_stream_kernel(StreamArgs a) {
     }
   }
 
-  // ---- reduce the 4 wavefronts through LDS; wave w finishes rows 4*kq + w ----
-  __shared__ float red[4][4 * NT][64];
+  // ---- reduce the W wavefronts through LDS.  A lane holds 4 rows (4 kq + i)
+  // x NT columns per 16-row tile; wavefront w sums and stores CW of those
+  // 4 NT values: row i = w CW / NT, columns (w CW) % NT .. + CW ----
+  constexpr int CW = 4 * NT / W > 0 ? 4 * NT / W : 1;
+  __shared__ float red[W][4 * NT][64];
   const int Mpad = 16 * MT;
-  float fin[MT][NT];
+  const bool fin_wave = wave * CW < 4 * NT;          // NT = 1 with 8 wavefronts: the upper four only contribute
+  const int q0 = fin_wave ? wave * CW : 0, ri = q0 / NT, tc = q0 % NT;
+  float fin[MT][CW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -353,16 +393,19 @@ w4a16_stream_kernel(StreamArgs a) {
       for (int i = 0; i < 4; ++i) red[wave][i * NT + t][lane] = acc[mt][t][i];
     __syncthreads();
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
-      fin[mt][t] = ((red[0][wave * NT + t][lane] + red[1][wave * NT + t][lane]) +
-                    red[2][wave * NT + t][lane]) + red[3][wave * NT + t][lane];
+    for (int t = 0; t < CW; ++t) {
+      float v = red[0][q0 + t][lane];
+#pragma unroll
+      for (int w = 1; w < W; ++w) v += red[w][q0 + t][lane];
+      fin[mt][t] = v;
+    }
     __syncthreads();
-    const int m = 16 * mt + 4 * kq + wave;
-    if (m < a.M) {
+    const int m = 16 * mt + 4 * kq + ri;
+    if (fin_wave && m < a.M) {
       if (a.splits == 1)
-        store_out_row<DT, NT>(a.out + (size_t)m * N + ncol, a.bias, ncol, fin[mt]);
+        store_out_row<DT, CW>(a.out + (size_t)m * N + ncol + tc, a.bias, ncol + tc, fin[mt]);
       else
-        store_partial<NT>(a.partial + ((size_t)split * Mpad + m) * N + ncol, fin[mt]);
+        store_partial<CW>(a.partial + ((size_t)split * Mpad + m) * N + ncol + tc, fin[mt]);
     }
   }
   if (a.splits == 1) return;
@@ -382,14 +425,14 @@ w4a16_stream_kernel(StreamArgs a) {
   if (!is_last) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = 16 * mt + 4 * kq + wave;
-    if (m >= a.M) continue;
-    float v[NT];
+    const int m = 16 * mt + 4 * kq + ri;
+    if (!fin_wave || m >= a.M) continue;
+    float v[CW];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) v[t] = 0.f;
+    for (int t = 0; t < CW; ++t) v[t] = 0.f;
     for (int sp = 0; sp < a.splits; ++sp)
-      load_partial_add<NT>(a.partial + ((size_t)sp * Mpad + m) * N + ncol, v);
-    store_out_row<DT, NT>(a.out + (size_t)m * N + ncol, a.bias, ncol, v);
+      load_partial_add<CW>(a.partial + ((size_t)sp * Mpad + m) * N + ncol + tc, v);
+    store_out_row<DT, CW>(a.out + (size_t)m * N + ncol + tc, a.bias, ncol + tc, v);
   }
   if (threadIdx.x == 0)
     __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -402,8 +445,13 @@ static void launch_spf(const StreamArgs& a, int nt, hipStream_t st) {
   dim3 grid(a.N / 128 * (8 / nt), a.splits), block(256);
 #define MQ_STREAM_LAUNCH(SPF, NT) \
   hipLaunchKernelGGL((w4a16_stream_kernel<DT, MT, ZK, SPF, NT>), grid, block, 0, st, a)
-  if (a.gs % 128 != 0) MQ_STREAM_LAUNCH(1, 8);
-  else if (nt == 8) MQ_STREAM_LAUNCH(4, 8);
+  if (a.gs % 128 != 0) {
+    // 32 scale rows per K block: callers keep these launches to 32 rows (64 rows x 8 tiles spill)
+    if constexpr (MT <= 2) MQ_STREAM_LAUNCH(1, 8);
+  }
+  else if (nt == 8) {
+    if constexpr (MT <= 2) MQ_STREAM_LAUNCH(4, 8);    // 64 rows x 8 tiles do not fit the register file
+  }
   else if (nt == 4) MQ_STREAM_LAUNCH(4, 4);
   else if (nt == 2) MQ_STREAM_LAUNCH(4, 2);
   else MQ_STREAM_LAUNCH(4, 1);
@@ -472,12 +520,17 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
   int G = K / 128;
   StreamPlan plan = w4a16_stream_auto_plan(M, K, N, group_size);
   const int force_s = split_k & 0xff, force_nt = (split_k >> 8) & 0xff;
+  MQ_REQUIRE(group_size % 128 == 0 || M <= 32, "w4a16_gemm(stream): group sizes below 128 take at most 32 rows per launch, got %d", M);
+  MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 31) && (size_t)(K / group_size) * N * 2 < ((size_t)1 << 31) &&
+                 (size_t)K * group_size < ((size_t)1 << 32),
+             "w4a16_gemm(stream): activations and scales must each stay below 2 GiB (M=%d K=%d N=%d)", M, K, N);
+  a.gs_magic = (uint32_t)((((uint64_t)1 << 32) + group_size - 1) / group_size);
   if (force_nt) {
     MQ_REQUIRE(force_nt == 1 || force_nt == 2 || force_nt == 4 || force_nt == 8,
                "w4a16_gemm: tiles per workgroup must be 1, 2, 4 or 8, got %d", force_nt);
     MQ_REQUIRE(force_nt == 8 || group_size % 128 == 0,
                "w4a16_gemm: tile groups below 8 need group_size %% 128 == 0");
-    plan.nt = force_nt;
+    plan.nt = (force_nt == 8 && M > 32) ? 4 : force_nt;
     if (!force_s) plan.splits = 1;
   }
   int splits = force_s ? force_s : plan.splits;
