@@ -245,8 +245,12 @@ w4a16_stream_kernel(StreamArgs a) {
   uint32_t xlane[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
+    // Activations are fetched with 4 consecutive lanes on 64 contiguous bytes of one row (lane =
+    // 4 * row + chunk): the MFMA wants lane 16 * chunk + row, whose neighbours sit a whole row
+    // pitch apart, and 64 single 16-byte requests per instruction cost the L1 more than the weight
+    // stream itself.  compute_block moves each register to its MFMA lane (xperm).
     // rows past M repeat the last row: output rows are independent and rows >= M are never stored
-    xlane[mt] = ((uint32_t)min(16 * mt + c, a.M - 1) * K + 8 * kq) * 2u;
+    xlane[mt] = ((uint32_t)min(16 * mt + (lane >> 2), a.M - 1) * K + 8 * (lane & 3)) * 2u;
   // block i of this wavefront's order; i >= nb loads nothing (zeros, no memory traffic)
   auto load_block = [&](Block& b, int i) {
     const bool have = i < nb;
@@ -284,6 +288,7 @@ w4a16_stream_kernel(StreamArgs a) {
       for (int s = 0; s < 4; ++s) x.xr[mt][s] = buf_load16(xres, xlane[mt] + (uint32_t)(128 * g + 32 * s) * 2u);
   };
 
+  const int xperm = 4 * (4 * c + kq);                // byte index of the lane that fetched this lane's MFMA chunk
   auto compute_block = [&](const Block& b, const Acts& xa) {
 #pragma unroll
     for (int f = 0; f < 4 / SPF; ++f) {
@@ -298,7 +303,10 @@ w4a16_stream_kernel(StreamArgs a) {
         corr[mt] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < SPF; ++s) {
-          const u4 raw = XA ? b.xr[XA ? 4 * mt + SPF * f + s : 0] : xa.xr[XA ? 0 : mt][SPF * f + s];
+          const u4 got = XA ? b.xr[XA ? 4 * mt + SPF * f + s : 0] : xa.xr[XA ? 0 : mt][SPF * f + s];
+          u4 raw;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) raw[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(xperm, (int)got[d]);
           av[mt][s] = MM::prep_a(raw);
           xs[mt] = MM::run(bitcast<vec>(raw), MM::splat(1.0f), xs[mt]);
           if (MM::kScaledA) corr[mt] = MM::run(av[mt][s], MM::splat(MM::kBase), corr[mt]);
