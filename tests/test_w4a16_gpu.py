@@ -137,6 +137,22 @@ def test_stream_gemm_exact_and_split_invariant(ops, rearrange, split_k):
     assert torch.equal(got.cpu(), want)
 
 
+def test_split_k_layers_of_different_width_share_a_workspace(ops, rearrange):
+    # one workspace serves every layer: a narrow layer's split-K partial tiles must not land on
+    # the arrival counters a wider layer uses afterwards.  The output allocation is poisoned
+    # first, so a launch that never stores (a corrupted counter) cannot pass on stale memory.
+    g = 128
+    cases = [(4, 1024, 256, 4 | (2 << 8)), (4, 1024, 2048, 2 | (1 << 8)), (4, 1024, 256, 2 | (1 << 8))]
+    for i, (M, K, N, split_k) in enumerate(cases):
+        print(f"case shared workspace M={M} K={K} N={N} split_k={split_k:#x}", flush=True)
+        q, z, s, x = make_case(40 + i, M, K, N, g, exact=True)
+        want = torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16)
+        poison = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        del poison
+        got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, split_k=split_k)
+        assert torch.equal(got.cpu(), want)
+
+
 @pytest.mark.parametrize("g", [32, 64, 128, 256, -1])
 def test_stream_gemm_group_sizes_and_bias(ops, rearrange, g):
     M, K, N = 5, 512, 128

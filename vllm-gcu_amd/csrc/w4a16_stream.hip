@@ -505,9 +505,15 @@ StreamPlan w4a16_stream_auto_plan(int M, int K, int N, int gs) {
   return p;
 }
 
+// The arrival counters own a fixed region at the start of the workspace, whatever the shape:
+// one workspace serves layers of different widths, and the counters must stay zero between
+// launches -- a width-dependent boundary would let one layer's partial tiles land on the
+// counters of a wider layer.
+static constexpr size_t STREAM_COUNTER_BYTES = (size_t)64 << 10;
+
 size_t w4a16_stream_workspace_bytes(int M, int N) {
   const int Mpad = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
-  return ((size_t)(N / 16) * sizeof(int) + 255) / 256 * 256 + (size_t)32 * Mpad * N * sizeof(float);
+  return STREAM_COUNTER_BYTES + (size_t)32 * Mpad * N * sizeof(float);
 }
 
 // split_k: bits 0..7 force the split factor, bits 8..15 the tiles per
@@ -551,7 +557,8 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
   a.counters = nullptr;
   if (splits > 1) {
     const int Mpad = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
-    size_t cbytes = ((size_t)(N / 16) * sizeof(int) + 255) / 256 * 256;
+    const size_t cbytes = STREAM_COUNTER_BYTES;
+    MQ_REQUIRE((size_t)(N / 16) * sizeof(int) <= cbytes, "w4a16_gemm(stream): N=%d needs more arrival counters than the workspace holds", N);
     size_t need = cbytes + (size_t)splits * Mpad * N * sizeof(float);
     MQ_REQUIRE(workspace && workspace_bytes >= need,
                "w4a16_gemm: workspace of %zu bytes needed for split_k=%d, got %zu", need, splits,
