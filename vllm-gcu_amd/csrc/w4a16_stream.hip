@@ -225,7 +225,7 @@ w4a16_stream_kernel(StreamArgs a) {
     uint32_t zword[4 / SPF];
     u4 xr[XA ? 4 * MT : 1];
   };
-  constexpr int W = 4;                                // wavefronts per workgroup (eight were measured: not faster)
+  constexpr int W = 4;                                // wavefronts per workgroup (8 and 16 were measured: not faster)
   // K blocks of this wavefront: gb + wave, + W, ...; visited from a
   // workgroup-dependent start (see the loop below)
   const int g0 = gb + wave;

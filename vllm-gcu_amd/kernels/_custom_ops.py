@@ -1077,6 +1077,57 @@ _register("_C", "weight_only_quant",
           _weight_only_quant_impl)
 
 
+# ---------------------------------------------------------------------------
+# fused q / kv projections (csrc/src/fused_qkv_proj.cpp:14-23,
+# fused_qkv_gemm_quant.cpp:12-20; defs torch_bindings.cpp:1204-1217)
+# ---------------------------------------------------------------------------
+# The reference forwards both straight to its vendor library and has neither a
+# Python caller nor a test nor a description of them, so their arithmetic is
+# unpinned.  They are built as what the signatures say: one quantised GEMM over
+# the merged weight whose output columns are split into ``q`` (the first
+# q.shape[-1]) and ``kv`` (the rest) -- the merged q_a / kv_a projection of an
+# MLA layer.
+def _split_qkv(q, kv, merged):
+    nq, nkv = q.shape[-1], kv.shape[-1]
+    if merged.shape[-1] != nq + nkv:
+        raise RuntimeError(f"fused qkv: weight has {merged.shape[-1]} output columns, q + kv need {nq} + {nkv}")
+    q.copy_(merged[:, :nq].reshape(q.shape))
+    kv.copy_(merged[:, nq:].reshape(kv.shape))
+
+
+def _fused_qkv_proj_impl(q, kv, x, weight, x_scale, weight_scale, group_size):
+    """fp8 block-scaled: x fp8 [.., K] with scales [.., K/128], weight fp8 [Nq + Nkv, K] with scales
+    [(Nq + Nkv)/128, K/128]; the arithmetic of linear_quant."""
+    rt.require_gpu(q, kv, x, weight, x_scale, weight_scale)
+    if x.numel() == 0:
+        return
+    if int(group_size) != 128:
+        raise RuntimeError(f"fused_qkv_proj: group_size {group_size}: the fp8 block size is 128")
+    x2 = x.reshape(-1, x.shape[-1])
+    merged = torch.empty((x2.shape[0], weight.shape[0]), dtype=q.dtype, device=q.device)
+    _linear_quant_impl(merged, x2, weight, None, x_scale, weight_scale)
+    _split_qkv(q, kv, merged)
+
+
+def _fused_qkv_gemm_quant_impl(q, kv, x, weight, scale, zeros, group_size):
+    """W4A16: the operands of gptq_gemm_gcu (int4 weight in the slab or any reference layout,
+    group scales, zeros in any of the accepted forms)."""
+    rt.require_gpu(q, kv, x, weight, scale, zeros)
+    if x.numel() == 0:
+        return
+    merged = w4a16_gemm(x.reshape(-1, x.shape[-1]), weight, scale, zeros if zeros.numel() else None, None,
+                        int(group_size))
+    _split_qkv(q, kv, merged.to(q.dtype))
+
+
+_register("_C", "fused_qkv_proj",
+          "(Tensor(a!) q, Tensor(a!) kv, Tensor x, Tensor weight, Tensor x_scale, Tensor weight_scale, "
+          "int group_size) -> ()", _fused_qkv_proj_impl)
+_register("_C", "fused_qkv_gemm_quant",
+          "(Tensor(a!) q, Tensor(a!) kv, Tensor x, Tensor weight, Tensor scale, Tensor zeros, "
+          "int group_size) -> ()", _fused_qkv_gemm_quant_impl)
+
+
 # vllm_gcu/kernels/_custom_ops.py:564-579
 def w8a8_block_fp8_matmul(A: torch.Tensor, B: torch.Tensor, As: torch.Tensor, Bs: torch.Tensor,
                           block_size: List[int], output_dtype: torch.dtype = torch.float16,
