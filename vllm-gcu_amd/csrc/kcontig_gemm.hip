@@ -104,7 +104,11 @@ __device__ __forceinline__ void s8x16_to_bf16(const u4& v, u4& lo, u4& hi) {
   hi = (u4){o[4], o[5], o[6], o[7]};
 }
 
-template <int MODE, int ODT, int MT, bool GROUPED>
+// KS (dense launches of at most 32 rows): the four wavefronts of a workgroup share one group of 64
+// columns and take its K blocks round-robin, partial sums meet in LDS.  With a single row block
+// there are only N / 64 column groups; one wavefront each leaves most of the chip idle and every
+// wavefront with the whole of K as one dependent chain of loads.
+template <int MODE, int ODT, int MT, bool GROUPED, bool KS = false>
 __global__ void __launch_bounds__(256, 1)
 kcontig_gemm_kernel(KcArgs a) {
   typedef Kc<MODE> T;
@@ -128,7 +132,7 @@ kcontig_gemm_kernel(KcArgs a) {
     for (int r = tid; r < BM; r += 256) tok[r] = a.sorted_ids[m0 + r];
     __syncthreads();
   }
-  const int n0 = blockIdx.x * 256 + wave * 64;
+  const int n0 = KS ? blockIdx.x * 64 : blockIdx.x * 256 + wave * 64;
   if (n0 >= N) return;
   const char* wbase = (const char*)a.w + expert * a.w_stride * T::WBYTES;
 
@@ -284,20 +288,59 @@ kcontig_gemm_kernel(KcArgs a) {
   };
 
   {
-    Blk b0, b1;
-    load_blk(b0, 0);
-    int kb = 0;
-    while (true) {
-      load_blk(b1, min(kb + 1, KB - 1));
-      __builtin_amdgcn_sched_barrier(0);
-      compute_blk(b0, kb);
-      __builtin_amdgcn_sched_barrier(0);
-      if (++kb >= KB) break;
-      load_blk(b0, min(kb + 1, KB - 1));
-      __builtin_amdgcn_sched_barrier(0);
-      compute_blk(b1, kb);
-      __builtin_amdgcn_sched_barrier(0);
-      if (++kb >= KB) break;
+    constexpr int kstep = KS ? 4 : 1;
+    const int kfirst = KS ? wave : 0;
+    if (kfirst < KB) {
+      const int klast = kfirst + (KB - 1 - kfirst) / kstep * kstep;   // this wavefront's last block
+      Blk b0, b1;
+      load_blk(b0, kfirst);
+      int kb = kfirst;
+      while (true) {
+        load_blk(b1, min(kb + kstep, klast));
+        __builtin_amdgcn_sched_barrier(0);
+        compute_blk(b0, kb);
+        __builtin_amdgcn_sched_barrier(0);
+        kb += kstep;
+        if (kb >= KB) break;
+        load_blk(b0, min(kb + kstep, klast));
+        __builtin_amdgcn_sched_barrier(0);
+        compute_blk(b1, kb);
+        __builtin_amdgcn_sched_barrier(0);
+        kb += kstep;
+        if (kb >= KB) break;
+      }
+    }
+  }
+
+  // KS: wavefront w sums the four partial sums of column tile w (in wavefront order) and stores it
+  __shared__ uint32_t red[KS ? 4 : 1][KS ? 16 * MT : 1][64];
+  if (KS) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) red[KS ? wave : 0][KS ? (i * MT + j) * 4 + e : 0][lane] = bitcast<u4>(acc[i][j])[e];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      u4 t;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int slot = (wave * MT + j) * 4 + e;
+        if (MODE == KC_INT8) {
+          int v = (int)red[0][KS ? slot : 0][lane];
+#pragma unroll
+          for (int w = 1; w < 4; ++w) v += (int)red[KS ? w : 0][KS ? slot : 0][lane];
+          t[e] = (uint32_t)v;
+        } else {
+          float v = bitcast<float>(red[0][KS ? slot : 0][lane]);
+#pragma unroll
+          for (int w = 1; w < 4; ++w) v += bitcast<float>(red[KS ? w : 0][KS ? slot : 0][lane]);
+          t[e] = bitcast<uint32_t>(v);
+        }
+      }
+      acc[0][j] = bitcast<acc_t>(t);
     }
   }
 
@@ -320,8 +363,8 @@ kcontig_gemm_kernel(KcArgs a) {
     float xs = 1.0f;
     if (MODE == KC_INT8 && a.a_scale) xs = a.a_scale[arow[j]];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + 16 * i + 4 * q;
+    for (int i = 0; i < (KS ? 1 : 4); ++i) {
+      const int n = n0 + 16 * (KS ? wave : i) + 4 * q;
       if (n >= N) continue;
       float v[4];
 #pragma unroll
@@ -369,6 +412,15 @@ kslab_repack_kernel(const u4* src, u4* dst, long chunks, int N, int K, int wb) {
 template <int MODE, int ODT, bool GROUPED>
 void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
   dim3 grid((a.N + 255) / 256, row_blocks), block(256);
+  if constexpr (!GROUPED) {
+    // a single row block and too few column groups to fill the chip: split K inside the workgroup
+    if (row_blocks == 1 && mt <= 2 && (a.N + 255) / 256 < 2 * device_cu_count()) {
+      dim3 gks((a.N + 63) / 64, 1);
+      if (mt == 1) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true>), gks, block, 0, st, a);
+      else hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true>), gks, block, 0, st, a);
+      return;
+    }
+  }
   switch (mt) {
     case 1: hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, GROUPED>), grid, block, 0, st, a); break;
     case 2: hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, GROUPED>), grid, block, 0, st, a); break;
