@@ -104,10 +104,10 @@ __device__ __forceinline__ void s8x16_to_bf16(const u4& v, u4& lo, u4& hi) {
   hi = (u4){o[4], o[5], o[6], o[7]};
 }
 
-// KS (dense launches of at most 32 rows): the four wavefronts of a workgroup share one group of 64
-// columns and take its K blocks round-robin, partial sums meet in LDS.  With a single row block
-// there are only N / 64 column groups; one wavefront each leaves most of the chip idle and every
-// wavefront with the whole of K as one dependent chain of loads.
+// KS (dense launches of few row blocks): the four wavefronts of a workgroup share one group of 64
+// columns and take its K blocks round-robin, partial sums meet in LDS.  With one or two row blocks
+// there are only a few hundred wavefronts of 64 columns each; that leaves most of the chip idle
+// and every wavefront with the whole of K as one dependent chain of loads.
 template <int MODE, int ODT, int MT, bool GROUPED, bool KS = false>
 __global__ void __launch_bounds__(256, 1)
 kcontig_gemm_kernel(KcArgs a) {
@@ -312,35 +312,43 @@ kcontig_gemm_kernel(KcArgs a) {
     }
   }
 
-  // KS: wavefront w sums the four partial sums of column tile w (in wavefront order) and stores it
-  __shared__ uint32_t red[KS ? 4 : 1][KS ? 16 * MT : 1][64];
+  acc_t fin[MT];
+  // KS: wavefront w sums the four partial sums of column tile w (in wavefront order) and stores
+  // it; two row tiles at a time go through LDS
+  constexpr int RJ = MT < 2 ? MT : 2;
+  __shared__ uint32_t red[KS ? 4 : 1][KS ? 16 * RJ : 1][64];
   if (KS) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int jc = 0; jc < MT; jc += RJ) {
+      if (jc) __syncthreads();
 #pragma unroll
-      for (int j = 0; j < MT; ++j)
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) red[KS ? wave : 0][KS ? (i * MT + j) * 4 + e : 0][lane] = bitcast<u4>(acc[i][j])[e];
-    __syncthreads();
+        for (int j = 0; j < RJ; ++j)
 #pragma unroll
-    for (int j = 0; j < MT; ++j) {
-      u4 t;
+          for (int e = 0; e < 4; ++e)
+            red[KS ? wave : 0][KS ? (i * RJ + j) * 4 + e : 0][lane] = bitcast<u4>(acc[i][jc + j])[e];
+      __syncthreads();
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int slot = (wave * MT + j) * 4 + e;
-        if (MODE == KC_INT8) {
-          int v = (int)red[0][KS ? slot : 0][lane];
+      for (int j = 0; j < RJ; ++j) {
+        u4 t;
 #pragma unroll
-          for (int w = 1; w < 4; ++w) v += (int)red[KS ? w : 0][KS ? slot : 0][lane];
-          t[e] = (uint32_t)v;
-        } else {
-          float v = bitcast<float>(red[0][KS ? slot : 0][lane]);
+        for (int e = 0; e < 4; ++e) {
+          const int slot = (wave * RJ + j) * 4 + e;
+          if (MODE == KC_INT8) {
+            int v = (int)red[0][KS ? slot : 0][lane];
 #pragma unroll
-          for (int w = 1; w < 4; ++w) v += bitcast<float>(red[KS ? w : 0][KS ? slot : 0][lane]);
-          t[e] = bitcast<uint32_t>(v);
+            for (int w = 1; w < 4; ++w) v += (int)red[KS ? w : 0][KS ? slot : 0][lane];
+            t[e] = (uint32_t)v;
+          } else {
+            float v = bitcast<float>(red[0][KS ? slot : 0][lane]);
+#pragma unroll
+            for (int w = 1; w < 4; ++w) v += bitcast<float>(red[KS ? w : 0][KS ? slot : 0][lane]);
+            t[e] = bitcast<uint32_t>(v);
+          }
         }
+        fin[jc + j] = bitcast<acc_t>(t);
       }
-      acc[0][j] = bitcast<acc_t>(t);
     }
   }
 
@@ -371,13 +379,13 @@ kcontig_gemm_kernel(KcArgs a) {
       for (int e = 0; e < 4; ++e) {
         if (MODE == KC_INT8) {
           const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + n + e];
-          v[e] = ((float)bitcast<i4>(acc[i][j])[e] * xs) * ws;
+          v[e] = ((float)bitcast<i4>(KS ? fin[j] : acc[i][j])[e] * xs) * ws;
         } else if ((W8H || W8B) && !GW) {
           const uint16_t raw = ((const uint16_t*)a.w_scale)[expert * a.ws_stride + n + e];
           const float ws = W8H ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw);
-          v[e] = bitcast<f4>(acc[i][j])[e] * ws;
+          v[e] = bitcast<f4>(KS ? fin[j] : acc[i][j])[e] * ws;
         } else {
-          v[e] = bitcast<f4>(acc[i][j])[e];
+          v[e] = bitcast<f4>(KS ? fin[j] : acc[i][j])[e];
         }
         v[e] *= rw;
         if (!GROUPED && a.bias) v[e] += Elem<ODT>::to_f32(((const uint16_t*)a.bias)[n + e]);
@@ -413,11 +421,15 @@ template <int MODE, int ODT, bool GROUPED>
 void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
   dim3 grid((a.N + 255) / 256, row_blocks), block(256);
   if constexpr (!GROUPED) {
-    // a single row block and too few column groups to fill the chip: split K inside the workgroup
-    if (row_blocks == 1 && mt <= 2 && (a.N + 255) / 256 < 2 * device_cu_count()) {
-      dim3 gks((a.N + 63) / 64, 1);
+    // too few workgroups to fill the chip: split K inside the workgroup
+    // (64-row launches only for one-byte weights x one-byte activations: the others run out of registers)
+    if ((mt <= 2 || MODE == KC_FP8_BLOCK || MODE == KC_INT8) &&
+        (a.N + 255) / 256 * row_blocks < 2 * device_cu_count()) {
+      dim3 gks((a.N + 63) / 64, row_blocks);
       if (mt == 1) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true>), gks, block, 0, st, a);
-      else hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true>), gks, block, 0, st, a);
+      else if (mt == 2) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true>), gks, block, 0, st, a);
+      else if constexpr (MODE == KC_FP8_BLOCK || MODE == KC_INT8)
+        hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true>), gks, block, 0, st, a);
       return;
     }
   }

@@ -187,7 +187,7 @@ def _gptq_gemm_gcu_fake(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bi
 # ---------------------------------------------------------------------------
 # W8A8 int8 (csrc/torch_bindings.cpp:734-766, 1002-1019)
 # ---------------------------------------------------------------------------
-_INT8_STREAM_MAX_M = 48      # measured on MI355X (K 8192, N 28672): 49-67 us against 94 us up to M = 32, equal at 64
+_INT8_STREAM_MAX_M = 64      # measured on MI355X (K 8192, N 28672): 40-51 us against 90 us for the MFMA tile kernel
 
 
 def _int8_weight_nk(weight: torch.Tensor):
