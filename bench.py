@@ -33,7 +33,7 @@ INT8_PEAK_TOPS = 5000.0
 # then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy of --calibrate-copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per
 # unit).  Keyed by (M, --split-k); other settings were not profiled.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 35169011}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 34011114}
 
 
 def w4a16_bytes(M, K, N, g=GROUP):
