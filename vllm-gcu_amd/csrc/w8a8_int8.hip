@@ -198,8 +198,12 @@ w8a8_int8_gemm_kernel(I8Args a) {
   auto lds_wait = [&](Frag& f) {
     // "s_waitcnt lgkmcnt(0)" with every operand register as an in/out operand
     // (each register exactly once: a duplicate would come back as a stale copy)
-    static_assert((NJ == 8 && NI == 4) || (NJ == 4 && NI == 7), "operand lists are written out");
-    if constexpr (NJ == 8) {
+    static_assert((NJ == 8 && NI == 4) || (NJ == 4 && NI == 7) || (NJ == 4 && NI == 4), "operand lists are written out");
+    if constexpr (NJ == 4 && NI == 4) {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(f.bx[0]), "+v"(f.bx[1]), "+v"(f.bx[2]), "+v"(f.bx[3]), "+v"(f.aw[0]), "+v"(f.aw[1]),
+                     "+v"(f.aw[2]), "+v"(f.aw[3]));
+    } else if constexpr (NJ == 8) {
       asm volatile("s_waitcnt lgkmcnt(0)"
                    : "+v"(f.bx[0]), "+v"(f.bx[1]), "+v"(f.bx[2]), "+v"(f.bx[3]), "+v"(f.bx[4]), "+v"(f.bx[5]),
                      "+v"(f.bx[6]), "+v"(f.bx[7]), "+v"(f.aw[0]), "+v"(f.aw[1]), "+v"(f.aw[2]), "+v"(f.aw[3]));
@@ -239,7 +243,9 @@ w8a8_int8_gemm_kernel(I8Args a) {
       }
   };
   constexpr int NM = NI * NJ;
-  static_assert(NM > 3 + 3 * (NSLOT - 1) && NM >= RE * (NJ + NI), "not enough MFMAs to spread the copies and reads");
+  // copy slots: the first after MFMA C0, then one every CE MFMAs (closer together in the narrow tile)
+  constexpr int CP0 = NM >= 24 ? 3 : 1, CPE = NM >= 24 ? 3 : 2;
+  static_assert(NM > CP0 + CPE * (NSLOT - 1) && NM >= RE * (NJ + NI), "not enough MFMAs to spread the copies and reads");
 
   // The K tiles of all the output tiles of this workgroup form one stream;
   // stream element g lives in LDS stage g % 2.  Half 0 of element g multiplies
@@ -284,7 +290,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
       const int want = tile + ahead * (int)gridDim.x;
       if (want >= total_tiles) kt = nt - 1;        // past the end: harmless re-read, never consumed
       else if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
-      half(f1, f0, st ^ 1, 0, 0, NSLOT, 3, 3, st, kt * TKB);
+      half(f1, f0, st ^ 1, 0, 0, NSLOT, CP0, CPE, st, kt * TKB);
       lds_wait(f0);
     }
 
@@ -463,6 +469,10 @@ int launch_gemm(const I8Args& a, hipStream_t st) {
   const long cus = device_cu_count(), mtiles = (a.M + TM - 1) / TM;
   const long t256 = mtiles * ((a.N + 255) / 256), t224 = mtiles * ((a.N + 223) / 224);
   const long cost256 = (t256 + cus - 1) / cus * 256, cost224 = (t224 + cus - 1) / cus * 224;
+  // a single row of tiles that leaves most CUs idle: tiles half as wide (the launch is bound by
+  // the weight stream, which then comes in over twice as many CUs)
+  const long t128 = mtiles * ((a.N + 127) / 128);
+  if (mtiles == 1 && (t224 < cost224 ? t224 : t256) * 3 <= cus * 2 && t128 > t224) return launch_tile<DT, 4, 2, 4, 4>(a, st);
   if (cost224 < cost256) return launch_tile<DT, 4, 2, 7, 4>(a, st);
   return launch_tile<DT, 2, 4, 4, 8>(a, st);
 }
