@@ -94,6 +94,18 @@ int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          int dtype, void* workspace, size_t workspace_bytes,
                          int split_k, int family, void* stream);
 
+/* fp8-e4m3 block-scaled GEMM for prefill-sized M: the arithmetic of linear_quant
+ * (csrc/src/linear_quant.cpp:16-95; vllm_gcu/kernels/quantization/fp8.py:169-205) on an MFMA
+ * tile kernel,
+ *   out[m, n] = sum_kb x_scale[m, kb] * w_scale[n / 128, kb] * (sum over K block kb of x[m, k] * w[n, k]) (+ bias[n])
+ * x is [M, K] fp8 with row stride ldx bytes and scales f32 [M, K/128]; w is [N, K] fp8 with row
+ * stride ldw bytes, or in the kslab order when ldw = 0 (see mi355q_kslab_repack), scales f32
+ * [N/128, K/128]; bias in the output dtype (f16 / bf16) or NULL.  K %% 128 == 0, N %% 128 == 0.
+ * mi355q_kcontig_gemm (quant_mode 1) computes the same and is the faster one up to about 128 rows. */
+int mi355q_fp8_block_gemm(void* out, const void* x, const void* w, const float* x_scale,
+                          const float* w_scale, const void* bias, int M, int N, int K, long ldx,
+                          long ldw, long ldo, int out_dtype, void* stream);
+
 /* ---- W8A8 int8 -------------------------------------------------------------
  * Replaces topsatenDotBiasQuant as called by cutlass_scaled_mm
  * (csrc/src/cutlass_scaled_mm.cpp:12-36) and dot_bias_quant

@@ -381,3 +381,31 @@ def test_fused_qkv_ops_equal_the_unfused_gemm_split_by_columns():
     want = ow4.w4a16_gemm(xh.float().numpy(), qw, z, sh, g)
     got = torch.cat([q, kv], dim=1).float().cpu().numpy()
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("M,K,N", [(129, 128, 128), (300, 512, 384), (513, 1024, 256), (2050, 256, 1152)])
+@pytest.mark.parametrize("kslab", [False, True])
+def test_fp8_block_gemm_tile_kernel(M, K, N, kslab, monkeypatch):
+    """linear_quant above 128 rows runs the MFMA tile kernel; checked against the oracle of the
+    block-scaled GEMM and, bit for bit, between the two weight orders."""
+    from vllm_gcu_amd.kernels import _custom_ops
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print(f"case fp8 tile M={M} K={K} N={N} kslab={kslab}", flush=True)
+    monkeypatch.setattr(_custom_ops, "_FP8_TILE_MIN_TILES", 1)      # small shapes: take the tile kernel anyway
+    rng = np.random.default_rng(M + K + N)
+    w = of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 0.5, -448, 448).astype(np.float32))
+    ws = rng.uniform(0.02, 0.1, size=(N // 128, K // 128)).astype(np.float32)
+    xq, xs = of8.per_token_group_quant_fp8(rng.standard_normal((M, K)).astype(np.float32), 128)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.bfloat16)
+    wd = dev(w).view(torch.float8_e4m3fn)
+    if kslab:
+        wd = rearrange.to_kslab(wd)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(out, dev(xq).view(torch.float8_e4m3fn), wd, bias.cuda(), dev(xs), dev(ws))
+    want = of8.block_fp8_gemm(xq, xs, w, ws) + bias.float().numpy()
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    if kslab:
+        ref = torch.empty_like(out)
+        torch.ops._C.linear_quant(ref, dev(xq).view(torch.float8_e4m3fn), dev(w).view(torch.float8_e4m3fn),
+                                  bias.cuda(), dev(xs), dev(ws))
+        assert torch.equal(out, ref)

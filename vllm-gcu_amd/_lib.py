@@ -31,6 +31,8 @@ SIGNATURES = {
     "mi355q_w8a8_int8_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                       c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_int,
                                       c_void_p]),
+    "mi355q_fp8_block_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                      c_int, c_long, c_long, c_long, c_int, c_void_p]),
     "mi355q_dynamic_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355q_silu_mul_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_void_p]),

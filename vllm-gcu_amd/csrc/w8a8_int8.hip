@@ -257,13 +257,15 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // while the epilogue of this one runs; past the last output tile the copies
   // re-read its last K tile into a stage nobody reads.
   const int nt = K / TKB;
+  // (kept in a register: read through the dispatch packet it is fetched again in every iteration)
+  const int gdim = __builtin_amdgcn_readfirstlane((int)gridDim.x);
   int tile = blockIdx.x;
   set_copy_tile(tile);
   issue(0, 0);
   issue(1, min(1, nt - 1) * TKB);
   int copy_tile = tile;
-  if (nt == 1 && tile + (int)gridDim.x < total_tiles) {      // element 1 already belongs to the next output tile
-    copy_tile = tile + gridDim.x;
+  if (nt == 1 && tile + gdim < total_tiles) {      // element 1 already belongs to the next output tile
+    copy_tile = tile + gdim;
     set_copy_tile(copy_tile);
     issue(1, 0);
   }
@@ -273,7 +275,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   read_frag(f0, 0, 0);
   lds_wait(f0);
   int g = 0;                                       // stream position of the current K tile
-  for (; tile < total_tiles; tile += gridDim.x) {
+  for (; tile < total_tiles; tile += gdim) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -287,7 +289,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
       // element g + 2: K tile (T + 2) % nt of output tile number (T + 2) / nt after this one
       int kt = T + 2, ahead = 0;
       while (kt >= nt) { kt -= nt; ++ahead; }
-      const int want = tile + ahead * (int)gridDim.x;
+      const int want = tile + ahead * gdim;
       if (want >= total_tiles) kt = nt - 1;        // past the end: harmless re-read, never consumed
       else if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
       half(f1, f0, st ^ 1, 0, 0, NSLOT, CP0, CPE, st, kt * TKB);

@@ -1023,6 +1023,12 @@ def _kcontig(out, a, w, a_scale, w_scale, bias, mode, group):
                   layout, rt.stream_ptr())
 
 
+# the MFMA tile kernel beats the weight-streaming kernel above 128 rows once its tiles fill a good part of
+# the chip (measured: K 7168 N 4096, M 512: 81 us against 60 us; M 2048: 96 us against 202 us)
+_FP8_TILE_MIN_M = 128
+_FP8_TILE_MIN_TILES = 96
+
+
 def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
     """fp8 block-scaled GEMM (linear_quant.cpp:16-95): lhs fp8 [.., K] with
     scales [.., K/128]; rhs fp8 [N, K] with scales [N/128, K/128]."""
@@ -1030,6 +1036,26 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
         return
     if lhs.dtype != torch.float8_e4m3fn or rhs.dtype != torch.float8_e4m3fn:
         raise RuntimeError("linear_quant: operands must be float8_e4m3fn")
+    M, N, K = lhs.numel() // lhs.shape[-1], rhs.shape[0], lhs.shape[-1]
+    tiles = -(-M // 256) * (N // 128)               # 256 x 128 output tiles, one workgroup each
+    if M > _FP8_TILE_MIN_M and tiles >= _FP8_TILE_MIN_TILES and N % 128 == 0 and K % 128 == 0 \
+            and out.dtype in (torch.float16, torch.bfloat16) \
+            and rhs.dim() == 2 and rhs.is_contiguous() and out.is_contiguous():
+        # prefill-sized M: the MFMA tile kernel (the weight-streaming kernel re-reads the weights per 64 rows)
+        rt.require_gpu(out, lhs, rhs, bias, lhs_scale, rhs_scale)
+        from .quantization import rearrange
+        a2 = lhs.reshape(M, K).contiguous()
+        xs = lhs_scale.to(torch.float32).reshape(M, -1).contiguous()
+        ws = rhs_scale.to(torch.float32).contiguous()
+        if tuple(xs.shape) != (M, K // 128) or tuple(ws.shape) != (N // 128, K // 128):
+            raise RuntimeError(f"linear_quant: scales {tuple(xs.shape)} / {tuple(ws.shape)} do not match "
+                               f"M={M} N={N} K={K} with 128 x 128 blocks")
+        b = None if bias is None else bias.to(out.dtype).contiguous()
+        with torch.cuda.device(lhs.device):
+            _lib.call("mi355q_fp8_block_gemm", out.data_ptr(), a2.data_ptr(), rhs.data_ptr(), xs.data_ptr(),
+                      ws.data_ptr(), rt.ptr(b), M, N, K, K, 0 if rearrange.is_kslab(rhs) else K, N,
+                      rt.dtype_code(out.dtype), rt.stream_ptr())
+        return
     _kcontig(out, lhs, rhs, lhs_scale.to(torch.float32).reshape(-1, lhs_scale.shape[-1]).contiguous(),
              rhs_scale.to(torch.float32).contiguous(), bias, _lib.Q_FP8_BLOCK, 128)
 
