@@ -247,6 +247,8 @@ def main():
         out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")
         torch.cuda.empty_cache()
         out["norm_quant"] = glue_bench(ops, dev, stream)
+        torch.cuda.empty_cache()
+        out["fp8_dense"] = fp8_dense_bench(ops, dev, stream)
     if args.sweep:
         out["sweep"] = sweep(ops, dev, stream, args)
     if args.calibrate_copy:
@@ -401,6 +403,31 @@ def glue_bench(ops, dev, stream, iters=50):
         out[name] = {"shape": [rows, K], "us": round(t * 1e6, 2), "GBps": round(nbytes / t / 1e9, 1),
                      "frac_hbm": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4)}
     return out
+
+
+def fp8_dense_bench(ops, dev, stream, iters=12):
+    """fp8 block-scaled dense linear (linear_quant), K=8192 N=28672, weights in the kslab order,
+    three copies in turn: decode (M=16, weight-streaming kernel, HBM-bound) and prefill
+    (M=2048, MFMA tile kernel)."""
+    import torch
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    K, N = 8192, 28672
+    ws_ = [rearrange.to_kslab((torch.randn(N, K, device=dev) * 0.5).to(torch.float8_e4m3fn)) for _ in range(3)]
+    wsc = torch.rand(N // 128, K // 128, device=dev) * 0.05 + 0.02
+    out = {}
+    for M in (16, 2048):
+        x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+        xq, xs = ops.per_token_group_quant_fp8(x, 128)
+        o = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        fns = [(lambda w=w: torch.ops._C.linear_quant(o, xq, w, None, xs, wsc)) for w in ws_]
+        time_graph(fns, iters, 3, stream)
+        t = time_graph(fns, iters, 0, stream) / iters
+        nbytes = N * K + M * K + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128) + 2 * M * N
+        out[f"M{M}"] = {"us": round(t * 1e6, 1), "GBps": round(nbytes / t / 1e9, 1),
+                        "frac_hbm": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
+                        "TFLOPs": round(2.0 * M * N * K / t / 1e12, 1),
+                        "frac_fp8_mfma_peak": round(2.0 * M * N * K / t / 1e12 / 5000.0, 4)}
+    return {"workload": "fp8 block-scaled dense linear K=8192 N=28672, bf16 out", **out}
 
 
 def sweep(ops, dev, stream, args):
