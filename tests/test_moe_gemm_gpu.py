@@ -192,6 +192,21 @@ def test_dense_block_fp8_and_w8a16(ops):
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("M", [1, 5, 17, 33])
+def test_dense_w8a16_ragged_width_splits_k_inside_the_workgroup(ops, M):
+    # few rows and a width that is no multiple of 64 (row-major weights): the launch splits K over
+    # the wavefronts of a workgroup, the last column group is partly outside the matrix
+    rng = np.random.default_rng(50 + M)
+    K, N = 640, 100
+    print(f"case dense w8a16 ragged M={M} K={K} N={N}", flush=True)
+    w8 = rng.integers(-128, 128, size=(N, K), dtype=np.int8)
+    s16 = rng.uniform(0.001, 0.01, N).astype(np.float16)
+    xh = rng.standard_normal((M, K)).astype(np.float16)
+    out = ops.gptq_gemm_gcu(dev(xh), dev(w8), torch.empty(0, device="cuda"), dev(s16), torch.empty(0, device="cuda"), 8, None, -1)
+    want = o8.weight_only_int8(xh, w8, s16, -1)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("dtype,shape", [(np.uint8, (3, 128, 256)), (np.uint16, (2, 64, 384)), (np.uint8, (192, 128))])
 def test_kslab_repack_bit_exact(rearrange, dtype, shape):
     print(f"case kslab repack {dtype.__name__} {shape}", flush=True)
