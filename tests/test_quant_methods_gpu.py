@@ -409,3 +409,35 @@ def test_fp8_block_gemm_tile_kernel(M, K, N, kslab, monkeypatch):
         torch.ops._C.linear_quant(ref, dev(xq).view(torch.float8_e4m3fn), dev(w).view(torch.float8_e4m3fn),
                                   bias.cuda(), dev(xs), dev(ws))
         assert torch.equal(out, ref)
+
+
+def test_fp8_full_size_layer_tile_kernel_against_streaming_kernel(monkeypatch):
+    """K = 8192, N = 28672, 300 rows: the MFMA tile kernel and the weight-streaming kernel are
+    independent implementations of the same block-scaled sum; they must agree to fp32
+    accumulation-order accuracy, and sampled entries must match the oracle."""
+    from vllm_gcu_amd.kernels import _custom_ops
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print("case fp8 full size tile vs streamer", flush=True)
+    M, K, N = 300, 8192, 28672
+    g = torch.Generator(device="cuda").manual_seed(5)
+    w = (torch.randn(N, K, device="cuda", generator=g) * 0.5).to(torch.float8_e4m3fn)
+    ws = torch.rand(N // 128, K // 128, device="cuda", generator=g) * 0.05 + 0.02
+    x = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    xq, xs = _custom_ops.per_token_group_quant_fp8(x, 128)
+    wk = rearrange.to_kslab(w)
+    tile = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(tile, xq, wk, None, xs, ws)
+    monkeypatch.setattr(_custom_ops, "_FP8_TILE_MIN_M", 1 << 30)
+    stream = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(stream, xq, wk, None, xs, ws)
+    d = (tile.float() - stream.float()).abs()
+    scale = stream.float().abs().max().item()
+    assert d.max().item() <= 2 ** -7 * scale + 1e-3          # one bf16 ulp of the largest output
+    rows = np.array([0, 150, 299])
+    cols = np.random.default_rng(1).integers(0, N, size=48)
+    want = of8.block_fp8_gemm(xq.view(torch.uint8)[rows].cpu().numpy(), xs[rows].cpu().numpy(),
+                              w.view(torch.uint8).cpu().numpy()[np.concatenate([np.arange(c // 128 * 128, c // 128 * 128 + 128) for c in cols])],
+                              np.repeat(ws.cpu().numpy()[cols // 128], 1, axis=0))
+    want = want.reshape(3, len(cols), 128)[:, np.arange(len(cols)), cols % 128]
+    got = tile[rows][:, cols].float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))

@@ -80,7 +80,7 @@ def test_int8_gemm_accumulators_bit_exact_both_layouts(ops, M, K, N):
 @pytest.mark.parametrize("M,K,N", [(1, 128, 64), (33, 384, 320), (300, 1024, 448), (513, 2048, 1024)])
 def test_int8_gemm_kslab_weights(ops, M, K, N):
     """Weights re-ordered by rearrange.to_kslab: the MFMA tile kernel reads them in place (raw
-    accumulators bit-exact), and up to 48 rows the operator switches to the weight-streaming kernel,
+    accumulators bit-exact), and up to 64 rows the operator switches to the weight-streaming kernel,
     whose outputs must equal the tile kernel's on row-major weights bit for bit."""
     from vllm_gcu_amd.kernels.quantization import rearrange
     print(f"case i8 kslab {M}x{K}x{N}", flush=True)
@@ -101,6 +101,39 @@ def test_int8_gemm_kslab_weights(ops, M, K, N):
         assert torch.equal(a, r)
         wantf = o8.scaled_mm_epilogue(want, xs, ws, None if b is None else b.float().cpu().numpy())
         np.testing.assert_allclose(a.float().cpu().numpy(), wantf, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("M", [16, 64, 200])
+def test_int8_full_size_layer_three_kernels_agree_bit_for_bit(ops, M):
+    """K = 8192, N = 28672 (the Llama-3-70B MLP layer of the config): the weight-streaming kernel
+    (kslab weights, M <= 64), the MFMA tile kernel on kslab weights and the MFMA tile kernel on
+    row-major weights are three independent paths over the same int32 sums and epilogue; their
+    outputs must be identical, and sampled entries must match the oracle."""
+    from vllm_gcu_amd.kernels import _custom_ops
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print(f"case i8 full size M={M}", flush=True)
+    K, N = 8192, 28672
+    g = torch.Generator(device="cuda").manual_seed(M)
+    w = torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+    x = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda", generator=g)
+    xs = torch.rand(M, 1, device="cuda", generator=g) * 0.01 + 0.001
+    ws = torch.rand(N, device="cuda", generator=g) * 0.02 + 0.001
+    wk = rearrange.to_kslab(w)
+    a = ops.cutlass_scaled_mm(x, wk.t(), xs, ws, torch.float16, None)          # streaming kernel up to 64 rows
+    r = ops.cutlass_scaled_mm(x, w.t(), xs, ws, torch.float16, None)           # tile kernel, row-major
+    limit = _custom_ops._INT8_STREAM_MAX_M
+    try:
+        _custom_ops._INT8_STREAM_MAX_M = 0
+        t = ops.cutlass_scaled_mm(x, wk.t(), xs, ws, torch.float16, None)      # tile kernel, kslab
+    finally:
+        _custom_ops._INT8_STREAM_MAX_M = limit
+    assert torch.equal(a, r) and torch.equal(t, r)
+    rows = np.array([0, M // 2, M - 1])
+    cols = np.random.default_rng(M).integers(0, N, size=64)
+    acc = x[rows].cpu().numpy().astype(np.int64) @ w[cols].cpu().numpy().astype(np.int64).T
+    want = (acc.astype(np.float32) * xs[rows].cpu().numpy()) * ws[cols].cpu().numpy()[None, :]
+    got = r[rows][:, cols].float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
