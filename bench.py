@@ -242,6 +242,8 @@ def main():
     if args.moe:
         out["moe_w4a16"] = moe_bench(ops, dev, stream, "w4a16")
         torch.cuda.empty_cache()
+        out["moe_w4a16_decode"] = moe_bench(ops, dev, stream, "w4a16", tokens=16)
+        torch.cuda.empty_cache()
         out["moe_fp8_block"] = moe_bench(ops, dev, stream, "fp8")
         torch.cuda.empty_cache()
         out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")

@@ -30,6 +30,13 @@ struct StreamArgs {
   int splits;
   float* partial;    // [splits][16*MT][N]
   int* counters;     // one per blockIdx.x (<= N/16), zero between launches
+  // grouped (fused-MoE) launches: blockIdx.z = block of 16 sorted token slots, all of one expert
+  const int32_t* sorted_ids;    // [.. padded ..] slot ids, pads >= numel
+  const int32_t* expert_ids;    // [blocks]
+  const int32_t* npp;           // device scalar: slots after padding
+  const float* topk_weights;    // [numel] or null
+  int numel, topk;
+  long w_stride, s_stride, z_stride;   // per expert, in elements of the respective arrays (weights: 16-byte units)
 };
 
 // (a & mask) | orv.  Callers launder `mask` into an SGPR and `orv` into a VGPR
@@ -184,11 +191,24 @@ __device__ __forceinline__ void buf_load_halves(rsrc_t r, uint32_t off, uint32_t
   else dst[0] = __builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0);
 }
 
-template <int DT, int MT, int ZK, int SPF, int NT>
+// GR: fused-MoE grouped launch -- the 16 MT rows of a workgroup are the token slots of block
+// blockIdx.z (gathered from x by slot id / topk, scattered to out by slot id, optionally times the
+// routing weight) and the weights are those of the block's expert.  The same stream as a dense
+// decode launch: a decode-sized MoE layer is bound by the experts' weights in exactly the same way.
+template <int DT, int MT, int ZK, int SPF, int NT, bool GR = false>
 __global__ void __launch_bounds__(256, (MT == 1 || (MT == 2 && NT <= 4)) ? 2 : 1)
 w4a16_stream_kernel(StreamArgs a) {
   typedef Mma<DT> MM;
   typedef typename MM::vec vec;
+  static_assert(!GR || MT <= 2, "grouped launches take blocks of 16 or 32 slots");
+  if (GR) {
+    if ((int)blockIdx.z * 16 * MT >= *a.npp) return;
+    const long e = a.expert_ids[blockIdx.z];
+    a.qw += e * a.w_stride;
+    a.scales += e * a.s_stride;
+    if (ZK == MI355Q_ZP_PACKED) a.zeros = (const uint32_t*)a.zeros + e * a.z_stride;
+    if (ZK == MI355Q_ZP_PRESCALED) a.zeros = (const uint16_t*)a.zeros + e * a.z_stride;
+  }
   // the wavefront index is made visibly uniform: K-block indices and loop control then live in scalar registers
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, kq = lane >> 4;
@@ -250,6 +270,11 @@ w4a16_stream_kernel(StreamArgs a) {
     // pitch apart, and 64 single 16-byte requests per instruction cost the L1 more than the weight
     // stream itself.  compute_block moves each register to its MFMA lane (xperm).
     // rows past M repeat the last row: output rows are independent and rows >= M are never stored
+    if (GR) {
+      // slot id -> row of x (pads repeat the last valid slot: their results are never stored)
+      const int id = a.sorted_ids[(int)blockIdx.z * 16 * MT + 16 * mt + (lane >> 2)];
+      xlane[mt] = ((uint32_t)(min(id, a.numel - 1) / a.topk) * K + 8 * (lane & 3)) * 2u;
+    } else
     xlane[mt] = ((uint32_t)min(16 * mt + (lane >> 2), a.M - 1) * K + 8 * (lane & 3)) * 2u;
   // block i of this wavefront's order; i >= nb loads nothing (zeros, no memory traffic)
   auto load_block = [&](Block& b, int i) {
@@ -409,6 +434,20 @@ w4a16_stream_kernel(StreamArgs a) {
     }
     __syncthreads();
     const int m = 16 * mt + 4 * kq + ri;
+    if (GR) {
+      if (fin_wave) {
+        const int id = a.sorted_ids[(int)blockIdx.z * 16 * MT + m];
+        if (id < a.numel) {
+          if (a.topk_weights) {
+            const float rw = a.topk_weights[id];
+#pragma unroll
+            for (int t = 0; t < CW; ++t) fin[mt][t] *= rw;
+          }
+          store_out_row<DT, CW>(a.out + (size_t)id * N + ncol + tc, nullptr, ncol + tc, fin[mt]);
+        }
+      }
+      continue;
+    }
     if (fin_wave && m < a.M) {
       if (a.splits == 1)
         store_out_row<DT, CW>(a.out + (size_t)m * N + ncol + tc, a.bias, ncol + tc, fin[mt]);
@@ -416,7 +455,7 @@ w4a16_stream_kernel(StreamArgs a) {
         store_partial<CW>(a.partial + ((size_t)split * Mpad + m) * N + ncol + tc, fin[mt]);
     }
   }
-  if (a.splits == 1) return;
+  if (GR || a.splits == 1) return;
 
   // ---- cross-workgroup split-K ---------------------------------------------
   // Partial tiles travel as device-scope relaxed accesses (they bypass the
@@ -572,6 +611,70 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
   if (dtype == MI355Q_F16) launch_mt<MI355Q_F16>(a, zeros_kind, plan.nt, st);
   else launch_mt<MI355Q_BF16>(a, zeros_kind, plan.nt, st);
   MQ_LAUNCH_CHECK("w4a16_gemm(stream)");
+  return 0;
+}
+
+// Fused-MoE grouped GEMM for blocks of 16 or 32 slots (decode-sized token counts): one launch over
+// (tile groups, blocks); K is never split, so there is no workspace.
+template <int DT, int ZK>
+static void launch_grouped_nt(const StreamArgs& a, int mt, int nt, int blocks, hipStream_t st) {
+  dim3 grid(a.N / 128 * (8 / nt), 1, blocks), block(256);
+#define MQ_GR_LAUNCH(MT, NT) hipLaunchKernelGGL((w4a16_stream_kernel<DT, MT, ZK, 4, NT, true>), grid, block, 0, st, a)
+  if (mt == 1) {
+    if (nt == 8) MQ_GR_LAUNCH(1, 8);
+    else if (nt == 4) MQ_GR_LAUNCH(1, 4);
+    else MQ_GR_LAUNCH(1, 2);
+  } else {
+    if (nt == 8) MQ_GR_LAUNCH(2, 8);
+    else if (nt == 4) MQ_GR_LAUNCH(2, 4);
+    else MQ_GR_LAUNCH(2, 2);
+  }
+#undef MQ_GR_LAUNCH
+}
+
+int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                                const void* zeros, int zeros_kind, const float* topk_weights,
+                                const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
+                                int numel, int topk, int block_size, int max_blocks, int K, int N,
+                                int group_size, int dtype, hipStream_t st) {
+  MQ_REQUIRE(block_size == 16 || block_size == 32, "moe_w4a16(stream): blocks of 16 or 32 slots, got %d", block_size);
+  const int mt = block_size / 16;
+  MQ_REQUIRE(group_size % 128 == 0 && K % 128 == 0 && N % 128 == 0,
+             "moe_w4a16(stream): K=%d, N=%d and group_size=%d must be multiples of 128", K, N, group_size);
+  const int rows = numel / (topk > 0 ? topk : 1) + 1;
+  MQ_REQUIRE((size_t)rows * K * 2 < ((size_t)1 << 31) && (size_t)(K / group_size) * N * 2 < ((size_t)1 << 31) &&
+                 (size_t)K * group_size < ((size_t)1 << 32),
+             "moe_w4a16(stream): activations and one expert's scales must each stay below 2 GiB (K=%d N=%d)", K, N);
+  StreamArgs a = {};
+  a.out = (uint16_t*)out;
+  a.x = (const uint16_t*)x;
+  a.qw = (const u4*)qweight;
+  a.scales = (const uint16_t*)scales;
+  a.zeros = zeros;
+  a.bias = nullptr;
+  a.M = (numel + topk - 1) / topk;                 // rows of x
+  a.K = K; a.N = N; a.gs = group_size;
+  a.gs_magic = (uint32_t)((((uint64_t)1 << 32) + group_size - 1) / group_size);
+  a.splits = 1;
+  a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
+  a.numel = numel; a.topk = topk;
+  a.w_stride = (long)(K / 8) * N / 4;
+  a.s_stride = (long)(K / group_size) * N;
+  a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
+  // tiles per workgroup: all eight of a slab unless that leaves the chip short of workgroups
+  const int slabs = N / 128, cus = device_cu_count();
+  int nt = 8;
+  while (nt > 2 && (long)slabs * (8 / nt) * max_blocks < 2L * cus) nt >>= 1;
+#define MQ_GR_ZK(DT)                                                                          \
+  do {                                                                                        \
+    if (zeros_kind == MI355Q_ZP_NONE) launch_grouped_nt<DT, MI355Q_ZP_NONE>(a, mt, nt, max_blocks, st);    \
+    else if (zeros_kind == MI355Q_ZP_PACKED) launch_grouped_nt<DT, MI355Q_ZP_PACKED>(a, mt, nt, max_blocks, st); \
+    else launch_grouped_nt<DT, MI355Q_ZP_PRESCALED>(a, mt, nt, max_blocks, st);               \
+  } while (0)
+  if (dtype == MI355Q_F16) MQ_GR_ZK(MI355Q_F16);
+  else MQ_GR_ZK(MI355Q_BF16);
+#undef MQ_GR_ZK
+  MQ_LAUNCH_CHECK("moe_w4a16(stream)");
   return 0;
 }
 

@@ -548,6 +548,12 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   return 0;
 }
 
+int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
+                                const void* zeros, int zeros_kind, const float* topk_weights,
+                                const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
+                                int numel, int topk, int block_size, int max_blocks, int K, int N,
+                                int group_size, int dtype, hipStream_t st);
+
 int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                          const float* scales_f32, const float* out_scale,
                          const void* zeros, int zeros_kind, const float* topk_weights,
@@ -559,6 +565,12 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
              "moe_w4a16: activation matrix of %d rows x %d is 4 GiB or more", numel / (topk > 0 ? topk : 1), K);
   MQ_REQUIRE(block_size == 16 || block_size == 32 || block_size == 64 || block_size == 128,
              "moe_w4a16: block_size=%d must be 16, 32, 64 or 128", block_size);
+  // blocks of 16 or 32 slots (decode-sized token counts): the layer is bound by the experts' weights,
+  // which the streaming kernel reads faster than the MFMA tile kernel with one or two row tiles
+  if (block_size <= 32 && !scales_f32 && !out_scale)
+    return w4a16_stream_grouped_launch(out, x, qweight, scales, zeros, zeros_kind, topk_weights, sorted_ids,
+                                       expert_ids, npp, numel, topk, block_size, max_blocks, K, N, group_size,
+                                       dtype, st);
   TileArgs a = {};
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;

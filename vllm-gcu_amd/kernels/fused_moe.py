@@ -23,8 +23,8 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
     per_expert = (M * topk) / max(E, 1)
     if per_expert <= 16:
         bm = 16
-    elif per_expert <= 32:
-        bm = 32
+    elif per_expert <= 28:      # measured on the Mixtral-8x7B W4A16 layer: at 32 rows per expert on average
+        bm = 32                 # half of the experts already need a second block of 32
     else:
         bm = 64
     return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
