@@ -93,9 +93,12 @@ def test_grouped_w4a16_both_gemms(fmoe, rearrange, block, dtype):
     np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
 
 
-def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe):
+@pytest.mark.parametrize("block", [16, 32, 64])
+def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe, block):
     # what the reference's moe_wna16 loader leaves on the layer: uint8 [E, N, K/2]
     # half-group bytes (moe_wna16.py:464-466) and fp16 zeros = z * scales
+    # (blocks of 16 / 32 slots run the weight-streaming kernel, 64 the MFMA tile kernel)
+    print(f"case grouped w4a16 reference layout block={block}", flush=True)
     rng = np.random.default_rng(5)
     M, E, T, K, N = 20, 3, 2, 256, 256
     q, z, s = make_int4_experts(rng, E, K, N)
@@ -104,9 +107,16 @@ def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe):
     x = rng.standard_normal((M, K)).astype(np.float16)
     tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
     C = torch.empty((M, T, N), dtype=torch.float16, device="cuda")
-    run_grouped(fmoe, dev(x), dev(rw), C, None, dev(s), dev(zs), dev(tw), dev(ids), E, 64, False, T,
+    run_grouped(fmoe, dev(x), dev(rw), C, None, dev(s), dev(zs), dev(tw), dev(ids), E, block, False, T,
                 use_int4_w4a16=True, block_shape=[0, 128])
     want = om.fused_moe_gemm(x.astype(np.float32), lambda e: ow4.dequantize_prescaled_zeros(q[e], zs[e], s[e], 128), ids, T)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # symmetric experts: no zero-point tensor, implicit zero 8
+    C = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
+    run_grouped(fmoe, dev(x), dev(rw), C, None, dev(s), None, dev(tw), dev(ids), E, block, False, T,
+                use_int4_w4a16=True, block_shape=[0, 128])
+    z8 = np.full_like(z, 8)
+    want = om.fused_moe_gemm(x.astype(np.float32), lambda e: ow4.dequantize(q[e], z8[e], s[e].astype(np.float32), 128), ids, T)
     np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
