@@ -103,6 +103,19 @@ def test_int8_gemm_kslab_weights(ops, M, K, N):
         np.testing.assert_allclose(a.float().cpu().numpy(), wantf, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("M,N", [(2305, 2048), (4200, 1792), (2049, 4096)])
+def test_int8_gemm_more_than_eight_row_tiles(ops, M, N):
+    # above 2048 rows the XCD-aware tile order walks the row tiles in chunks of eight (with a
+    # shorter last chunk): every output tile must still be visited exactly once
+    print(f"case i8 many row tiles {M}x{N}", flush=True)
+    K = 128
+    rng = np.random.default_rng(M + N)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    acc = ops.int8_gemm_accumulators(dev(x), dev(w_nk).t())
+    assert np.array_equal(acc.cpu().numpy(), o8.int8_gemm_i32(x, np.ascontiguousarray(w_nk.T)))
+
+
 @pytest.mark.parametrize("M", [16, 64, 200])
 def test_int8_full_size_layer_three_kernels_agree_bit_for_bit(ops, M):
     """K = 8192, N = 28672 (the Llama-3-70B MLP layer of the config): the weight-streaming kernel

@@ -63,13 +63,26 @@ fp8_block_gemm_kernel(F8Args a) {
   const int M = a.M, N = a.N, K = a.K, KB = K >> 7;
 
   const int mtiles = (M + FTM - 1) / FTM;
-  const int total_tiles = mtiles * (N / FTN);
+  const int ntiles_n = N / FTN;
+  const int total_tiles = mtiles * ntiles_n;
   auto tile_origin = [&](int tile, int& m0, int& n0) {
     int tm, tn;
     if (a.n_panels_swizzle) {
+      // XCD x takes the weight panels tn = x, x + 8, ...; it sweeps them for a chunk of 8 row tiles
+      // (2048 rows of x: what its L2 can keep warm next to a panel) before the next chunk
       const int x = tile & 7, j = tile >> 3;
-      tm = j % mtiles;
-      tn = (j / mtiles) * 8 + x;
+      const int P = ntiles_n >> 3, full = (mtiles >> 3) << 3;           // panels per XCD, row tiles in whole chunks
+      int tj;
+      if (j < full * P) {
+        const int c = j / (8 * P), r = j - c * 8 * P;
+        tj = r >> 3;
+        tm = c * 8 + (r & 7);
+      } else {
+        const int rem = mtiles - full, r = j - full * P;
+        tj = r / rem;
+        tm = full + r % rem;
+      }
+      tn = tj * 8 + x;
     } else {
       tm = tile % mtiles;
       tn = tile / mtiles;
