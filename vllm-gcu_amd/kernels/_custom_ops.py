@@ -474,10 +474,17 @@ def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: i
     M = gating_output.shape[0]
     topk_weights = torch.empty(M, topk, dtype=torch.float32, device=gating_output.device)
     topk_ids = torch.empty(M, topk, dtype=torch.int32, device=gating_output.device)
-    token_expert_indices = torch.empty(M, topk, dtype=torch.int32, device=gating_output.device)
-    topk_softmax(topk_weights, topk_ids, token_expert_indices, gating_output.float())
-    if renormalize:
-        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+    rt.require_gpu(gating_output)
+    if gating_output.numel() == 0:
+        return topk_weights, topk_ids
+    # one launch: the kernel reads f16 / bf16 / f32 logits as they are and divides by the row sum
+    # itself (the reference's caller does both in separate PyTorch kernels)
+    g = gating_output.contiguous()
+    if g.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        g = g.float()
+    with torch.cuda.device(g.device):
+        _lib.call("mi355q_topk_softmax", topk_weights.data_ptr(), topk_ids.data_ptr(), None, g.data_ptr(),
+                  M, g.shape[1], topk, int(bool(renormalize)), rt.dtype_code(g.dtype), rt.stream_ptr())
     return topk_weights, topk_ids
 
 
@@ -536,7 +543,15 @@ def _leading_rows_to_flat(t: torch.Tensor, size: torch.Tensor) -> torch.Tensor:
     size = size.to(torch.int32)
     lead = t.shape[0]
     inner = (t.numel() // t.shape[-1]) // max(lead, 1)
-    return size * inner if inner != 1 else size
+    if inner == 1:
+        return size
+    # the product is kept on the count tensor (one tiny kernel less per call for counts that live
+    # across calls, like the cached token counts of prepare_finalize); redone if it was written since
+    hit = getattr(size, "_mi355q_scaled", None)
+    if hit is None or hit[0] != (size._version, inner):
+        hit = ((size._version, inner), size * inner)
+        size._mi355q_scaled = hit
+    return hit[1]
 
 
 def _silu_and_mul_pad_impl(out, input, size):

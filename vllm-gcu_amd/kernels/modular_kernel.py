@@ -28,7 +28,8 @@ class FusedMoEModularKernel(torch.nn.Module):
                 a1_scale_rec: Optional[torch.Tensor] = None,
                 a2_scale_rec: Optional[torch.Tensor] = None) -> torch.Tensor:
         a1 = hidden_states
-        output = a1 if inplace else torch.zeros_like(a1)
+        # every element is written by finalize (a copy or the shared experts' output plus an add)
+        output = a1 if inplace else torch.empty_like(a1)
         if a1.numel() == 0:
             return output
         fe = self.fused_experts
@@ -42,7 +43,11 @@ class FusedMoEModularKernel(torch.nn.Module):
                                                                          global_num_experts, E)
         workspace13 = torch.empty(ws13_shape, device=a1.device, dtype=ws_dtype)
         workspace2 = torch.empty(ws2_shape, device=a1.device, dtype=ws_dtype)
-        fused_out = torch.empty(out_shape, device=a1.device, dtype=a1.dtype)
+        # without shared experts the experts' final sum can land in the output directly: a1 is last
+        # read by the first GEMM, long before that sum is written
+        direct = (getattr(self.prepare_finalize, "shared_experts", None) is None and shared_output is None
+                  and tuple(out_shape) == tuple(output.shape) and output.is_contiguous())
+        fused_out = output if direct else torch.empty(out_shape, device=a1.device, dtype=a1.dtype)
         fe.apply(fused_out, a1q, w1, w2, topk_weights, topk_ids, activation, global_num_experts, expert_map,
                  w1_scale, w2_scale, w1_zp, w2_zp, a1q_scale, a2_scale, workspace13, workspace2,
                  expert_num_tokens, apply_router_weight_on_input, a1_scale_rec, a2_scale_rec)

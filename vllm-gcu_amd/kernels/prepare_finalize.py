@@ -26,6 +26,22 @@ def moe_kernel_quantize_input(A: torch.Tensor, A_scale: Optional[torch.Tensor], 
     return A, A_scale
 
 
+_TOKEN_COUNTS = {}
+
+
+def _token_count(n: int, device: torch.device) -> torch.Tensor:
+    """Device scalar ``int32 [1]`` holding ``n``: one per (device, value), never written again
+    (a fresh ``torch.full`` per forward is a kernel launch of its own)."""
+    key = (device.type, device.index, int(n))
+    t = _TOKEN_COUNTS.get(key)
+    if t is None:
+        if len(_TOKEN_COUNTS) > 4096:
+            _TOKEN_COUNTS.clear()
+        t = torch.full((1,), int(n), dtype=torch.int32, device=device)
+        _TOKEN_COUNTS[key] = t
+    return t
+
+
 class MoEPrepareAndFinalizeNoEP:
 
     def __init__(self):
@@ -56,7 +72,7 @@ class MoEPrepareAndFinalizeNoEP:
             a1q, a1q_scale = moe_kernel_quantize_input(a1, a1_scale, quant_config.quant_dtype,
                                                        quant_config.per_act_token_quant,
                                                        quant_config.block_shape)
-        total_tokens = torch.full((1,), a1.shape[0], dtype=torch.int32, device=a1.device)
+        total_tokens = _token_count(a1.shape[0], a1.device)
         shared_output = None
         if self.shared_experts is not None:
             shared_output = self.shared_experts(a1)
@@ -64,7 +80,8 @@ class MoEPrepareAndFinalizeNoEP:
 
     def finalize(self, output, fused_expert_output, topk_weights, topk_ids, apply_router_weight_on_input) -> None:
         if self.shared_experts is None:
-            output.copy_(fused_expert_output)
+            if fused_expert_output is not output:          # the experts may have written into it directly
+                output.copy_(fused_expert_output)
         else:
             fused_expert_output.mul_(self.routed_scaling_factor)
             output.add_(fused_expert_output)
