@@ -414,7 +414,7 @@ def test_fused_experts_fp8_block_sequence(ops, fmoe):
 
 
 def test_config3_full_size_properties_and_sample(ops, rearrange):
-    # BASELINE config 3: 512 tokens, hidden 4096, 8 experts, intermediate 14336, top-2, int4 g=128
+    # benchmark configuration 3: 512 tokens, hidden 4096, 8 experts, intermediate 14336, top-2, int4 g=128
     print("case config3", flush=True)
     M, E, T, H, I = 512, 8, 2, 4096, 14336
     g = torch.Generator().manual_seed(0)

@@ -165,7 +165,7 @@ def test_stream_gemm_group_sizes_and_bias(ops, rearrange, g):
 
 
 def test_config0_full_size_and_determinism(ops, rearrange):
-    # BASELINE config 0: x f16 [16, 4096], int4 [4096, 4096], g = 128
+    # benchmark configuration 0: x f16 [16, 4096], int4 [4096, 4096], g = 128
     M, K, N, g = 16, 4096, 4096, 128
     print("case config0", flush=True)
     q, z, s, x = make_case(0, M, K, N, g)

@@ -183,7 +183,7 @@ def test_dot_bias_quant_single_scale(ops):
 
 
 def test_config2_full_size_sampled_rows(ops):
-    # BASELINE config 2: x f16 [2048, 8192] -> per-token int8; W int8 [8192, 28672];
+    # benchmark configuration 2: x f16 [2048, 8192] -> per-token int8; W int8 [8192, 28672];
     # int32 accumulate bit-exact.  The oracle checks 96 rows spread over every
     # 256-row tile, all 28672 columns.
     M, K, N = 2048, 8192, 28672

@@ -4,7 +4,7 @@ Mirrors vllm_gcu/kernels/quantization/utils.py:10-13
 (``register_gcu_quantization_config``): configs are registered under
 ``<name>_gcu`` and HF ``quant_method`` names are overridden to them.  vLLM is
 not imported; a deployment wires ``QUANTIZATION_METHODS`` into vLLM's own
-registry.
+registry (``register_quantization_config`` for each entry).
 """
 QUANTIZATION_METHODS = {}
 
