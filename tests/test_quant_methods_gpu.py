@@ -442,3 +442,20 @@ def test_fp8_full_size_layer_tile_kernel_against_streaming_kernel(monkeypatch):
     want = want.reshape(3, len(cols), 128)[:, np.arange(len(cols)), cols % 128]
     got = tile[rows][:, cols].float().cpu().numpy()
     np.testing.assert_allclose(got, want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+
+
+@pytest.mark.parametrize("M", [65, 100, 128])
+def test_fp8_dense_65_to_128_rows_single_block(M):
+    """65..128 rows of the fp8 block-scaled linear run as one 128-row block of the weight-streaming
+    kernel with K split over the workgroup's wavefronts."""
+    print(f"case fp8 dense 128-row block M={M}", flush=True)
+    rng = np.random.default_rng(M)
+    K, N = 1024, 384
+    w = of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 0.5, -448, 448).astype(np.float32))
+    ws = rng.uniform(0.02, 0.1, size=(N // 128, K // 128)).astype(np.float32)
+    xq, xs = of8.per_token_group_quant_fp8(rng.standard_normal((M, K)).astype(np.float32), 128)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(out, dev(xq).view(torch.float8_e4m3fn), dev(w).view(torch.float8_e4m3fn), None,
+                              dev(xs), dev(ws))
+    want = of8.block_fp8_gemm(xq, xs, w, ws)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
