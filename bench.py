@@ -126,6 +126,46 @@ def cpu_baseline_w4a16(M, target_s=12.0):
                       f"four layers at M={M}; {tot_t:.1f} s of CPU work"}
 
 
+def device_report(dev):
+    """Peaks re-derived from what the device reports, beside the published ones the fractions use:
+    matrix peak = compute units x core clock x dense MFMA operations per unit and clock (4096 for
+    fp16 / bf16, 8192 for fp8 / int8 on CDNA4), HBM peak = 2 x memory clock x bus width."""
+    import torch
+    p = torch.cuda.get_device_properties(dev)
+    cus, ghz = p.multi_processor_count, getattr(p, "clock_rate", 0) / 1e6
+    if not ghz:
+        # the runtime reports no clock here: take the GPU agent's "Max Clock Freq. (MHz)" of rocminfo
+        import re
+        import subprocess
+        try:
+            txt = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=30).stdout
+            for agent in txt.split("*******")[1:]:
+                if re.search(r"Device Type:\s+GPU", agent):
+                    m = re.search(r"Max Clock Freq\. \(MHz\):\s*(\d+)", agent)
+                    if m:
+                        ghz = int(m.group(1)) / 1e3
+                        break
+        except (OSError, subprocess.SubprocessError):
+            pass
+    rep = {"name": p.name, "arch": getattr(p, "gcnArchName", ""), "compute_units": cus, "core_clock_GHz": round(ghz, 3),
+           "hbm_GiB": round(p.total_memory / 2**30, 1),
+           "derived_peak_TFLOPs": {"f16_bf16": round(cus * ghz * 4096 / 1e3, 1), "fp8_int8": round(cus * ghz * 8192 / 1e3, 1)}}
+    mem_khz, width = getattr(p, "memory_clock_rate", 0), getattr(p, "memory_bus_width", 0)
+    if mem_khz and width:
+        rep["derived_peak_hbm_GBps"] = round(2 * mem_khz * 1e3 * width / 8 / 1e9, 1)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    rep["host_cpu"] = {"model": model, "os_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()}
+    return rep
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -237,6 +277,7 @@ def main():
                        "step_time_over_floor": round(ms_per_step * 1e3 / floor_us, 3)},
         "roofline": roofline,
     }
+    out["device"] = device_report(dev)
     if not args.no_w8a8:
         out["w8a8_int8"] = w8a8_gemm_bench(ops, dev, stream)
     if args.moe:

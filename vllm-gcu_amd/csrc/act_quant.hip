@@ -53,6 +53,26 @@ __device__ __forceinline__ u2 to_fp8x8(const float* y) {
 
 __device__ __forceinline__ float clamp448(float y) { return fminf(fmaxf(y, -FP8_MAX), FP8_MAX); }
 
+// a / s for many a and one s, with the result of the IEEE division: the reciprocal estimate and
+// its Newton step are made once per divisor, the quotient estimate and its two residual
+// corrections once per dividend -- the same fused multiply-adds the division expands to, without
+// the operand scaling and special-case fix-up that only matter when s, 1 / s, a / s or a residual
+// leave the normal range.  For the dynamic scales here s = max(absmax, 1e-10) / 448 is normal,
+// |a / s| <= 448, and a residual can only underflow where the quotient is far below the smallest
+// fp8 step; a group that holds an infinity or a NaN comes out as NaN throughout.
+struct SharedDivisor {
+  float s, y;
+  __device__ __forceinline__ explicit SharedDivisor(float s_) : s(s_) {
+    const float y0 = __builtin_amdgcn_rcpf(s_);
+    y = __builtin_fmaf(__builtin_fmaf(-s_, y0, 1.0f), y0, y0);
+  }
+  __device__ __forceinline__ float div(float a) const {
+    const float q0 = a * y;
+    const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, a), y, q0);
+    return __builtin_fmaf(__builtin_fmaf(-s, q1, a), y, q1);
+  }
+};
+
 // ---- silu_and_mul: out[r, :d] = silu(x[r, :d]) * x[r, d:] -------------------
 template <int DT>
 __global__ void __launch_bounds__(256)
@@ -105,9 +125,10 @@ group_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, long rows
     if (!live) mx = 0.f;
     for (int o = 1; o < lpg; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
     const float s = fmaxf(mx, 1e-10f) / FP8_MAX;
+    const SharedDivisor by_s(s);
     float q[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) q[e] = clamp448(y[e] / s);
+    for (int e = 0; e < 8; ++e) q[e] = clamp448(by_s.div(y[e]));
     if (live) {
       *(u2*)(out + r * K + 8 * c) = to_fp8x8(q);
       if ((c % lpg) == 0) scales[r * (K / gs) + c / lpg] = s;
@@ -131,8 +152,9 @@ token_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, int K, co
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   const float s = fmaxf(mx, 1e-10f) / FP8_MAX;
   if (threadIdx.x == 0) scales[row] = s;
+  const SharedDivisor by_s(s);
   for (int k = threadIdx.x; k < K; k += 256) {
-    const float y = clamp448(Elem<DT>::to_f32(x[row * K + k]) / s);
+    const float y = clamp448(by_s.div(Elem<DT>::to_f32(x[row * K + k])));
     int w = __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
     out[row * K + k] = (uint8_t)(w & 0xff);
   }
@@ -276,9 +298,10 @@ rms_norm_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* resid
       if (!live) mx = 0.f;
       for (int o = 1; o < lpg; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
       const float sg = fmaxf(mx, 1e-10f) / FP8_MAX;
+      const SharedDivisor by_sg(sg);
       float q[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) q[e] = clamp448(v[e] / sg);
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(by_sg.div(v[e]));
       if (live) {
         *(u2*)((uint8_t*)out + row * K + 8 * c) = to_fp8x8(q);
         if ((c % lpg) == 0) out_scales[row * (K / gs) + c / lpg] = sg;
