@@ -261,6 +261,24 @@ def test_tile_gemm_split_k_small_grid(ops, rearrange, M, K, N):
     assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16))
 
 
+def test_tile_gemm_three_way_split_between_half_and_full_round(ops, rearrange):
+    # 288 output tiles over a long K (more than half of the 512 resident workgroups, fewer than 0.7
+    # of them): K is split three ways; sampled rows against the oracle, exact inputs bit for bit
+    M, K, N, g = 1152, 8192, 4096, 128
+    print(f"case tile 3-way split M={M} K={K} N={N}", flush=True)
+    q, z, s, x = make_case(77, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).float().cpu().numpy()
+    rows = np.random.default_rng(3).choice(M, size=48, replace=False)
+    rows[:3] = (0, 63, M - 1)
+    want = oracle(q, z, s, x[rows], g, torch.float16)
+    np.testing.assert_allclose(got[rows], want, rtol=RTOL, atol=ATOL)
+    assert np.isfinite(got).all()
+    q, z, s, x = make_case(78, M, K, N, g, exact=True)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).cpu()
+    want = torch.from_numpy(oracle(q, z, s, x[rows], g, torch.float16)).to(torch.float16)
+    assert torch.equal(got[torch.from_numpy(rows)], want)
+
+
 def test_tile_gemm_zero_kinds_and_group_256(ops, rearrange):
     M, K, N, g = 130, 512, 256, 256
     q, z, s, x = make_case(77, M, K, N, g)

@@ -495,10 +495,19 @@ static int tile_splits(int M, int K, int N) {
   const long wgs = (long)((M + 16 * mt - 1) / (16 * mt)) * ((N + BN - 1) / BN);
   // 64-row tiles run two workgroups per CU
   const long target = (long)device_cu_count() * (mt == 4 ? 2 : 1);
-  if (wgs * 2 > target) return 1;
-  // 128-row tiles: the nearest count; 64-row tiles must all be resident at once (a second
-  // round of a few workgroups would double the time), so never above the target
-  long s = mt == 4 ? target / wgs : (target + wgs / 2) / wgs;
+  long s;
+  if (wgs * 2 > target) {
+    // More than half a round already.  A workgroup alone on its CU runs a K block in about 60 %
+    // of the time of two that share one, so between 1/2 and 0.7 of a round over a long K three
+    // splits (two even rounds of a third of K) beat one uneven round: K 14336, N 4096,
+    // M 1100..1280: 203 -> 167..175 us; above that, and for K 4096, no split count gained.
+    if (mt != 4 || wgs * 10 > target * 7 || G < 64) return 1;
+    s = 3;
+  } else {
+    // 128-row tiles: the nearest count; 64-row tiles must all be resident at once (a second
+    // round of a few workgroups would double the time), so never above the target
+    s = mt == 4 ? target / wgs : (target + wgs / 2) / wgs;
+  }
   if (s > G / 4) s = G / 4;
   while (s > 1 && (size_t)s * M * N * sizeof(float) > TILE_SPLITK_BYTES) --s;
   return s < 1 ? 1 : (int)s;
