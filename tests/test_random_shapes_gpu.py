@@ -1,0 +1,124 @@
+"""Seeded random shapes through the dense operators: every kernel family, row count and ragged
+edge that the routing inside the operators can pick, checked against the oracle.  Outputs are
+allocated full of NaN (or land in memory that was just filled with NaN), so a tile that no
+workgroup writes shows up as NaN instead of as a stale correct value."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8 as of8
+from oracle import w4 as ow4
+from oracle import w8a8 as o8
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2        # fp16 / bf16 outputs of fp32 accumulation
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def poison(nbytes):
+    """Fill and free a block of the size the operator is about to allocate: the caching allocator
+    hands the same block out again."""
+    t = torch.full((max(nbytes // 2, 1),), float("nan"), dtype=torch.float16, device="cuda")
+    del t
+
+
+def draw_rows(rng):
+    # decode sizes, the 16/32/64/128/256-row boundaries of the kernels, and prefill sizes
+    kind = rng.integers(0, 4)
+    if kind == 0:
+        return int(rng.integers(1, 18))
+    if kind == 1:
+        return int(rng.choice([31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257]))
+    if kind == 2:
+        return int(rng.integers(18, 300))
+    return int(rng.integers(300, 1200))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_w4a16_random_shapes(seed):
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    rng = np.random.default_rng(1000 + seed)
+    M = draw_rows(rng)
+    K = 128 * int(rng.integers(1, 25))
+    N = 128 * int(rng.integers(1, 13))
+    g = int(rng.choice([32, 64, 128, 128, 128, -1]))
+    if g == -1 and K > 1024:
+        g = 128
+    dtype = torch.float16 if rng.integers(0, 2) else torch.bfloat16
+    with_bias = bool(rng.integers(0, 2))
+    sym = bool(rng.integers(0, 4) == 0)
+    print(f"case w4a16 random seed={seed} M={M} K={K} N={N} g={g} {dtype} bias={with_bias} sym={sym}", flush=True)
+    G = 1 if g == -1 else K // g
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = np.full((G, N), 8, dtype=np.uint8) if sym else rng.integers(0, 16, size=(G, N), dtype=np.uint8)
+    s = torch.from_numpy(rng.uniform(0.001, 0.01, size=(G, N)).astype(np.float32)).to(dtype)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(dtype) if with_bias else None
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    poison(M * N * 2)
+    out = ops.w4a16_gemm(x.cuda(), w, s.cuda(), None if sym else zp, None if bias is None else bias.cuda(), g)
+    torch.cuda.synchronize()
+    want = ow4.w4a16_gemm(x.float().numpy(), q, z, s.float().numpy(), g,
+                          bias=None if bias is None else bias.float().numpy())
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_w8a8_int8_random_shapes(seed):
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    rng = np.random.default_rng(2000 + seed)
+    M = draw_rows(rng)
+    K = 128 * int(rng.integers(1, 17))
+    kslab = bool(rng.integers(0, 2))
+    N = 64 * int(rng.integers(1, 20)) if kslab else 4 * int(rng.integers(1, 300))
+    dtype = torch.float16 if rng.integers(0, 2) else torch.bfloat16
+    with_bias = bool(rng.integers(0, 2))
+    per_row = bool(rng.integers(0, 4) != 0)
+    print(f"case w8a8 random seed={seed} M={M} K={K} N={N} kslab={kslab} {dtype} bias={with_bias} "
+          f"per_row={per_row}", flush=True)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    xs = rng.uniform(0.001, 0.01, size=(M, 1) if per_row else (1, 1)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(dtype) if with_bias else None
+    wd = dev(w_nk)
+    if kslab:
+        wd = rearrange.to_kslab(wd)
+    out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    torch.ops._C.cutlass_scaled_mm(out, dev(x), wd.t(), dev(xs), dev(ws), None if bias is None else bias.cuda())
+    torch.cuda.synchronize()
+    acc = o8.int8_gemm_i32(x, np.ascontiguousarray(w_nk.T))
+    want = o8.scaled_mm_epilogue(acc, xs, ws, None if bias is None else bias.float().numpy())
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_fp8_block_random_shapes(seed):
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    rng = np.random.default_rng(3000 + seed)
+    M = draw_rows(rng)
+    K = 128 * int(rng.integers(1, 13))
+    N = 128 * int(rng.integers(1, 10))
+    kslab = bool(rng.integers(0, 2))
+    with_bias = bool(rng.integers(0, 2))
+    print(f"case fp8 block random seed={seed} M={M} K={K} N={N} kslab={kslab} bias={with_bias}", flush=True)
+    w = of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 0.5, -448, 448).astype(np.float32))
+    ws = rng.uniform(0.02, 0.1, size=(N // 128, K // 128)).astype(np.float32)
+    xq, xs = of8.per_token_group_quant_fp8(rng.standard_normal((M, K)).astype(np.float32), 128)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.bfloat16) if with_bias else None
+    wd = dev(w).view(torch.float8_e4m3fn)
+    if kslab:
+        wd = rearrange.to_kslab(wd)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(out, dev(xq).view(torch.float8_e4m3fn), wd, None if bias is None else bias.cuda(),
+                              dev(xs), dev(ws))
+    torch.cuda.synchronize()
+    want = of8.block_fp8_gemm(xq, xs, w, ws)
+    if bias is not None:
+        want = want + bias.float().numpy()
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL,
+                               atol=ATOL * max(1.0, np.abs(want).max()))
