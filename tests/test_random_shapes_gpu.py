@@ -1,4 +1,4 @@
-"""Seeded random shapes through the dense operators: every kernel family, row count and ragged
+"""Seeded random shapes through the dense and grouped operators: every kernel family, row count and ragged
 edge that the routing inside the operators can pick, checked against the oracle.  Outputs are
 allocated full of NaN (or land in memory that was just filled with NaN), so a tile that no
 workgroup writes shows up as NaN instead of as a stale correct value."""
@@ -122,3 +122,49 @@ def test_fp8_block_random_shapes(seed):
         want = want + bias.float().numpy()
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL,
                                atol=ATOL * max(1.0, np.abs(want).max()))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_grouped_w4a16_random_shapes(seed):
+    """Both GEMM forms of the fused-MoE W4A16 layer over random token counts, expert counts, top-k
+    and block sizes, with a routing skewed so that some experts receive nothing."""
+    from oracle import moe as om
+    from vllm_gcu_amd.kernels import fused_moe as fmoe
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    rng = np.random.default_rng(4000 + seed)
+    M = int(rng.choice([1, 2, 7, 16, 33, 100, 257]))
+    E = int(rng.choice([2, 4, 8, 16]))
+    T = int(rng.integers(1, min(E, 4) + 1))
+    K = 128 * int(rng.integers(1, 7))
+    N = 128 * int(rng.integers(1, 6))
+    block = int(rng.choice([16, 32, 64, 128]))
+    dtype = torch.float16 if rng.integers(0, 2) else torch.bfloat16
+    print(f"case grouped w4a16 random seed={seed} M={M} E={E} T={T} K={K} N={N} block={block} {dtype}", flush=True)
+    q = rng.integers(0, 16, size=(E, K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(E, K // 128, N), dtype=np.uint8)
+    sd = torch.from_numpy(rng.uniform(0.001, 0.01, size=(E, K // 128, N)).astype(np.float32)).to(dtype)
+    qw = np.stack([ow4.gptq_pack_weight(q[e]) for e in range(E)])
+    qz = np.stack([ow4.gptq_pack_zeros(z[e]) for e in range(E)])
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(qw), dev(qz))
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    logits[:, : max(1, E // 2)] += 4.0                      # the upper half of the experts is rarely chosen
+    tw, ids, _ = om.topk_softmax(logits, T, True)
+    wf = lambda e: ow4.dequantize(q[e], z[e], sd[e].float().numpy(), 128)
+
+    def run(A, C, mul, topk):
+        s, e, n = fmoe.moe_align_block_size(dev(ids), block, E)
+        fmoe.invoke_fused_moe_kernel(A, w, C, None, sd.cuda(), zp, dev(tw), dev(ids), s, e, n, mul, topk,
+                                     {"BLOCK_SIZE_M": block}, use_fp8_w8a8=False, use_int8_w8a8=False,
+                                     use_int8_w8a16=False, use_int4_w4a16=True, block_shape=[0, 128])
+        torch.cuda.synchronize()
+
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    C = torch.full((M, T, N), float("nan"), dtype=dtype, device="cuda")
+    run(x.cuda(), C, False, T)
+    want = om.fused_moe_gemm(x.float().numpy(), wf, ids, T)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    x2 = torch.from_numpy(rng.standard_normal((M * T, K)).astype(np.float32)).to(dtype)
+    C2 = torch.full((M, T, N), float("nan"), dtype=dtype, device="cuda")
+    run(x2.cuda(), C2, True, 1)
+    want2 = om.fused_moe_gemm(x2.float().numpy(), wf, ids, 1, tw, True)
+    np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
