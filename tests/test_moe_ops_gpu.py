@@ -198,6 +198,29 @@ def test_per_token_group_quant_fp8_bit_exact(ops, dtype, rows, K, gs):
     assert np.all(qb.view(torch.uint8).cpu().numpy()[nv:] == 0) and np.all(sb.cpu().numpy()[nv:] == -1.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_per_token_group_quant_fp8_rounding_boundaries_bit_exact(ops, dtype):
+    """Quotients at and next to the midpoints between fp8 codes, group scales over 30 binades:
+    the kernel divides through a shared reciprocal with residual corrections and must produce the
+    codes of the IEEE division the oracle uses."""
+    rng = np.random.default_rng(11)
+    rows, K, gs = 384, 2048, 128
+    table = of8.e4m3fn_decode_table().astype(np.float64)
+    pos = np.sort(table[np.isfinite(table) & (table >= 0)])
+    mids = (pos[:-1] + pos[1:]) / 2                         # rounding boundaries of e4m3fn
+    lo, hi = (-14, 15) if dtype == torch.float16 else (-20, 20)
+    scale = np.exp2(rng.uniform(lo, hi - 9, size=(rows, K // gs, 1))) * rng.uniform(1, 2, size=(rows, K // gs, 1))
+    target = rng.choice(mids, size=(rows, K // gs, gs)) * rng.choice([1 - 2.0 ** -12, 1.0, 1 + 2.0 ** -12],
+                                                                     size=(rows, K // gs, gs))
+    x = target * scale * rng.choice([-1.0, 1.0], size=target.shape)
+    x[:, :, 0] = 448.0 * scale[:, :, 0]                     # the element that sets the group's scale
+    xt = torch.from_numpy(x.reshape(rows, K).astype(np.float32)).to(dtype)
+    q, s = ops.per_token_group_quant_fp8(xt.cuda(), gs)
+    qo, so = of8.per_token_group_quant_fp8(xt.float().numpy(), gs)
+    assert np.array_equal(s.cpu().numpy(), so)
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy(), qo)
+
+
 def test_silu_mul_group_quant_equals_unfused_sequence(ops):
     # csrc equivalence table: silu_mul_per_token_group_quant == silu_and_mul then
     # dynamic_per_token_group_fp8_quant (vllm_gcu/compilation/fx_fusion.py:102-108)

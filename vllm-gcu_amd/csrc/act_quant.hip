@@ -56,10 +56,9 @@ __device__ __forceinline__ float clamp448(float y) { return fminf(fmaxf(y, -FP8_
 // a / s for many a and one s, with the result of the IEEE division: the reciprocal estimate and
 // its Newton step are made once per divisor, the quotient estimate and its two residual
 // corrections once per dividend -- the same fused multiply-adds the division expands to, without
-// the operand scaling and special-case fix-up that only matter when s, 1 / s, a / s or a residual
-// leave the normal range.  For the dynamic scales here s = max(absmax, 1e-10) / 448 is normal,
-// |a / s| <= 448, and a residual can only underflow where the quotient is far below the smallest
-// fp8 step; a group that holds an infinity or a NaN comes out as NaN throughout.
+// the operand scaling that only matters when s, 1 / s, a / s or a residual leave the normal range.
+// For the dynamic scales here s = max(absmax, 1e-10) / 448 is normal, |a / s| <= 448, and a
+// residual can only underflow where the quotient is far below the smallest fp8 step.
 struct SharedDivisor {
   float s, y;
   __device__ __forceinline__ explicit SharedDivisor(float s_) : s(s_) {
@@ -69,7 +68,8 @@ struct SharedDivisor {
   __device__ __forceinline__ float div(float a) const {
     const float q0 = a * y;
     const float q1 = __builtin_fmaf(__builtin_fmaf(-s, q0, a), y, q0);
-    return __builtin_fmaf(__builtin_fmaf(-s, q1, a), y, q1);
+    // the division's own last instruction: signed zeros, infinities and NaN as IEEE has them
+    return __builtin_amdgcn_div_fixupf(__builtin_fmaf(__builtin_fmaf(-s, q1, a), y, q1), s, a);
   }
 };
 
