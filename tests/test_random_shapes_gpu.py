@@ -168,3 +168,67 @@ def test_grouped_w4a16_random_shapes(seed):
     run(x2.cuda(), C2, True, 1)
     want2 = om.fused_moe_gemm(x2.float().numpy(), wf, ids, 1, tw, True)
     np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_grouped_fp8_and_int8_random_shapes(seed):
+    """The K-contiguous grouped GEMM (fp8 block-scaled and int8 per-token x per-channel experts),
+    row-major and kslab weights, random routing with idle experts, all block sizes."""
+    from oracle import moe as om
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    from vllm_gcu_amd.kernels import fused_moe as fmoe
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    rng = np.random.default_rng(5000 + seed)
+    M = int(rng.choice([1, 3, 16, 40, 130, 300]))
+    E = int(rng.choice([2, 4, 8, 32]))
+    T = int(rng.integers(1, min(E, 4) + 1))
+    K = 128 * int(rng.integers(1, 7))
+    N = 128 * int(rng.integers(1, 5))
+    block = int(rng.choice([16, 32, 64, 128]))
+    kslab = bool(rng.integers(0, 2))
+    mul = bool(rng.integers(0, 2))
+    fp8 = bool(seed % 2)
+    print(f"case grouped {'fp8' if fp8 else 'int8'} random seed={seed} M={M} E={E} T={T} K={K} N={N} "
+          f"block={block} kslab={kslab} mul={mul}", flush=True)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    logits[:, : max(1, E // 2)] += 3.0
+    tw, ids, _ = om.topk_softmax(logits, T, True)
+    flat = ids.reshape(-1)
+    s, e, n = fmoe.moe_align_block_size(dev(ids), block, E)
+    want = np.zeros((M * T, N), dtype=np.float32)
+    if fp8:
+        wq = np.stack([of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 2, -448, 448).astype(np.float32))
+                       for _ in range(E)])
+        ws = rng.uniform(0.005, 0.02, size=(E, N // 128, K // 128)).astype(np.float32)
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+        xq, xs = ops.per_token_group_quant_fp8(x.cuda(), 128)
+        wd = dev(wq).view(torch.float8_e4m3fn)
+        if kslab:
+            wd = rearrange.to_kslab(wd)
+        C = torch.full((M, T, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        fmoe.invoke_fused_moe_kernel(xq, wd, C, xs, dev(ws), None, dev(tw), dev(ids), s, e, n, mul, T,
+                                     {"BLOCK_SIZE_M": block}, use_fp8_w8a8=True, use_int8_w8a8=False,
+                                     use_int8_w8a16=False, use_int4_w4a16=False, block_shape=[128, 128])
+        xq_c, xs_c = xq.view(torch.uint8).cpu().numpy(), xs.cpu().numpy()
+        for t in range(M * T):
+            want[t] = of8.block_fp8_gemm(xq_c[t // T:t // T + 1], xs_c[t // T:t // T + 1], wq[flat[t]], ws[flat[t]])[0]
+    else:
+        x = rng.standard_normal((M, K)).astype(np.float16)
+        xq, xs = o8.dynamic_scaled_int8_quant(x)
+        wq = rng.integers(-127, 128, size=(E, N, K), dtype=np.int8)
+        ws = rng.uniform(0.001, 0.02, size=(E, N, 1)).astype(np.float32)
+        wd = dev(wq)
+        if kslab:
+            wd = rearrange.to_kslab(wd)
+        C = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
+        fmoe.invoke_fused_moe_kernel(dev(xq), wd, C, dev(xs), dev(ws), None, dev(tw), dev(ids), s, e, n, mul, T,
+                                     {"BLOCK_SIZE_M": block}, use_fp8_w8a8=False, use_int8_w8a8=True,
+                                     use_int8_w8a16=False, use_int4_w4a16=False)
+        for t in range(M * T):
+            acc = o8.int8_gemm_i32(xq[t // T:t // T + 1], np.ascontiguousarray(wq[flat[t]].T))
+            want[t] = o8.scaled_mm_epilogue(acc, xs[t // T], ws[flat[t], :, 0])[0]
+    torch.cuda.synchronize()
+    if mul:
+        want = want * tw.reshape(-1, 1)
+    got = C.view(-1, N).float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
