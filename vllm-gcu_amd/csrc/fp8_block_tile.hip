@@ -46,18 +46,18 @@ __device__ __forceinline__ void dma4(const void* gptr, void* lds_wave_base) {
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 4, 0, 0);
 }
 
-__device__ __forceinline__ long lo64(i4 v) { return (long)((unsigned long)(uint32_t)v[0] | ((unsigned long)(uint32_t)v[1] << 32)); }
-__device__ __forceinline__ long hi64(i4 v) { return (long)((unsigned long)(uint32_t)v[2] | ((unsigned long)(uint32_t)v[3] << 32)); }
+typedef int i8v __attribute__((ext_vector_type(8)));
 
 template <int DT>
 __global__ void __launch_bounds__(F8_THREADS, 1)
 fp8_block_gemm_kernel(F8Args a) {
   constexpr int WN = 2, NI = 4, NJ = 4;                 // 4 x 2 wavefronts of 64 x 64
   constexpr int X_BYTES = FTM * FTKB, W_BYTES = FTN * FTKB, XS_BYTES = FTM * 4;
-  constexpr int STAGE_BYTES = X_BYTES + W_BYTES + XS_BYTES;
+  constexpr int WS_BYTES = 256;                         // the tile's weight scale of a K block, 64 copies
+  constexpr int STAGE_BYTES = X_BYTES + W_BYTES + XS_BYTES + WS_BYTES;
   constexpr int XCOPIES = FTM / 8 / 8, WCOPIES = FTN / 8 / 8;       // 1 KiB copies per wavefront
   extern __shared__ __align__(16) unsigned char lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15, kq = lane >> 4;
   const int wm = wave / WN, wn = wave % WN;
   const int M = a.M, N = a.N, K = a.K, KB = K >> 7;
@@ -91,12 +91,13 @@ fp8_block_gemm_kernel(F8Args a) {
     n0 = tn * FTN;
   };
 
-  f4 acc[NI][NJ], part[NI][NJ];
+  f4 acc[NI][NJ];
 
   // global -> LDS: lane = 8 * row + slot, slot p of row r receives chunk p ^ (r & 7); kslab weights
   // chunk-major (lane = 8 * position + row, position p of an odd 8-row group holding chunk p ^ 1)
   const int crow = lane >> 3, cchunk = (lane & 7) ^ (crow & 7);
   uint32_t xo[XCOPIES], wo[WCOPIES], xso = 0;
+  int wsbase = 0;
   const uint8_t *xtile, *wtile;
   auto set_copy_tile = [&](int tile) {
     int m0, n0;
@@ -120,6 +121,7 @@ fp8_block_gemm_kernel(F8Args a) {
     }
     // activation scales: wavefronts 0..3 copy 64 rows each (index in floats)
     xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB;
+    wsbase = (n0 >> 7) * KB;                       // wavefront 4 copies the tile's weight scale
     xtile = a.x + (long)m0 * a.ldx;
     wtile = a.w_kslab ? a.w : a.w + (long)n0 * a.ldw;
   };
@@ -134,14 +136,15 @@ fp8_block_gemm_kernel(F8Args a) {
             xs + X_BYTES + (wave + 8 * p) * 1024);
     } else if (wave < 4) {
       dma4(a.x_scale + xso + kt, xs + X_BYTES + W_BYTES + wave * 256);
+    } else if (wave == 4) {
+      dma4(a.w_scale + wsbase + kt, xs + X_BYTES + W_BYTES + XS_BYTES);
     }
   };
-  auto issue = [&](int stage, int kt) {
-#pragma unroll
-    for (int s = 0; s < NSLOT; ++s) copy_slot(s, stage, kt);
-  };
 
-  // operand reads (assembly, waited for by hand: see the int8 kernel)
+  // operand reads (assembly, waited for by hand: see the int8 kernel).  Lane (l16, kq) takes the
+  // 16-byte chunks kq and 4 + kq of row l16 of a 16-row tile: together the 32 bytes of K it feeds
+  // to the 128-deep MFMA.  Which 32 of the 128 a lane holds does not matter as long as both
+  // operands hold the same ones.
   const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds;
   uint32_t lo[2], wlo[2];
 #pragma unroll
@@ -152,119 +155,166 @@ fp8_block_gemm_kernel(F8Args a) {
   }
   const uint32_t xwave = wm * (16 * NJ) * FTKB, wwave = X_BYTES + wn * (16 * NI) * FTKB;
   const uint32_t xsaddr = lds_base + X_BYTES + W_BYTES + (uint32_t)(wm * 64 + l16) * 4u;
-  struct Frag { i4 bx[NJ]; i4 aw[NI]; };
-  auto read_one = [&](Frag& f, int r, uint32_t xb, uint32_t wb) {
+  // The operands of one K block: two 16-byte halves per 16-row tile.  The x tiles and the
+  // activation scales of this lane's four row tiles (rows wm * 64 + 16 j + l16) have two register
+  // sets that swap roles every K block.  The w tiles of rows 0..2 have one: the MFMAs walk the w
+  // tiles in order, so tile i is re-read for the next K block as soon as its four MFMAs are under
+  // way; only the last w tile, in use until the end of the K block, has two sets.  (Two full sets
+  // would need 128 registers of the 256 a wavefront has at two wavefronts per SIMD.)
+  struct XOps { i4 bx[2][NJ]; float xs[NJ]; float ws; };
+  typedef i4 WTile[2];
+  auto read_x = [&](XOps& f, int h, int j, uint32_t stage_off) {
+    const uint32_t xb = lo[h] + stage_off + xwave;
+#pragma unroll
+    for (int jj = 0; jj < NJ; ++jj)
+      if (jj == j) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.bx[h][jj]) : "v"(xb), "n"(jj * 16 * FTKB));
+  };
+  auto read_w = [&](WTile& t, int i, uint32_t stage_off) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint32_t wb = wlo[h] + stage_off + wwave;
+#pragma unroll
+      for (int ii = 0; ii < NI; ++ii)
+        if (ii == i) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(t[h]) : "v"(wb), "n"(ii * 16 * FTKB));
+    }
+  };
+  auto read_xs = [&](XOps& f, uint32_t stage_off) {
+    const uint32_t ad = xsaddr + stage_off;
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
-      if (r == j) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.bx[j]) : "v"(xb), "n"(j * 16 * FTKB));
-#pragma unroll
-    for (int i = 0; i < NI; ++i)
-      if (r == NJ + i) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.aw[i]) : "v"(wb), "n"(i * 16 * FTKB));
+      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(f.xs[j]) : "v"(ad), "n"(j * 64));
+    asm volatile("ds_read_b32 %0, %1" : "=v"(f.ws) : "v"(lds_base + (uint32_t)(X_BYTES + W_BYTES + XS_BYTES) + stage_off));
   };
-  auto read_frag = [&](Frag& f, int stage, int h) {
-    const uint32_t xb = lo[h] + (uint32_t)(stage * STAGE_BYTES) + xwave;
-    const uint32_t wb = wlo[h] + (uint32_t)(stage * STAGE_BYTES) + wwave;
-#pragma unroll
-    for (int r = 0; r < NJ + NI; ++r) read_one(f, r, xb, wb);
-  };
-  auto lds_wait = [&](Frag& f) {
+  WTile w012[3];
+  auto lds_wait = [&](XOps& f, WTile& w3) {
+    // every register the reads of a step write, exactly once each
     asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f.bx[0]), "+v"(f.bx[1]), "+v"(f.bx[2]), "+v"(f.bx[3]), "+v"(f.aw[0]), "+v"(f.aw[1]),
-                   "+v"(f.aw[2]), "+v"(f.aw[3]));
-  };
-  // the activation scales of this lane's four row tiles (rows wm * 64 + 16 j + l16) for one K block
-  float xsv[NJ];
-  auto read_xs = [&](int stage) {
-    const uint32_t ad = xsaddr + (uint32_t)(stage * STAGE_BYTES);
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-      asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(xsv[j]) : "v"(ad), "n"(j * 64));
-  };
-  auto xs_wait = [&]() {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xsv[0]), "+v"(xsv[1]), "+v"(xsv[2]), "+v"(xsv[3]));
+                 : "+v"(f.bx[0][0]), "+v"(f.bx[0][1]), "+v"(f.bx[0][2]), "+v"(f.bx[0][3]), "+v"(f.bx[1][0]),
+                   "+v"(f.bx[1][1]), "+v"(f.bx[1][2]), "+v"(f.bx[1][3]), "+v"(w012[0][0]), "+v"(w012[0][1]),
+                   "+v"(w012[1][0]), "+v"(w012[1][1]), "+v"(w012[2][0]), "+v"(w012[2][1]), "+v"(w3[0]),
+                   "+v"(w3[1]), "+v"(f.xs[0]), "+v"(f.xs[1]), "+v"(f.xs[2]), "+v"(f.xs[3]), "+v"(f.ws));
   };
 
-  // One half of a K block: 2 MFMAs (k = 32 each) per (w tile i, x tile j).  Between them: the
-  // LDS reads of the next operand set, one per pair for the first eight pairs, and copy slots
-  // SB .. SE-1 of a later K block, one after every other pair.  The second half adds the block's
-  // partial sums to the running sums with the block's scale.
-  float sc[NJ];
-  auto half = [&](const Frag& cur, Frag& nxt, int rstage, int rh, bool second, int SB, int SE, int cstage, int kt) {
-    const uint32_t xb = lo[rh] + (uint32_t)(rstage * STAGE_BYTES) + xwave;
-    const uint32_t wb = wlo[rh] + (uint32_t)(rstage * STAGE_BYTES) + wwave;
+  // One K block: one 128-deep MFMA per (w tile i, x tile j), started from zero; its result joins
+  // the running sum with the block's scale two MFMAs later, when the matrix pipe has delivered it.
+  // Between the MFMAs: the operand and scale reads of the next K block (a w tile one MFMA after
+  // the last one that used it) and the copy slots of the K block three ahead.
+  auto step = [&](const XOps& cur, XOps& nxt, const WTile& w3cur, WTile& w3nxt, uint32_t rso, int cstage, int kt) {
+    float sc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) sc[j] = cur.xs[j] * cur.ws;
+    f4 ring[4];
     int n = 0;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        f4 c = second ? part[i][j] : (f4){0.f, 0.f, 0.f, 0.f};
-        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(lo64(cur.aw[i]), lo64(cur.bx[j]), c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(hi64(cur.aw[i]), hi64(cur.bx[j]), c, 0, 0, 0);
-        part[i][j] = c;
-        // the block's partial sum joins the running sum one pair later, when the MFMA has delivered it
-        if (second && n > 0) {
-          const int pi = (n - 1) / NJ, pj = (n - 1) % NJ;
-          acc[pi][pj] += sc[pj] * part[pi][pj];
+        const i4 a0 = i < 3 ? w012[i < 3 ? i : 0][0] : w3cur[0], a1 = i < 3 ? w012[i < 3 ? i : 0][1] : w3cur[1];
+        const i8v av = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+        const i8v bv = __builtin_shufflevector(cur.bx[0][j], cur.bx[1][j], 0, 1, 2, 3, 4, 5, 6, 7);
+        ring[n & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+        if (n >= 2) {
+          const int pn = n - 2;
+          acc[pn / NJ][pn % NJ] += sc[pn % NJ] * ring[pn & 3];
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (n < NJ + NI) read_one(nxt, n, xb, wb);
-        if ((n & 1) && SB + (n >> 1) < SE) copy_slot(SB + (n >> 1), cstage, kt);
+        if (n == 0) read_w(w3nxt, 3, rso);
+        if (n == 4) read_w(w012[0], 0, rso);
+        if (n == 8) read_w(w012[1], 1, rso);
+        if (n == 12) read_w(w012[2], 2, rso);
+        // x tiles: one read after each of MFMAs 1 2 3, 5 6 7, 9 10; the scales after 13
+        if ((n & 3) != 0 && n < 11) {
+          const int r = n - 1 - (n >> 2);             // 0..7
+          read_x(nxt, r >> 2, r & 3, rso);
+        }
+        if (n == 13) read_xs(nxt, rso);
+        if ((n & 1) && (n >> 1) < NSLOT) copy_slot(n >> 1, cstage, kt);
         __builtin_amdgcn_sched_barrier(0);
         ++n;
       }
-    if (second) acc[NI - 1][NJ - 1] += sc[NJ - 1] * part[NI - 1][NJ - 1];
+#pragma unroll
+    for (int pn = NI * NJ - 2; pn < NI * NJ; ++pn) acc[pn / NJ][pn % NJ] += sc[pn % NJ] * ring[pn & 3];
   };
-  static_assert(NI * NJ >= NJ + NI && NI * NJ / 2 >= NSLOT, "not enough MFMA pairs to spread the copies and reads");
+  static_assert(NI == 4 && NJ == 4 && NSLOT <= 8, "the read and copy schedule is written for 16 MFMAs per K block");
 
-  // Stream of K blocks across this workgroup's output tiles, two LDS stages
-  // (element g in stage g % 2): half 0 of element g multiplies (g, 0) while it
-  // reads (g, 1) and the block's activation scales; half 1 multiplies (g, 1),
-  // reads (g + 1, 0) and issues the copy of element g + 2 into g's stage.
+  // Stream of K blocks across this workgroup's output tiles, three LDS stages (element g in stage
+  // g % 3).  Step g multiplies element g from registers, reads element g + 1 from LDS into the
+  // other register set, and issues the copy of element g + 3 into g's stage (every wavefront
+  // finished reading g before the barrier that opened the step).  The step ends when this
+  // wavefront's copies of element g + 2 have landed -- those of g + 3 stay in flight -- and a
+  // barrier makes that true for everybody's.
   const int nt = KB;
   // (kept in a register: read through the dispatch packet it is fetched again in every iteration)
   const int gdim = __builtin_amdgcn_readfirstlane((int)gridDim.x);
   int tile = blockIdx.x;
-  set_copy_tile(tile);
-  issue(0, 0);
-  issue(1, min(1, nt - 1));
   int copy_tile = tile;
-  if (nt == 1 && tile + gdim < total_tiles) {
-    copy_tile = tile + gdim;
-    set_copy_tile(copy_tile);
-    issue(1, 0);
+  set_copy_tile(tile);
+  // element (T + d) of the stream seen from K block T of `tile`: its K block, after moving the copy
+  // offsets to its output tile; past the last output tile a harmless re-read that nobody consumes
+  auto ahead_kt = [&](int T, int d) {
+    int kt = T + d, ahead = 0;
+    while (kt >= nt) { kt -= nt; ++ahead; }
+    const int want = tile + ahead * gdim;
+    if (want >= total_tiles) return nt - 1;
+    if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
+    return kt;
+  };
+  auto wait_all_but_last_step = [&]() {
+    // copies per step and wavefront: 4 x + 2 w, and one of scales in wavefronts 0..4
+    if (wave <= 4) __builtin_amdgcn_s_waitcnt(0x0f77);  // vmcnt(7)
+    else __builtin_amdgcn_s_waitcnt(0x0f76);            // vmcnt(6)
+  };
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    const int kt = ahead_kt(0, d);
+#pragma unroll
+    for (int s = 0; s < NSLOT; ++s) copy_slot(s, d, kt);
   }
-  __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
+  wait_all_but_last_step();                        // elements 0 and 1 landed
   __builtin_amdgcn_s_barrier();
-  Frag f0, f1;
-  read_frag(f0, 0, 0);
-  lds_wait(f0);
-  int g = 0;
+  XOps o0, o1;
+  WTile w3a, w3b;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) read_x(o0, r >> 2, r & 3, 0);
+#pragma unroll
+  for (int i = 0; i < 3; ++i) read_w(w012[i], i, 0);
+  read_w(w3a, 3, 0);
+  read_xs(o0, 0);
+  lds_wait(o0, w3a);
+  __builtin_amdgcn_s_barrier();                    // nobody still reads element 0 when step 0 overwrites its stage
+  int st = 0;                                      // stage of the current element
   for (; tile < total_tiles; tile += gdim) {
     int m0, n0;
     tile_origin(tile, m0, n0);
-    const float* wsp = a.w_scale + (long)(n0 >> 7) * KB;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
-    for (int T = 0; T < nt; ++T, ++g) {
-      const int st = g & 1;
-      const float wsv = wsp[T];
-      read_xs(st);
-      half(f0, f1, st, 1, false, 0, 0, st, 0);
-      lds_wait(f1);
-      xs_wait();
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) sc[j] = xsv[j] * wsv;
-      __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): my copies of element g + 1 landed
-      __builtin_amdgcn_s_barrier();
-      int kt = T + 2, ahead = 0;
-      while (kt >= nt) { kt -= nt; ++ahead; }
-      const int want = tile + ahead * gdim;
-      if (want >= total_tiles) kt = nt - 1;        // past the end: harmless re-read, never consumed
-      else if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
-      half(f1, f0, st ^ 1, 0, true, 0, NSLOT, st, kt);
-      lds_wait(f0);
+    // two K blocks per iteration so that the register sets swap roles without copies
+    for (int T = 0; T < nt; T += 2) {
+      {
+        const int kt = ahead_kt(T, 3);
+        const int nst = st == 2 ? 0 : st + 1;
+        step(o0, o1, w3a, w3b, (uint32_t)(nst * STAGE_BYTES), st, kt);
+        lds_wait(o1, w3b);
+        wait_all_but_last_step();
+        __builtin_amdgcn_s_barrier();
+        st = nst;
+      }
+      if (T + 1 < nt) {
+        const int kt = ahead_kt(T + 1, 3);
+        const int nst = st == 2 ? 0 : st + 1;
+        step(o1, o0, w3b, w3a, (uint32_t)(nst * STAGE_BYTES), st, kt);
+        lds_wait(o0, w3a);
+        wait_all_but_last_step();
+        __builtin_amdgcn_s_barrier();
+        st = nst;
+      } else {
+        // odd number of K blocks: the next element sits in the other set, move it where the next tile expects it
+        o0 = o1;
+        w3a[0] = w3b[0];
+        w3a[1] = w3b[1];
+      }
     }
 
     // ---- epilogue: lane holds, per (w tile i, x tile j), output row m = .. + l16 and columns
@@ -289,8 +339,9 @@ fp8_block_gemm_kernel(F8Args a) {
         *(u2*)((uint16_t*)a.out + (long)m * a.ldo + n) = o;
       }
     }
-    read_frag(f0, g & 1, 0);
-    lds_wait(f0);
+    // the stores above count in vmcnt too and need not finish in order with the copies: start the
+    // next tile's counting from zero
+    __builtin_amdgcn_s_waitcnt(0x0f70);            // vmcnt(0)
   }
   // no copy may still be writing LDS when the workgroup retires
   __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
@@ -301,7 +352,7 @@ int launch_f8(const F8Args& a, hipStream_t st) {
   const int mtiles = (a.M + FTM - 1) / FTM, ntiles = a.N / FTN;
   F8Args b = a;
   b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
-  const size_t shmem = 2 * (size_t)(FTM * FTKB + FTN * FTKB + FTM * 4);
+  const size_t shmem = 3 * (size_t)(FTM * FTKB + FTN * FTKB + FTM * 4 + 256);
   static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   MQ_REQUIRE(attr == hipSuccess, "fp8_block_gemm: cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
