@@ -204,6 +204,7 @@ fp8_block_gemm_kernel(F8Args a) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) sc[j] = cur.xs[j] * cur.ws;
     f4 ring[4];
+    const bool odd_slots = wave < 4;
     int n = 0;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -228,7 +229,9 @@ fp8_block_gemm_kernel(F8Args a) {
           read_x(nxt, r >> 2, r & 3, rso);
         }
         if (n == 13) read_xs(nxt, rso);
-        if ((n & 1) && (n >> 1) < NSLOT) copy_slot(n >> 1, cstage, kt);
+        // copy slot k after MFMA 2 k + 1 in wavefronts 0..3, after MFMA 2 k + 2 in wavefronts 4..7: the
+        // address unit takes one copy (1 KiB) at a time, and eight in the same cycle queue up
+        if (n >= 1 && n <= 2 * NSLOT && ((n & 1) != 0) == odd_slots) copy_slot((n - 1) >> 1, cstage, kt);
         __builtin_amdgcn_sched_barrier(0);
         ++n;
       }
