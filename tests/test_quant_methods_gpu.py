@@ -383,11 +383,11 @@ def test_fused_qkv_ops_equal_the_unfused_gemm_split_by_columns():
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("M,K,N", [(129, 128, 128), (300, 512, 384), (513, 1024, 256), (2050, 256, 1152),
+@pytest.mark.parametrize("M,K,N", [(65, 384, 256), (129, 128, 128), (300, 512, 384), (513, 1024, 256), (2050, 256, 1152),
                                    (2305, 128, 1024), (4200, 128, 2048)])     # > 8 row tiles, XCD-aware order
 @pytest.mark.parametrize("kslab", [False, True])
 def test_fp8_block_gemm_tile_kernel(M, K, N, kslab, monkeypatch):
-    """linear_quant above 128 rows runs the MFMA tile kernel; checked against the oracle of the
+    """linear_quant above 64 rows (and enough output tiles) runs the MFMA tile kernel; checked against the oracle of the
     block-scaled GEMM and, bit for bit, between the two weight orders."""
     from vllm_gcu_amd.kernels import _custom_ops
     from vllm_gcu_amd.kernels.quantization import rearrange

@@ -96,9 +96,14 @@ def test_w8a8_int8_random_shapes(seed):
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("seed", range(16))
-def test_fp8_block_random_shapes(seed):
+@pytest.mark.parametrize("seed", range(24))
+def test_fp8_block_random_shapes(seed, monkeypatch):
+    from vllm_gcu_amd.kernels import _custom_ops
     from vllm_gcu_amd.kernels.quantization import rearrange
+    if seed % 3:
+        # shapes this small would all go to the weight-streaming kernel: send two thirds of them (above
+        # 64 rows) to the MFMA tile kernel
+        monkeypatch.setattr(_custom_ops, "_FP8_TILE_MIN_TILES", 1)
     rng = np.random.default_rng(3000 + seed)
     M = draw_rows(rng)
     K = 128 * int(rng.integers(1, 13))

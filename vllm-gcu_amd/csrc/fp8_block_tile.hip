@@ -1,20 +1,22 @@
-// fp8-e4m3 block-scaled GEMM for prefill-sized M on the gfx950 fp8 MFMA
-// (v_mfma_f32_16x16x32_fp8_fp8), with the 128 x 128 block scales applied to
-// the fp32 partial sum of every K block.
+// fp8-e4m3 block-scaled GEMM for more than 64 rows on the 128-deep fp8 MFMA of gfx950
+// (v_mfma_f32_16x16x128_f8f6f4, twice the rate of the 32-deep one), with the 128 x 128 block
+// scales applied to the fp32 partial sum of every K block.
 //
 //   out[m, n] = sum_kb x_scale[m, kb] * w_scale[n / 128, kb] * sum_{k in block kb} x[m, k] * w[n, k]
 //
 // Same machinery as the int8 GEMM next door: a workgroup of eight wavefronts
 // (4 x 2, each 64 rows of x by 64 rows of w) owns a 256 x 128 output tile; K
-// advances in LDS tiles of 128 bytes per row, which is exactly one scale block;
-// tiles go from global memory straight into LDS (16 B per lane, no staging
-// registers; 16-byte-chunk XOR swizzle, or chunk-major for kslab weights) in
-// two stages; operand reads are hand-written and hand-waited for.  The tile is
-// 128 columns wide because each K block needs its own set of partial
-// accumulators next to the running sum (2 x 64 registers per lane); 128 columns
-// are also exactly one scale block, so the weight scale of a tile and K block
-// is a single number.  The activation scales of a K block (one per row) travel
-// with the x tile through LDS (4-byte direct-to-LDS copies).
+// advances in LDS tiles of 128 bytes per row, which is exactly one scale block
+// and one MFMA deep; tiles go from global memory straight into LDS (16 B per
+// lane, no staging registers; 16-byte-chunk XOR swizzle, or chunk-major for
+// kslab weights) in three stages; operand reads are hand-written and
+// hand-waited for.  A K block's MFMA starts from zero and its result joins the
+// running sum multiplied by the block's scale.  128 columns are exactly one
+// scale block, so the weight scale of a tile and K block is a single number;
+// it and the activation scales of the K block (one per row) travel with the
+// tiles through LDS (4-byte direct-to-LDS copies).  Two wavefronts per SIMD
+// leave each 256 registers: 64 running sums, two sets of x operands, one set
+// of w operands that is re-read tile by tile behind the MFMAs (see `step`).
 #include "common.h"
 
 namespace mi355q {

@@ -1038,9 +1038,11 @@ def _kcontig(out, a, w, a_scale, w_scale, bias, mode, group):
                   layout, rt.stream_ptr())
 
 
-# the MFMA tile kernel beats the weight-streaming kernel above 128 rows once its tiles fill a good part of
-# the chip (measured: K 7168 N 4096, M 512: 81 us against 60 us; M 2048: 96 us against 202 us)
-_FP8_TILE_MIN_M = 128
+# the MFMA tile kernel beats the weight-streaming kernel above 64 rows once its tiles fill a good part of
+# the chip (measured, K 8192 N 28672 = 224 tiles: M 65..128 69..73 us against 87..119 us, M 64 68 us
+# against 73 us for the streamer's last single-block size; K 7168 N 4096 = 32 tiles: 52 us against
+# 37..53 us at M 65..128, so few tiles stay with the streamer)
+_FP8_TILE_MIN_M = 64
 _FP8_TILE_MIN_TILES = 96
 
 
