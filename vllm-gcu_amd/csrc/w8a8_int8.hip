@@ -74,6 +74,8 @@ w8a8_int8_gemm_kernel(I8Args a) {
   static_assert(WM * WN == 8 && WM * NJ * 16 == TM, "eight wavefronts cover 256 rows of x");
   constexpr int TN = WN * NI * 16;
   constexpr int X_BYTES = TM * TKB, W_BYTES = TN * TKB, STAGE_BYTES = X_BYTES + W_BYTES;
+  // LDS stages: three where they fit (the 128-column tile: 3 x 48 KiB), else two
+  constexpr int STAGES = 3 * STAGE_BYTES <= 160 * 1024 ? 3 : 2;
   constexpr int XCOPIES = TM / 8 / 8;                   // 1 KiB copies (8 rows) per wavefront, x tile
   constexpr int WGROUPS = TN / 8;                       // 8-row groups of the w tile
   constexpr int WCOPIES = (WGROUPS + 7) / 8;
@@ -261,52 +263,62 @@ w8a8_int8_gemm_kernel(I8Args a) {
   static_assert(NM > CP0 + CPE * (NSLOT - 1) && NM >= RE * (NJ + NI), "not enough MFMAs to spread the copies and reads");
 
   // The K tiles of all the output tiles of this workgroup form one stream;
-  // stream element g lives in LDS stage g % 2.  Half 0 of element g multiplies
+  // stream element g lives in LDS stage g % STAGES.  Half 0 of element g multiplies
   // (g, 0) while it reads (g, 1); half 1 multiplies (g, 1) while it reads
-  // (g + 1, 0) and issues the copy of element g + 2 into g's stage.  The
+  // (g + 1, 0) and issues the copy of element g + STAGES into g's stage.  The
   // barrier between the halves means: everybody's copies of element g + 1 have
-  // landed, and everybody has finished reading element g.  The stream runs
-  // across output tiles, so the first K tiles of the next output tile arrive
-  // while the epilogue of this one runs; past the last output tile the copies
-  // re-read its last K tile into a stage nobody reads.
+  // landed, and everybody has finished reading element g.  With two stages that
+  // is a wait for every copy of this wavefront; with three the copies of
+  // element g + 2, issued one element ago, stay in flight (the wait leaves the
+  // last NSLOT: every wavefront issues exactly NSLOT copies per element there).
+  // The stream runs across output tiles, so the first K tiles of the next
+  // output tile arrive while the epilogue of this one runs; past the last
+  // output tile the copies re-read its last K tile into a stage nobody reads.
+  static_assert(STAGES == 2 || (WCOPIES * 8 == WGROUPS && NSLOT == 6), "the three-stage wait counts six copies per wavefront and element");
   const int nt = K / TKB;
   // (kept in a register: read through the dispatch packet it is fetched again in every iteration)
   const int gdim = __builtin_amdgcn_readfirstlane((int)gridDim.x);
   int tile = blockIdx.x;
-  set_copy_tile(tile);
-  issue(0, 0);
-  issue(1, min(1, nt - 1) * TKB);
   int copy_tile = tile;
-  if (nt == 1 && tile + gdim < total_tiles) {      // element 1 already belongs to the next output tile
-    copy_tile = tile + gdim;
-    set_copy_tile(copy_tile);
-    issue(1, 0);
-  }
-  __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
+  set_copy_tile(tile);
+  // K tile of the element d ahead of K tile T of `tile`, after moving the copy offsets to its
+  // output tile; past the last output tile a harmless re-read that is never consumed
+  auto ahead_k0 = [&](int T, int d) {
+    int kt = T + d, ahead = 0;
+    while (kt >= nt) { kt -= nt; ++ahead; }
+    const int want = tile + ahead * gdim;
+    if (want >= total_tiles) return (nt - 1) * TKB;
+    if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
+    return kt * TKB;
+  };
+  auto wait_landed = [&]() {
+    if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f76);   // vmcnt(6): all but the newest element
+    else __builtin_amdgcn_s_waitcnt(0x0f70);                          // vmcnt(0)
+  };
+#pragma unroll
+  for (int d = 0; d < STAGES; ++d) issue(d, ahead_k0(0, d));
+  if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f7c);     // vmcnt(12): element 0 landed
+  else __builtin_amdgcn_s_waitcnt(0x0f70);
   __builtin_amdgcn_s_barrier();
   Frag f0, f1;
   read_frag(f0, 0, 0);
   lds_wait(f0);
-  int g = 0;                                       // stream position of the current K tile
+  int st = 0;                                      // stage of the current K tile
   for (; tile < total_tiles; tile += gdim) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) acc[i][j] = (i4){0, 0, 0, 0};
-    for (int T = 0; T < nt; ++T, ++g) {
-      const int st = g & 1;
+    for (int T = 0; T < nt; ++T) {
+      const int nst = st + 1 == STAGES ? 0 : st + 1;
       half(f0, f1, st, 1, 0, 0, 0, 1, st, 0);
       lds_wait(f1);
-      __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): my copies of element g + 1 landed
+      wait_landed();                               // my copies of the next element landed
       __builtin_amdgcn_s_barrier();                // bare barrier: the waits are explicit, no fence needed
-      // element g + 2: K tile (T + 2) % nt of output tile number (T + 2) / nt after this one
-      int kt = T + 2, ahead = 0;
-      while (kt >= nt) { kt -= nt; ++ahead; }
-      const int want = tile + ahead * gdim;
-      if (want >= total_tiles) kt = nt - 1;        // past the end: harmless re-read, never consumed
-      else if (want != copy_tile) { set_copy_tile(want); copy_tile = want; }
-      half(f1, f0, st ^ 1, 0, 0, NSLOT, CP0, CPE, st, kt * TKB);
+      const int k0 = ahead_k0(T, STAGES);
+      half(f1, f0, nst, 0, 0, NSLOT, CP0, CPE, st, k0);
       lds_wait(f0);
+      st = nst;
     }
 
     // ---- epilogue: lane holds, per (n tile i, m tile j), output row
@@ -354,7 +366,8 @@ w8a8_int8_gemm_kernel(I8Args a) {
     // rather than kept from the last half above: that frees their registers
     // for the epilogue (the copy has landed: it was waited for at the last
     // barrier of the K loop).
-    read_frag(f0, g & 1, 0);
+    if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f70);   // the stores counted too: start again from zero
+    read_frag(f0, st, 0);
     lds_wait(f0);
   }
   // no copy may still be writing LDS when the workgroup retires
@@ -464,7 +477,8 @@ int launch_tile(const I8Args& a, hipStream_t st) {
   const int mtiles = (a.M + TM - 1) / TM, ntiles = (a.N + TN - 1) / TN;
   I8Args b = a;
   b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
-  const size_t shmem = 2 * (size_t)(TM + TN) * TKB;      // two stages, 120 or 128 KiB
+  const size_t stage = (size_t)(TM + TN) * TKB;
+  const size_t shmem = (3 * stage <= 160 * 1024 ? 3 : 2) * stage;   // 144 KiB (three stages), 120 or 128 KiB (two)
   static hipError_t attr = hipFuncSetAttribute((const void*)w8a8_int8_gemm_kernel<DT, WM, WN, NI, NJ>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   MQ_REQUIRE(attr == hipSuccess, "w8a8_int8_gemm: cannot reserve %zu bytes of LDS: %s", shmem,
