@@ -1041,9 +1041,12 @@ def _kcontig(out, a, w, a_scale, w_scale, bias, mode, group):
 # the MFMA tile kernel beats the weight-streaming kernel above 64 rows once its tiles fill a good part of
 # the chip (measured, K 8192 N 28672 = 224 tiles: M 65..128 69..73 us against 87..119 us, M 64 68 us
 # against 73 us for the streamer's last single-block size; K 7168 N 4096 = 32 tiles: 52 us against
-# 37..53 us at M 65..128, so few tiles stay with the streamer)
+# 37..53 us at M 65..128, so few tiles stay with the streamer).  The tile kernel needs about 1 us
+# per K block however few tiles there are; the streamer's time grows with the rows: they cross at
+# 48..64 tiles (K 7168 N 4096: 32 tiles 56 against 31 us, 64 tiles 55 against 58 us, 96 tiles 56
+# against 85 us; the same on K 4096 N 4096, K 2048 N 7168 and K 7168 N 2048)
 _FP8_TILE_MIN_M = 64
-_FP8_TILE_MIN_TILES = 96
+_FP8_TILE_MIN_TILES = 64
 
 
 def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
