@@ -175,9 +175,12 @@ int mi355q_moe_align_block_size(const void* topk_ids, int ids_are_int64, int num
 
 /* ---- activation glue --------------------------------------------------------
  * silu_and_mul / silu_and_mul_pad (csrc/src/silu_and_mul.cpp:29-109,
- * silu_and_mul_pad.cpp:27-90): out[r, :d] = silu(x[r, :d]) * x[r, d:2d]. */
+ * silu_and_mul_pad.cpp:27-90): out[r, :d] = silu(x[r, :d]) * x[r, d:2d].
+ * valid_rows (device int32[1], optional) counts leading units of rows_per_count rows each (tokens of
+ * top-k slot rows): only the first *valid_rows * rows_per_count rows are processed; the product is
+ * taken on the device, so a captured graph may change the count between replays. */
 int mi355q_silu_and_mul(void* out, const void* x, long rows, int d, int dtype,
-                        const int32_t* valid_rows, void* stream);
+                        const int32_t* valid_rows, int rows_per_count, void* stream);
 /* dynamic_per_token_group_fp8_quant(_with_size) and, with fuse_silu_mul,
  * silu_mul_per_token_group_quant(_with_size)
  * (csrc/src/dynamic_per_token_group_fp8_quant.cpp:15-84,
@@ -185,7 +188,8 @@ int mi355q_silu_and_mul(void* out, const void* x, long rows, int d, int dtype,
  * s = max(absmax, 1e-10) / 448, q = e4m3fn(clamp(x / s)).  x is [rows, K]
  * (or [rows, 2K] when fused); scales [rows, K / group_size] row-major. */
 int mi355q_fp8_group_quant(uint8_t* out, float* scales, const void* x, long rows, int K, int group_size,
-                           int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream);
+                           int fuse_silu_mul, int dtype, const int32_t* valid_rows, int rows_per_count,
+                           void* stream);
 /* dynamic_per_token_scaled_fp8_quant (csrc/src/dynamic_per_token_scaled_fp8_quant.cpp): one scale per row */
 int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x, int rows, int K, int dtype,
                            const int32_t* valid_rows, void* stream);
@@ -194,7 +198,8 @@ int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x, int rows,
  * q = e4m3fn(clamp(v / scale)) with one fp32 scale; fuse_silu_mul 0: v = x [rows, K];
  * 1: v = silu(x[:, :K]) * x[:, K:] of x [rows, 2K]; 2: v = x[:, :K] * x[:, K:] */
 int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, long rows, int K,
-                            int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream);
+                            int fuse_silu_mul, int dtype, const int32_t* valid_rows, int rows_per_count,
+                            void* stream);
 /* rms_norm / fused_add_rms_norm and their fusions with the activation quantisers
  * (csrc/torch_bindings.cpp:254-272 rms_norm, fused_add_rms_norm; :277-317 *_static_fp8_quant;
  * :852-871 *_static_int8_quant; :1124-1143 *_per_token_group_quant_fp8; equivalences

@@ -449,3 +449,57 @@ def test_config3_full_size_properties_and_sample(ops, rearrange):
     want = om.fused_experts(x[tok:tok + 1].float().numpy(), lambda e: expert(w13, z13, s13, e),
                             lambda e: expert(w2, z2, s2, e), two[tok:tok + 1], e_tok[None, :], f16)
     np.testing.assert_allclose(out[tok:tok + 1].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("block", [16, 32, 64])
+def test_expert_map_with_non_local_experts_zeroes_their_rows(fmoe, ops, rearrange, block):
+    """Under an expert map the reference maps non-local experts to -1 (fused_moe.py:70-71, 106-107).
+    Blocks of such experts must read no weights and leave zeros in their slot rows; local experts are
+    renumbered.  Checked through both align paths and the three grouped kernels (int4 streaming /
+    MFMA tile by block size, K-contiguous fp16)."""
+    print(f"case expert_map -1 block={block}", flush=True)
+    rng = np.random.default_rng(40 + block)
+    M, E, T, K, N = 45, 6, 2, 256, 384
+    emap = np.array([-1, 0, -1, 1, 2, -1], dtype=np.int32)      # 3 local experts
+    L = 3
+    q, z, s = make_int4_experts(rng, L, K, N)
+    w, zp = int4_to_device(rearrange, q, z)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    flat = ids.reshape(-1)
+    assert (emap[flat] < 0).any() and (emap[flat] >= 0).any()
+    wf = lambda e: ow4.dequantize(q[e], z[e], s[e].astype(np.float32), 128)
+    want = np.zeros((M * T, N), dtype=np.float32)
+    for t in range(M * T):
+        le = emap[flat[t]]
+        if le >= 0:
+            want[t] = x[t // T].astype(np.float32) @ wf(le)
+    cfg = {"BLOCK_SIZE_M": block}
+    count = torch.full((1,), M, dtype=torch.int32, device="cuda")
+    for topk_ids_size in (None, count):      # plain align + host-side map; exts align with the map inside
+        so, eo, no = fmoe.moe_align_block_size(dev(ids), block, E, dev(emap), topk_ids_size)
+        assert (eo[: int(no.item()) // block].cpu().numpy() < L).all()
+        C = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
+        fmoe.invoke_fused_moe_kernel(dev(x), w, C, None, dev(s), zp, dev(tw), dev(ids), so, eo, no, False, T, cfg,
+                                     use_fp8_w8a8=False, use_int8_w8a8=False, use_int8_w8a16=False,
+                                     use_int4_w4a16=True, block_shape=[0, 128])
+        torch.cuda.synchronize()
+        got = C.view(-1, N).float().cpu().numpy()
+        assert np.isfinite(got).all()
+        assert (got[emap[flat] < 0] == 0).all()
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+    # the K-contiguous kernel (unquantised fp16 experts)
+    wf16 = (rng.standard_normal((L, N, K)) * 0.05).astype(np.float16)
+    so, eo, no = fmoe.moe_align_block_size(dev(ids), block, E, dev(emap), None)
+    C = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
+    fmoe.invoke_fused_moe_kernel(dev(x), dev(wf16), C, None, None, None, dev(tw), dev(ids), so, eo, no, False, T, cfg,
+                                 use_fp8_w8a8=False, use_int8_w8a8=False, use_int8_w8a16=False, use_int4_w4a16=False)
+    torch.cuda.synchronize()
+    got = C.view(-1, N).float().cpu().numpy()
+    want = np.zeros((M * T, N), dtype=np.float32)
+    for t in range(M * T):
+        le = emap[flat[t]]
+        if le >= 0:
+            want[t] = x[t // T].astype(np.float32) @ wf16[le].astype(np.float32).T
+    assert (got[emap[flat] < 0] == 0).all()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)

@@ -301,3 +301,44 @@ def test_moe_sum_pad(ops, dtype, odtype):
     else:
         assert np.array_equal(got[:41], torch.from_numpy(want[:41]).to(odtype).float().numpy())
     assert np.all(got[41:] == 3.0)
+
+
+def test_valid_token_count_is_read_on_the_device_under_graph_replay(ops):
+    """The ``*_pad`` / ``*_with_size`` operators take a device count so that a captured graph can be
+    replayed with another number of valid tokens: the count (tokens) times the slots per token must
+    be taken inside the kernel, not on the host at capture time."""
+    rng = np.random.default_rng(3)
+    M, T, D = 24, 4, 256
+    x = dev(rng.standard_normal((M, T, 2 * D)).astype(np.float16))
+    count = torch.full((1,), M, dtype=torch.int32, device="cuda")
+    out = torch.zeros((M, T, D), dtype=torch.float16, device="cuda")
+    q = torch.zeros((M, T, D), dtype=torch.float8_e4m3fn, device="cuda")
+    qs = torch.zeros((M, T, D // 128), dtype=torch.float32, device="cuda")
+
+    def step():
+        torch.ops._C.silu_and_mul_pad(out, x, count)
+        torch.ops._C.silu_mul_per_token_group_quant_with_size(q, qs, x, count, 128)
+
+    step()                                      # eager warm-up, as a serving loop does before capturing
+    torch.cuda.synchronize()
+    full = out.clone()
+    full_q = q.view(torch.uint8).clone()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for n in (M, 5, 17, 0, M):
+        count.fill_(n)
+        out.fill_(-1.0)
+        q.view(torch.uint8).fill_(0x7f)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out[:n], full[:n]), n
+        assert (out[n:] == -1.0).all(), n       # rows past the count are left alone
+        assert torch.equal(q.view(torch.uint8)[:n], full_q[:n]), n
+        assert (q.view(torch.uint8)[n:] == 0x7f).all(), n

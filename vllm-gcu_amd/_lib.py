@@ -41,11 +41,12 @@ SIGNATURES = {
                                     c_int, c_int, c_void_p]),
     "mi355q_moe_align_block_size": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_void_p]),
-    "mi355q_silu_and_mul": (c_int, [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_silu_and_mul": (c_int, [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_void_p]),
     "mi355q_fp8_group_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p,
-                                       c_void_p]),
+                                       c_int, c_void_p]),
     "mi355q_fp8_token_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "mi355q_fp8_static_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi355q_fp8_static_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int,
+                                        c_void_p]),
     "mi355q_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_long, c_int,
                                 c_int, c_int, c_int, c_void_p]),
     "mi355q_fp8_to_half": (c_int, [c_void_p, c_void_p, c_long, c_int, c_void_p]),

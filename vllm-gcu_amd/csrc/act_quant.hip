@@ -76,8 +76,8 @@ struct SharedDivisor {
 // ---- silu_and_mul: out[r, :d] = silu(x[r, :d]) * x[r, d:] -------------------
 template <int DT>
 __global__ void __launch_bounds__(256)
-silu_and_mul_kernel(uint16_t* out, const uint16_t* x, long rows, int d, const int* valid_rows) {
-  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+silu_and_mul_kernel(uint16_t* out, const uint16_t* x, long rows, int d, const int* valid_rows, int rpc) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows) * rpc) : rows;
   const int chunks = d / 8;
   const long total = nrow * chunks;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
@@ -97,8 +97,8 @@ silu_and_mul_kernel(uint16_t* out, const uint16_t* x, long rows, int d, const in
 template <int DT, bool SILU>
 __global__ void __launch_bounds__(256)
 group_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, long rows, int K, int gs,
-                       const int* valid_rows) {
-  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+                       const int* valid_rows, int rpc) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows) * rpc) : rows;
   const int chunks = K / 8;                      // 8-element chunks per output row
   const int lpg = gs / 8;                        // lanes per group (power of two <= 64)
   const long total = nrow * chunks;
@@ -164,8 +164,8 @@ token_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, int K, co
 template <int DT, int FUSE>
 __global__ void __launch_bounds__(256)
 static_fp8_quant_kernel(uint8_t* out, const uint16_t* x, const float* scale, long rows, int K,
-                        const int* valid_rows) {
-  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows)) : rows;
+                        const int* valid_rows, int rpc) {
+  const long nrow = valid_rows ? min(rows, (long)max(0, *valid_rows) * rpc) : rows;
   const float s = *scale;
   if ((K & 7) == 0) {
     // 8 elements per lane and step: 16-byte loads, 8-byte stores
@@ -351,15 +351,16 @@ using namespace mi355q;
   } while (0)
 
 extern "C" int mi355q_silu_and_mul(void* out, const void* x, long rows, int d, int dtype,
-                                   const int32_t* valid_rows, void* stream) {
+                                   const int32_t* valid_rows, int rows_per_count, void* stream) {
+  if (rows_per_count < 1) rows_per_count = 1;
   MQ_REQUIRE(rows >= 0 && d > 0 && d % 8 == 0, "silu_and_mul: bad shape rows=%ld d=%d (d %% 8 == 0)", rows, d);
   if (rows == 0) return 0;
   MQ_REQUIRE(out && x, "silu_and_mul: null pointer");
   hipStream_t st = as_stream(stream);
   unsigned g = grid_for(rows * (d / 8));
   MQ_DISPATCH_16(dtype,
-    hipLaunchKernelGGL((silu_and_mul_kernel<MI355Q_F16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint16_t*)x, rows, d, valid_rows),
-    hipLaunchKernelGGL((silu_and_mul_kernel<MI355Q_BF16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint16_t*)x, rows, d, valid_rows),
+    hipLaunchKernelGGL((silu_and_mul_kernel<MI355Q_F16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint16_t*)x, rows, d, valid_rows, rows_per_count),
+    hipLaunchKernelGGL((silu_and_mul_kernel<MI355Q_BF16>), dim3(g), dim3(256), 0, st, (uint16_t*)out, (const uint16_t*)x, rows, d, valid_rows, rows_per_count),
     "silu_and_mul");
   MQ_LAUNCH_CHECK("silu_and_mul");
   return 0;
@@ -367,7 +368,8 @@ extern "C" int mi355q_silu_and_mul(void* out, const void* x, long rows, int d, i
 
 extern "C" int mi355q_fp8_group_quant(uint8_t* out, float* scales, const void* x, long rows, int K,
                                       int group_size, int fuse_silu_mul, int dtype,
-                                      const int32_t* valid_rows, void* stream) {
+                                      const int32_t* valid_rows, int rows_per_count, void* stream) {
+  if (rows_per_count < 1) rows_per_count = 1;
   MQ_REQUIRE(rows >= 0 && K > 0, "fp8_group_quant: bad shape rows=%ld K=%d", rows, K);
   if (rows == 0) return 0;
   MQ_REQUIRE(out && scales && x, "fp8_group_quant: null pointer");
@@ -379,13 +381,13 @@ extern "C" int mi355q_fp8_group_quant(uint8_t* out, float* scales, const void* x
   unsigned g = grid_for(rows * (K / 8));
   if (fuse_silu_mul) {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_F16, true>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
-      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_BF16, true>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_F16, true>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows, rows_per_count),
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_BF16, true>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows, rows_per_count),
       "fp8_group_quant");
   } else {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_F16, false>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
-      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_BF16, false>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows),
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_F16, false>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows, rows_per_count),
+      hipLaunchKernelGGL((group_fp8_quant_kernel<MI355Q_BF16, false>), dim3(g), dim3(256), 0, st, out, scales, (const uint16_t*)x, rows, K, group_size, valid_rows, rows_per_count),
       "fp8_group_quant");
   }
   MQ_LAUNCH_CHECK("fp8_group_quant");
@@ -407,7 +409,9 @@ extern "C" int mi355q_fp8_token_quant(uint8_t* out, float* scales, const void* x
 }
 
 extern "C" int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float* scale, long rows, int K,
-                                       int fuse_silu_mul, int dtype, const int32_t* valid_rows, void* stream) {
+                                       int fuse_silu_mul, int dtype, const int32_t* valid_rows,
+                                       int rows_per_count, void* stream) {
+  if (rows_per_count < 1) rows_per_count = 1;
   MQ_REQUIRE(rows >= 0 && K > 0, "fp8_static_quant: bad shape rows=%ld K=%d", rows, K);
   if (rows == 0) return 0;
   MQ_REQUIRE(out && scale && x, "fp8_static_quant: null pointer");
@@ -416,18 +420,18 @@ extern "C" int mi355q_fp8_static_quant(uint8_t* out, const void* x, const float*
   MQ_REQUIRE(fuse_silu_mul >= 0 && fuse_silu_mul <= 2, "fp8_static_quant: unknown fusion %d", fuse_silu_mul);
   if (fuse_silu_mul == 1) {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 1>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 1>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 1>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows, rows_per_count),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 1>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows, rows_per_count),
       "fp8_static_quant");
   } else if (fuse_silu_mul == 2) {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 2>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 2>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 2>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows, rows_per_count),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 2>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows, rows_per_count),
       "fp8_static_quant");
   } else {
     MQ_DISPATCH_16(dtype,
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 0>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
-      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 0>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_F16, 0>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows, rows_per_count),
+      hipLaunchKernelGGL((static_fp8_quant_kernel<MI355Q_BF16, 0>), dim3(g), dim3(256), 0, st, out, (const uint16_t*)x, scale, rows, K, valid_rows, rows_per_count),
       "fp8_static_quant");
   }
   MQ_LAUNCH_CHECK("fp8_static_quant");

@@ -86,6 +86,20 @@ __device__ __forceinline__ void use_agpr_accumulators() {
   asm volatile("" : "+a"(t));
 }
 
+// Fused-MoE grouped GEMMs: a block whose expert id lies outside [0, E) -- a non-local expert under an
+// expert map, -1 in the reference (vllm_gcu/kernels/fused_moe.py:70-71, 106-107) -- contributes
+// nothing.  Its workgroups read no weights and zero the columns [col0, col0 + ncols) (ncols % 4 == 0)
+// of every valid slot row of the block; `ids` are the block's `rows` slot ids, pads >= numel.
+__device__ __forceinline__ void zero_block_columns(uint16_t* out, const int* ids, int rows, int numel, int N,
+                                                   int col0, int ncols, int nthreads) {
+  const int per_row = ncols >> 2;
+  for (int i = threadIdx.x; i < rows * per_row; i += nthreads) {
+    const int r = i / per_row, piece = i - r * per_row;
+    const int id = ids[r];
+    if (id < numel) *(uint2*)(out + (size_t)id * N + col0 + 4 * piece) = make_uint2(0u, 0u);
+  }
+}
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 int device_cu_count();

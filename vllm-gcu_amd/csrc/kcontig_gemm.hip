@@ -44,7 +44,7 @@ struct KcArgs {
   const int* expert_ids;
   const int* npp;
   const float* topk_weights;
-  int numel, topk, block_size;
+  int numel, topk, block_size, E;
   long w_stride, ws_stride;    // per-expert strides (elements)
 };
 
@@ -129,6 +129,11 @@ kcontig_gemm_kernel(KcArgs a) {
   if (GROUPED) {
     if (m0 >= *a.npp) return;
     expert = a.expert_ids[m0 / a.block_size];
+    if (expert < 0 || expert >= a.E) {             // not one of this rank's experts: zero rows, no weights read
+      const int col0 = blockIdx.x * 256;
+      zero_block_columns((uint16_t*)a.out, a.sorted_ids + m0, BM, a.numel, N, col0, min(256, N - col0), 256);
+      return;
+    }
     for (int r = tid; r < BM; r += 256) tok[r] = a.sorted_ids[m0 + r];
     __syncthreads();
   }
@@ -516,7 +521,7 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = nullptr;
   g.M = numel; g.N = N; g.K = K; g.kslab = w_layout;
   g.sorted_ids = sorted_token_ids; g.expert_ids = expert_ids; g.npp = num_tokens_post_pad;
-  g.topk_weights = topk_weights; g.numel = numel; g.topk = topk; g.block_size = block_size;
+  g.topk_weights = topk_weights; g.numel = numel; g.topk = topk; g.block_size = block_size; g.E = E;
   g.w_stride = (long)N * K;
   int mode;
   if (quant_mode == 1) {

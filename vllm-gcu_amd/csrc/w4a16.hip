@@ -18,6 +18,13 @@ using namespace mi355q;
 
 static constexpr size_t TILE_WS_OFFSET = (size_t)1 << 20;
 
+// streaming kernel up to 32 rows; 33..64 rows: the MFMA kernel where its pipelined loop exists
+// (fp16, integer zero-points; measured equal or up to 22 % faster there), else streaming again
+static int auto_family(int M, int group_size, int zeros_kind, int dtype) {
+  const bool piped = dtype == MI355Q_F16 && zeros_kind != MI355Q_ZP_PRESCALED;
+  return (group_size % 128 != 0 || M <= 32 || (M <= 64 && !piped)) ? 1 : 2;
+}
+
 extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const size_t s = w4a16_stream_workspace_bytes(M > 64 ? 64 : M, N);
@@ -48,12 +55,7 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
              "w4a16_gemm: unknown zeros_kind %d", zeros_kind);
   MQ_REQUIRE(zeros_kind == MI355Q_ZP_NONE || zeros, "w4a16_gemm: zeros pointer missing");
   MQ_REQUIRE(family >= 0 && family <= 2, "w4a16_gemm: unknown kernel family %d", family);
-  if (family == 0) {
-    // streaming kernel up to 32 rows; 33..64 rows: the MFMA kernel where its pipelined loop exists
-    // (fp16, integer zero-points; measured equal or up to 22 % faster there), else streaming again
-    const bool piped = dtype == MI355Q_F16 && zeros_kind != MI355Q_ZP_PRESCALED;
-    family = (group_size % 128 != 0 || M <= 32 || (M <= 64 && !piped)) ? 1 : 2;
-  }
+  if (family == 0) family = auto_family(M, group_size, zeros_kind, dtype);
   MQ_REQUIRE(family != 2 || group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   if (family == 1) {

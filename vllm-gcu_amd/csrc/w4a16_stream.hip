@@ -35,7 +35,7 @@ struct StreamArgs {
   const int32_t* expert_ids;    // [blocks]
   const int32_t* npp;           // device scalar: slots after padding
   const float* topk_weights;    // [numel] or null
-  int numel, topk;
+  int numel, topk, E;
   long w_stride, s_stride, z_stride;   // per expert, in elements of the respective arrays (weights: 16-byte units)
 };
 
@@ -204,6 +204,19 @@ w4a16_stream_kernel(StreamArgs a) {
   if (GR) {
     if ((int)blockIdx.z * 16 * MT >= *a.npp) return;
     const long e = a.expert_ids[blockIdx.z];
+    if (e < 0 || e >= a.E) {
+      // not one of this rank's experts (-1 under an expert map): zero the block's valid slot rows in this
+      // workgroup's columns and read no weights
+      const int zr = threadIdx.x >> 4, zc = threadIdx.x & 15;
+      const float zero[NT] = {};
+      const int col = 128 * (int)(blockIdx.x / (8 / NT)) + 8 * zc + (int)(blockIdx.x % (8 / NT)) * NT;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int id = a.sorted_ids[(int)blockIdx.z * 16 * MT + 16 * mt + zr];
+        if (id < a.numel) store_out_row<DT, NT>(a.out + (size_t)id * a.N + col, nullptr, col, zero);
+      }
+      return;
+    }
     a.qw += e * a.w_stride;
     a.scales += e * a.s_stride;
     if (ZK == MI355Q_ZP_PACKED) a.zeros = (const uint32_t*)a.zeros + e * a.z_stride;
@@ -459,10 +472,14 @@ w4a16_stream_kernel(StreamArgs a) {
 
   // ---- cross-workgroup split-K ---------------------------------------------
   // Partial tiles travel as device-scope relaxed accesses (they bypass the
-  // per-XCD L2 instead of flushing it); the barrier's wait for outstanding
-  // stores orders them before the arrival count.  The last workgroup to
-  // arrive adds the tiles in split order, so the sum is reproducible.
+  // per-XCD L2 instead of flushing it).  Every wavefront waits until its own
+  // partial stores have been acknowledged (vmcnt counts stores on gfx9) and
+  // only then joins the barrier that precedes the arrival count -- the
+  // barrier alone does not wait for memory operations in flight.  The last
+  // workgroup to arrive adds the tiles in split order, so the sum is
+  // reproducible.
   __shared__ int is_last;
+  __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
   __syncthreads();
   if (threadIdx.x == 0) {
     int old = __hip_atomic_fetch_add(a.counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -635,7 +652,7 @@ static void launch_grouped_nt(const StreamArgs& a, int mt, int nt, int blocks, h
 int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                                 const void* zeros, int zeros_kind, const float* topk_weights,
                                 const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
-                                int numel, int topk, int block_size, int max_blocks, int K, int N,
+                                int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                                 int group_size, int dtype, hipStream_t st) {
   MQ_REQUIRE(block_size == 16 || block_size == 32, "moe_w4a16(stream): blocks of 16 or 32 slots, got %d", block_size);
   const int mt = block_size / 16;
@@ -657,7 +674,7 @@ int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight
   a.gs_magic = (uint32_t)((((uint64_t)1 << 32) + group_size - 1) / group_size);
   a.splits = 1;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
-  a.numel = numel; a.topk = topk;
+  a.numel = numel; a.topk = topk; a.E = E;
   a.w_stride = (long)(K / 8) * N / 4;
   a.s_stride = (long)(K / group_size) * N;
   a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;

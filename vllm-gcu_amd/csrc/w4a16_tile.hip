@@ -38,7 +38,7 @@ struct TileArgs {
   const int* expert_ids;      // [blocks]
   const int* npp;             // device scalar: padded id count
   const float* topk_weights;  // [numel] or null
-  int numel, topk;
+  int numel, topk, E;
   // dense split-K: blockIdx.z takes K blocks [z * kper, (z + 1) * kper) and writes an fp32
   // partial tile to partial[z][M][N]; a second kernel adds the partials up
   int kper;                   // K blocks per split (G when there is no split)
@@ -131,6 +131,11 @@ w4a16_tile_kernel(TileArgs a) {
   if (GROUPED) {
     if (m0 >= *a.npp) return;                       // block beyond the padded ids
     const long e = a.expert_ids[blockIdx.y];
+    if (e < 0 || e >= a.E) {                        // not one of this rank's experts: zero rows, no weights read
+      const int col0 = blockIdx.x * BN;
+      zero_block_columns(a.out, a.sorted_ids + m0, BM, a.numel, N, col0, min(BN, N - col0), NTHR);
+      return;
+    }
     qw += e * a.w_stride;
     if (SF32) scales32 += e * a.s_stride;
     else scales += e * a.s_stride;
@@ -560,7 +565,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
 int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                                 const void* zeros, int zeros_kind, const float* topk_weights,
                                 const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
-                                int numel, int topk, int block_size, int max_blocks, int K, int N,
+                                int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                                 int group_size, int dtype, hipStream_t st);
 
 int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
@@ -578,7 +583,7 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   // which the streaming kernel reads faster than the MFMA tile kernel with one or two row tiles
   if (block_size <= 32 && !scales_f32 && !out_scale)
     return w4a16_stream_grouped_launch(out, x, qweight, scales, zeros, zeros_kind, topk_weights, sorted_ids,
-                                       expert_ids, npp, numel, topk, block_size, max_blocks, K, N, group_size,
+                                       expert_ids, npp, numel, topk, block_size, max_blocks, E, K, N, group_size,
                                        dtype, st);
   TileArgs a = {};
   a.out = (uint16_t*)out;
@@ -592,12 +597,11 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   a.zeros = zeros;
   a.M = numel; a.K = K; a.N = N; a.gs = group_size;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
-  a.numel = numel; a.topk = topk;
+  a.numel = numel; a.topk = topk; a.E = E;
   a.kper = K / 128; a.partial = nullptr;
   a.w_stride = (long)(K / 8) * N / 4;              // u4 elements per expert
   a.s_stride = (long)(K / group_size) * N;
   a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
-  (void)E;
   hipError_t e = (dtype == MI355Q_F16)
                      ? launch_mt<MI355Q_F16, true>(a, zeros_kind, block_size / 16, max_blocks, st)
                      : launch_mt<MI355Q_BF16, true>(a, zeros_kind, block_size / 16, max_blocks, st);

@@ -95,14 +95,16 @@ def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     """out[M, N] = x[M, K] @ dequant(qweight) (+ bias); allocates the output
     like gptq_gemm_gcu (csrc/src/gptq_gemm_gcu.cpp:35)."""
     rt.require_gpu(x, qweight, scales, zeros, bias)
-    if x.dim() != 2:
-        raise RuntimeError(f"w4a16_gemm expects a 2-D activation, got {tuple(x.shape)}")
+    if x.dim() < 1:
+        raise RuntimeError(f"w4a16_gemm expects activations [.., K], got {tuple(x.shape)}")
     qw = _slab_weight(qweight)
+    lead = x.shape[:-1]
+    x = x.reshape(-1, x.shape[-1])
     M, K = x.shape
     N = qw.shape[-1]
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     if x.numel() == 0:
-        return out
+        return out.reshape(lead + (N,))
     if qw.shape[-2] * 8 != K:
         raise RuntimeError(f"w4a16_gemm: activation K={K} does not match weight K={qw.shape[-2] * 8}")
     x = x.contiguous()
@@ -122,10 +124,29 @@ def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
             out.data_ptr(), x.data_ptr(), qw.data_ptr(), scales.data_ptr(), rt.ptr(z), zk, rt.ptr(bias),
             M, K, N, int(group_size), rt.dtype_code(x.dtype), ws.data_ptr(), ws.numel(),
             int(split_k), int(family), rt.stream_ptr()), "w4a16_gemm")
-    return out
+    return out.reshape(lead + (N,))
+
+
+def _require_trivial_g_idx(g_idx: Optional[torch.Tensor], group_size: int) -> None:
+    """The kernels take groups of consecutive rows (gptq.py:141-143 rejects act-order at load time);
+    an operator caller that hands over a permuting ``g_idx`` must not get silently wrong sums.  The
+    check reads the tensor back once and is remembered on it."""
+    if g_idx is None or g_idx.numel() == 0:
+        return
+    tag = (g_idx.data_ptr(), g_idx._version, int(group_size))
+    if getattr(g_idx, "_mi355q_trivial", None) == tag:
+        return
+    K = g_idx.numel()
+    gs = int(group_size) if group_size > 0 else K
+    want = torch.arange(K, device=g_idx.device, dtype=g_idx.dtype) // gs
+    if not bool(torch.equal(g_idx.reshape(-1), want)):
+        raise RuntimeError("gptq_gemm_gcu: act-order checkpoints (a g_idx that is not k // group_size) are "
+                           "not supported")
+    g_idx._mi355q_trivial = tag
 
 
 def _gptq_gemm_gcu_impl(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bit, bias, group_size):
+    _require_trivial_g_idx(b_g_idx, group_size)
     if bit != 4:
         raise RuntimeError("gptq_gemm_gcu: only bit == 4 takes this operator "
                            "(8-bit goes through weight_only_quant)")
@@ -520,7 +541,7 @@ def _rows_last(t: torch.Tensor):
     return t.numel() // t.shape[-1], t.shape[-1]
 
 
-def _silu_and_mul_common(out, input, size):
+def _silu_and_mul_common(out, input, size, rows_per_count=1):
     rt.require_gpu(out, input, size)
     if input.numel() == 0:
         return
@@ -530,32 +551,27 @@ def _silu_and_mul_common(out, input, size):
         raise RuntimeError("silu_and_mul: out must be contiguous [..., d] of the input dtype for input [..., 2d]")
     with torch.cuda.device(x.device):
         _lib.call("mi355q_silu_and_mul", out.data_ptr(), x.data_ptr(), rows, d2 // 2, rt.dtype_code(x.dtype),
-                  rt.ptr(size), rt.stream_ptr())
+                  rt.ptr(size), rows_per_count, rt.stream_ptr())
 
 
 def _silu_and_mul_impl(result, input):
     _silu_and_mul_common(result, input, None)
 
 
-def _leading_rows_to_flat(t: torch.Tensor, size: torch.Tensor) -> torch.Tensor:
-    """``size`` counts entries of the leading dimension (tokens); the kernels
-    work on rows flattened over every dimension but the last."""
-    size = size.to(torch.int32)
+def _leading_rows_to_flat(t: torch.Tensor, size: torch.Tensor):
+    """``size`` counts entries of the leading dimension (tokens); the kernels work on rows flattened
+    over every dimension but the last.  -> (count tensor, rows per counted entry): the product is
+    taken inside the kernel, so a captured graph whose count tensor is rewritten between replays
+    sees the new value."""
+    if size.dtype != torch.int32:
+        size = size.to(torch.int32)
     lead = t.shape[0]
     inner = (t.numel() // t.shape[-1]) // max(lead, 1)
-    if inner == 1:
-        return size
-    # the product is kept on the count tensor (one tiny kernel less per call for counts that live
-    # across calls, like the cached token counts of prepare_finalize); redone if it was written since
-    hit = getattr(size, "_mi355q_scaled", None)
-    if hit is None or hit[0] != (size._version, inner):
-        hit = ((size._version, inner), size * inner)
-        size._mi355q_scaled = hit
-    return hit[1]
+    return size, max(int(inner), 1)
 
 
 def _silu_and_mul_pad_impl(out, input, size):
-    _silu_and_mul_common(out, input, _leading_rows_to_flat(input, size))
+    _silu_and_mul_common(out, input, *_leading_rows_to_flat(input, size))
 
 
 def _fp8_out_ok(out, shape):
@@ -563,7 +579,7 @@ def _fp8_out_ok(out, shape):
         raise RuntimeError(f"fp8 output must be a contiguous float8_e4m3fn tensor of shape {tuple(shape)}")
 
 
-def _group_quant_common(out, scale, input, real_size, group_size, fuse):
+def _group_quant_common(out, scale, input, real_size, group_size, fuse, rows_per_count=1):
     rt.require_gpu(out, scale, input, real_size)
     if input.numel() == 0:
         return
@@ -577,7 +593,8 @@ def _group_quant_common(out, scale, input, real_size, group_size, fuse):
         real_size = real_size.to(torch.int32)
     with torch.cuda.device(x.device):
         _lib.call("mi355q_fp8_group_quant", out.data_ptr(), scale.data_ptr(), x.data_ptr(), rows, K,
-                  int(group_size), int(fuse), rt.dtype_code(x.dtype), rt.ptr(real_size), rt.stream_ptr())
+                  int(group_size), int(fuse), rt.dtype_code(x.dtype), rt.ptr(real_size), rows_per_count,
+                  rt.stream_ptr())
 
 
 def _dynamic_per_token_group_fp8_quant_impl(out, scale, input, group_size):
@@ -585,7 +602,8 @@ def _dynamic_per_token_group_fp8_quant_impl(out, scale, input, group_size):
 
 
 def _dynamic_per_token_group_fp8_quant_with_size_impl(out, scale, input, real_size, group_size):
-    _group_quant_common(out, scale, input, _leading_rows_to_flat(input, real_size), group_size, False)
+    cnt, rpc = _leading_rows_to_flat(input, real_size)
+    _group_quant_common(out, scale, input, cnt, group_size, False, rpc)
 
 
 def _silu_mul_per_token_group_quant_impl(out, scale, input, group_size):
@@ -593,7 +611,8 @@ def _silu_mul_per_token_group_quant_impl(out, scale, input, group_size):
 
 
 def _silu_mul_per_token_group_quant_with_size_impl(out, scale, input, size, group_size):
-    _group_quant_common(out, scale, input, _leading_rows_to_flat(input, size), group_size, True)
+    cnt, rpc = _leading_rows_to_flat(input, size)
+    _group_quant_common(out, scale, input, cnt, group_size, True, rpc)
 
 
 def _dynamic_per_token_scaled_fp8_quant_impl(result, input, scale, scale_ub):
@@ -609,7 +628,7 @@ def _dynamic_per_token_scaled_fp8_quant_impl(result, input, scale, scale_ub):
                   rt.dtype_code(x.dtype), 0, rt.stream_ptr())
 
 
-def _static_fp8_common(out, input, scale, real_rows, fuse):
+def _static_fp8_common(out, input, scale, real_rows, fuse, rows_per_count=1):
     rt.require_gpu(out, input, scale, real_rows)
     if input.numel() == 0:
         return
@@ -622,7 +641,7 @@ def _static_fp8_common(out, input, scale, real_rows, fuse):
         raise RuntimeError("static fp8 quant takes a single scale")
     with torch.cuda.device(x.device):
         _lib.call("mi355q_fp8_static_quant", out.data_ptr(), x.data_ptr(), sc.data_ptr(), rows, K, int(fuse),
-                  rt.dtype_code(x.dtype), rt.ptr(real_rows), rt.stream_ptr())
+                  rt.dtype_code(x.dtype), rt.ptr(real_rows), rows_per_count, rt.stream_ptr())
 
 
 def _static_scaled_fp8_quant_impl(result, input, scale):
@@ -630,11 +649,13 @@ def _static_scaled_fp8_quant_impl(result, input, scale):
 
 
 def _silu_mul_static_fp8_quant_impl(out, input, scale, real_num_tokens):
-    _static_fp8_common(out, input, scale, _leading_rows_to_flat(input, real_num_tokens), 1)
+    cnt, rpc = _leading_rows_to_flat(input, real_num_tokens)
+    _static_fp8_common(out, input, scale, cnt, 1, rpc)
 
 
 def _mul_static_fp8_quant_impl(out, input, scale, real_num_tokens):
-    _static_fp8_common(out, input, scale, _leading_rows_to_flat(input, real_num_tokens), 2)
+    cnt, rpc = _leading_rows_to_flat(input, real_num_tokens)
+    _static_fp8_common(out, input, scale, cnt, 2, rpc)
 
 
 def _silu_mul_static_int8_quant_impl(result, input, scale):
@@ -883,9 +904,12 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
                 raise RuntimeError(f"fp8 expert weights must be [E, N, K]; got {tuple(w.shape)} for K={K}")
         elif A.dtype == torch.int8:
             mode = _lib.Q_INT8
-            a_scale = A_scale.to(torch.float32).reshape(-1).contiguous()
-            if a_scale.numel() not in (A.shape[0],):
-                raise RuntimeError("int8 MoE needs one activation scale per token")
+            a_scale = A_scale.to(torch.float32).reshape(-1)
+            if a_scale.numel() == 1:                    # one static scale for every token
+                a_scale = a_scale.expand(A.shape[0])
+            a_scale = a_scale.contiguous()
+            if a_scale.numel() != A.shape[0]:
+                raise RuntimeError("int8 MoE needs one activation scale, or one per token")
             w_scale = B_scale.to(torch.float32).reshape(B.shape[0], -1).contiguous()
             w = B.contiguous()
         else:

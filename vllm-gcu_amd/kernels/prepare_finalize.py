@@ -31,14 +31,15 @@ _TOKEN_COUNTS = {}
 
 def _token_count(n: int, device: torch.device) -> torch.Tensor:
     """Device scalar ``int32 [1]`` holding ``n``: one per (device, value), never written again
-    (a fresh ``torch.full`` per forward is a kernel launch of its own)."""
+    (a fresh ``torch.full`` per forward is a kernel launch of its own).  A cached scalar is never
+    freed -- a captured graph may hold its address --; past 65536 distinct values new ones are
+    simply not cached (their owner is the caller, or the capturing graph's pool)."""
     key = (device.type, device.index, int(n))
     t = _TOKEN_COUNTS.get(key)
     if t is None:
-        if len(_TOKEN_COUNTS) > 4096:
-            _TOKEN_COUNTS.clear()
         t = torch.full((1,), int(n), dtype=torch.int32, device=device)
-        _TOKEN_COUNTS[key] = t
+        if len(_TOKEN_COUNTS) < 65536:
+            _TOKEN_COUNTS[key] = t
     return t
 
 
