@@ -94,6 +94,20 @@ int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          int dtype, void* workspace, size_t workspace_bytes,
                          int split_k, int family, void* stream);
 
+/* No counterpart in the reference.  mi355q_w4a16_gemm for callers that cannot allocate device memory
+ * or pass a workspace (code under HIP graph capture, serving loops and harnesses that forbid
+ * allocation): same arguments without the workspace, same kernels, bit-identical results.  The
+ * split-K partial tiles and arrival counters live in a fixed array of
+ * mi355q_w4a16_noalloc_scratch_bytes() = 32 MiB of device memory that every GPU running the library
+ * holds until the process ends.  A shape whose split-K plan needs more is rejected with an error
+ * (use mi355q_w4a16_gemm then).  All calls on one GPU share the array: calls that may overlap in time
+ * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ * Calls no allocating routine; enqueues one small clearing kernel before a split-K launch. */
+size_t mi355q_w4a16_noalloc_scratch_bytes(void);
+int mi355q_w4a16_gemm_noalloc(void* out, const void* x, const int32_t* qweight, const void* scales,
+                              const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
+                              int group_size, int dtype, void* stream);
+
 /* fp8-e4m3 block-scaled GEMM for prefill-sized M: the arithmetic of linear_quant
  * (csrc/src/linear_quant.cpp:16-95; vllm_gcu/kernels/quantization/fp8.py:169-205) on an MFMA
  * tile kernel,

@@ -2,12 +2,15 @@
 // streaming (small M) and the LDS-staged MFMA (large M) kernels.
 #include "common.h"
 
+#include <mutex>
+
 namespace mi355q {
 int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                         const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
                         int group_size, int dtype, void* workspace, size_t workspace_bytes,
                         int split_k, hipStream_t st);
 size_t w4a16_stream_workspace_bytes(int M, int N);
+size_t w4a16_stream_plan_workspace_bytes(int M, int K, int N, int gs);
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
                       int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
@@ -85,4 +88,84 @@ extern "C" int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweigh
                                  size_t workspace_bytes, void* stream) {
   return mi355q_w4a16_gemm_ex(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size,
                               dtype, workspace, workspace_bytes, 0, 0, stream);
+}
+
+// ---- the same GEMM for callers that cannot allocate ----------------------------------------------
+// Split-K partial tiles and arrival counters live in a fixed array in device memory instead of a
+// caller's workspace.  Every GPU holds its own copy of the array (at its own address) from the
+// moment the library is loaded there until the process ends; every call on a GPU shares it.
+static constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+namespace {
+__global__ void __launch_bounds__(256) noalloc_clear_kernel(uint32_t* p, int words) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < words) p[i] = 0u;
+}
+
+// device address of `scratch` on the current device, looked up once per device
+int noalloc_scratch_ptr(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64];
+  int dev = 0;
+  MQ_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64, "w4a16_gemm_noalloc: no current device");
+  std::lock_guard<std::mutex> lk(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    MQ_REQUIRE(e == hipSuccess && p, "w4a16_gemm_noalloc: cannot resolve the scratch array on device %d: %s", dev,
+               hipGetErrorString(e));
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return 0;
+}
+}  // namespace
+
+extern "C" size_t mi355q_w4a16_noalloc_scratch_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
+
+extern "C" int mi355q_w4a16_gemm_noalloc(void* out, const void* x, const int32_t* qweight, const void* scales,
+                                         const void* zeros, int zeros_kind, const void* bias, int M, int K,
+                                         int N, int group_size, int dtype, void* stream) {
+  MQ_REQUIRE(M >= 0 && K > 0 && N > 0, "w4a16_gemm_noalloc: bad shape M=%d K=%d N=%d", M, K, N);
+  if (M == 0) return 0;
+  MQ_REQUIRE(K % 128 == 0 && N % 128 == 0,
+             "w4a16_gemm_noalloc: K=%d and N=%d must be multiples of 128 (slab layout)", K, N);
+  const int gs = group_size <= 0 ? K : group_size;
+  MQ_REQUIRE(gs % 32 == 0 && K % gs == 0 && (gs % 128 == 0 || 128 % gs == 0),
+             "w4a16_gemm_noalloc: group_size=%d must be a multiple of 32 dividing K=%d and dividing or a multiple of 128",
+             gs, K);
+  // what the plan of this shape needs, exactly -- the same plan mi355q_w4a16_gemm takes when its
+  // workspace is large enough, so both entry points give bit-identical results
+  const int family = auto_family(M, gs, zeros_kind, dtype);
+  size_t need;
+  bool counters = false;
+  if (family == 1) {
+    const int chunk = gs % 128 == 0 ? 64 : 32;
+    need = w4a16_stream_plan_workspace_bytes(M < chunk ? M : chunk, K, N, gs);
+    if (M > chunk && M % chunk) {
+      const size_t tail = w4a16_stream_plan_workspace_bytes(M % chunk, K, N, gs);
+      need = tail > need ? tail : need;
+    }
+    counters = need > 0;
+  } else {
+    const size_t t = w4a16_tile_workspace_bytes(M, K, N);
+    need = t ? t + TILE_WS_OFFSET : 0;
+  }
+  MQ_REQUIRE(need <= NOALLOC_SCRATCH_BYTES,
+             "w4a16_gemm_noalloc: M=%d K=%d N=%d splits K through %zu bytes of scratch, the fixed array holds %zu; "
+             "use mi355q_w4a16_gemm with a workspace",
+             M, K, N, need, NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = noalloc_scratch_ptr(&ws)) return rc;
+  if (counters) {
+    // the arrival counters must start at zero whatever an earlier call left behind (a fill kernel, not
+    // a memset: callers may be capturing a graph)
+    const int words = N / 16;
+    hipLaunchKernelGGL(noalloc_clear_kernel, dim3((words + 255) / 256), dim3(256), 0, as_stream(stream),
+                       (uint32_t*)ws, words);
+    MQ_LAUNCH_CHECK("w4a16_gemm_noalloc(clear)");
+  }
+  return mi355q_w4a16_gemm_ex(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, ws,
+                              NOALLOC_SCRATCH_BYTES, 0, 0, stream);
 }

@@ -575,6 +575,18 @@ size_t w4a16_stream_workspace_bytes(int M, int N) {
   return STREAM_COUNTER_BYTES + (size_t)32 * Mpad * N * sizeof(float);
 }
 
+// exactly what the automatic plan of a launch of up to 64 rows uses (0: K is not split)
+size_t w4a16_stream_plan_workspace_bytes(int M, int K, int N, int gs) {
+  const StreamPlan plan = w4a16_stream_auto_plan(M, K, N, gs);
+  const int G = K / 128;
+  int splits = plan.splits > G ? G : plan.splits;
+  if (splits > 32) splits = 32;
+  while (splits > 1 && ((G + splits - 1) / splits) * (splits - 1) >= G) --splits;
+  if (splits <= 1) return 0;
+  const int Mpad = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+  return STREAM_COUNTER_BYTES + (size_t)splits * Mpad * N * sizeof(float);
+}
+
 // split_k: bits 0..7 force the split factor, bits 8..15 the tiles per
 // workgroup (1, 2, 4 or 8); 0 in a field = automatic.
 int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
