@@ -237,8 +237,9 @@ def dequantize(q: np.ndarray, z: np.ndarray, s: np.ndarray, group_size: int) -> 
     K, N = q.shape
     g = K if group_size in (-1, 0) else group_size
     zi = np.full((K // g, N), 8, np.float32) if z is None else z.astype(np.float32)
-    qf = q.astype(np.float32).reshape(K // g, g, N)
-    w = (qf - zi[:, None, :]) * s.astype(np.float32)[:, None, :]
+    w = q.astype(np.float32).reshape(K // g, g, N)
+    w -= zi[:, None, :]                    # in place: the same two roundings, no full-size temporaries
+    w *= s.astype(np.float32)[:, None, :]
     return w.reshape(K, N)
 
 

@@ -117,7 +117,7 @@ def test_awq_linear_method(M, dtype):
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
     out = method.apply(layer, x.cuda())
     want = ow4.w4a16_gemm(x.float().numpy(), q, z, sd.float().numpy(), g)
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL * max(1.0, np.abs(want).max() / 8))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
 def test_w8a8_linear_method_static_input_scales():
@@ -186,7 +186,7 @@ def test_fp8_linear_method_block_scaled():
     xq, xs = of8.per_token_group_quant_fp8(x.float().numpy(), 128)
     want = of8.block_fp8_gemm(xq, xs, w, ws) + bias.float().numpy()
     assert out.dtype == torch.bfloat16 and out.shape == (M, N)
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("fmt", ["gptq", "awq"])
@@ -255,7 +255,7 @@ def test_fp8_and_int8_moe_methods_grouped_routing():
 
     want = om.fused_experts(qdq(x.float().numpy()), lambda e: deq(w13[e], s13[e]), lambda e: deq(w2[e], s2[e]),
                             two, ido, bf16, quant_a2=qdq)
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
     # int8 per-channel experts, per-token dynamic activations
     w13i = rng.integers(-127, 128, size=(E, 2 * I, H), dtype=np.int8)
@@ -278,8 +278,8 @@ def test_fp8_and_int8_moe_methods_grouped_routing():
 
     want8 = om.fused_experts(qdq8(x.float().numpy()), lambda e: (w13i[e].astype(np.float32) * c13[e][:, None]).T,
                              lambda e: (w2i[e].astype(np.float32) * c2[e][:, None]).T, two, ido, bf16, quant_a2=qdq8)
-    np.testing.assert_allclose(out8.float().cpu().numpy(), want8, rtol=2 * RTOL,
-                               atol=ATOL * max(1.0, np.abs(want8).max()))
+    np.testing.assert_allclose(out8.float().cpu().numpy(), want8, rtol=RTOL,
+                               atol=ATOL)
 
     # the same experts under the compressed-tensors parameter names
     from vllm_gcu_amd.kernels.quantization.w8a8 import GCUCompressedTensorsW8A8Int8MoEMethod
@@ -341,7 +341,7 @@ def test_moe_w4a8_method(rearranged):
                             lambda e: (w13[e].astype(np.float32) - 8) * np.repeat(s13[e], 128, 0),
                             lambda e: (w2[e].astype(np.float32) - 8) * np.repeat(s2[e], 128, 0),
                             two, ido, bf16, quant_a2=lambda v: fake_quant(v, a2))
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
 def test_fused_qkv_ops_equal_the_unfused_gemm_split_by_columns():
@@ -365,7 +365,7 @@ def test_fused_qkv_ops_equal_the_unfused_gemm_split_by_columns():
                                 dev(xs), dev(ws), 128)
     want = of8.block_fp8_gemm(xq, xs, w, ws)
     got = torch.cat([q, kv], dim=1).float().cpu().numpy()
-    np.testing.assert_allclose(got, want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
     # W4A16, GPTQ checkpoint tensors
     g = 128
     qw = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
@@ -404,7 +404,7 @@ def test_fp8_block_gemm_tile_kernel(M, K, N, kslab, monkeypatch):
     out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     torch.ops._C.linear_quant(out, dev(xq).view(torch.float8_e4m3fn), wd, bias.cuda(), dev(xs), dev(ws))
     want = of8.block_fp8_gemm(xq, xs, w, ws) + bias.float().numpy()
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
     if kslab:
         ref = torch.empty_like(out)
         torch.ops._C.linear_quant(ref, dev(xq).view(torch.float8_e4m3fn), dev(w).view(torch.float8_e4m3fn),
@@ -441,7 +441,7 @@ def test_fp8_full_size_layer_tile_kernel_against_streaming_kernel(monkeypatch):
                               np.repeat(ws.cpu().numpy()[cols // 128], 1, axis=0))
     want = want.reshape(3, len(cols), 128)[:, np.arange(len(cols)), cols % 128]
     got = tile[rows][:, cols].float().cpu().numpy()
-    np.testing.assert_allclose(got, want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("M", [65, 100, 128])
@@ -458,4 +458,4 @@ def test_fp8_dense_65_to_128_rows_single_block(M):
     torch.ops._C.linear_quant(out, dev(xq).view(torch.float8_e4m3fn), dev(w).view(torch.float8_e4m3fn), None,
                               dev(xs), dev(ws))
     want = of8.block_fp8_gemm(xq, xs, w, ws)
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)

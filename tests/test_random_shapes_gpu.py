@@ -1,7 +1,7 @@
 """Seeded random shapes through the dense and grouped operators: every kernel family, row count and ragged
 edge that the routing inside the operators can pick, checked against the oracle.  Outputs are
-allocated full of NaN (or land in memory that was just filled with NaN), so a tile that no
-workgroup writes shows up as NaN instead of as a stale correct value."""
+handed over full of NaN, so a tile that no workgroup writes shows up as NaN instead of as a stale
+correct value."""
 import numpy as np
 import pytest
 import torch
@@ -16,13 +16,6 @@ RTOL = ATOL = 1e-2        # fp16 / bf16 outputs of fp32 accumulation
 
 def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
-
-
-def poison(nbytes):
-    """Fill and free a block of the size the operator is about to allocate: the caching allocator
-    hands the same block out again."""
-    t = torch.full((max(nbytes // 2, 1),), float("nan"), dtype=torch.float16, device="cuda")
-    del t
 
 
 def draw_rows(rng):
@@ -59,8 +52,8 @@ def test_w4a16_random_shapes(seed):
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
     bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(dtype) if with_bias else None
     w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
-    poison(M * N * 2)
-    out = ops.w4a16_gemm(x.cuda(), w, s.cuda(), None if sym else zp, None if bias is None else bias.cuda(), g)
+    out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    ops.w4a16_gemm(x.cuda(), w, s.cuda(), None if sym else zp, None if bias is None else bias.cuda(), g, out=out)
     torch.cuda.synchronize()
     want = ow4.w4a16_gemm(x.float().numpy(), q, z, s.float().numpy(), g,
                           bias=None if bias is None else bias.float().numpy())
@@ -125,8 +118,8 @@ def test_fp8_block_random_shapes(seed, monkeypatch):
     want = of8.block_fp8_gemm(xq, xs, w, ws)
     if bias is not None:
         want = want + bias.float().numpy()
-    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=2 * RTOL,
-                               atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL,
+                               atol=ATOL)
 
 
 @pytest.mark.parametrize("seed", range(16))
@@ -236,4 +229,4 @@ def test_grouped_fp8_and_int8_random_shapes(seed):
     if mul:
         want = want * tw.reshape(-1, 1)
     got = C.view(-1, N).float().cpu().numpy()
-    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL * max(1.0, np.abs(want).max()))
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)

@@ -86,8 +86,11 @@ def test_repack_batched_experts_and_zeros(rearrange):
 # --------------------------------------------------------------- GEMM ----
 def run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=None, split_k=0, family=0):
     w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    # the output starts full of NaN: a tile that no workgroup stores cannot pass as a stale value
+    out = torch.full((x.shape[0], q.shape[1]), float("nan"), dtype=dtype, device="cuda")
     out = ops.w4a16_gemm(to_act(x, dtype).cuda(), w, to_act(s, dtype).cuda(), zp,
-                         None if bias is None else to_act(bias, dtype).cuda(), g, split_k=split_k, family=family)
+                         None if bias is None else to_act(bias, dtype).cuda(), g, split_k=split_k, family=family,
+                         out=out)
     torch.cuda.synchronize()
     return out
 
@@ -139,16 +142,14 @@ def test_stream_gemm_exact_and_split_invariant(ops, rearrange, split_k):
 
 def test_split_k_layers_of_different_width_share_a_workspace(ops, rearrange):
     # one workspace serves every layer: a narrow layer's split-K partial tiles must not land on
-    # the arrival counters a wider layer uses afterwards.  The output allocation is poisoned
-    # first, so a launch that never stores (a corrupted counter) cannot pass on stale memory.
+    # the arrival counters a wider layer uses afterwards.  run_gemm hands over an output full of NaN,
+    # so a launch that never stores (a corrupted counter) cannot pass on stale memory.
     g = 128
     cases = [(4, 1024, 256, 4 | (2 << 8)), (4, 1024, 2048, 2 | (1 << 8)), (4, 1024, 256, 2 | (1 << 8))]
     for i, (M, K, N, split_k) in enumerate(cases):
         print(f"case shared workspace M={M} K={K} N={N} split_k={split_k:#x}", flush=True)
         q, z, s, x = make_case(40 + i, M, K, N, g, exact=True)
         want = torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16)
-        poison = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
-        del poison
         got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, split_k=split_k)
         assert torch.equal(got.cpu(), want)
 

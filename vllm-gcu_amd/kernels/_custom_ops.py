@@ -91,9 +91,10 @@ def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype):
 
 def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
                zeros: Optional[torch.Tensor], bias: Optional[torch.Tensor], group_size: int,
-               split_k: int = 0, family: int = 0) -> torch.Tensor:
+               split_k: int = 0, family: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[M, N] = x[M, K] @ dequant(qweight) (+ bias); allocates the output
-    like gptq_gemm_gcu (csrc/src/gptq_gemm_gcu.cpp:35)."""
+    like gptq_gemm_gcu (csrc/src/gptq_gemm_gcu.cpp:35) unless the caller brings
+    a contiguous ``out [M, N]`` of the activation dtype."""
     rt.require_gpu(x, qweight, scales, zeros, bias)
     if x.dim() < 1:
         raise RuntimeError(f"w4a16_gemm expects activations [.., K], got {tuple(x.shape)}")
@@ -102,7 +103,10 @@ def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     x = x.reshape(-1, x.shape[-1])
     M, K = x.shape
     N = qw.shape[-1]
-    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if out is None:
+        out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    elif out.dtype != x.dtype or out.numel() != M * N or not out.is_contiguous() or not out.is_cuda:
+        raise RuntimeError(f"w4a16_gemm: out must be a contiguous GPU tensor of {M} x {N} {x.dtype} values")
     if x.numel() == 0:
         return out.reshape(lead + (N,))
     if qw.shape[-2] * 8 != K:
