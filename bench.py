@@ -11,6 +11,11 @@ timed with HIP events on the launch stream.
 
 Prints ONE JSON line: whole-job GB/s of algorithmic bytes, the roofline
 fraction of the dominant kernel, and the CPU oracle timed on the host cores.
+The same line carries the rest of the metric: the M = 1 .. 2048 sweep over the
+four shapes (``sweep``), the W8A8 int8 GEMM of configs[2] with its own roofline
+block and CPU baseline (``w8a8_int8``), and the two fused-MoE layers of
+configs[3] / configs[4] (``moe_w4a16``, ``moe_fp8_block``), each with the CPU
+oracle timed on a stated sample.  ``--quick`` leaves those legs out.
 """
 import argparse
 import json
@@ -34,6 +39,9 @@ INT8_PEAK_TOPS = 5000.0
 # copy of --calibrate-copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per
 # unit).  Keyed by (M, --split-k); other settings were not profiled.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 34011114}
+# when and on which build the figure above was taken; it must be re-measured (profiles/ names the
+# commands) whenever the streaming kernel's work split changes
+MEASURED_TRAFFIC_PROVENANCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, 2026-11-25, work split unchanged since"
 
 
 def w4a16_bytes(M, K, N, g=GROUP):
@@ -173,12 +181,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--m", type=int, default=16, help="activation rows of the default workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sweep", action="store_true", help="also time every (shape, M) of the config")
+    ap.add_argument("--sweep", action="store_true", help="(default now) time every (shape, M) of the config")
+    ap.add_argument("--quick", action="store_true",
+                    help="headline, per-layer detail and CPU baseline only: no sweep, no W8A8, no MoE legs")
+    ap.add_argument("--extras", action="store_true",
+                    help="also the decode-sized MoE layer, the w4a8 experts, norm + quant and the fp8 dense linear")
     ap.add_argument("--split-k", type=int, default=0)
     ap.add_argument("--no-w8a8", action="store_true", help="skip the W8A8 int8 GEMM leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a 256 MiB device copy at the end (reference reading for rocprofv3 --pmc)")
-    ap.add_argument("--moe", action="store_true", help="also time the two fused-MoE layers of the config")
+    ap.add_argument("--moe", action="store_true", help="(default now) time the two fused-MoE layers of the config")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); "
@@ -213,6 +225,10 @@ def main():
     step_bytes = sum(w4a16_bytes(M, K, N) for _, K, N in LLAMA3_8B)
     ms_per_step = secs / args.steps * 1e3
     value = step_bytes * args.steps / secs / 1e9
+    # the same step timed over at least 200 steps after at least 20 warm-up steps, whatever --steps says
+    # (a short --steps run is one or two graph replays: consistent, but noisier)
+    n_long = max(args.steps, 200)
+    secs_long = time_graph(step_fns, n_long, max(args.warmup, 20), stream)
 
     # per-layer detail (each layer timed alone, its weights rotating the same way)
     per_layer = {}
@@ -223,23 +239,31 @@ def main():
         b = w4a16_bytes(M, K, N)
         per_layer[name] = {"K": K, "N": N, "us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
                            "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBPS, 4)}
-    # floor: a plain streaming read (no arithmetic, 16-byte loads, 512 workgroups)
-    # of each layer's packed weights, timed the same way
-    from vllm_gcu_amd import _lib
+    # floor: a plain streaming read (no arithmetic, 16-byte loads, nothing stored) of each layer's
+    # packed weights, timed the same way; the best of several grid sizes is quoted
+    import ctypes
     from vllm_gcu_amd.kernels import _runtime as rt
+    probe = ctypes.CDLL(os.path.join(ROOT, "vllm-gcu_amd", "libmi355q_bench.so"))
+    probe.mi355q_bench_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                                               ctypes.c_void_p]
     sink = torch.zeros(16, dtype=torch.uint8, device=dev)
     floor_us = 0.0
     for name, K, N in LLAMA3_8B:
         nbytes = K * N // 2
-        wgs = 512
-        while nbytes % (wgs * 32768):
-            wgs //= 2
-        fns = [(lambda name=name, c=c, nbytes=nbytes, wgs=wgs: _lib.call(
-            "mi355q_probe_stream_read", layers[name][c][0].data_ptr(), nbytes, wgs, sink.data_ptr(),
-            rt.stream_ptr())) for c in range(copies)]
-        n = max(args.steps, 100)
-        t = time_graph(fns, n, args.warmup, stream) / n
+        best = None
+        for wgs in (256, 512, 1024, 2048):
+            def read(c, name=name, nbytes=nbytes, wgs=wgs):
+                rc = probe.mi355q_bench_stream_read(layers[name][c][0].data_ptr(), nbytes, wgs, sink.data_ptr(),
+                                                    rt.stream_ptr())
+                assert rc == 0
+            fns = [(lambda c=c, read=read: read(c)) for c in range(copies)]
+            n = max(args.steps, 100)
+            t = time_graph(fns, n, args.warmup, stream) / n
+            if best is None or t < best[0]:
+                best = (t, wgs)
+        t = best[0]
         per_layer[name]["read_floor_us"] = round(t * 1e6, 3)
+        per_layer[name]["read_floor_workgroups"] = best[1]
         per_layer[name]["time_over_read_floor"] = round(per_layer[name]["us"] / (t * 1e6), 3)
         floor_us += t * 1e6
     # Every launch of a step is the same kernel (w4a16_stream_kernel), so the
@@ -252,7 +276,8 @@ def main():
     roofline = {"bound": "hbm", "kernel": "w4a16_stream_kernel", "launches_per_step": launches,
                 "avg_launch_us": round(launch_us, 3), "algorithmic_bytes_per_launch": step_bytes // launches,
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic}
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                "traffic_provenance": MEASURED_TRAFFIC_PROVENANCE if traffic else None}
     if M > 64:
         # --m above the decode range: the launches are the MFMA tile kernel and the bound is the fp16 matrix peak
         step_flops = sum(2.0 * M * K * N for _, K, N in LLAMA3_8B)
@@ -272,28 +297,33 @@ def main():
                    "weight_copies_rotated": copies, "bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "per_layer": per_layer,
-        "read_floor": {"what": "plain streaming read of the packed weights only, one launch per layer, same graph timing",
+        "stable": {"steps": n_long, "ms_per_step": round(secs_long / n_long * 1e3, 5),
+                   "value": round(step_bytes * n_long / secs_long / 1e9, 2),
+                   "frac_hbm_peak": round(step_bytes * n_long / secs_long / 1e9 / HBM_PEAK_GBPS, 4)},
+        "read_floor": {"what": "plain streaming read of the packed weights only (best of 256..2048 workgroups), one launch "
+                               "per layer, same graph timing",
                        "us_per_step": round(floor_us, 3),
                        "step_time_over_floor": round(ms_per_step * 1e3 / floor_us, 3)},
         "roofline": roofline,
     }
     out["device"] = device_report(dev)
-    if not args.no_w8a8:
-        out["w8a8_int8"] = w8a8_gemm_bench(ops, dev, stream)
-    if args.moe:
-        out["moe_w4a16"] = moe_bench(ops, dev, stream, "w4a16")
+    if not args.no_w8a8 and not args.quick:
+        out["w8a8_int8"] = w8a8_gemm_bench(ops, dev, stream, cpu=not args.no_cpu)
         torch.cuda.empty_cache()
+    if not args.quick:
+        out["sweep"] = sweep(ops, dev, stream, args)
+        out["moe_w4a16"] = moe_bench(ops, dev, stream, "w4a16", cpu=not args.no_cpu)
+        torch.cuda.empty_cache()
+        out["moe_fp8_block"] = moe_bench(ops, dev, stream, "fp8", cpu=not args.no_cpu)
+        torch.cuda.empty_cache()
+    if args.extras:
         out["moe_w4a16_decode"] = moe_bench(ops, dev, stream, "w4a16", tokens=16)
-        torch.cuda.empty_cache()
-        out["moe_fp8_block"] = moe_bench(ops, dev, stream, "fp8")
         torch.cuda.empty_cache()
         out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")
         torch.cuda.empty_cache()
         out["norm_quant"] = glue_bench(ops, dev, stream)
         torch.cuda.empty_cache()
         out["fp8_dense"] = fp8_dense_bench(ops, dev, stream)
-    if args.sweep:
-        out["sweep"] = sweep(ops, dev, stream, args)
     if args.calibrate_copy:
         # a plain copy of known size: its FETCH_SIZE / WRITE_SIZE readings scale
         # the counters of the profiled kernels to bytes
@@ -308,7 +338,29 @@ def main():
     print(json.dumps(out))
 
 
-def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40):
+def cpu_baseline_w8a8(x16, w_nk, ws, rows=2048):
+    """The CPU oracle of configs[2] on the first `rows` token rows against the whole weight: dynamic
+    per-token quantisation, exact int32 GEMM (fp32 matmul over K chunks of 1024), scale epilogue."""
+    import numpy as np
+    import torch
+    from oracle import w8a8 as o8
+    torch.set_num_threads(os.cpu_count() or 1)
+    x = x16[:rows].cpu().numpy()
+    w_kn = np.ascontiguousarray(w_nk.cpu().numpy().T)
+    wsn = ws.cpu().numpy()
+    t0 = time.time()
+    xq, xs = o8.dynamic_scaled_int8_quant(x)
+    acc = o8.int8_gemm_i32(xq, w_kn)
+    o8.scaled_mm_epilogue(acc, xs, wsn).astype(np.float16)
+    dt = time.time() - t0
+    K, N = w_kn.shape
+    return {"value": round(2.0 * rows * K * N / dt / 1e12, 4), "unit": "TOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"oracle.w8a8 (per-token quant + exact int32 GEMM + epilogue) on {rows} of the 2048 token rows "
+                      f"against the whole [8192, 28672] weight, 1 repetition, {dt:.2f} s of CPU work"}
+
+
+def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40, cpu=False):
     """BASELINE configs[2]: W8A8 int8 GEMM, M=2048, K=8192, N=28672 (one
     Llama-3-70B MLP layer), per-token x per-channel scales fused, fp16 out."""
     import torch
@@ -333,16 +385,90 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40):
     outd = torch.empty(Md, N, dtype=torch.float16, device=dev)
     fns = [(lambda w=w: torch.ops._C.cutlass_scaled_mm(outd, xq[:Md], w.t(), xs[:Md], ws, None)) for w in ksl]
     td = time_graph(fns, iters, 3, stream) / iters
+    res_cpu = cpu_baseline_w8a8(x, w_nk, ws) if cpu else None
     return {"workload": "W8A8 int8 GEMM M=2048 K=8192 N=28672, fused per-token x per-channel scales, fp16 out",
             "gemm_us": round(t * 1e6, 1), "TOPs": round(ops_ / t / 1e12, 1),
             "frac_int8_mfma_peak": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
+            "roofline": {"bound": "mfma", "kernel": "w8a8_int8_gemm_kernel", "avg_launch_us": round(t * 1e6, 1),
+                         "algorithmic_ops_per_launch": ops_, "achieved": round(ops_ / t / 1e12, 1),
+                         "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
+                         "timed_launches": iters, "warmup_launches": warmup},
+            "cpu_baseline": res_cpu,
             "dynamic_quant_us": round(tq * 1e6, 1),
             "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1),
             "decode_m16_us": round(td * 1e6, 1),
             "decode_m16_GBps": round((N * K + Md * K + 2 * Md * N) / td / 1e9, 1)}
 
 
-def moe_bench(ops, dev, stream, which, iters=10, tokens=None):
+def cpu_baseline_moe_w4a16(x, logits, w13, z13, s13, w2, z2, s2, T):
+    """The CPU oracle of configs[3]: routing + the naive per-expert loop over dequantised experts, all 512
+    tokens, 1 repetition (the experts are dequantised inside the timed region, as the oracle does)."""
+    import numpy as np
+    import torch
+    from oracle import moe as om
+    from oracle import w4 as ow4
+    torch.set_num_threads(os.cpu_count() or 1)
+    xh = x.cpu().numpy()
+    lg = logits.cpu().numpy()
+    W13, Z13, S13 = w13.cpu().numpy(), z13.cpu().numpy(), s13.cpu().numpy()
+    W2, Z2, S2 = w2.cpu().numpy(), z2.cpu().numpy(), s2.cpu().numpy()
+
+    def expert(wq, zq, sc, e):
+        # the bench's random words are slab-order words; as a timing of unpack + dequantise they stand
+        # for any int4 matrix (values are not compared here)
+        return ow4.dequantize(ow4.gptq_unpack_weight(wq[e]), ow4.gptq_unpack_zeros(zq[e]), sc[e], GROUP)
+
+    def f16(a):
+        return a.astype(np.float16).astype(np.float32)
+    t0 = time.time()
+    tw, ids, _ = om.topk_softmax(lg, T, True)
+    om.fused_experts(xh.astype(np.float32), lambda e: expert(W13, Z13, S13, e), lambda e: expert(W2, Z2, S2, e),
+                     tw, ids, f16)
+    dt = time.time() - t0
+    M, H = xh.shape
+    I = W2.shape[1] * 8
+    flops = 2.0 * M * T * (H * 2 * I + I * H)
+    return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle.moe.fused_experts on all {M} tokens (routing, unpack + dequantise of the 8 experts, fp32 "
+                      f"matmuls, SiLU gate, weighted sum), 1 repetition, {dt:.1f} s of CPU work"}
+
+
+def cpu_baseline_moe_fp8(x, tw, ids, w13, s13, w2, s2, tokens=2):
+    """The CPU oracle of configs[4] on the first `tokens` tokens (their 8 experts each are dequantised)."""
+    import numpy as np
+    import torch
+    from oracle import fp8 as of8
+    from oracle import moe as om
+    torch.set_num_threads(os.cpu_count() or 1)
+    xf = x[:tokens].float().cpu().numpy()
+    twn, idn = tw[:tokens].cpu().numpy(), ids[:tokens].cpu().numpy()
+    need = sorted(set(idn.reshape(-1).tolist()))
+    c13 = {e: w13[e].view(torch.uint8).cpu().numpy() for e in need}
+    c2 = {e: w2[e].view(torch.uint8).cpu().numpy() for e in need}
+    b13 = {e: s13[e].cpu().numpy() for e in need}
+    b2 = {e: s2[e].cpu().numpy() for e in need}
+
+    def deq(codes, sc):
+        return (of8.from_e4m3fn(codes) * np.repeat(np.repeat(sc, 128, 0), 128, 1)).T
+
+    def qdq(a):
+        qa, sa = of8.per_token_group_quant_fp8(a, 128)
+        return of8.from_e4m3fn(qa) * np.repeat(sa, 128, -1)
+
+    def bf16(a):
+        return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+    t0 = time.time()
+    om.fused_experts(qdq(xf), lambda e: deq(c13[e], b13[e]), lambda e: deq(c2[e], b2[e]), twn, idn, bf16, quant_a2=qdq)
+    dt = time.time() - t0
+    H, I = xf.shape[1], w2.shape[2]
+    nbytes = len(need) * (3 * H * I)
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle.moe.fused_experts on the first {tokens} of 256 tokens ({len(need)} experts dequantised from "
+                      f"fp8 codes and block scales, fp32 matmuls), 1 repetition, {dt:.1f} s of CPU work; bytes = those "
+                      f"experts' weights"}
+
+
+def moe_bench(ops, dev, stream, which, iters=10, tokens=None, cpu=False):
     """BASELINE configs[3] (Mixtral-8x7B layer, W4A16) and configs[4]
     (DeepSeek-V3-style layer, fp8 block-scaled): routing + the whole
     fused-experts sequence, one layer."""
@@ -419,9 +545,15 @@ def moe_bench(ops, dev, stream, which, iters=10, tokens=None):
             + M * H + M * H // 128 * 4 + M * H * 2
         name = f"fused MoE fp8 block-scaled, DeepSeek-V3-style layer: 256 tok, hidden 7168, 256 experts ({hit} hit), inter 2048, top-8"
     t = time_graph([step], iters, 2, stream) / iters
-    return {"workload": name, "us": round(t * 1e6, 1), "compulsory_bytes": int(bytes_),
-            "GBps": round(bytes_ / t / 1e9, 1), "frac_hbm": round(bytes_ / t / 1e9 / HBM_PEAK_GBPS, 4),
-            "TFLOPs": round(flops / t / 1e12, 1)}
+    res = {"workload": name, "us": round(t * 1e6, 1), "compulsory_bytes": int(bytes_),
+           "GBps": round(bytes_ / t / 1e9, 1), "frac_hbm": round(bytes_ / t / 1e9 / HBM_PEAK_GBPS, 4),
+           "TFLOPs": round(flops / t / 1e12, 1),
+           "frac_mfma_peak": round(flops / t / 1e12 / (5000.0 if which == "fp8" else FP16_PEAK_TFLOPS), 4)}
+    if cpu and which == "w4a16" and tokens is None:
+        res["cpu_baseline"] = cpu_baseline_moe_w4a16(x, logits, w13, z13, s13, w2, z2, s2, T)
+    if cpu and which == "fp8":
+        res["cpu_baseline"] = cpu_baseline_moe_fp8(x, tw, ids, w13, s13, w2, s2)
+    return res
 
 
 def glue_bench(ops, dev, stream, iters=50):

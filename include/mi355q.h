@@ -277,14 +277,6 @@ int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_
  * the reference (load-time conversion, like its int4 rearrange). */
 int mi355q_kslab_repack(const void* src, void* dst, int batch, int N, int K, int elem_bytes, void* stream);
 
-/* ---- measurement probe -------------------------------------------------------
- * No counterpart in the reference.  Streams `bytes` of device memory through
- * `workgroups` workgroups of 256 threads with 16-byte loads and no arithmetic:
- * the time of this read of a kernel's weight bytes is the floor the benchmark
- * quotes next to the weight-streaming kernels.  bytes must be a multiple of
- * workgroups * 32 KiB; sink is 16 writable bytes (never written in practice). */
-int mi355q_probe_stream_read(const void* src, size_t bytes, int workgroups, void* sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -58,7 +58,6 @@ SIGNATURES = {
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_void_p]),
     "mi355q_kslab_repack": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
-    "mi355q_probe_stream_read": (c_int, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
     "mi355q_kcontig_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_int, c_int, c_void_p]),
 }

@@ -226,31 +226,18 @@ moe_align_kernel(const IdT* __restrict__ topk_ids, int numel, int top, const int
     const int total = __shfl(incl, 63);
     // estart[e] must not be overwritten before the lane that reads estart[e + 1] = old count
     // of expert e has consumed it: every lane first reads its own run, then all write
+    // a lane's run is at most 16 experts: the launch caps E at what 64 KiB of LDS hold (below 1024)
     int vals[16];
-    const bool small = per <= 16;
-    if (small) {
 #pragma unroll
-      for (int k = 0; k < 16; ++k) vals[k] = (e0 + k < e1) ? estart[e0 + k + 1] : 0;
-    }
+    for (int k = 0; k < 16; ++k) vals[k] = (e0 + k < e1) ? estart[e0 + k + 1] : 0;
     __builtin_amdgcn_wave_barrier();
-    if (small) {
 #pragma unroll
-      for (int k = 0; k < 16; ++k)
-        if (e0 + k < e1) {
-          estart[e0 + k] = run;
-          run += vals[k];
-        }
-      if (lane == 63) estart[E] = total;
-    } else if (lane == 0) {
-      // more than 1024 experts: plain serial scan
-      int r = 0;
-      for (int e = 0; e < E; ++e) {
-        const int c = estart[e + 1];
-        estart[e] = r;
-        r += c;
+    for (int k = 0; k < 16; ++k)
+      if (e0 + k < e1) {
+        estart[e0 + k] = run;
+        run += vals[k];
       }
-      estart[E] = r;
-    }
+    if (lane == 63) estart[E] = total;
     if (lane == 0) *npp = total;
   }
   __syncthreads();
@@ -348,7 +335,7 @@ extern "C" int mi355q_moe_align_block_size(const void* topk_ids, int ids_are_int
   MQ_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_pad && (topk_ids || numel == 0),
              "moe_align_block_size: null pointer");
   const size_t shmem = ((size_t)ALIGN_WAVES * num_experts + num_experts + 1) * sizeof(int);
-  MQ_REQUIRE(shmem <= 64 * 1024, "moe_align_block_size: num_experts=%d too large", num_experts);
+  MQ_REQUIRE(shmem <= 64 * 1024 && num_experts <= 1024, "moe_align_block_size: num_experts=%d too large", num_experts);
   const int cap = numel + num_experts * (block_size - 1);
   const int nblocks = cap / block_size;
   hipStream_t st = as_stream(stream);

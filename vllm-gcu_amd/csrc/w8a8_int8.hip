@@ -236,10 +236,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // behind the workgroup barrier, so a phase of reads or copies of its own
   // would idle the matrix pipes of the whole CU (a burst of copies also blocks
   // every wavefront in the address unit, 64 B/clk per CU).
-#ifndef MQ_I8_RE
-#define MQ_I8_RE 2
-#endif
-  constexpr int RE = MQ_I8_RE;                      // one LDS read every RE MFMAs
+  constexpr int RE = 2;                             // one LDS read every RE MFMAs (1 and 3 were measured: slower)
   auto half = [&](const Frag& cur, Frag& nxt, int rstage, int rh, int SB, int SE, int C0, int CE,
                   int cstage, int k0) {
     const uint32_t xb = lo[rh] + (uint32_t)(rstage * STAGE_BYTES) + xwave;
