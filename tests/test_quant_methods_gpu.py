@@ -459,3 +459,132 @@ def test_fp8_dense_65_to_128_rows_single_block(M):
                               dev(xs), dev(ws))
     want = of8.block_fp8_gemm(xq, xs, w, ws)
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_moe_wna16_create_weights_then_load_8bit_gptq_experts():
+    """8-bit GPTQ experts (moe_wna16.py:364-401): ``create_weights`` registers int32 ``[E, K/4, N]`` words,
+    symmetric zero-points stored as 127, scales ``[E, K/g, N]``; after loading they become int8
+    ``[E, N, K]`` = byte - 128 and take the W8A16 grouped GEMM with group scales."""
+    from vllm_gcu_amd.kernels.quantization.moe_wna16 import MoeWNA16GCUConfig
+    print("case moe_wna16 8-bit", flush=True)
+    M, E, T, H, I, g = 36, 4, 2, 256, 384, 128
+    rng = np.random.default_rng(21)
+    cfg = MoeWNA16GCUConfig.from_config({"quant_method": "gptq", "bits": 8, "group_size": g, "sym": True})
+    assert cfg.weight_bits == 8 and not cfg.has_zp and int(cfg.pack_factor) == 4
+    method = cfg.get_quant_method()
+    layer = torch.nn.Module()
+    method.create_weights(layer, E, H, I, torch.float16, weight_loader=None)
+    assert tuple(layer.w13_qweight.shape) == (E, H // 4, 2 * I) and tuple(layer.w2_qweight.shape) == (E, I // 4, H)
+    assert tuple(layer.w13_scales.shape) == (E, H // g, 2 * I) and tuple(layer.w13_qzeros.shape) == (E, H // g, 2 * I // 4)
+    assert layer.w13_qweight.is_transposed and layer.w13_qweight.quant_method == "group"
+    layer.cuda()
+    u13 = rng.integers(0, 256, size=(E, H, 2 * I), dtype=np.uint8)       # stored bytes: w + 128
+    u2 = rng.integers(0, 256, size=(E, I, H), dtype=np.uint8)
+    s13 = rng.uniform(0.001, 0.004, size=(E, H // g, 2 * I)).astype(np.float16)
+    s2 = rng.uniform(0.001, 0.004, size=(E, I // g, H)).astype(np.float16)
+
+    def pack8(u):                         # [E, K, N] bytes -> int32 [E, K/4, N], byte i of a word = k 4r + i
+        Ex, K, N = u.shape
+        v = u.reshape(Ex, K // 4, 4, N).astype(np.uint32)
+        return (v[:, :, 0] | (v[:, :, 1] << 8) | (v[:, :, 2] << 16) | (v[:, :, 3] << 24)).view(np.int32)
+    load(layer, "w13_qweight", dev(pack8(u13))); load(layer, "w2_qweight", dev(pack8(u2)))
+    load(layer, "w13_scales", dev(s13)); load(layer, "w2_scales", dev(s2))
+    layer.w13_qzeros.data.fill_(0x7f7f7f7f); layer.w2_qzeros.data.fill_(0x7f7f7f7f)
+    method.process_weights_after_loading(layer)
+    assert layer.w13_qweight.dtype == torch.int8 and tuple(layer.w13_qweight.shape) == (E, 2 * I, H)
+    x = rng.standard_normal((M, H)).astype(np.float16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    out = method.apply(layer, dev(x).clone(), dev(logits), top_k=T, renormalize=True)
+    two, ido, _ = om.topk_softmax(logits, T, True)
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)   # noqa: E731
+
+    def wf(u, s, e):
+        return (u[e].astype(np.float32) - 128.0) * np.repeat(s[e].astype(np.float32), g, 0)
+    want = om.fused_experts(x.astype(np.float32), lambda e: wf(u13, s13, e), lambda e: wf(u2, s2, e), two, ido, f16)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # a zero-point that is not the symmetric one is refused, as in the reference
+    bad = torch.nn.Module()
+    method.create_weights(bad, E, H, I, torch.float16)
+    bad.cuda()
+    bad.w13_qzeros.data.fill_(0x7f7f7f7e); bad.w2_qzeros.data.fill_(0x7f7f7f7f)
+    with pytest.raises(AssertionError):
+        method.process_weights_after_loading(bad)
+
+
+def test_moe_wna16_create_weights_4bit_and_act_order_refused():
+    from vllm_gcu_amd.kernels.quantization.moe_wna16 import MoeWNA16GCUConfig
+    E, H, I, g = 2, 256, 256, 128
+    for fmt, shapes in (("gptq", ((E, H // 8, 2 * I), (E, I // 8, H))), ("awq", ((E, H, 2 * I // 8), (E, I, H // 8)))):
+        conf = {"quant_method": fmt, "bits": 4, "group_size": g, "sym": True, "zero_point": True}
+        method = MoeWNA16GCUConfig.from_config(conf).get_quant_method()
+        layer = torch.nn.Module()
+        method.create_weights(layer, E, H, I, torch.bfloat16)
+        assert tuple(layer.w13_qweight.shape) == shapes[0] and tuple(layer.w2_qweight.shape) == shapes[1]
+        assert tuple(layer.w13_qzeros.shape) == (E, H // g, 2 * I // 8) and layer.w2_scales.dtype == torch.bfloat16
+        assert hasattr(layer, "w13_g_idx") == (fmt == "gptq")
+    # GPTQ: a g_idx that is not made of consecutive runs (act-order) is refused at load time
+    method = MoeWNA16GCUConfig.from_config({"quant_method": "gptq", "bits": 4, "group_size": g, "sym": False}).get_quant_method()
+    layer = torch.nn.Module()
+    method.create_weights(layer, E, H, I, torch.float16)
+    layer.cuda()
+    layer.w13_g_idx.data.copy_((torch.arange(H, device="cuda") // g).expand(E, H))
+    layer.w2_g_idx.data.copy_((torch.arange(I, device="cuda") // g).flip(0).expand(E, I))
+    for n in ("w13_qweight", "w2_qweight", "w13_qzeros", "w2_qzeros"):
+        getattr(layer, n).data.zero_()
+    with pytest.raises(AssertionError):
+        method.process_weights_after_loading(layer)
+
+
+def test_fp8_create_weights_shapes():
+    from vllm_gcu_amd.kernels.quantization.fp8 import Fp8GCUConfig
+    moe = Fp8GCUConfig().get_quant_method(moe=True)
+    layer = torch.nn.Module()
+    moe.create_weights(layer, 4, 512, 384, torch.bfloat16)
+    assert tuple(layer.w13_weight.shape) == (4, 768, 512) and layer.w13_weight.dtype == torch.float8_e4m3fn
+    assert tuple(layer.w13_weight_scale_inv.shape) == (4, 6, 4) and tuple(layer.w2_weight_scale_inv.shape) == (4, 4, 3)
+    lin = Fp8GCUConfig().get_quant_method()
+    l2 = torch.nn.Module()
+    lin.create_weights(l2, 512, [256, 128], 512, 384, torch.bfloat16)
+    assert tuple(l2.weight.shape) == (384, 512) and tuple(l2.weight_scale_inv.shape) == (3, 4)
+
+
+def test_modular_kernel_chunks_tokens(monkeypatch):
+    """``VLLM_FUSED_MOE_CHUNK_SIZE`` (modular_kernel.py:167-286): with workspaces sized for one chunk the
+    layer gives what one pass gives, for a token count that is no multiple of the chunk, in place and
+    out of place.  (Not bit for bit: a chunk of 64 tokens picks smaller align blocks than 150 tokens
+    do, hence another kernel and another fp32 summation order; both are held to the oracle.)"""
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    from vllm_gcu_amd.kernels.modular_experts import TritonExpertsPad
+    from vllm_gcu_amd.kernels.modular_kernel import FusedMoEModularKernel
+    from vllm_gcu_amd.kernels.prepare_finalize import MoEPrepareAndFinalizeNoEP
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print("case modular kernel chunking", flush=True)
+    M, E, T, H, I, g = 150, 8, 2, 256, 384, 128
+    rng = np.random.default_rng(33)
+    q13 = rng.integers(0, 16, size=(E, H, 2 * I), dtype=np.uint8)
+    q2 = rng.integers(0, 16, size=(E, I, H), dtype=np.uint8)
+    z13 = rng.integers(0, 16, size=(E, H // g, 2 * I), dtype=np.uint8)
+    z2 = rng.integers(0, 16, size=(E, I // g, H), dtype=np.uint8)
+    s13 = dev(rng.uniform(0.001, 0.01, size=(E, H // g, 2 * I)).astype(np.float16))
+    s2 = dev(rng.uniform(0.001, 0.01, size=(E, I // g, H)).astype(np.float16))
+    w13, zp13 = rearrange.rearrange_uint4_int32_gptq(dev(np.stack([ow4.gptq_pack_weight(a) for a in q13])),
+                                                     dev(np.stack([ow4.gptq_pack_zeros(a) for a in z13])))
+    w2, zp2 = rearrange.rearrange_uint4_int32_gptq(dev(np.stack([ow4.gptq_pack_weight(a) for a in q2])),
+                                                   dev(np.stack([ow4.gptq_pack_zeros(a) for a in z2])))
+    x = dev(rng.standard_normal((M, H)).astype(np.float16))
+    tw, ids = ops.fused_topk(x, dev(rng.standard_normal((M, E)).astype(np.float32)), T, True)
+    moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad(use_int4_w4a16=True, block_shape=[0, g]))
+    kw = dict(w1_scale=s13, w2_scale=s2, w1_zp=zp13, w2_zp=zp2)
+    whole = moe(x, w13, w2, tw, ids, **kw)
+    monkeypatch.setenv("VLLM_FUSED_MOE_CHUNK_SIZE", "64")
+    chunked = moe(x, w13, w2, tw, ids, **kw)
+    two, ido = tw.cpu().numpy(), ids.cpu().numpy()
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)   # noqa: E731
+    sn13, sn2 = s13.cpu().numpy().astype(np.float32), s2.cpu().numpy().astype(np.float32)
+    want = om.fused_experts(x.float().cpu().numpy(), lambda e: ow4.dequantize(q13[e], z13[e], sn13[e], g),
+                            lambda e: ow4.dequantize(q2[e], z2[e], sn2[e], g), two, ido, f16)
+    np.testing.assert_allclose(whole.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(chunked.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    xin = x.clone()
+    inplace = moe(xin, w13, w2, tw, ids, inplace=True, **kw)
+    assert inplace.data_ptr() == xin.data_ptr() and torch.equal(inplace, chunked)

@@ -66,3 +66,31 @@ def test_golden_list_covers_every_registered_op():
     have = {(ns, torch._C.parse_schema(f"{ns}::{t}").name.split("::")[-1]) for ns, _, t in golden_rows()}
     registered = {tuple(q.split("::")) for q in _custom_ops.SCHEMAS}
     assert registered == have
+
+
+def test_moe_wna16_config_parsing_and_compatibility():
+    """MoeWNA16GCUConfig.from_config / is_moe_wna16_gcu_compatible / override_quantization_method
+    (vllm_gcu/kernels/quantization/moe_wna16.py:67-158): host logic, no GPU work."""
+    import pytest
+    try:
+        from vllm_gcu_amd.kernels.quantization.moe_wna16 import MoeWNA16GCUConfig
+    except Exception as e:                                     # library not built in this environment
+        pytest.skip(f"package not importable here: {e}")
+    c = MoeWNA16GCUConfig.from_config({"quant_method": "gptq", "bits": 4, "group_size": 128, "sym": True})
+    assert c.has_zp and c.weight_bits == 4 and int(c.pack_factor) == 8 and c.get_name() == "moe_wna16_gcu"
+    c = MoeWNA16GCUConfig.from_config({"quant_method": "gptq", "bits": 8, "group_size": -1, "sym": True})
+    assert not c.has_zp and int(c.pack_factor) == 4
+    c = MoeWNA16GCUConfig.from_config({"quant_method": "awq", "bits": 4, "group_size": 64, "zero_point": True,
+                                       "modules_to_not_convert": ["gate"]})
+    assert c.has_zp and c.modules_to_not_convert == ["gate"]
+    with pytest.raises(ValueError):
+        MoeWNA16GCUConfig.from_config({"quant_method": "fp8", "bits": 8, "group_size": 128})
+    ok = MoeWNA16GCUConfig.is_moe_wna16_gcu_compatible
+    assert ok({"quant_method": "gptq", "bits": 4, "desc_act": False})
+    assert ok({"quant_method": "gptq", "bits": 8, "desc_act": True, "static_groups": True})
+    assert not ok({"quant_method": "gptq", "bits": 4, "desc_act": True})
+    assert not ok({"quant_method": "gptq", "bits": 3})
+    assert ok({"quant_method": "awq", "bits": 4}) and not ok({"quant_method": "awq", "bits": 8})
+    over = MoeWNA16GCUConfig.override_quantization_method
+    assert over({"quant_method": "gptq", "bits": 4}, "moe_wna16_gcu") == "moe_wna16_gcu"
+    assert over({"quant_method": "gptq", "bits": 4}, None) is None

@@ -61,6 +61,24 @@ class Fp8GCULinearMethod:
         self.quant_config = quant_config
         self.block_quant = quant_config.weight_block_size is not None
 
+    def create_weights(self, layer, input_size_per_partition: int, output_partition_sizes: List[int],
+                       input_size: int, output_size: int, params_dtype: torch.dtype, **extra_weight_attrs):
+        """Block-quantised checkpoint tensors as upstream vLLM 0.9.2's ``Fp8LinearMethod.create_weights``
+        registers them (the reference inherits it, fp8.py:49-70): ``weight`` fp8 ``[N, K]``,
+        ``weight_scale_inv`` f32 ``[ceil(N / 128), ceil(K / 128)]``, no static input scale."""
+        bn, bk = self.quant_config.weight_block_size
+        N, K = sum(output_partition_sizes), input_size_per_partition
+
+        def reg(name, t):
+            p = torch.nn.Parameter(t, requires_grad=False)
+            for k, v in extra_weight_attrs.items():
+                setattr(p, k, v)
+            layer.register_parameter(name, p)
+        reg("weight", torch.empty(N, K, dtype=torch.float8_e4m3fn))
+        reg("weight_scale_inv", torch.empty(-(-N // bn), -(-K // bk), dtype=torch.float32))
+        layer.input_scale = None
+        layer.orig_dtype = params_dtype
+
     def process_weights_after_loading(self, layer) -> None:
         # the reference keeps the checkpoint tensors as they are (fp8.py:72-166);
         # here the weight bytes are re-ordered once for contiguous wavefront loads
@@ -87,6 +105,26 @@ class Fp8GCUMoEMethod:
 
     def select_gemm_impl(self, prepare_finalize=None, moe=None):
         return TritonExpertsPad(use_fp8_w8a8=True, block_shape=self.quant_config.weight_block_size)
+
+    def create_weights(self, layer, num_experts: int, hidden_size: int, intermediate_size_per_partition: int,
+                       params_dtype: torch.dtype, **extra_weight_attrs):
+        """Block-quantised experts as upstream vLLM 0.9.2's ``Fp8MoEMethod.create_weights`` registers them
+        (inherited by the reference, fp8.py:72-79): fp8 ``w13_weight [E, 2I, H]`` / ``w2_weight [E, H, I]``,
+        f32 ``*_weight_scale_inv`` with one value per 128 x 128 block, dynamic activation scales."""
+        bn, bk = self.quant_config.weight_block_size
+        E, H, I = num_experts, hidden_size, intermediate_size_per_partition
+
+        def reg(name, t):
+            p = torch.nn.Parameter(t, requires_grad=False)
+            for k, v in extra_weight_attrs.items():
+                setattr(p, k, v)
+            layer.register_parameter(name, p)
+        reg("w13_weight", torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn))
+        reg("w2_weight", torch.empty(E, H, I, dtype=torch.float8_e4m3fn))
+        reg("w13_weight_scale_inv", torch.ones(E, 2 * (-(-I // bn)), -(-H // bk), dtype=torch.float32))
+        reg("w2_weight_scale_inv", torch.ones(E, -(-H // bn), -(-I // bk), dtype=torch.float32))
+        layer.w13_input_scale = None
+        layer.w2_input_scale = None
 
     def process_weights_after_loading(self, layer) -> None:
         rearrange.kslab_parameters_(layer, ("w13_weight", "w2_weight"))
