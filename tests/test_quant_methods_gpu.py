@@ -588,3 +588,59 @@ def test_modular_kernel_chunks_tokens(monkeypatch):
     xin = x.clone()
     inplace = moe(xin, w13, w2, tw, ids, inplace=True, **kw)
     assert inplace.data_ptr() == xin.data_ptr() and torch.equal(inplace, chunked)
+
+
+def test_vllm_wiring_pieces_without_vllm():
+    """init_prepare_finalize / shared-experts hook (patch_0_9_2/moe_layer.py:21-79), the x_scale
+    pass-through forward (kernels/linear.py:117-129) and the int8 hook (patch_0_9_2/utils.py:13-15),
+    on stand-ins for the vLLM objects they read."""
+    import types
+    from vllm_gcu_amd.kernels import linear, moe_layer
+    from vllm_gcu_amd.kernels.modular_kernel import FusedMoEModularKernel
+    from vllm_gcu_amd.kernels.prepare_finalize import MoEPrepareAndFinalizeNoEP
+    from vllm_gcu_amd.kernels.quantization.fp8 import Fp8GCUConfig
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    moe_cfg = types.SimpleNamespace(use_pplx_kernels=False, use_deepep_ht_kernels=False, use_deepep_ll_kernels=False,
+                                    moe_parallel_config=types.SimpleNamespace(ep_size=1, dp_size=1))
+    method = Fp8GCUConfig().get_quant_method(moe=True)
+    method.fused_experts = None
+    moe_layer.init_prepare_finalize(method, moe_cfg, None)
+    assert isinstance(method.fused_experts, FusedMoEModularKernel)
+    assert isinstance(method.fused_experts.prepare_finalize, MoEPrepareAndFinalizeNoEP)
+    assert method.topk_indices_dtype is None
+    moe_cfg.moe_parallel_config.ep_size = 2
+    with pytest.raises(NotImplementedError):
+        moe_layer.init_prepare_finalize(method, moe_cfg, None)
+    shared = lambda a: a          # noqa: E731
+    layer = types.SimpleNamespace(quant_method=method, shared_experts=shared, routed_scaling_factor=2.5)
+    moe_layer.set_shared_experts(layer)
+    assert method.fused_experts.prepare_finalize.shared_experts is shared
+    assert method.fused_experts.prepare_finalize.routed_scaling_factor == 2.5
+    with pytest.raises(ImportError):
+        moe_layer.install()
+    x = torch.randn(5, 256, device="cuda", dtype=torch.float16)
+    q, s = moe_layer.per_token_quant_int8_gcu(x)
+    q2, s2, _ = ops.scaled_int8_quant(x)
+    assert torch.equal(q, q2) and torch.equal(s, s2)
+
+    # x_scale pass-through: pre-quantised fp8 activations + their group scales give what the method
+    # gives when it quantises the bf16 activations itself
+    rng = np.random.default_rng(5)
+    N, K = 256, 512
+    lin_method = Fp8GCUConfig().get_quant_method()
+
+    class Lin(linear.MergedReplicatedLinearMixin, torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.bias, self.skip_bias_add, self.return_bias, self.quant_method = None, False, False, lin_method
+    lin = Lin()
+    lin_method.create_weights(lin, K, [N], K, N, torch.bfloat16)
+    lin.cuda()
+    lin.weight.data = (torch.randn(N, K, device="cuda") * 0.5).to(torch.float8_e4m3fn)
+    lin.weight_scale_inv.data = torch.rand(N // 128, K // 128, device="cuda") * 0.05 + 0.02
+    lin_method.process_weights_after_loading(lin)
+    xb = torch.from_numpy(rng.standard_normal((7, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    plain = lin(xb)
+    xq, xs = ops.per_token_group_quant_fp8(xb, 128)
+    passed = lin(xq, xs)
+    assert passed.dtype == torch.bfloat16 and torch.equal(plain, passed)
