@@ -156,6 +156,21 @@ int mi355q_static_int8_quant(int8_t* out, const void* x, const float* scale, int
 int mi355q_silu_mul_static_int8_quant(int8_t* out, const void* x, const float* scale, int per_channel,
                                       long rows, int d, int dtype, void* stream);
 
+/* The static int8 experts of FusedW8A8MoEMethod (vllm_gcu/kernels/quantization/w8a8.py:174-342) hand the
+ * vendor grouped GEMM 16-bit activations together with per-expert, per-input-channel reciprocal input
+ * scales [E, K] (w13_in_scales / w2_in_scales, w8a8.py:226-236; vllm_gcu/kernels/prepare_finalize.py:62-64
+ * passes them through un-quantised).  Here that quantisation is a kernel of its own in front of the int8
+ * grouped GEMM: for every (token, slot) id t < numel listed in the first *num_tokens_post_pad entries of
+ * sorted_token_ids, with e = expert_ids[position / block_size],
+ *   out[t, :] = sat_s8(rne(x[t / topk, :] * scale_rec[e, :]))   (product in fp32),
+ * out is int8 [numel, K]; x and scale_rec share dtype (f16 / bf16); rows of blocks whose expert is outside
+ * [0, E) are zero; max_sorted = entries of sorted_token_ids.  The vendor kernel's own rounding is not
+ * part of the reference: parity with it is unpinned. */
+int mi355q_moe_expert_int8_quant(int8_t* out, const void* x, const void* scale_rec,
+                                 const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                 const int32_t* num_tokens_post_pad, int max_sorted, int block_size, int numel,
+                                 int topk, int E, int K, int dtype, void* stream);
+
 /* ---- MoE routing ------------------------------------------------------------
  * Replaces topsvllm's topk_softmax (csrc/src/topk_softmax.cpp:27-34):
  * softmax over E experts in fp32, top-k descending (ties to the lower index);

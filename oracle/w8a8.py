@@ -42,6 +42,22 @@ def static_scaled_int8_quant(x: np.ndarray, scale: np.ndarray):
     return np.clip(np.rint(y), -128, 127).astype(np.int8)
 
 
+def moe_expert_int8_quant(x: np.ndarray, scale_rec: np.ndarray, topk_ids: np.ndarray) -> np.ndarray:
+    """Static per-expert, per-input-channel quantisation of fused-MoE activations: for every
+    (token, slot) id t with expert e, ``q[t] = sat_s8(rne(x[t // topk] * scale_rec[e]))``, product in
+    float32.  ``scale_rec [E, K]`` holds reciprocals, as the reference's loader stores
+    ``w13_in_scales`` / ``w2_in_scales`` (vllm_gcu/kernels/quantization/w8a8.py:226-236, 277-289) and
+    hands them, with the un-quantised activations, to its vendor grouped GEMM
+    (vllm_gcu/kernels/prepare_finalize.py:62-64, w8a8.py:339-340).  Parity unpinned: the vendor
+    kernel's rounding is not in the reference; this is the build's own definition."""
+    M, K = x.shape
+    flat = topk_ids.reshape(-1)
+    topk = topk_ids.shape[-1] if topk_ids.ndim > 1 else 1
+    rows = np.arange(flat.size) // topk
+    y = x[rows].astype(np.float32) * scale_rec[flat].astype(np.float32)
+    return np.clip(np.rint(y), -128, 127).astype(np.int8)
+
+
 def int8_gemm_i32(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     """Exact ``a[M, K] @ b[K, N]`` in int32 for int8 operands.
 

@@ -644,3 +644,54 @@ def test_vllm_wiring_pieces_without_vllm():
     xq, xs = ops.per_token_group_quant_fp8(xb, 128)
     passed = lin(xq, xs)
     assert passed.dtype == torch.bfloat16 and torch.equal(plain, passed)
+
+
+def test_w8a8_moe_static_per_expert_input_scales():
+    """FusedW8A8MoEMethod as the reference runs it (w8a8.py:174-342): ``w13_in_scales [E, H]`` /
+    ``w2_in_scales [E, I]`` hold reciprocal scales, 16-bit activations are quantised per (token, slot)
+    with the expert's vector, int8 GEMM, per-channel output scales.  int8 codes and int32 sums are exact,
+    so the result is held to the oracle of the same definition (the vendor kernel itself is unpinned)."""
+    from vllm_gcu_amd.kernels.quantization.w8a8 import W8A8Config
+    print("case w8a8 moe static in-scales", flush=True)
+    M, E, T, H, I = 30, 4, 2, 256, 384
+    rng = np.random.default_rng(44)
+    m8 = W8A8Config().get_quant_method(moe=True)
+    layer = torch.nn.Module()
+    m8.create_weights(layer, E, H, I, torch.float16, static_in_scales=True)
+    assert tuple(layer.w13_in_scales.shape) == (E, H) and layer.w2_in_scales.dtype == torch.float16
+    layer.cuda()
+    w13 = rng.integers(-127, 128, size=(E, 2 * I, H), dtype=np.int8)
+    w2 = rng.integers(-127, 128, size=(E, H, I), dtype=np.int8)
+    c13 = rng.uniform(1e-4, 4e-4, size=(E, 2 * I)).astype(np.float32)
+    c2 = rng.uniform(1e-4, 4e-4, size=(E, H)).astype(np.float32)
+    in13 = rng.uniform(0.02, 0.05, size=(E, H)).astype(np.float32)      # checkpoint scales
+    in2 = rng.uniform(0.02, 0.06, size=(E, I)).astype(np.float32)
+    load(layer, "w13_weight", dev(w13)); load(layer, "w2_weight", dev(w2))
+    load(layer, "w13_out_scales", dev(c13)); load(layer, "w2_out_scales", dev(c2))
+    for e in range(E):
+        m8.load_in_scales(layer.w13_in_scales, e, dev(in13[e]))
+        m8.load_in_scales(layer.w2_in_scales, e, dev(in2[e]))
+    m8.process_weights_after_loading(layer)
+    x = rng.standard_normal((M, H)).astype(np.float16)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    out = m8.apply(layer, dev(x).clone(), dev(logits), top_k=T, renormalize=True)
+    tw, ids, _ = om.topk_softmax(logits, T, True)
+    rec13 = layer.w13_in_scales.float().cpu().numpy()
+    rec2 = layer.w2_in_scales.float().cpu().numpy()
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)   # noqa: E731
+    flat = ids.reshape(-1)
+    q1 = o8.moe_expert_int8_quant(x, rec13, ids)                                  # [M*T, H]
+    c1 = np.zeros((M * T, 2 * I), dtype=np.float32)
+    for t in range(M * T):
+        e = flat[t]
+        c1[t] = o8.int8_gemm_i32(q1[t:t + 1], np.ascontiguousarray(w13[e].T))[0].astype(np.float32) * c13[e]
+    a2 = f16(om.silu_and_mul(f16(c1))).astype(np.float16)
+    q2 = o8.moe_expert_int8_quant(a2, rec2, flat.reshape(-1, 1))                  # one row per slot
+    c3 = np.zeros((M * T, H), dtype=np.float32)
+    for t in range(M * T):
+        e = flat[t]
+        c3[t] = o8.int8_gemm_i32(q2[t:t + 1], np.ascontiguousarray(w2[e].T))[0].astype(np.float32) * c2[e]
+    c3 = f16(c3 * tw.reshape(-1, 1))
+    want = f16(c3.reshape(M, T, H).sum(1))
+    assert np.abs(want).max() > 0.05
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)

@@ -468,6 +468,36 @@ silu_mul_static_int8_quant_kernel(int8_t* out, const uint16_t* x, const float* s
   out[i] = sat_rne_s8(act * inv);
 }
 
+// static per-expert, per-input-channel quantisation of the rows a fused-MoE GEMM is about to read:
+// out[t, :] = sat_s8(rne(x[t / topk, :] * rec[e, :])) for every (token, slot) id t listed in
+// sorted_ids, e being the expert of its align block; the product is taken in fp32.  One workgroup
+// per sorted position; ids of blocks whose expert lies outside [0, E) get zero rows.
+template <int DT>
+__global__ void __launch_bounds__(256)
+moe_expert_int8_quant_kernel(int8_t* out, const uint16_t* x, const uint16_t* rec, const int* sorted_ids,
+                             const int* expert_ids, const int* npp, int block_size, int numel, int topk, int E, int K) {
+  const int p = blockIdx.x;
+  if (p >= *npp) return;
+  const long t = sorted_ids[p];
+  if (t >= numel) return;                                      // pad
+  const int e = expert_ids[p / block_size];
+  const bool local = e >= 0 && e < E;
+  const uint16_t* xr = x + (t / topk) * (long)K;
+  const uint16_t* rr = rec + (long)(local ? e : 0) * K;
+  for (int c = threadIdx.x; c < (K >> 3); c += 256) {
+    const u4 xv = *(const u4*)(xr + 8 * c), rv = *(const u4*)(rr + 8 * c);
+    uint32_t q[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t xw = xv[i >> 1], rw = rv[i >> 1];
+      const float y = ld_half<DT>((uint16_t)((i & 1) ? (xw >> 16) : (xw & 0xffffu))) *
+                      ld_half<DT>((uint16_t)((i & 1) ? (rw >> 16) : (rw & 0xffffu)));
+      q[i >> 2] |= ((uint32_t)(uint8_t)(local ? sat_rne_s8(y) : (int8_t)0)) << (8 * (i & 3));
+    }
+    *(u2*)(out + t * (long)K + 8 * c) = (u2){q[0], q[1]};
+  }
+}
+
 template <int DT, int WM, int WN, int NI, int NJ>
 int launch_tile(const I8Args& a, hipStream_t st) {
   constexpr int TN = WN * NI * 16;
@@ -570,6 +600,30 @@ extern "C" int mi355q_static_int8_quant(int8_t* out, const void* x, const float*
   else
     MQ_REQUIRE(false, "static_int8_quant: bad dtype %d", dtype);
   MQ_LAUNCH_CHECK("static_int8_quant");
+  return 0;
+}
+
+extern "C" int mi355q_moe_expert_int8_quant(int8_t* out, const void* x, const void* scale_rec,
+                                            const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                            const int32_t* num_tokens_post_pad, int max_sorted, int block_size,
+                                            int numel, int topk, int E, int K, int dtype, void* stream) {
+  MQ_REQUIRE(numel >= 0 && topk > 0 && E > 0 && K > 0 && K % 8 == 0 && block_size > 0 && max_sorted >= 0,
+             "moe_expert_int8_quant: bad shape numel=%d topk=%d E=%d K=%d block=%d (K %% 8 == 0)", numel, topk, E, K,
+             block_size);
+  if (numel == 0 || max_sorted == 0) return 0;
+  MQ_REQUIRE(out && x && scale_rec && sorted_token_ids && expert_ids && num_tokens_post_pad,
+             "moe_expert_int8_quant: null pointer");
+  MQ_REQUIRE(dtype == MI355Q_F16 || dtype == MI355Q_BF16, "moe_expert_int8_quant: dtype %d must be f16 or bf16", dtype);
+  hipStream_t st = as_stream(stream);
+  if (dtype == MI355Q_F16)
+    hipLaunchKernelGGL((moe_expert_int8_quant_kernel<MI355Q_F16>), dim3(max_sorted), dim3(256), 0, st, out,
+                       (const uint16_t*)x, (const uint16_t*)scale_rec, sorted_token_ids, expert_ids,
+                       num_tokens_post_pad, block_size, numel, topk, E, K);
+  else
+    hipLaunchKernelGGL((moe_expert_int8_quant_kernel<MI355Q_BF16>), dim3(max_sorted), dim3(256), 0, st, out,
+                       (const uint16_t*)x, (const uint16_t*)scale_rec, sorted_token_ids, expert_ids,
+                       num_tokens_post_pad, block_size, numel, topk, E, K);
+  MQ_LAUNCH_CHECK("moe_expert_int8_quant");
   return 0;
 }
 

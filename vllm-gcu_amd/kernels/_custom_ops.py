@@ -898,7 +898,25 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
         raise RuntimeError("fused_moe: C must be contiguous")
     zk, zp, group = _lib.ZP_NONE, None, int(gs)
     a_scale = w_scale = None
-    if A_scale is not None:
+    if A_scale is not None and A.dtype in (torch.float16, torch.bfloat16) and B.dtype == torch.int8 \
+            and A_scale.dim() == 2 and A_scale.shape[-1] == K and A_scale.dtype == A.dtype:
+        # static int8 experts (w8a8.py:174-342): 16-bit activations plus per-expert, per-channel reciprocal
+        # input scales [E, K].  Each (token, slot) row is quantised with its expert's vector, then the
+        # int8 grouped GEMM reads one row per slot.
+        rec = A_scale.contiguous()
+        # rows of pads and of non-local experts are never read by the GEMM (zeros, so that nothing is undefined)
+        Aq = torch.zeros((numel, K), dtype=torch.int8, device=A.device)
+        with torch.cuda.device(A.device):
+            _lib.call("mi355q_moe_expert_int8_quant", Aq.data_ptr(), A.data_ptr(), rec.data_ptr(),
+                      sorted_token_ids.data_ptr(), experts_ids.data_ptr(), num_tokens_post_pad.data_ptr(),
+                      sorted_token_ids.numel(), int(block_size), numel, int(topk), rec.shape[0], K,
+                      rt.dtype_code(A.dtype), rt.stream_ptr())
+        A, A_scale, topk = Aq, None, 1
+        mode = _lib.Q_INT8
+        w_scale = B_scale.to(torch.float32).reshape(B.shape[0], -1).contiguous()
+        w = B.contiguous()
+        act_code = _lib.F16
+    elif A_scale is not None:
         if A.dtype == torch.float8_e4m3fn:
             mode = _lib.Q_FP8_BLOCK
             a_scale = A_scale.to(torch.float32).contiguous()

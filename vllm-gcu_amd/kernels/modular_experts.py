@@ -120,7 +120,12 @@ class TritonExpertsPad:
         elif self.use_int8_w8a8:
             tmp = torch.empty((num_tokens * top_k_num, N // 2), dtype=act_dtype, device=cache1.device)
             torch.ops._C.silu_and_mul_pad(tmp.view(-1, top_k_num, N // 2), cache1, expert_num_tokens)
-            if a2_scale is not None:
+            if a2_scale is not None and a2_scale.dim() == 2 and a2_scale.dtype == act_dtype \
+                    and a2_scale.shape[-1] == N // 2:
+                # per-expert, per-channel reciprocal input scales [E, I] (modular_experts.py:232-240 of the
+                # reference): the 16-bit activations go to the grouped GEMM together with the scales
+                cache2 = tmp
+            elif a2_scale is not None:
                 torch.ops._C.static_scaled_int8_quant(cache2, tmp, a2_scale, None)
                 a2_scale = a2_scale.expand(tmp.shape[0]).contiguous() if a2_scale.numel() == 1 else a2_scale
             else:

@@ -89,9 +89,16 @@ class CompressedTensorMMLinearKernel:
 
 class FusedW8A8MoEMethod:
     """int8 experts ``w13_weight [E, 2I, H]`` / ``w2_weight [E, H, I]`` with
-    per-channel ``*_out_scales`` (w8a8.py:174-345).  Activations are quantised
-    per token on the fly; ``*_in_scales`` of the checkpoint (static per-channel
-    smoothing scales) are forwarded when the layer carries them."""
+    per-channel ``*_out_scales`` (w8a8.py:174-345).
+
+    The reference's layer always carries static input scales: ``w13_in_scales [E, H]`` /
+    ``w2_in_scales [E, I]`` in the activation dtype, holding the *reciprocals* of the checkpoint's
+    per-expert, per-input-channel scales (its loader inverts them, w8a8.py:226-236), and hands
+    them with the un-quantised activations to the grouped GEMM.  ``create_weights(...,
+    static_in_scales=True)`` registers them the same way and ``load_in_scales`` does the loader's
+    inversion; each (token, slot) row is then quantised with its expert's vector in front of the
+    int8 GEMM (``mi355q_moe_expert_int8_quant``; the vendor kernel's own rounding is unpinned).
+    Without them (the default here, an extension) activations are quantised per token on the fly."""
 
     def __init__(self, quant_config: W8A8Config):
         self.quant_config = quant_config
@@ -106,7 +113,7 @@ class FusedW8A8MoEMethod:
         rearrange.kslab_parameters_(layer, ("w13_weight", "w2_weight"))
 
     def create_weights(self, layer, num_experts, hidden_size, intermediate_size_per_partition, params_dtype,
-                       **extra_weight_attrs):
+                       static_in_scales: bool = False, **extra_weight_attrs):
         E, H, I = num_experts, hidden_size, intermediate_size_per_partition
 
         def reg(name, t):
@@ -115,6 +122,15 @@ class FusedW8A8MoEMethod:
         reg("w2_weight", torch.empty(E, H, I, dtype=torch.int8))
         reg("w13_out_scales", torch.zeros(E, 2 * I, dtype=torch.float32))
         reg("w2_out_scales", torch.zeros(E, H, dtype=torch.float32))
+        if static_in_scales:                       # w8a8.py:277-289
+            reg("w13_in_scales", torch.ones(E, H, dtype=params_dtype))
+            reg("w2_in_scales", torch.ones(E, I, dtype=params_dtype))
+
+    @staticmethod
+    def load_in_scales(param: torch.Tensor, expert_id: int, loaded_scale: torch.Tensor) -> None:
+        """The reference's loader for ``*_in_scales`` (w8a8.py:226-236): the stored value is the reciprocal
+        of the checkpoint's scale."""
+        param.data[expert_id].copy_(loaded_scale.to(param.dtype).reciprocal())
 
     def apply(self, layer, x, router_logits, top_k: int, renormalize: bool, use_grouped_topk: bool = False,
               global_num_experts: int = -1, expert_map=None, topk_group=None, num_expert_group=None,
