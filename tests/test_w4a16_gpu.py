@@ -302,3 +302,20 @@ def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):
     q, z, s, x = make_case(5, M, K, N, g)
     got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).float().cpu().numpy()
     np.testing.assert_allclose(got, oracle(q, z, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)
+
+
+def test_operand_shapes_are_checked_on_the_host(ops, rearrange):
+    """The kernels index scales, zero-points and bias by (group row, column) without bounds checks, so
+    the wrapper refuses operands whose sizes do not fit K / group_size x N before anything is launched."""
+    print("case w4a16 operand shape checks", flush=True)
+    q, z, s, x = make_case(5, 4, 256, 256, 128)
+    qw, qz = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    xs, sc = to_act(x, torch.float16).cuda(), to_act(s, torch.float16).cuda()
+    good = ops.w4a16_gemm(xs, qw, sc, qz, None, 128)
+    assert good.shape == (4, 256)
+    with pytest.raises(RuntimeError, match="zero-points"):
+        ops.w4a16_gemm(xs, qw, sc, qz.to(torch.float16), None, 128)       # [K/g, N/8] values, not [K/g, N]
+    with pytest.raises(RuntimeError, match="scales"):
+        ops.w4a16_gemm(xs, qw, sc[:1], qz, None, 128)
+    with pytest.raises(RuntimeError, match="bias"):
+        ops.w4a16_gemm(xs, qw, sc, qz, torch.zeros(8, dtype=torch.float16, device="cuda"), 128)

@@ -58,7 +58,8 @@ SIGNATURES = {
     "mi355q_moe_sum": (c_int, [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_moe_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                c_int, c_int, c_int, c_int, c_void_p]),
+                                c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "mi355q_moe_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "mi355q_kslab_repack": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355q_kcontig_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -476,11 +476,18 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
                          const void* zeros, int zeros_kind, const float* topk_weights,
                          const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
-                         int group_size, int dtype, hipStream_t st);
+                         int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
+size_t w4a16_grouped_workspace_bytes(int numel, int block_size, int max_blocks, int E, int K, int N);
 
 }  // namespace mi355q
 
 using namespace mi355q;
+
+extern "C" size_t mi355q_moe_gemm_workspace_bytes(int quant_mode, int numel, int block_size, int max_blocks, int E,
+                                                  int K, int N) {
+  if (quant_mode != 0 || numel <= 0 || K <= 0 || N <= 0 || K % 128 || N % 128) return 0;
+  return w4a16_grouped_workspace_bytes(numel, block_size, max_blocks, E, K, N);
+}
 
 // quant_mode of the MoE / dense entry points
 //   0 = W4A16 (slab-layout int4), 1 = fp8 block-scaled, 2 = int8 per-token x per-channel,
@@ -490,7 +497,8 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
                                int group_size, const float* topk_weights, const int32_t* sorted_token_ids,
                                const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int numel,
                                int topk, int block_size, int max_blocks, int E, int K, int N, int act_dtype,
-                               int out_dtype, int w_layout, void* stream) {
+                               int out_dtype, int w_layout, void* workspace, size_t workspace_bytes,
+                               void* stream) {
   MQ_REQUIRE(numel >= 0 && topk > 0 && E > 0 && K > 0 && N > 0, "moe_gemm: bad shape");
   if (numel == 0 || max_blocks == 0) return 0;
   MQ_REQUIRE(out && a && w && sorted_token_ids && expert_ids && num_tokens_post_pad, "moe_gemm: null pointer");
@@ -503,7 +511,8 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
     MQ_REQUIRE(out_dtype == act_dtype, "moe_gemm(w4a16): output dtype must equal the activation dtype");
     return w4a16_grouped_launch(out, a, (const int32_t*)w, w_scale, nullptr, nullptr, w_zeros, zeros_kind,
                                 topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, numel, topk,
-                                block_size, max_blocks, E, K, N, group_size <= 0 ? K : group_size, act_dtype, st);
+                                block_size, max_blocks, E, K, N, group_size <= 0 ? K : group_size, act_dtype,
+                                workspace, workspace_bytes, st);
   }
   if (quant_mode == 5) {
     MQ_REQUIRE(N % 128 == 0, "moe_gemm(w4, fp32 scales): N=%d must be a multiple of 128", N);
@@ -513,7 +522,7 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
     return w4a16_grouped_launch(out, a, (const int32_t*)w, nullptr, (const float*)w_scale, a_scale, nullptr,
                                 MI355Q_ZP_NONE, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad,
                                 numel, topk, block_size, max_blocks, E, K, N, group_size <= 0 ? K : group_size,
-                                act_dtype, st);
+                                act_dtype, nullptr, 0, st);
   }
   MQ_REQUIRE(N % 4 == 0, "moe_gemm: N=%d must be a multiple of 4", N);
   MQ_REQUIRE(w_layout == 0 || (w_layout == 1 && N % 64 == 0), "moe_gemm: weight layout %d needs N=%d %% 64 == 0", w_layout, N);

@@ -39,8 +39,9 @@ struct TileArgs {
   const int* npp;             // device scalar: padded id count
   const float* topk_weights;  // [numel] or null
   int numel, topk, E;
-  // dense split-K: blockIdx.z takes K blocks [z * kper, (z + 1) * kper) and writes an fp32
-  // partial tile to partial[z][M][N]; a second kernel adds the partials up
+  // split-K: blockIdx.z takes K blocks [z * kper, (z + 1) * kper) and writes an fp32 partial
+  // tile to partial[z][M][N] (grouped: M = numel, rows indexed by slot id, routing weight not yet
+  // applied); a second kernel adds the partials up
   int kper;                   // K blocks per split (G when there is no split)
   float* partial;             // null: write the output directly
   long w_stride, s_stride, z_stride;   // per-expert strides in elements of the respective arrays
@@ -118,6 +119,7 @@ w4a16_tile_kernel(TileArgs a) {
   constexpr int A_BUF = BM * A_ROW;
   extern __shared__ __align__(16) unsigned char lds[];
   __shared__ int tok[GROUPED ? BM : 1];
+  __shared__ int live_s;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = (tid >> 6) & 3, wmh = tid >> 8;
   const int c = lane & 15, kq = lane >> 4;
@@ -128,21 +130,49 @@ w4a16_tile_kernel(TileArgs a) {
   const uint16_t* scales = a.scales;
   const float* scales32 = a.scales_f32;
   const char* zeros = (const char*)a.zeros;
+  // row tiles of the block that hold at least one real slot (the pads of an expert's last block
+  // are skipped by the matrix instructions); bit = row tile
+  int live_tiles = (1 << MT) - 1;
   if (GROUPED) {
     if (m0 >= *a.npp) return;                       // block beyond the padded ids
     const long e = a.expert_ids[blockIdx.y];
     if (e < 0 || e >= a.E) {                        // not one of this rank's experts: zero rows, no weights read
-      const int col0 = blockIdx.x * BN;
-      zero_block_columns(a.out, a.sorted_ids + m0, BM, a.numel, N, col0, min(BN, N - col0), NTHR);
+      const int col0 = blockIdx.x * BN, ncols = min(BN, N - col0);
+      if (a.partial) {
+        // split K: the reduction sums every split's rows, so each split zeroes its own
+        const int per_row = ncols >> 2;
+        for (int i = tid; i < BM * per_row; i += NTHR) {
+          const int r = i / per_row, piece = i - r * per_row;
+          const int id = a.sorted_ids[m0 + r];
+          if (id < a.numel)
+            *(f4*)(a.partial + ((size_t)blockIdx.z * a.numel + id) * N + col0 + 4 * piece) = (f4){0.f, 0.f, 0.f, 0.f};
+        }
+      } else {
+        zero_block_columns(a.out, a.sorted_ids + m0, BM, a.numel, N, col0, ncols, NTHR);
+      }
       return;
     }
     qw += e * a.w_stride;
     if (SF32) scales32 += e * a.s_stride;
     else scales += e * a.s_stride;
     if (zeros) zeros += e * a.z_stride * (ZK == MI355Q_ZP_PACKED ? 4 : 2);
+    if (tid == 0) live_s = 0;
     for (int r = tid; r < BM; r += NTHR) tok[r] = a.sorted_ids[m0 + r];
     __syncthreads();
+    if (tid < BM) {
+      const unsigned long long valid = __ballot(tok[tid] < a.numel);
+      if (lane == 0) {
+        int m = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) m |= ((valid >> (16 * t)) & 0xffffull) ? (1 << t) : 0;
+        if (m) atomicOr(&live_s, m << (4 * (tid >> 6)));
+      }
+    }
+    __syncthreads();
+    live_tiles = live_s;
+    if (live_tiles == 0) return;                    // pads only
   }
+  auto tile_live = [&](int mt) { return !GROUPED || ((live_tiles >> (wmh * MTW + mt)) & 1); };
   // N may end in the middle of the 256-column tile: the two wavefronts of a
   // missing slab compute on the previous one and skip the epilogue
   const bool live = (blockIdx.x * 2 + (wave >> 1)) < (N >> 7);
@@ -199,11 +229,15 @@ w4a16_tile_kernel(TileArgs a) {
     if (ZK == MI355Q_ZP_PRESCALED) zsreg = *(const uint2*)((const uint16_t*)zeros + (size_t)qrow * N + ncol);
   };
 
-  const int gb = GROUPED ? 0 : (int)blockIdx.z * a.kper, ge = GROUPED ? G : min(G, gb + a.kper);
+  const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
   // The pipelined loop needs nearly the whole register file; it is used where it fits
   // (fp16, 128-row tiles), the plain loop elsewhere.
   constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED && !SF32;
-  if constexpr (PIPE) {
+  // (a grouped block with row tiles of pads only takes the plain loop, which skips them: the
+  // pipelined loop has no room for branches)
+  bool done = false;
+  if constexpr (PIPE) if (!GROUPED || live_tiles == (1 << MT) - 1) {
+    done = true;
     // Software pipeline, written out because the compiler otherwise sinks every
     // load next to its use.  Activations: global loads at the top of the K block
     // before their use, stored into the other LDS buffer near its end.  Weights:
@@ -314,7 +348,8 @@ w4a16_tile_kernel(TileArgs a) {
       kblock(g + 1, w1, w0);
       if (g + 2 >= ge) break;
     }
-  } else {
+  }
+  if (!done) {
     // Plain loop: operands of the whole K block dequantised up front, the next block's loads
     // pinned at the top, one partial tile per row tile.  Two wavefronts per SIMD cover each
     // other's dequantisation bursts.
@@ -362,6 +397,7 @@ w4a16_tile_kernel(TileArgs a) {
       const unsigned char* abase = lds + buf + (wmh * MTW * 16 + c) * A_ROW + kq * 16;
 #pragma unroll
       for (int mt = 0; mt < MTW; ++mt) {
+        if (!tile_live(mt)) continue;
         f4 part[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
@@ -404,7 +440,7 @@ w4a16_tile_kernel(TileArgs a) {
         m = m0 + (wmh * MTW + mt) * 16 + 4 * kq + i;
         ok = m < M;
       }
-      if (!GROUPED && a.partial) {
+      if (a.partial) {
         if (ok) {
           float* pp = a.partial + ((size_t)blockIdx.z * M + m) * N + ncol;
           *(f4*)pp = (f4){acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]};
@@ -421,13 +457,16 @@ w4a16_tile_kernel(TileArgs a) {
 }
 
 // out[m, n] = sum over splits of partial[s][m][n] (+ bias[n]), added in split order
+// times row_weight[m] when given (the routing weights of a grouped launch)
 template <int DT>
 __global__ void __launch_bounds__(256)
-w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* bias, long MN, int N, int splits) {
+w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* bias, const float* row_weight,
+                           long MN, int N, int splits) {
   const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= MN) return;
   f4 v = *(const f4*)(partial + i);
   for (int s = 1; s < splits; ++s) v += *(const f4*)(partial + (size_t)s * MN + i);
+  if (row_weight) v *= row_weight[i / N];
   if (bias) {
     const int n = (int)(i % N);
 #pragma unroll
@@ -443,7 +482,7 @@ template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32>
 hipError_t launch_wm(const TileArgs& a, int row_blocks, hipStream_t st) {
   constexpr int BM = 16 * MT;
   const int G = a.K >> 7;
-  dim3 grid((a.N + BN - 1) / BN, row_blocks, GROUPED ? 1 : (G + a.kper - 1) / a.kper), block(256 * WM);
+  dim3 grid((a.N + BN - 1) / BN, row_blocks, (G + a.kper - 1) / a.kper), block(256 * WM);
   const size_t shmem = 2 * BM * A_ROW;             // up to 72 KiB: above the 64 KiB default
   static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -553,10 +592,10 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
     const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
     if (dtype == MI355Q_F16)
       hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, (const uint16_t*)bias, MN, N, splits);
+                         (const float*)workspace, (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
     else
       hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, (const uint16_t*)bias, MN, N, splits);
+                         (const float*)workspace, (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
     MQ_LAUNCH_CHECK("w4a16_gemm(split-K reduce)");
   }
   return 0;
@@ -568,12 +607,35 @@ int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight
                                 int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                                 int group_size, int dtype, hipStream_t st);
 
+// Split-K plan of a grouped launch.  The host does not know how many blocks the alignment filled, so
+// the grid is estimated as every slot in a full block plus half a block of pads per expert.  A long K
+// with a narrow N (the second expert GEMM of a gated MLP) leaves the chip part empty and makes its few
+// workgroups very long; K is split until about two and a half workgroups per resident slot exist,
+// keeping at least 16 K blocks per split (Mixtral-8x7B layer, 512 tokens, second GEMM: 4 splits
+// measured best of 1..7; every further split adds 17 MB of partial tiles).
+static int grouped_splits(int numel, int block_size, int max_blocks, int E, int K, int N) {
+  if (block_size != 64) return 1;                  // the 64-row pipelined kernel only
+  const int G = K / 128;
+  long blocks = (numel + block_size - 1) / block_size + (E + 1) / 2;
+  if (blocks > max_blocks) blocks = max_blocks;
+  const long wgs = blocks * ((N + BN - 1) / BN), slots = 2L * device_cu_count();
+  if (wgs >= 2 * slots || G < 32) return 1;
+  long s = (5 * slots / 2 + wgs - 1) / wgs;
+  if (s > G / 16) s = G / 16;
+  while (s > 1 && (size_t)s * numel * N * sizeof(float) > TILE_SPLITK_BYTES * 2) --s;
+  return s < 1 ? 1 : (int)s;
+}
+size_t w4a16_grouped_workspace_bytes(int numel, int block_size, int max_blocks, int E, int K, int N) {
+  const int s = grouped_splits(numel, block_size, max_blocks, E, K, N);
+  return s > 1 ? (size_t)s * numel * N * sizeof(float) : 0;
+}
+
 int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                          const float* scales_f32, const float* out_scale,
                          const void* zeros, int zeros_kind, const float* topk_weights,
                          const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
-                         int group_size, int dtype, hipStream_t st) {
+                         int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
   MQ_REQUIRE(group_size % 128 == 0, "moe_w4a16: group_size=%d must be a multiple of 128", group_size);
   MQ_REQUIRE((size_t)(numel / (topk > 0 ? topk : 1)) * K * 2 < ((size_t)1 << 32),
              "moe_w4a16: activation matrix of %d rows x %d is 4 GiB or more", numel / (topk > 0 ? topk : 1), K);
@@ -598,7 +660,12 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   a.M = numel; a.K = K; a.N = N; a.gs = group_size;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
   a.numel = numel; a.topk = topk; a.E = E;
-  a.kper = K / 128; a.partial = nullptr;
+  const int G = K / 128;
+  int splits = (scales_f32 || out_scale) ? 1 : grouped_splits(numel, block_size, max_blocks, E, K, N);
+  if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * numel * N * sizeof(float))) splits = 1;
+  a.kper = (G + splits - 1) / splits;
+  splits = (G + a.kper - 1) / a.kper;              // no empty splits
+  a.partial = splits > 1 ? (float*)workspace : nullptr;
   a.w_stride = (long)(K / 8) * N / 4;              // u4 elements per expert
   a.s_stride = (long)(K / group_size) * N;
   a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
@@ -607,6 +674,18 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
                      : launch_mt<MI355Q_BF16, true>(a, zeros_kind, block_size / 16, max_blocks, st);
   MQ_REQUIRE(e == hipSuccess, "moe_w4a16: cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("moe_w4a16");
+  if (splits > 1) {
+    // every slot id below numel sits in exactly one block, so every row of the partial tiles is written
+    const long MN = (long)numel * N;
+    const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
+    if (dtype == MI355Q_F16)
+      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
+                         (const float*)workspace, (const uint16_t*)nullptr, topk_weights, MN, N, splits);
+    else
+      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
+                         (const float*)workspace, (const uint16_t*)nullptr, topk_weights, MN, N, splits);
+    MQ_LAUNCH_CHECK("moe_w4a16(split-K reduce)");
+  }
   return 0;
 }
 

@@ -19,6 +19,9 @@ from .. import _lib
 from . import _runtime as rt
 from .quantization import rearrange
 
+# start of the shared scratch reserved for arrival counters (they must stay zero between launches)
+_WS_COUNTER_BYTES = 1 << 20
+
 _lib.load()          # fail at import time when the HIP library is missing
 
 _libs = {
@@ -120,6 +123,14 @@ def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
         z = z.contiguous()
     if bias is not None:
         bias = bias.to(x.dtype).contiguous()
+    # the kernels index these by (group row, column): sizes are checked here, not on the device
+    groups = K // int(group_size) if int(group_size) > 0 else 1
+    if scales.numel() != groups * N:
+        raise RuntimeError(f"w4a16_gemm: scales hold {scales.numel()} values, expected {groups} x {N}")
+    if z is not None and z.numel() != (groups * N // 8 if zk == _lib.ZP_PACKED else groups * N):
+        raise RuntimeError(f"w4a16_gemm: zero-points of shape {tuple(z.shape)} do not fit {groups} groups x {N} columns")
+    if bias is not None and bias.numel() != N:
+        raise RuntimeError(f"w4a16_gemm: bias holds {bias.numel()} values, expected {N}")
     lib = _lib.load()
     with torch.cuda.device(x.device):
         ws_bytes = lib.mi355q_w4a16_workspace_bytes(M, K, N)
@@ -940,6 +951,8 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
     elif B.dtype == torch.int32 or (B.dtype in (torch.uint8, torch.int8) and B.shape[-1] * 2 == K):
         mode = _lib.Q_W4A16
         w = _slab_weight(B, transposed=True)
+        if w.shape[-2] * 8 != K or w.shape[-1] != N:
+            raise RuntimeError(f"fused_moe: int4 experts of shape {tuple(w.shape)} do not fit K={K}, N={N}")
         w_scale = B_scale.contiguous()
         if w_scale.dtype != A.dtype:
             w_scale = w_scale.to(A.dtype)
@@ -981,10 +994,16 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
     if sorted_token_ids.numel() < experts_ids.numel() * block_size:
         raise RuntimeError("fused_moe: sorted_token_ids is shorter than experts_ids * block_size")
     with torch.cuda.device(A.device):
+        ws_ptr = ws_bytes = 0
+        need = _lib.load().mi355q_moe_gemm_workspace_bytes(mode, numel, int(block_size), experts_ids.numel(), E, K, N)
+        if need:
+            # behind the first MiB of the shared scratch, which holds arrival counters that stay zero
+            ws = rt.workspace(A.device, need + _WS_COUNTER_BYTES)
+            ws_ptr, ws_bytes = ws.data_ptr() + _WS_COUNTER_BYTES, ws.numel() - _WS_COUNTER_BYTES
         _lib.call("mi355q_moe_gemm", C.data_ptr(), A.data_ptr(), w.data_ptr(), rt.ptr(a_scale), rt.ptr(w_scale),
                   rt.ptr(zp), zk, mode, group, rt.ptr(tw), sorted_token_ids.data_ptr(), experts_ids.data_ptr(),
                   num_tokens_post_pad.data_ptr(), numel, int(topk), int(block_size), experts_ids.numel(), E, K, N,
-                  act_code, rt.dtype_code(C.dtype), layout, rt.stream_ptr())
+                  act_code, rt.dtype_code(C.dtype), layout, ws_ptr, ws_bytes, rt.stream_ptr())
 
 
 def _fused_moe_quant_kernel_impl(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorted_token_ids,
@@ -1056,7 +1075,7 @@ def _fused_moe_quant_kernel_ex_impl(C, A, B, A_scale, B_scale, B_zero, bias, top
         _lib.call("mi355q_moe_gemm", C.data_ptr(), a16.data_ptr(), w.data_ptr(), out_scale.data_ptr(),
                   w_scale.data_ptr(), 0, _lib.ZP_NONE, _lib.Q_W4_F32SCALE, int(group_k), rt.ptr(tw),
                   sorted_token_ids.data_ptr(), experts_ids.data_ptr(), num_tokens_post_pad.data_ptr(), numel,
-                  int(topk), int(block_size), experts_ids.numel(), E, K, N, code, code, 0, rt.stream_ptr())
+                  int(topk), int(block_size), experts_ids.numel(), E, K, N, code, code, 0, 0, 0, rt.stream_ptr())
 
 
 def _fused_moe_kernel_impl(C, A, B, topk_weights, topk_ids, sorted_topk_ids, expert_ids, num_tokens_post_pad,
