@@ -311,6 +311,8 @@ def main():
         out["w8a8_int8"] = w8a8_gemm_bench(ops, dev, stream, cpu=not args.no_cpu)
         torch.cuda.empty_cache()
     if not args.quick:
+        out["yardsticks"] = yardsticks(dev, stream)
+        torch.cuda.empty_cache()
         out["sweep"] = sweep(ops, dev, stream, args)
         out["moe_w4a16"] = moe_bench(ops, dev, stream, "w4a16", cpu=not args.no_cpu)
         torch.cuda.empty_cache()
@@ -603,6 +605,59 @@ def fp8_dense_bench(ops, dev, stream, iters=12):
                         "TFLOPs": round(2.0 * M * N * K / t / 1e12, 1),
                         "frac_fp8_mfma_peak": round(2.0 * M * N * K / t / 1e12 / 5000.0, 4)}
     return {"workload": "fp8 block-scaled dense linear K=8192 N=28672, bf16 out", **out}
+
+
+def yardsticks(dev, stream, iters=30):
+    """What the chip and the vendor's own library reach on the same shapes and the same kind of data,
+    beside the published peaks: (a) a loop of matrix instructions on register-resident operands
+    (nothing loaded or stored in the loop; fp16: A ~ N(0,1), B ~ N(0, 0.02); int8: uniform), two
+    wavefronts per SIMD; (b) torch.matmul (fp16, dense weights, no dequantisation) at the Llama-3-8B shapes for
+    M = 128 and 2048 and torch._int_mm (int8 -> int32, no scales) at the W8A8 shape."""
+    import ctypes
+    import torch
+    from vllm_gcu_amd.kernels import _runtime as rt
+    probe = ctypes.CDLL(os.path.join(ROOT, "vllm-gcu_amd", "libmi355q_bench.so"))
+    probe.mi355q_bench_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                             ctypes.c_void_p]
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    # launches of about half a millisecond, timed like the GEMMs (the sustained rate over tens of
+    # milliseconds is lower still: the clock keeps dropping under matrix load)
+    wgs, loops = 2 * 256, 800
+    res = {"what": yardsticks.__doc__.split("\n\n")[0].replace("\n    ", " ")}
+    # operands as the GEMMs see them: activations N(0,1), weights N(0, 0.02) (fp16); uniform int8 on both sides
+    f16_src = torch.cat([torch.randn(1 << 20, device=dev), torch.randn(1 << 20, device=dev) * 0.02]).half()
+    for kind, name, src, per in ((0, "mfma_f32_16x16x32_f16", f16_src, 2 * 16 * 16 * 32),
+                                 (1, "mfma_i32_16x16x64_i8",
+                                  torch.randint(-127, 128, (4 << 20,), dtype=torch.int8, device=dev), 2 * 16 * 16 * 64)):
+        def run(kind=kind, src=src):
+            assert probe.mi355q_bench_mfma_rate(src.data_ptr(), kind, wgs, loops, sink.data_ptr(), rt.stream_ptr()) == 0
+        t = time_graph([run], iters, 10, stream) / iters
+        rate = wgs * 4 * loops * 32 * per / t / 1e12
+        peak = FP16_PEAK_TFLOPS if kind == 0 else INT8_PEAK_TOPS
+        res[name] = {"T_per_s": round(rate, 1), "frac_of_published_peak": round(rate / peak, 4)}
+    vend = []
+    for name, K, N in LLAMA3_8B:
+        w = [(torch.randn(K, N, device=dev) * 0.02).half() for _ in range(2)]
+        for M in (128, 2048):
+            x = torch.randn(M, K, device=dev).half()
+            outs = [torch.empty(M, N, dtype=torch.float16, device=dev) for _ in range(2)]
+            fns = [(lambda c=c: torch.matmul(x, w[c], out=outs[c])) for c in range(2)]
+            n = 100 if M <= 128 else iters
+            t = time_graph(fns, n, 10, stream) / n
+            vend.append({"layer": name, "K": K, "N": N, "M": M, "us": round(t * 1e6, 2),
+                         "TFLOPs": round(2.0 * M * K * N / t / 1e12, 1)})
+        del w
+        torch.cuda.empty_cache()
+    res["vendor_fp16_gemm"] = vend
+    M, K, N = 2048, 8192, 28672
+    a = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev)
+    b = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev).t()
+    try:
+        t = time_graph([lambda: torch._int_mm(a, b)], iters, 40, stream) / iters
+        res["vendor_int8_mm"] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1), "TOPs": round(2.0 * M * K * N / t / 1e12, 1)}
+    except RuntimeError as e:
+        res["vendor_int8_mm"] = {"error": str(e)[:120]}
+    return res
 
 
 def sweep(ops, dev, stream, args):

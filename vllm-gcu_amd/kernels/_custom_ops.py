@@ -961,6 +961,13 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
             zp = zp.contiguous()
         if group <= 0:
             group = K
+        ne, groups = w.shape[0], K // group
+        if w_scale.numel() != ne * groups * N:
+            raise RuntimeError(f"fused_moe: int4 expert scales of shape {tuple(w_scale.shape)} do not fit "
+                               f"{ne} experts x {groups} groups x {N} columns")
+        if zp is not None and zp.numel() != ne * groups * (N // 8 if zk == _lib.ZP_PACKED else N):
+            raise RuntimeError(f"fused_moe: int4 expert zero-points of shape {tuple(zp.shape)} do not fit "
+                               f"{ne} experts x {groups} groups x {N} columns")
         act_code = rt.dtype_code(A.dtype)
     elif B.dtype == torch.int8:
         mode = _lib.Q_W8A16
