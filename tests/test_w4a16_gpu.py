@@ -297,6 +297,34 @@ def test_tile_gemm_zero_kinds_and_group_256(ops, rearrange):
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("M", [33, 64, 100, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_narrow_tiles_mid_rows(ops, rearrange, M, dtype):
+    """33..128 rows on layers up to 8192 wide run 32-row x 64-column workgroups (one tile per wavefront,
+    two K blocks in flight), with K split up to four ways on a narrow layer: packed, absent and float
+    zero-points, group 128 and 256, bias, ragged last row block, exact inputs bit for bit."""
+    print(f"case narrow tiles M={M} {dtype}", flush=True)
+    for K, N, g in ((4096, 512, 128), (1024, 1152, 256)):
+        q, z, s, x = make_case(M + K + N, M, K, N, g)
+        bias = np.random.default_rng(4).standard_normal(N).astype(np.float32)
+        got = run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias, family=2)
+        assert torch.equal(got, run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias, family=2))
+        np.testing.assert_allclose(got.float().cpu().numpy(), oracle(q, z, s, x, g, dtype, bias=bias), rtol=RTOL, atol=ATOL)
+        w, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
+        xs, sd = to_act(x, dtype).cuda(), to_act(s, dtype).cuda()
+        out = ops.w4a16_gemm(xs, w, sd, None, None, g, family=2)
+        np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, None, s, x, g, dtype), rtol=RTOL, atol=ATOL)
+        sf = to_act(s, dtype).float().numpy()
+        zs = to_act(z.astype(np.float32) * sf, dtype)
+        out = ops.w4a16_gemm(xs, w, sd, zs.cuda(), None, g, family=2)
+        # the kernels recover the integer zero-point from z * s (rounded to the activation type), so the
+        # result is that of the integer form; q * s - round(z * s) differs from it by the rounding of z * s
+        np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, z, s, x, g, dtype), rtol=RTOL, atol=ATOL)
+    q, z, s, x = make_case(6, M, 4096, 256, 128, exact=True)
+    got = run_gemm(ops, rearrange, q, z, s, x, 128, torch.float16, family=2)
+    assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, 128, torch.float16)).to(torch.float16))
+
+
 def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):
     M, K, N, g = 150, 256, 128, 64
     q, z, s, x = make_case(5, M, K, N, g)

@@ -43,6 +43,7 @@ struct TileArgs {
   // tile to partial[z][M][N] (grouped: M = numel, rows indexed by slot id, routing weight not yet
   // applied); a second kernel adds the partials up
   int kper;                   // K blocks per split (G when there is no split)
+  uint32_t gpk_magic;         // narrow kernel: ceil(2^32 / (gs / 128)), 0 when a group is one K block
   float* partial;             // null: write the output directly
   long w_stride, s_stride, z_stride;   // per-expert strides in elements of the respective arrays
 };
@@ -499,6 +500,202 @@ hipError_t launch_one(const TileArgs& a, int row_blocks, hipStream_t st) {
   return launch_wm<DT, ZK, MT, GROUPED, WM, SF32>(a, row_blocks, st);
 }
 
+// ---- narrow column tiles for mid-sized M ---------------------------------------------------------
+// Between the decode kernel's 32 rows and a few hundred rows the weights are read about once (a
+// streaming problem) while a 256-column tile leaves a narrow layer with a handful of workgroups, which
+// K then has to be split many ways to occupy the chip: at M = 128 on a 4096-column layer eight splits
+// wrote and re-read 17 MB of fp32 partial tiles, more time than the GEMM itself.  Here a wavefront
+// owns NTW = 1 or 2 of the 16-column tiles (64 or 128 columns per workgroup), so the columns supply
+// the workgroups and K is split little or not at all; the 16 MT activation rows are still shared by the
+// four wavefronts through LDS.  Plain loop (the compiler schedules it), several workgroups per CU.
+template <int DT, int ZK, int MT, int NTW, int D>
+__global__ void __launch_bounds__(256, 2)
+w4a16_tile_narrow_kernel(TileArgs a) {
+  typedef TileMma<DT> MM;
+  typedef typename MM::vec vec;
+  constexpr int BM = 16 * MT, A_BUF = BM * A_ROW;
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, kq = lane >> 4;
+  const int N = a.N, K = a.K, M = a.M;
+  const int G = K >> 7;
+  const int m0 = blockIdx.y * BM;
+  // tile index inside the matrix: 8 tiles per 128-column slab; tile t of a slab holds its columns 8 c + t
+  const int tile = ((int)blockIdx.x * 4 + wave) * NTW;
+  const bool live = tile < (N >> 4);
+  const int slab = live ? tile >> 3 : 0;
+  const int t0 = live ? tile & 7 : 0;
+  const int ncol = 128 * slab + 8 * c + t0;          // first of this lane's NTW adjacent columns
+
+  f4 acc[MT][NTW];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
+  const DqConst dqk = dq_consts();
+
+  const int arow = tid >> 4, achunk = tid & 15;
+  // Buffer loads: lane offset in a register, block offset in a scalar, so a load costs no vector
+  // arithmetic, and a block index past the matrix reads zeros instead of faulting (the ring runs D
+  // blocks ahead of the last one).
+  typedef __amdgpu_buffer_rsrc_t rsrc_t;
+  auto make_rsrc = [](const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+  };
+  const int rows_q = K / a.gs;
+  const rsrc_t xres = make_rsrc(a.x, (uint32_t)M * (uint32_t)K * 2u);
+  const rsrc_t wres = make_rsrc(a.qw + (size_t)slab * G * 512, (uint32_t)G * 8192u);
+  const rsrc_t sres = make_rsrc(a.scales, (uint32_t)rows_q * (uint32_t)N * 2u);
+  const rsrc_t zres = make_rsrc(a.zeros, ZK == MI355Q_ZP_PACKED ? (uint32_t)rows_q * (uint32_t)(N >> 3) * 4u
+                                                                 : (uint32_t)rows_q * (uint32_t)N * 2u);
+  uint32_t aofs[MT];
+#pragma unroll
+  for (int p = 0; p < MT; ++p)
+    aofs[p] = ((uint32_t)min(m0 + p * 16 + arow, M - 1) * (uint32_t)K + 8u * achunk) * 2u;
+  const uint32_t wofs = (uint32_t)(t0 * 64 + lane) * 16u;
+  // A K block is short here (a few hundred cycles), far shorter than a trip to memory: the loads of
+  // D blocks are in flight at any time, each block's in its own slot of a register ring (the loop
+  // is unrolled D times, so the slots are fixed registers).
+  u4 ar[D][MT], wr[D][NTW];
+  // scales (and float zero-points) of the aligned group of four tiles this wavefront's tiles lie in:
+  // whole 8-byte loads (a 16-bit load only writes half a register, which ties it to the register's
+  // previous load and serialises the ring)
+  uint2 sr[D], zsr[D];
+  uint32_t zr[D];
+  const int tsel = 16 * (t0 & 3), ncol4 = ncol - (t0 & 3);
+  auto pick = [&](uint2 v, int t) {
+    const unsigned long long q = ((unsigned long long)v.y << 32) | v.x;
+    return (uint16_t)(q >> (tsel + 16 * t));
+  };
+  const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
+  auto issue = [&](int d, int g) {
+#pragma unroll
+    for (int p = 0; p < MT; ++p)
+      ar[d][p] = bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(xres, (int)aofs[p], g * 256, 0));
+#pragma unroll
+    for (int t = 0; t < NTW; ++t)
+      wr[d][t] = bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(wres, (int)wofs, g * 8192 + t * 1024, 0));
+    const int qrow = a.gpk_magic ? (int)__umulhi((uint32_t)g, a.gpk_magic) : g;
+    sr[d] = bitcast<uint2>(__builtin_amdgcn_raw_buffer_load_b64(sres, ncol4 * 2, qrow * N * 2, 0));
+    if (ZK == MI355Q_ZP_PACKED)
+      zr[d] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(zres, (ncol >> 3) * 4, qrow * (N >> 3) * 4, 0);
+    if (ZK == MI355Q_ZP_PRESCALED)
+      zsr[d] = bitcast<uint2>(__builtin_amdgcn_raw_buffer_load_b64(zres, ncol4 * 2, qrow * N * 2, 0));
+  };
+  auto store_a = [&](int d, unsigned buf_off) {
+#pragma unroll
+    for (int p = 0; p < MT; ++p) *(u4*)(lds + buf_off + (p * 16 + arow) * A_ROW + achunk * 16) = ar[d][p];
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) issue(d, gb + d);
+  store_a(0, 0);
+  __syncthreads();
+  auto kblock = [&](int d, int g) {
+    const unsigned buf = ((g - gb) & 1) * A_BUF;
+    u4 wcur[NTW];
+    float sc[NTW];
+    h2 zz[NTW];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      wcur[t] = wr[d][t];
+      sc[t] = Elem<DT>::to_f32(pick(sr[d], t));
+      float zf;
+      if (ZK == MI355Q_ZP_PRESCALED) zf = __builtin_rintf(Elem<DT>::to_f32(pick(zsr[d], t)) / sc[t]);   // z * s -> z
+      else if (ZK == MI355Q_ZP_PACKED) zf = (float)((zr[d] >> (4 * (t0 + t))) & 15u);
+      else zf = 8.0f;
+      zz[t] = (h2){(_Float16)(1024.0f + zf), (_Float16)(64.0f + zf)};
+    }
+    vec bv[4][NTW];
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) bv[st][t] = MM::dequant(wcur[t][st], zz[t], dqk);
+    // the activations of block g went to LDS during block g - 1: the slot is free again
+    issue(d, g + D);
+    const unsigned char* abase = lds + buf + c * A_ROW + kq * 16;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      f4 part[NTW];
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const vec av = bitcast<vec>(*(const u4*)(abase + mt * 16 * A_ROW + st * 64));
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) part[t] = MM::run(av, bv[st][t], part[t]);
+      }
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) acc[mt][t] += sc[t] * part[t];
+    }
+    // block g + 1 into the other buffer (last read during block g - 1: every wavefront has passed
+    // the barrier since)
+    store_a((d + 1) % D, A_BUF - buf);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);               // blocks stay apart: merged, their operands overflow the registers
+  };
+  // whole rounds of the ring without a branch inside (a branch between the blocks makes the
+  // compiler wait for every load in flight at each of them), then the remaining blocks one by one
+  int g0 = gb;
+  for (; g0 + D <= ge; g0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) kblock(d, g0 + d);
+  }
+#pragma unroll
+  for (int d = 0; d < D - 1; ++d) {
+    if (g0 + d < ge) kblock(d, g0 + d);
+  }
+
+  if (!live) return;
+  float bs[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) bs[t] = a.bias ? Elem<DT>::to_f32(a.bias[ncol + t]) : 0.f;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + mt * 16 + 4 * kq + i;
+      if (m >= M) continue;
+      if (a.partial) {
+        float* pp = a.partial + ((size_t)blockIdx.z * M + m) * N + ncol;
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) pp[t] = acc[mt][t][i];
+      } else {
+        uint16_t* po = a.out + (size_t)m * N + ncol;
+        if (NTW == 2) {
+          *(uint32_t*)po = (uint32_t)Elem<DT>::from_f32(acc[mt][0][i] + bs[0]) |
+                           ((uint32_t)Elem<DT>::from_f32(acc[mt][NTW - 1][i] + bs[NTW - 1]) << 16);
+        } else {
+#pragma unroll
+          for (int t = 0; t < NTW; ++t) po[t] = Elem<DT>::from_f32(acc[mt][t][i] + bs[t]);
+        }
+      }
+    }
+}
+
+template <int DT, int ZK, int MT, int NTW, int D>
+hipError_t launch_narrow_one(const TileArgs& a, int row_blocks, hipStream_t st) {
+  const int G = a.K >> 7;
+  dim3 grid((a.N / 16 + 4 * NTW - 1) / (4 * NTW), row_blocks, (G + a.kper - 1) / a.kper), block(256);
+  const size_t shmem = 2 * 16 * MT * A_ROW;
+  hipLaunchKernelGGL((w4a16_tile_narrow_kernel<DT, ZK, MT, NTW, D>), grid, block, shmem, st, a);
+  return hipSuccess;
+}
+template <int DT, int ZK>
+hipError_t launch_narrow_zk(const TileArgs& a, int mt, int ntw, int row_blocks, hipStream_t st) {
+  // measured on the Llama-3-8B layers for 33..128 rows: 32-row blocks of one tile per wavefront with two
+  // K blocks in flight; rings of 4 and 8 blocks and 64-row blocks were no faster (the deeper rings spill)
+  (void)mt;
+  (void)ntw;
+  return launch_narrow_one<DT, ZK, 2, 1, 2>(a, row_blocks, st);
+}
+template <int DT>
+hipError_t launch_narrow(const TileArgs& a, int zk, int mt, int ntw, int row_blocks, hipStream_t st) {
+  if (zk == MI355Q_ZP_NONE) return launch_narrow_zk<DT, MI355Q_ZP_NONE>(a, mt, ntw, row_blocks, st);
+  if (zk == MI355Q_ZP_PACKED) return launch_narrow_zk<DT, MI355Q_ZP_PACKED>(a, mt, ntw, row_blocks, st);
+  return launch_narrow_zk<DT, MI355Q_ZP_PRESCALED>(a, mt, ntw, row_blocks, st);
+}
+
 template <int DT, int MT, bool GROUPED>
 hipError_t launch_zk(const TileArgs& a, int zk, int row_blocks, hipStream_t st) {
   if constexpr (GROUPED) {
@@ -540,8 +737,9 @@ static int tile_splits(int M, int K, int N) {
   // 64-row tiles run two workgroups per CU
   const long target = (long)device_cu_count() * (mt == 4 ? 2 : 1);
   long s;
-  if (wgs * 2 > target) {
-    // More than half a round already.  A workgroup alone on its CU runs a K block in about 60 %
+  if (wgs * 5 >= target * 2) {
+    // 40 % of a round or more (a wide layer at about a hundred rows: N 28672, M 128: 47 -> 43 us
+    // without the two-way split).  A workgroup alone on its CU runs a K block in about 60 %
     // of the time of two that share one, so between 1/2 and 0.7 of a round over a long K three
     // splits (two even rounds of a third of K) beat one uneven round: K 14336, N 4096,
     // M 1100..1280: 203 -> 167..175 us; above that, and for K 4096, no split count gained.
@@ -556,8 +754,23 @@ static int tile_splits(int M, int K, int N) {
   while (s > 1 && (size_t)s * M * N * sizeof(float) > TILE_SPLITK_BYTES) --s;
   return s < 1 ? 1 : (int)s;
 }
+// 33..128 rows on a layer of moderate K whose 256-column tiles would need K split many ways: the
+// narrow kernel (32 rows x 64 columns per workgroup) with as few splits as bring the grid to about
+// two workgroups per CU, four at most.  Returns the split count, 0 = use the wide tiles.
+// (Llama-3-8B o / qkv, M = 64: 16.7 / 19.6 -> 13.9 / 16.7 us; M = 128: 22.1 / 23.4 -> 17.8 / 20.8 us;
+// K = 14336 and N = 28672 measured equal or slower and stay on the wide tiles.)
+static int tile_narrow_splits(int M, int K, int N) {
+  if (M <= 32 || M > 128 || K > 8192 || N > 8192) return 0;
+  const long wgs = (long)((M + 31) / 32) * (N / 64), target = 2L * device_cu_count();
+  if (wgs >= target) return 1;
+  long s = target / wgs;
+  if (s > 4) s = 4;
+  if (s > K / 128 / 4) s = K / 128 / 4;
+  return s < 1 ? 1 : (int)s;
+}
 size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
-  const int s = tile_splits(M, K, N);
+  const int narrow = tile_narrow_splits(M, K, N);
+  const int s = narrow ? narrow : tile_splits(M, K, N);
   return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
 }
 
@@ -575,16 +788,30 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   a.zeros = zeros;
   a.bias = (const uint16_t*)bias;
   a.M = M; a.K = K; a.N = N; a.gs = group_size;
-  const int mt = tile_rows_mt(M, N);
-  const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
+  int mt = tile_rows_mt(M, N);
+  int ntw = 4;
   const int G = K / 128;
   int splits = tile_splits(M, K, N);
+  const int narrow = tile_narrow_splits(M, K, N);
+  if (narrow) {
+    mt = 2;
+    ntw = 1;
+    splits = narrow;
+  }
+  const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
   if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * M * N * sizeof(float))) splits = 1;
   a.kper = (G + splits - 1) / splits;
   splits = (G + a.kper - 1) / a.kper;                // no empty splits
   a.partial = splits > 1 ? (float*)workspace : nullptr;
-  hipError_t e = (dtype == MI355Q_F16) ? launch_mt<MI355Q_F16, false>(a, zeros_kind, mt, row_blocks, st)
-                                       : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
+  hipError_t e;
+  const uint32_t gpk = (uint32_t)group_size / 128u;
+  a.gpk_magic = gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + gpk - 1) / gpk) : 0u;
+  if (ntw < 4)
+    e = (dtype == MI355Q_F16) ? launch_narrow<MI355Q_F16>(a, zeros_kind, mt, ntw, row_blocks, st)
+                              : launch_narrow<MI355Q_BF16>(a, zeros_kind, mt, ntw, row_blocks, st);
+  else
+    e = (dtype == MI355Q_F16) ? launch_mt<MI355Q_F16, false>(a, zeros_kind, mt, row_blocks, st)
+                              : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
   MQ_REQUIRE(e == hipSuccess, "w4a16_gemm(tile): cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("w4a16_gemm(tile)");
   if (splits > 1) {
