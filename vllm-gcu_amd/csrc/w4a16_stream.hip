@@ -28,6 +28,8 @@ struct StreamArgs {
   int gs;            // quantisation group size (rows of K per scale row)
   uint32_t gs_magic; // ceil(2^32 / gs): k / gs == umulhi(k, gs_magic) for every k < K
   int splits;
+  int per;           // K blocks per split: ceil(K / 128 / splits) (host-side: no division in the kernel's prologue)
+  int qrows;         // K / gs
   float* partial;    // [splits][16*MT][N]
   int* counters;     // one per blockIdx.x (<= N/16), zero between launches
   // grouped (fused-MoE) launches: blockIdx.z = block of 16 sorted token slots, all of one expert
@@ -229,7 +231,7 @@ w4a16_stream_kernel(StreamArgs a) {
   constexpr int HW = NT >= 2 ? NT / 2 : 1;            // packed 16-bit pairs per lane
   const int slab = blockIdx.x / TG, t0 = (blockIdx.x % TG) * NT, split = blockIdx.y;
   const int G = a.K >> 7;
-  const int per = (G + a.splits - 1) / a.splits;
+  const int per = a.per;
   const int gb = split * per;
   const int ge = min(G, gb + per);
   const int N = a.N, K = a.K;
@@ -259,20 +261,15 @@ w4a16_stream_kernel(StreamArgs a) {
     u4 xr[XA ? 4 * MT : 1];
   };
   constexpr int W = 4;                                // wavefronts per workgroup (8 and 16 were measured: not faster)
-  // K blocks of this wavefront: gb + wave, + W, ...; visited from a
-  // workgroup-dependent start (see the loop below)
+  // K blocks of this wavefront: gb + wave, + W, ... in order (starting each workgroup at a different
+  // block of its range was measured equal, and the modulo sat in front of the first loads)
   const int g0 = gb + wave;
   const int nb = (ge - g0 + W - 1) / W;
-  const int rot = nb > 0 ? (int)((blockIdx.x >> 3) * 5u % (unsigned)nb) : 0;
-  auto blk = [&](int i) {                            // i-th block in this workgroup's order, i < nb
-    int j = i + rot;
-    if (j >= nb) j -= nb;
-    return g0 + W * j;
-  };
+  auto blk = [&](int i) { return g0 + W * i; };      // i-th block of this wavefront, i < nb
   const rsrc_t wres = make_rsrc(a.qw + (size_t)slab * G * 512, (uint32_t)G * 8192u);
-  const rsrc_t sres = make_rsrc(a.scales, (uint32_t)(K / a.gs) * N * 2u);
-  const rsrc_t zres = make_rsrc(a.zeros, ZK == MI355Q_ZP_PACKED ? (uint32_t)(K / a.gs) * (N >> 3) * 4u
-                                                                 : (uint32_t)(K / a.gs) * N * 2u);
+  const rsrc_t sres = make_rsrc(a.scales, (uint32_t)a.qrows * N * 2u);
+  const rsrc_t zres = make_rsrc(a.zeros, ZK == MI355Q_ZP_PACKED ? (uint32_t)a.qrows * (N >> 3) * 4u
+                                                                 : (uint32_t)a.qrows * N * 2u);
   const rsrc_t xres = make_rsrc(a.x, (uint32_t)a.M * K * 2u);
   const uint32_t wlane = (uint32_t)(t0 * 64 + lane) * 16u;
   uint32_t xlane[MT];
@@ -624,6 +621,8 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
   // no empty splits: ceil(G / splits) * (splits - 1) < G
   while (splits > 1 && ((G + splits - 1) / splits) * (splits - 1) >= G) --splits;
   a.splits = splits;
+  a.per = (G + splits - 1) / splits;
+  a.qrows = K / group_size;
   a.partial = nullptr;
   a.counters = nullptr;
   if (splits > 1) {
@@ -685,6 +684,8 @@ int w4a16_stream_grouped_launch(void* out, const void* x, const int32_t* qweight
   a.K = K; a.N = N; a.gs = group_size;
   a.gs_magic = (uint32_t)((((uint64_t)1 << 32) + group_size - 1) / group_size);
   a.splits = 1;
+  a.per = K / 128;
+  a.qrows = K / group_size;
   a.sorted_ids = sorted_ids; a.expert_ids = expert_ids; a.npp = npp; a.topk_weights = topk_weights;
   a.numel = numel; a.topk = topk; a.E = E;
   a.w_stride = (long)(K / 8) * N / 4;
