@@ -38,10 +38,12 @@ INT8_PEAK_TOPS = 5000.0
 # then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy of --calibrate-copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per
 # unit).  Keyed by (M, --split-k); other settings were not profiled.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 34011114}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 34012173}
 # when and on which build the figure above was taken; it must be re-measured (profiles/ names the
 # commands) whenever the streaming kernel's work split changes
-MEASURED_TRAFFIC_PROVENANCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, 2026-11-25, work split unchanged since"
+MEASURED_TRAFFIC_PROVENANCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (commands and per-layer figures in "
+                               "profiles/w4a16_stream_kernel_llama3_8b_m16.txt), re-measured after the last change to the "
+                               "streaming kernel; work split unchanged since")
 
 
 def w4a16_bytes(M, K, N, g=GROUP):
@@ -618,7 +620,8 @@ def yardsticks(dev, stream, iters=30):
     from vllm_gcu_amd.kernels import _runtime as rt
     probe = ctypes.CDLL(os.path.join(ROOT, "vllm-gcu_amd", "libmi355q_bench.so"))
     probe.mi355q_bench_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
-                                             ctypes.c_void_p]
+                                             ctypes.c_void_p, ctypes.c_void_p]
+    clk = torch.zeros(2, dtype=torch.int64, device=dev)
     sink = torch.zeros(16, dtype=torch.uint8, device=dev)
     # launches of about half a millisecond, timed like the GEMMs (the sustained rate over tens of
     # milliseconds is lower still: the clock keeps dropping under matrix load)
@@ -630,11 +633,17 @@ def yardsticks(dev, stream, iters=30):
                                  (1, "mfma_i32_16x16x64_i8",
                                   torch.randint(-127, 128, (4 << 20,), dtype=torch.int8, device=dev), 2 * 16 * 16 * 64)):
         def run(kind=kind, src=src):
-            assert probe.mi355q_bench_mfma_rate(src.data_ptr(), kind, wgs, loops, sink.data_ptr(), rt.stream_ptr()) == 0
+            assert probe.mi355q_bench_mfma_rate(src.data_ptr(), kind, wgs, loops, sink.data_ptr(), clk.data_ptr(),
+                                                rt.stream_ptr()) == 0
         t = time_graph([run], iters, 10, stream) / iters
         rate = wgs * 4 * loops * 32 * per / t / 1e12
         peak = FP16_PEAK_TFLOPS if kind == 0 else INT8_PEAK_TOPS
-        res[name] = {"T_per_s": round(rate, 1), "frac_of_published_peak": round(rate / peak, 4)}
+        ticks = clk.cpu().tolist()
+        # core clock inside the loop: shader-clock ticks per tick of the 100 MHz reference counter
+        ghz = ticks[0] / max(1, ticks[1]) * 0.1
+        res[name] = {"T_per_s": round(rate, 1), "frac_of_published_peak": round(rate / peak, 4),
+                     "core_clock_GHz_in_loop": round(ghz, 3),
+                     "cycles_per_instruction_per_SIMD": round(ticks[0] / (2.0 * loops * 32), 2)}
     vend = []
     for name, K, N in LLAMA3_8B:
         w = [(torch.randn(K, N, device=dev) * 0.02).half() for _ in range(2)]

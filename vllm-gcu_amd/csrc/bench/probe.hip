@@ -43,8 +43,10 @@ typedef int i4 __attribute__((ext_vector_type(4)));
 // first 2 MiB of `src` and 4 B operands from the second 2 MiB once (whatever the caller put there: the
 // rate depends on the data, the chip being power-limited) and runs iters x 32 independent accumulations.
 template <int KIND>
-__global__ void __launch_bounds__(256) probe_mfma_kernel(const u4* src, int iters, u4* sink) {
+__global__ void __launch_bounds__(256) probe_mfma_kernel(const u4* src, int iters, u4* sink, unsigned long long* clk) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // core-clock ticks and 100 MHz reference ticks around the loop: the clock the chip grants under this load
+  const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
   u4 a[8], b[4];
 #pragma unroll
   for (int i = 0; i < 8; ++i) a[i] = src[((blockIdx.x * 4 + wave) * 8 + i) % 2048 * 64 + lane];
@@ -69,6 +71,10 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(const u4* src, int iter
         asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acci[c]) : "v"(a[c & 7]), "v"(b[c >> 3]));
     }
   }
+  if (clk && blockIdx.x == gridDim.x / 2 && threadIdx.x == 0) {
+    clk[0] = __builtin_amdgcn_s_memtime() - c0;
+    clk[1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
   f4 rf = {0.f, 0.f, 0.f, 0.f};
   i4 ri = {0, 0, 0, 0};
 #pragma unroll
@@ -83,11 +89,15 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(const u4* src, int iter
 // 0 on success.  src: 2 MiB of A then 2 MiB of B operand data (fp16 values or int8 values); one workgroup of four
 // wavefronts per launch slot, `workgroups` of them; operations done = workgroups * 4 * iters * 32 *
 // (2 * 16 * 16 * 32 for kind 0, 2 * 16 * 16 * 64 for kind 1).
-extern "C" int mi355q_bench_mfma_rate(const void* src, int kind, int workgroups, int iters, void* sink, void* stream) {
+// clk (optional): two 64-bit words, core-clock and 100 MHz reference ticks one wavefront spent in the loop.
+extern "C" int mi355q_bench_mfma_rate(const void* src, int kind, int workgroups, int iters, void* sink, void* clk,
+                                      void* stream) {
   if (!src || !sink || workgroups <= 0 || workgroups > 65536 || iters <= 0 || (kind != 0 && kind != 1)) return 1;
   if (kind == 0)
-    hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (const u4*)src, iters, (u4*)sink);
+    hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (const u4*)src, iters, (u4*)sink,
+                       (unsigned long long*)clk);
   else
-    hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (const u4*)src, iters, (u4*)sink);
+    hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (const u4*)src, iters, (u4*)sink,
+                       (unsigned long long*)clk);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
