@@ -590,7 +590,7 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
                         const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
                         int group_size, int dtype, void* workspace, size_t workspace_bytes,
                         int split_k, hipStream_t st) {
-  StreamArgs a;
+  StreamArgs a = {};
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;
   a.qw = (const u4*)qweight;
