@@ -125,17 +125,17 @@ __device__ __forceinline__ void store_partial(float* p, const float* v) {
   }
 }
 template <int NT>
-__device__ __forceinline__ void load_partial_add(const float* p, float* v) {
+__device__ __forceinline__ void load_partial(const float* p, float* v) {
   if (NT == 1) {
     uint32_t bits = __hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v[0] += bitcast<float>(bits);
+    v[0] = bitcast<float>(bits);
     return;
   }
 #pragma unroll
   for (int t = 0; t + 1 < NT; t += 2) {
     uint64_t bits = __hip_atomic_load((const uint64_t*)(p + t), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v[t] += bitcast<float>((uint32_t)bits);
-    v[t + 1] += bitcast<float>((uint32_t)(bits >> 32));
+    v[t] = bitcast<float>((uint32_t)bits);
+    v[t + 1 < NT ? t + 1 : t] = bitcast<float>((uint32_t)(bits >> 32));
   }
 }
 
@@ -491,8 +491,22 @@ w4a16_stream_kernel(StreamArgs a) {
     float v[CW];
 #pragma unroll
     for (int t = 0; t < CW; ++t) v[t] = 0.f;
-    for (int sp = 0; sp < a.splits; ++sp)
-      load_partial_add<CW>(a.partial + ((size_t)sp * Mpad + m) * N + ncol + tc, v);
+    // four splits' tiles are requested together and then added in split order: one trip to memory
+    // per four splits instead of one per split (a loop of load-then-add waits for every load in turn)
+    for (int sp = 0; sp < a.splits; sp += 4) {
+      float w[4][CW];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int spj = min(sp + j, a.splits - 1);   // past the end: a repeat that is not added
+        load_partial<CW>(a.partial + ((size_t)spj * Mpad + m) * N + ncol + tc, w[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (sp + j < a.splits) {
+#pragma unroll
+          for (int t = 0; t < CW; ++t) v[t] += w[j][t];
+        }
+    }
     store_out_row<DT, CW>(a.out + (size_t)m * N + ncol + tc, a.bias, ncol + tc, v);
   }
   if (threadIdx.x == 0)

@@ -469,7 +469,18 @@ w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* 
   const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= MN) return;
   f4 v = *(const f4*)(partial + i);
-  for (int s = 1; s < splits; ++s) v += *(const f4*)(partial + (size_t)s * MN + i);
+  // four splits requested together, added in split order (a loop of load-then-add would wait for a
+  // trip to memory per split)
+  int s = 1;
+  for (; s + 3 < splits; s += 4) {
+    const f4 p0 = *(const f4*)(partial + (size_t)s * MN + i), p1 = *(const f4*)(partial + (size_t)(s + 1) * MN + i);
+    const f4 p2 = *(const f4*)(partial + (size_t)(s + 2) * MN + i), p3 = *(const f4*)(partial + (size_t)(s + 3) * MN + i);
+    v += p0;
+    v += p1;
+    v += p2;
+    v += p3;
+  }
+  for (; s < splits; ++s) v += *(const f4*)(partial + (size_t)s * MN + i);
   if (row_weight) v *= row_weight[i / N];
   if (bias) {
     const int n = (int)(i % N);
