@@ -161,7 +161,7 @@ extern "C" int mi355q_w4a16_gemm_noalloc(void* out, const void* x, const int32_t
   if (counters) {
     // the arrival counters must start at zero whatever an earlier call left behind (a fill kernel, not
     // a memset: callers may be capturing a graph)
-    const int words = N / 16;
+    const int words = N / 16 * 4;                  // one counter per wavefront of every possible workgroup
     hipLaunchKernelGGL(noalloc_clear_kernel, dim3((words + 255) / 256), dim3(256), 0, as_stream(stream),
                        (uint32_t*)ws, words);
     MQ_LAUNCH_CHECK("w4a16_gemm_noalloc(clear)");

@@ -31,7 +31,7 @@ struct StreamArgs {
   int per;           // K blocks per split: ceil(K / 128 / splits) (host-side: no division in the kernel's prologue)
   int qrows;         // K / gs
   float* partial;    // [splits][16*MT][N]
-  int* counters;     // one per blockIdx.x (<= N/16), zero between launches
+  int* counters;     // four per blockIdx.x (<= N/16 workgroups, one per wavefront), zero between launches
   // grouped (fused-MoE) launches: blockIdx.z = block of 16 sorted token slots, all of one expert
   const int32_t* sorted_ids;    // [.. padded ..] slot ids, pads >= numel
   const int32_t* expert_ids;    // [blocks]
@@ -469,21 +469,21 @@ w4a16_stream_kernel(StreamArgs a) {
 
   // ---- cross-workgroup split-K ---------------------------------------------
   // Partial tiles travel as device-scope relaxed accesses (they bypass the
-  // per-XCD L2 instead of flushing it).  Every wavefront waits until its own
-  // partial stores have been acknowledged (vmcnt counts stores on gfx9) and
-  // only then joins the barrier that precedes the arrival count -- the
-  // barrier alone does not wait for memory operations in flight.  The last
-  // workgroup to arrive adds the tiles in split order, so the sum is
-  // reproducible.
-  __shared__ int is_last;
+  // per-XCD L2 instead of flushing it).  The exchange is per wavefront: each of
+  // the four wavefronts owns a slice of the workgroup's tile (its rows and
+  // columns of the LDS reduction above) and an arrival counter of its own.  A
+  // wavefront waits until its own partial stores have been acknowledged (vmcnt
+  // counts stores on gfx9), then counts itself in; the wavefront that arrives
+  // last at a slice adds that slice's tiles in split order, so the sum is
+  // reproducible.  No workgroup barrier: the wavefronts of a workgroup do not
+  // wait for each other's trips to memory.
+  if (!fin_wave) return;
   __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int old = __hip_atomic_fetch_add(a.counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    is_last = (old == a.splits - 1);
-  }
-  __syncthreads();
-  if (!is_last) return;
+  int* counter = a.counters + (int)blockIdx.x * W + wave;
+  int old = 0;
+  if (lane == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  old = __builtin_amdgcn_readfirstlane(old);
+  if (old != a.splits - 1) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + 4 * kq + ri;
@@ -509,8 +509,7 @@ w4a16_stream_kernel(StreamArgs a) {
     }
     store_out_row<DT, CW>(a.out + (size_t)m * N + ncol + tc, a.bias, ncol + tc, v);
   }
-  if (threadIdx.x == 0)
-    __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 struct StreamPlan { int nt, splits; };
@@ -642,7 +641,7 @@ int w4a16_stream_launch(void* out, const void* x, const int32_t* qweight, const 
   if (splits > 1) {
     const int Mpad = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
     const size_t cbytes = STREAM_COUNTER_BYTES;
-    MQ_REQUIRE((size_t)(N / 16) * sizeof(int) <= cbytes, "w4a16_gemm(stream): N=%d needs more arrival counters than the workspace holds", N);
+    MQ_REQUIRE((size_t)(N / 16) * 4 * sizeof(int) <= cbytes, "w4a16_gemm(stream): N=%d needs more arrival counters than the workspace holds", N);
     size_t need = cbytes + (size_t)splits * Mpad * N * sizeof(float);
     MQ_REQUIRE(workspace && workspace_bytes >= need,
                "w4a16_gemm: workspace of %zu bytes needed for split_k=%d, got %zu", need, splits,
