@@ -687,27 +687,24 @@ w4a16_tile_narrow_kernel(TileArgs a) {
     }
 }
 
-template <int DT, int ZK, int MT, int NTW, int D>
-hipError_t launch_narrow_one(const TileArgs& a, int row_blocks, hipStream_t st) {
+// The one configuration that is launched: 32-row blocks, one tile per wavefront, two K blocks in
+// flight.  Measured on the Llama-3-8B layers for 33..128 rows: rings of 4 and 8 blocks were no
+// faster (the deeper rings spill: every slot is live across the whole unrolled loop), nor were
+// 64-row blocks or two tiles per wavefront.
+template <int DT, int ZK>
+hipError_t launch_narrow_zk(const TileArgs& a, int row_blocks, hipStream_t st) {
+  constexpr int MT = 2, NTW = 1, D = 2;
   const int G = a.K >> 7;
   dim3 grid((a.N / 16 + 4 * NTW - 1) / (4 * NTW), row_blocks, (G + a.kper - 1) / a.kper), block(256);
   const size_t shmem = 2 * 16 * MT * A_ROW;
   hipLaunchKernelGGL((w4a16_tile_narrow_kernel<DT, ZK, MT, NTW, D>), grid, block, shmem, st, a);
   return hipSuccess;
 }
-template <int DT, int ZK>
-hipError_t launch_narrow_zk(const TileArgs& a, int mt, int ntw, int row_blocks, hipStream_t st) {
-  // measured on the Llama-3-8B layers for 33..128 rows: 32-row blocks of one tile per wavefront with two
-  // K blocks in flight; rings of 4 and 8 blocks and 64-row blocks were no faster (the deeper rings spill)
-  (void)mt;
-  (void)ntw;
-  return launch_narrow_one<DT, ZK, 2, 1, 2>(a, row_blocks, st);
-}
 template <int DT>
-hipError_t launch_narrow(const TileArgs& a, int zk, int mt, int ntw, int row_blocks, hipStream_t st) {
-  if (zk == MI355Q_ZP_NONE) return launch_narrow_zk<DT, MI355Q_ZP_NONE>(a, mt, ntw, row_blocks, st);
-  if (zk == MI355Q_ZP_PACKED) return launch_narrow_zk<DT, MI355Q_ZP_PACKED>(a, mt, ntw, row_blocks, st);
-  return launch_narrow_zk<DT, MI355Q_ZP_PRESCALED>(a, mt, ntw, row_blocks, st);
+hipError_t launch_narrow(const TileArgs& a, int zk, int row_blocks, hipStream_t st) {
+  if (zk == MI355Q_ZP_NONE) return launch_narrow_zk<DT, MI355Q_ZP_NONE>(a, row_blocks, st);
+  if (zk == MI355Q_ZP_PACKED) return launch_narrow_zk<DT, MI355Q_ZP_PACKED>(a, row_blocks, st);
+  return launch_narrow_zk<DT, MI355Q_ZP_PRESCALED>(a, row_blocks, st);
 }
 
 template <int DT, int MT, bool GROUPED>
@@ -821,8 +818,8 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   const uint32_t gpk = (uint32_t)group_size / 128u;
   a.gpk_magic = gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + gpk - 1) / gpk) : 0u;
   if (ntw < 4)
-    e = (dtype == MI355Q_F16) ? launch_narrow<MI355Q_F16>(a, zeros_kind, mt, ntw, row_blocks, st)
-                              : launch_narrow<MI355Q_BF16>(a, zeros_kind, mt, ntw, row_blocks, st);
+    e = (dtype == MI355Q_F16) ? launch_narrow<MI355Q_F16>(a, zeros_kind, row_blocks, st)
+                              : launch_narrow<MI355Q_BF16>(a, zeros_kind, row_blocks, st);
   else
     e = (dtype == MI355Q_F16) ? launch_mt<MI355Q_F16, false>(a, zeros_kind, mt, row_blocks, st)
                               : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
