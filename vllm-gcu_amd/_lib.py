@@ -65,6 +65,9 @@ SIGNATURES = {
                                     c_int, c_int, c_int, c_int, c_int, c_void_p]),
 }
 
+# must equal mi355q_abi_version() of the library (csrc/core.hip)
+ABI_VERSION = 2
+
 _lib = None
 
 
@@ -78,6 +81,10 @@ def load():
             f"{LIB_PATH} not found: build it first with "
             "`python -c 'import __graft_entry__ as g; g.build()'` (needs hipcc)")
     lib = ctypes.CDLL(LIB_PATH)
+    lib.mi355q_abi_version.restype = c_int
+    if lib.mi355q_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} has ABI version {lib.mi355q_abi_version()}, this binding needs {ABI_VERSION}: "
+                          "rebuild it with `python -c 'import __graft_entry__ as g; g.build()'`")
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
         fn.restype = res

@@ -32,4 +32,6 @@ int device_cu_count() {
 }  // namespace mi355q
 
 extern "C" const char* mi355q_last_error(void) { return mi355q::g_err; }
-extern "C" int mi355q_abi_version(void) { return 1; }
+// bumped whenever an entry point changes its arguments: the Python binding refuses a library of another version
+// (a stale build would be called with shifted arguments)
+extern "C" int mi355q_abi_version(void) { return 2; }
