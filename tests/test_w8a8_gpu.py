@@ -168,6 +168,32 @@ def test_cutlass_scaled_mm_epilogue(ops, dtype):
         np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N", [264, 488, 28672 // 8])
+def test_scaled_mm_wide_and_narrow_output_stores_agree(ops, dtype, N):
+    """16-bit outputs leave the tile kernel in 16-byte pieces when N, the output row stride and its address
+    allow, in 8-byte pieces otherwise; both orders of the same values, so the results are the same bits."""
+    rng = np.random.default_rng(11)
+    M, K = 300, 256
+    xq = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    xs = rng.uniform(0.5, 1.5, (M, 1)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(dtype).cuda()
+    want = o8.scaled_mm_epilogue(o8.int8_gemm_i32(xq, np.ascontiguousarray(w_nk.T)), xs, ws, bias.float().cpu().numpy())
+    wide = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    torch.ops._C.cutlass_scaled_mm(wide, dev(xq), dev(w_nk).t(), dev(xs), dev(ws), bias)
+    np.testing.assert_allclose(wide.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # a row stride of N + 4 elements and a base 8 bytes into the buffer: neither allows 16-byte stores
+    for buf, view in ((torch.full((M, N + 4), float("nan"), dtype=dtype, device="cuda"), lambda b: b[:, :N]),
+                      (torch.full((M * N + 4,), float("nan"), dtype=dtype, device="cuda"), lambda b: b[4:].view(M, N))):
+        narrow = view(buf)
+        torch.ops._C.cutlass_scaled_mm(narrow, dev(xq), dev(w_nk).t(), dev(xs), dev(ws), bias)
+        assert torch.equal(narrow, wide)
+    if N > 300:
+        assert bool(torch.isnan(buf[:4]).all())          # nothing written in front of the shifted base
+
+
 def test_dot_bias_quant_single_scale(ops):
     rng = np.random.default_rng(4)
     M, K, N = 20, 256, 132

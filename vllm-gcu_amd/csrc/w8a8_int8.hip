@@ -38,6 +38,7 @@ struct I8Args {
   int x_scale_per_row, w_scale_per_col, bias_f32;
   int n_panels_swizzle;     // non-zero: XCD-aware tile order
   int w_kslab;              // w is in the kslab order (see include/mi355q.h) instead of row-major
+  int wide_stores;          // N, ldo and the output address allow 16-byte stores of 8 adjacent 16-bit outputs
 };
 
 template <int DT>
@@ -341,22 +342,47 @@ w8a8_int8_gemm_kernel(I8Args a) {
         bia[i][e] = a.bias ? load_bias<DT>(a.bias, a.bias_f32, n + e) : 0.0f;
       }
     }
+    // 16-bit outputs leave in 16-byte pieces where the layout allows: the lanes of a row that hold
+    // columns 4 kq .. 4 kq + 3 of two neighbouring column tiles trade halves (v_permlane16_swap:
+    // lanes 16..31 of the first register with lanes 0..15 of the second, likewise 48..63 with
+    // 32..47), after which lane kq holds 8 adjacent columns of tile i + (kq & 1) -- a store
+    // instruction then writes 64 contiguous bytes per row instead of 32
+    const bool wide = DT != MI355Q_F32 && a.wide_stores;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
       if (m >= M) continue;
-#pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
-        if (n >= N) continue;                     // N is a multiple of 4
-        if (a.acc_out) *(i4*)(a.acc_out + (long)m * N + n) = acc[i][j];
-        float v[4];
+      auto scaled = [&](int i, float* v) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           v[e] = ((float)acc[i][j][e] * xsc[j]) * wsc[i][e];
           if (a.bias) v[e] += bia[i][e];
         }
-        store4<DT>(a.out, (long)m * a.ldo + n, v);
+      };
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+        if (a.acc_out && n < N) *(i4*)(a.acc_out + (long)m * N + n) = acc[i][j];
+        if (DT != MI355Q_F32 && wide && (i & 1) == 0 && i + 1 < NI) {
+          typedef Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT> E;
+          float v0[4], v1[4];
+          scaled(i, v0);
+          scaled(i + 1, v1);
+          uint32_t p[2][2];
+          p[0][0] = (uint32_t)E::from_f32(v0[0]) | ((uint32_t)E::from_f32(v0[1]) << 16);
+          p[0][1] = (uint32_t)E::from_f32(v0[2]) | ((uint32_t)E::from_f32(v0[3]) << 16);
+          p[1][0] = (uint32_t)E::from_f32(v1[0]) | ((uint32_t)E::from_f32(v1[1]) << 16);
+          p[1][1] = (uint32_t)E::from_f32(v1[2]) | ((uint32_t)E::from_f32(v1[3]) << 16);
+          const auto lo2 = __builtin_amdgcn_permlane16_swap(p[0][0], p[1][0], false, false);
+          const auto hi2 = __builtin_amdgcn_permlane16_swap(p[0][1], p[1][1], false, false);
+          const int nw = n0 + wn * (16 * NI) + (i + (kq & 1)) * 16 + 8 * (kq >> 1);
+          if (nw < N) *(u4*)((uint16_t*)a.out + (long)m * a.ldo + nw) = (u4){lo2[0], hi2[0], lo2[1], hi2[1]};
+        } else if (!(DT != MI355Q_F32 && wide && (i & 1) == 1)) {
+          if (n >= N) continue;                     // N is a multiple of 4
+          float v[4];
+          scaled(i, v);
+          store4<DT>(a.out, (long)m * a.ldo + n, v);
+        }
       }
     }
     // The operands of the next output tile's first half are read again here
@@ -560,6 +586,7 @@ extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* 
   a.x_scale_per_row = x_scale_per_row; a.w_scale_per_col = w_scale_per_col; a.bias_f32 = bias_f32;
   a.n_panels_swizzle = 0;
   a.w_kslab = kslab ? 1 : 0;
+  a.wide_stores = (N % 8 == 0 && ldo % 8 == 0 && ((size_t)out & 15) == 0) ? 1 : 0;
   if (out_dtype == MI355Q_F16) return launch_gemm<MI355Q_F16>(a, as_stream(stream));
   if (out_dtype == MI355Q_BF16) return launch_gemm<MI355Q_BF16>(a, as_stream(stream));
   return launch_gemm<MI355Q_F32>(a, as_stream(stream));
