@@ -378,8 +378,9 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40, cpu=False):
     wt = w_nk.t()
     # long warm-up: the core clock settles (it drops under sustained MFMA load and
     # recovers part of the way) only after some tens of launches
-    t = time_graph([lambda: torch.ops._C.cutlass_scaled_mm(out, xq, wt, xs, ws, None)], iters, warmup, stream) / iters
-    tq = time_graph([lambda: ops.scaled_int8_quant(x)], iters, 3, stream) / iters
+    # (several launches per graph: a graph of one short kernel would time the replay gap with it)
+    t = time_graph([lambda: torch.ops._C.cutlass_scaled_mm(out, xq, wt, xs, ws, None)] * 5, iters, warmup, stream) / iters
+    tq = time_graph([lambda: ops.scaled_int8_quant(x)] * 10, iters, 10, stream) / iters
     ops_ = 2.0 * M * K * N
     # decode: 16 tokens against the same layer, weights as the linear method keeps them after
     # loading (kslab order); three weight copies in turn so that none is served from a cache
@@ -388,7 +389,7 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40, cpu=False):
     ksl = [rearrange.to_kslab(w_nk if i == 0 else w_nk.roll(i, 0)) for i in range(3)]
     outd = torch.empty(Md, N, dtype=torch.float16, device=dev)
     fns = [(lambda w=w: torch.ops._C.cutlass_scaled_mm(outd, xq[:Md], w.t(), xs[:Md], ws, None)) for w in ksl]
-    td = time_graph(fns, iters, 3, stream) / iters
+    td = time_graph(fns * 2, iters, 6, stream) / iters
     res_cpu = cpu_baseline_w8a8(x, w_nk, ws) if cpu else None
     return {"workload": "W8A8 int8 GEMM M=2048 K=8192 N=28672, fused per-token x per-channel scales, fp16 out",
             "gemm_us": round(t * 1e6, 1), "TOPs": round(ops_ / t / 1e12, 1),
