@@ -10,15 +10,16 @@
 //                        expert with every expert's run padded to a multiple
 //                        of the block size.  One workgroup; each wavefront
 //                        owns a contiguous segment of ids, ranks inside a
-//                        64-id tile come from ballots (wavefront-level scan),
-//                        segment bases from an LDS scan over wavefronts.
+//                        64-id tile come from ballots over the bits of the
+//                        expert id (wavefront-level scan), segment bases from
+//                        an LDS scan over wavefronts.
 #include "common.h"
 
 namespace mi355q {
 namespace {
 
 constexpr int MAX_E = 1024;          // experts per token row handled by the routing kernels
-constexpr int EPL = MAX_E / 64;      // experts per lane
+// EPL (template parameter below) = experts per lane: 1, 4 or 16 for up to 64, 256 or 1024 experts
 
 template <int DT>
 __device__ __forceinline__ float ld_logit(const void* p, long i) {
@@ -26,28 +27,44 @@ __device__ __forceinline__ float ld_logit(const void* p, long i) {
   return Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT>::to_f32(((const uint16_t*)p)[i]);
 }
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-  return v;
+// Wavefront reductions on the data-parallel-primitive path (lane shifts inside the vector ALU, no trip
+// through the LDS crossbar): an inclusive scan within each row of 16 lanes (shifts by 1, 2, 4, 8; lanes a
+// shift does not reach keep the identity), then lane 15 of rows 0 and 2 joins rows 1 and 3, lane 31 joins
+// rows 2 and 3, and lane 63 holds the result, which is read back as a scalar.
+#define MQ_DPP_REDUCE(v, ident, OP)                                                                     \
+  do {                                                                                                  \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x111, 0xf, 0xf, false)); /* row_shr:1 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x112, 0xf, 0xf, false)); /* row_shr:2 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x114, 0xf, 0xf, false)); /* row_shr:4 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x118, 0xf, 0xf, false)); /* row_shr:8 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x142, 0xa, 0xf, false)); /* row_bcast:15 */        \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x143, 0xc, 0xf, false)); /* row_bcast:31 */        \
+    v = __builtin_amdgcn_readlane(v, 63);                                                               \
+  } while (0)
+__device__ __forceinline__ int op_fmax_bits(int a, int b) { return __float_as_int(fmaxf(__int_as_float(a), __int_as_float(b))); }
+__device__ __forceinline__ int op_fadd_bits(int a, int b) { return __float_as_int(__int_as_float(a) + __int_as_float(b)); }
+__device__ __forceinline__ int op_imin(int a, int b) { return a < b ? a : b; }
+__device__ __forceinline__ float wave_max(float x) {
+  int v = __float_as_int(x);
+  MQ_DPP_REDUCE(v, (int)0xff800000, op_fmax_bits);   // identity: -inf
+  return __int_as_float(v);
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
+__device__ __forceinline__ float wave_sum(float x) {
+  int v = __float_as_int(x);
+  MQ_DPP_REDUCE(v, 0, op_fadd_bits);
+  return __int_as_float(v);
 }
-// arg-max over the wavefront: larger value wins, lower index on ties
+// arg-max over the wavefront: larger value wins, lower index on ties; the result is the same in every lane
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    float ov = __shfl_xor(v, o);
-    int oi = __shfl_xor(idx, o);
-    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
-  }
+  const float m = wave_max(v);
+  int cand = (v == m) ? idx : 0x7fffffff;
+  MQ_DPP_REDUCE(cand, 0x7fffffff, op_imin);
+  v = m;
+  idx = cand;
 }
 
 // scores of one row, expert e = lane + 64 j in s[j]; -inf beyond E
-template <int DT>
+template <int DT, int EPL>
 __device__ __forceinline__ void row_scores(const void* gating, long row, int E, int lane, int sigmoid,
                                            float* s) {
   float mx = -INFINITY;
@@ -77,6 +94,7 @@ __device__ __forceinline__ void row_scores(const void* gating, long row, int E, 
 }
 
 // k rounds of arg-max over sel[]; weights are read from w[] at the winner
+template <int EPL>
 __device__ __forceinline__ void select_topk(float* sel, const float* w, int lane, int k, float* out_w,
                                             int* out_i, long base, bool renorm) {
   float total = 0.f;
@@ -91,12 +109,14 @@ __device__ __forceinline__ void select_topk(float* sel, const float* w, int lane
       if (sel[j] > bv) { bv = sel[j]; bi = e; }   // ascending e within a lane: first max wins
     }
     wave_argmax(bv, bi);
-    // the owner retires the winner and reports its (unbiased) weight
-    float wv = 0.f;
+    // the owner retires the winner; its (unbiased) weight is read from its lane (bi is uniform)
+    float cw = 0.f;
 #pragma unroll
-    for (int j = 0; j < EPL; ++j)
-      if (lane + 64 * j == bi) { wv = w[j]; sel[j] = -INFINITY; }
-    wv = wave_sum(wv);                             // exactly one lane contributes
+    for (int j = 0; j < EPL; ++j) {
+      if (j == (bi >> 6)) cw = w[j];
+      if (lane + 64 * j == bi) sel[j] = -INFINITY;
+    }
+    const float wv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cw), bi & 63));
     total += wv;
     if (lane == r) { mine_w = wv; mine_i = bi; }
   }
@@ -106,7 +126,7 @@ __device__ __forceinline__ void select_topk(float* sel, const float* w, int lane
   }
 }
 
-template <int DT>
+template <int DT, int EPL>
 __global__ void __launch_bounds__(256)
 topk_softmax_kernel(float* topk_w, int* topk_i, int* tok_exp, const void* gating, int M, int E, int k,
                     int renorm) {
@@ -114,23 +134,23 @@ topk_softmax_kernel(float* topk_w, int* topk_i, int* tok_exp, const void* gating
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= M) return;
   float s[EPL], w[EPL];
-  row_scores<DT>(gating, row, E, lane, 0, s);
+  row_scores<DT, EPL>(gating, row, E, lane, 0, s);
 #pragma unroll
   for (int j = 0; j < EPL; ++j) w[j] = s[j];
-  select_topk(s, w, lane, k, topk_w, topk_i, row * k, renorm != 0);
+  select_topk<EPL>(s, w, lane, k, topk_w, topk_i, row * k, renorm != 0);
   if (tok_exp && lane < k) tok_exp[row * k + lane] = lane * M + (int)row;
 }
 
-template <int DT>
+template <int DT, int EPL>
 __global__ void __launch_bounds__(256)
 grouped_topk_kernel(float* topk_w, int* topk_i, const void* gating, const float* bias, int M, int E, int k,
                     int ngroup, int topk_group, int renorm, int sigmoid) {
-  __shared__ float sh[4][MAX_E];
+  __shared__ float sh[4][64 * EPL];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const long row = (long)blockIdx.x * 4 + wv;
   if (row >= M) return;
   float s[EPL], sel[EPL];
-  row_scores<DT>(gating, row, E, lane, sigmoid, s);
+  row_scores<DT, EPL>(gating, row, E, lane, sigmoid, s);
 #pragma unroll
   for (int j = 0; j < EPL; ++j) {
     const int e = lane + 64 * j;
@@ -168,7 +188,7 @@ grouped_topk_kernel(float* topk_w, int* topk_i, const void* gating, const float*
     const int e = lane + 64 * j;
     if (e >= E || !((keep >> (e / per)) & 1ull)) sel[j] = -INFINITY;
   }
-  select_topk(sel, s, lane, k, topk_w, topk_i, row * k, renorm != 0);
+  select_topk<EPL>(sel, s, lane, k, topk_w, topk_i, row * k, renorm != 0);
 }
 
 // ---- align ------------------------------------------------------------------
@@ -249,6 +269,7 @@ moe_align_kernel(const IdT* __restrict__ topk_ids, int numel, int top, const int
     for (int b = estart[e] / B; b < estart[e + 1] / B; ++b) expert_ids[b] = me;
   }
   // stable scatter: tile by tile, rank inside the tile from ballots
+  const int ebits = E > 1 ? 32 - __builtin_clz((unsigned)(E - 1)) : 0;
   for (int t0 = seg_b; t0 < seg_e; t0 += 64) {
     const int i = t0 + lane;
     int e = -1;
@@ -256,20 +277,25 @@ moe_align_kernel(const IdT* __restrict__ topk_ids, int numel, int top, const int
       e = (int)topk_ids[i];
       if (e < 0 || e >= E) e = -1;
     }
-    unsigned long long todo = __ballot(e >= 0);
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const int e0 = __shfl(e, leader);
-      const unsigned long long same = __ballot(e == e0);
-      if (e == e0) {
-        const int rank = __popcll(same & ((1ull << lane) - 1ull));
-        sorted_ids[estart[e0] + cnt[wv * E + e0] + rank] = i;
-      }
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) cnt[wv * E + e0] += __popcll(same);
-      __builtin_amdgcn_wave_barrier();
-      todo &= ~same;
+    // lanes of the tile that hold the same expert: the ballots of the id's bits, each taken as it is or
+    // inverted according to the lane's own bit, intersected (no loop over the distinct experts of the tile)
+    unsigned long long same = __ballot(e >= 0);
+    for (int b = 0; b < ebits; ++b) {
+      const bool bit = (e >> b) & 1;
+      const unsigned long long set = __ballot(bit);
+      same &= bit ? set : ~set;
     }
+    int slot = 0, rank = 0;
+    if (e >= 0) {
+      rank = __popcll(same & ((1ull << lane) - 1ull));
+      slot = estart[e] + cnt[wv * E + e] + rank;   // read before the lowest lane of the set bumps the count
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (e >= 0) {
+      sorted_ids[slot] = i;
+      if (rank == 0) cnt[wv * E + e] += __popcll(same);
+    }
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -287,14 +313,16 @@ extern "C" int mi355q_topk_softmax(float* topk_weights, int32_t* topk_ids, int32
   MQ_REQUIRE(E <= MAX_E && topk <= 64 && topk <= E, "topk_softmax: E=%d (max %d) / topk=%d (max 64) unsupported", E, MAX_E, topk);
   dim3 grid((M + 3) / 4), block(256);
   hipStream_t st = as_stream(stream);
-  if (dtype == MI355Q_F32)
-    hipLaunchKernelGGL((topk_softmax_kernel<MI355Q_F32>), grid, block, 0, st, topk_weights, topk_ids, token_expert_indices, gating, M, E, topk, renormalize);
-  else if (dtype == MI355Q_F16)
-    hipLaunchKernelGGL((topk_softmax_kernel<MI355Q_F16>), grid, block, 0, st, topk_weights, topk_ids, token_expert_indices, gating, M, E, topk, renormalize);
-  else if (dtype == MI355Q_BF16)
-    hipLaunchKernelGGL((topk_softmax_kernel<MI355Q_BF16>), grid, block, 0, st, topk_weights, topk_ids, token_expert_indices, gating, M, E, topk, renormalize);
-  else
-    MQ_REQUIRE(false, "topk_softmax: bad dtype %d", dtype);
+  MQ_REQUIRE(dtype == MI355Q_F32 || dtype == MI355Q_F16 || dtype == MI355Q_BF16, "topk_softmax: bad dtype %d", dtype);
+#define MQ_TOPK_LAUNCH(DT, EPL) \
+  hipLaunchKernelGGL((topk_softmax_kernel<DT, EPL>), grid, block, 0, st, topk_weights, topk_ids, token_expert_indices, gating, M, E, topk, renormalize)
+#define MQ_TOPK_EPL(DT) \
+  do { if (E <= 64) MQ_TOPK_LAUNCH(DT, 1); else if (E <= 256) MQ_TOPK_LAUNCH(DT, 4); else MQ_TOPK_LAUNCH(DT, 16); } while (0)
+  if (dtype == MI355Q_F32) MQ_TOPK_EPL(MI355Q_F32);
+  else if (dtype == MI355Q_F16) MQ_TOPK_EPL(MI355Q_F16);
+  else MQ_TOPK_EPL(MI355Q_BF16);
+#undef MQ_TOPK_EPL
+#undef MQ_TOPK_LAUNCH
   MQ_LAUNCH_CHECK("topk_softmax");
   return 0;
 }
@@ -314,14 +342,16 @@ extern "C" int mi355q_grouped_topk(float* topk_weights, int32_t* topk_ids, const
   MQ_REQUIRE(!bias || E / num_expert_group >= 2, "grouped_topk: a correction bias needs at least 2 experts per group");
   dim3 grid((M + 3) / 4), block(256);
   hipStream_t st = as_stream(stream);
-  if (dtype == MI355Q_F32)
-    hipLaunchKernelGGL((grouped_topk_kernel<MI355Q_F32>), grid, block, 0, st, topk_weights, topk_ids, gating, bias, M, E, topk, num_expert_group, topk_group, renormalize, scoring_sigmoid);
-  else if (dtype == MI355Q_F16)
-    hipLaunchKernelGGL((grouped_topk_kernel<MI355Q_F16>), grid, block, 0, st, topk_weights, topk_ids, gating, bias, M, E, topk, num_expert_group, topk_group, renormalize, scoring_sigmoid);
-  else if (dtype == MI355Q_BF16)
-    hipLaunchKernelGGL((grouped_topk_kernel<MI355Q_BF16>), grid, block, 0, st, topk_weights, topk_ids, gating, bias, M, E, topk, num_expert_group, topk_group, renormalize, scoring_sigmoid);
-  else
-    MQ_REQUIRE(false, "grouped_topk: bad dtype %d", dtype);
+  MQ_REQUIRE(dtype == MI355Q_F32 || dtype == MI355Q_F16 || dtype == MI355Q_BF16, "grouped_topk: bad dtype %d", dtype);
+#define MQ_GTOPK_LAUNCH(DT, EPL) \
+  hipLaunchKernelGGL((grouped_topk_kernel<DT, EPL>), grid, block, 0, st, topk_weights, topk_ids, gating, bias, M, E, topk, num_expert_group, topk_group, renormalize, scoring_sigmoid)
+#define MQ_GTOPK_EPL(DT) \
+  do { if (E <= 64) MQ_GTOPK_LAUNCH(DT, 1); else if (E <= 256) MQ_GTOPK_LAUNCH(DT, 4); else MQ_GTOPK_LAUNCH(DT, 16); } while (0)
+  if (dtype == MI355Q_F32) MQ_GTOPK_EPL(MI355Q_F32);
+  else if (dtype == MI355Q_F16) MQ_GTOPK_EPL(MI355Q_F16);
+  else MQ_GTOPK_EPL(MI355Q_BF16);
+#undef MQ_GTOPK_EPL
+#undef MQ_GTOPK_LAUNCH
   MQ_LAUNCH_CHECK("grouped_topk");
   return 0;
 }
