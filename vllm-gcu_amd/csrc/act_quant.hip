@@ -123,7 +123,7 @@ group_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, long rows
 #pragma unroll
     for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(y[e]));
     if (!live) mx = 0.f;
-    for (int o = 1; o < lpg; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    mx = lane_group_max(mx, lpg);
     const float s = fmaxf(mx, 1e-10f) / FP8_MAX;
     const SharedDivisor by_s(s);
     float q[8];
@@ -145,8 +145,7 @@ token_fp8_quant_kernel(uint8_t* out, float* scales, const uint16_t* x, int K, co
   __shared__ float red[4];
   float mx = 0.f;
   for (int k = threadIdx.x; k < K; k += 256) mx = fmaxf(mx, fabsf(Elem<DT>::to_f32(x[row * K + k])));
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  mx = wave_max(mx);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
   __syncthreads();
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
@@ -264,8 +263,7 @@ rms_norm_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* resid
 #pragma unroll
     for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  ss = wave_sum(ss);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
   __syncthreads();
   ss = (red[0] + red[1]) + (red[2] + red[3]);
@@ -296,7 +294,7 @@ rms_norm_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* resid
 #pragma unroll
       for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
       if (!live) mx = 0.f;
-      for (int o = 1; o < lpg; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      mx = lane_group_max(mx, lpg);
       const float sg = fmaxf(mx, 1e-10f) / FP8_MAX;
       const SharedDivisor by_sg(sg);
       float q[8];

@@ -86,6 +86,48 @@ __device__ __forceinline__ void use_agpr_accumulators() {
   asm volatile("" : "+a"(t));
 }
 
+// Wavefront reductions on the data-parallel-primitive path (lane shifts inside the vector ALU, no trip
+// through the LDS crossbar).  Every lane of the wavefront must be active.
+// Whole wavefront: an inclusive scan within each row of 16 lanes (shifts by 1, 2, 4, 8; lanes a shift
+// does not reach keep the identity), then lane 15 of rows 0 and 2 joins rows 1 and 3, lane 31 joins
+// rows 2 and 3, and lane 63 holds the result, which is read back as a scalar.
+#define MQ_DPP_REDUCE(v, ident, OP)                                                                     \
+  do {                                                                                                  \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x111, 0xf, 0xf, false)); /* row_shr:1 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x112, 0xf, 0xf, false)); /* row_shr:2 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x114, 0xf, 0xf, false)); /* row_shr:4 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x118, 0xf, 0xf, false)); /* row_shr:8 */           \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x142, 0xa, 0xf, false)); /* row_bcast:15 */        \
+    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x143, 0xc, 0xf, false)); /* row_bcast:31 */        \
+    v = __builtin_amdgcn_readlane(v, 63);                                                               \
+  } while (0)
+__device__ __forceinline__ int op_fmax_bits(int a, int b) { return __float_as_int(fmaxf(__int_as_float(a), __int_as_float(b))); }
+__device__ __forceinline__ int op_fadd_bits(int a, int b) { return __float_as_int(__int_as_float(a) + __int_as_float(b)); }
+__device__ __forceinline__ int op_imin(int a, int b) { return a < b ? a : b; }
+__device__ __forceinline__ float wave_max(float x) {
+  int v = __float_as_int(x);
+  MQ_DPP_REDUCE(v, (int)0xff800000, op_fmax_bits);   // identity: -inf
+  return __int_as_float(v);
+}
+__device__ __forceinline__ float wave_sum(float x) {
+  int v = __float_as_int(x);
+  MQ_DPP_REDUCE(v, 0, op_fadd_bits);
+  return __int_as_float(v);
+}
+// max over aligned groups of `lanes` lanes (a power of two, 2 .. 64), the result in every lane of the
+// group: swaps inside quads, mirrors of the half row and of the row of 16 lanes, LDS shuffles only
+// for what crosses rows
+__device__ __forceinline__ float lane_group_max(float x, int lanes) {
+  int v = __float_as_int(x);
+  if (lanes >= 2) v = op_fmax_bits(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false));    // quad_perm [1,0,3,2]
+  if (lanes >= 4) v = op_fmax_bits(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false));    // quad_perm [2,3,0,1]
+  if (lanes >= 8) v = op_fmax_bits(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, false));   // row_half_mirror
+  if (lanes >= 16) v = op_fmax_bits(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false));  // row_mirror
+  float m = __int_as_float(v);
+  for (int o = 16; o < lanes; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
+  return m;
+}
+
 // Fused-MoE grouped GEMMs: a block whose expert id lies outside [0, E) -- a non-local expert under an
 // expert map, -1 in the reference (vllm_gcu/kernels/fused_moe.py:70-71, 106-107) -- contributes
 // nothing.  Its workgroups read no weights and zero the columns [col0, col0 + ncols) (ncols % 4 == 0)

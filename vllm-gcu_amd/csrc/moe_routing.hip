@@ -27,33 +27,6 @@ __device__ __forceinline__ float ld_logit(const void* p, long i) {
   return Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT>::to_f32(((const uint16_t*)p)[i]);
 }
 
-// Wavefront reductions on the data-parallel-primitive path (lane shifts inside the vector ALU, no trip
-// through the LDS crossbar): an inclusive scan within each row of 16 lanes (shifts by 1, 2, 4, 8; lanes a
-// shift does not reach keep the identity), then lane 15 of rows 0 and 2 joins rows 1 and 3, lane 31 joins
-// rows 2 and 3, and lane 63 holds the result, which is read back as a scalar.
-#define MQ_DPP_REDUCE(v, ident, OP)                                                                     \
-  do {                                                                                                  \
-    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x111, 0xf, 0xf, false)); /* row_shr:1 */           \
-    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x112, 0xf, 0xf, false)); /* row_shr:2 */           \
-    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x114, 0xf, 0xf, false)); /* row_shr:4 */           \
-    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x118, 0xf, 0xf, false)); /* row_shr:8 */           \
-    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x142, 0xa, 0xf, false)); /* row_bcast:15 */        \
-    v = OP(v, __builtin_amdgcn_update_dpp(ident, v, 0x143, 0xc, 0xf, false)); /* row_bcast:31 */        \
-    v = __builtin_amdgcn_readlane(v, 63);                                                               \
-  } while (0)
-__device__ __forceinline__ int op_fmax_bits(int a, int b) { return __float_as_int(fmaxf(__int_as_float(a), __int_as_float(b))); }
-__device__ __forceinline__ int op_fadd_bits(int a, int b) { return __float_as_int(__int_as_float(a) + __int_as_float(b)); }
-__device__ __forceinline__ int op_imin(int a, int b) { return a < b ? a : b; }
-__device__ __forceinline__ float wave_max(float x) {
-  int v = __float_as_int(x);
-  MQ_DPP_REDUCE(v, (int)0xff800000, op_fmax_bits);   // identity: -inf
-  return __int_as_float(v);
-}
-__device__ __forceinline__ float wave_sum(float x) {
-  int v = __float_as_int(x);
-  MQ_DPP_REDUCE(v, 0, op_fadd_bits);
-  return __int_as_float(v);
-}
 // arg-max over the wavefront: larger value wins, lower index on ties; the result is the same in every lane
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
   const float m = wave_max(v);

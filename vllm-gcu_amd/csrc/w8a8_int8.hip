@@ -438,8 +438,7 @@ dynamic_int8_quant_kernel(int8_t* out, float* scales, const void* x, int K, cons
   } else {
     for (int k = threadIdx.x; k < K; k += 256) mx = fmaxf(mx, fabsf(ld_act<DT>(x, (long)row * K + k)));
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  mx = wave_max(mx);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
   __syncthreads();
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
