@@ -86,6 +86,20 @@ __device__ __forceinline__ void use_agpr_accumulators() {
   asm volatile("" : "+a"(t));
 }
 
+// Buffer loads: an offset at or past the descriptor's size reads as zero
+// without touching memory, which makes "no such K block" a branch-free case
+// (callers add 2^31 to the lane offset; every buffer here is below 2 GiB).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u4 buf_load16(rsrc_t r, uint32_t off) {
+  return bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
+}
+// streamed once: non-temporal
+__device__ __forceinline__ u4 buf_load16_nt(rsrc_t r, uint32_t off) {
+  return bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 2));
+}
 // Wavefront reductions on the data-parallel-primitive path (lane shifts inside the vector ALU, no trip
 // through the LDS crossbar).  Every lane of the wavefront must be active.
 // Whole wavefront: an inclusive scan within each row of 16 lanes (shifts by 1, 2, 4, 8; lanes a shift

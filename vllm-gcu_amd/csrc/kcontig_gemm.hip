@@ -39,6 +39,7 @@ struct KcArgs {
   int M, N, K;
   int kslab;                   // weights are in the kslab layout (N % 64 == 0)
   int wgroup;                  // W8A16 group-wise modes: 64 or 128
+  int wide_stores;             // N % 8 == 0 and a 16-byte aligned output below 4 GiB: 16-byte stores of 8 adjacent outputs
   // grouped mode
   const int* sorted_ids;
   const int* expert_ids;
@@ -119,52 +120,53 @@ kcontig_gemm_kernel(KcArgs a) {
   constexpr bool GW = MODE == KC_W8A16G_F16 || MODE == KC_W8A16G_BF16;    // group-wise weight scales
   constexpr int AV = T::ABYTES * 2;               // 16-byte vectors per lane per K block (activations)
   constexpr int WV = T::WBYTES * 2;               // ... weights
-  __shared__ int tok[GROUPED ? BM : 1];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, q = lane >> 4;
   const int N = a.N, K = a.K;
   const int KB = K >> 7;
   const int m0 = blockIdx.y * BM;
   long expert = 0;
+  // slot ids of this lane's rows (row r16 of each row tile): one load per lane, in flight together with
+  // the expert id and the block count -- a chain of dependent loads in front of the weight stream costs
+  // one loaded memory latency each, per workgroup
+  int tok[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) tok[j] = 0;
   if (GROUPED) {
-    if (m0 >= *a.npp) return;
+    const int npp = *a.npp;
     expert = a.expert_ids[m0 / a.block_size];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) tok[j] = a.sorted_ids[m0 + 16 * j + r16];   // (the array is padded to whole blocks)
+    if (m0 >= npp) return;
     if (expert < 0 || expert >= a.E) {             // not one of this rank's experts: zero rows, no weights read
       const int col0 = blockIdx.x * 256;
       zero_block_columns((uint16_t*)a.out, a.sorted_ids + m0, BM, a.numel, N, col0, min(256, N - col0), 256);
       return;
     }
-    for (int r = tid; r < BM; r += 256) tok[r] = a.sorted_ids[m0 + r];
-    __syncthreads();
   }
   const int n0 = KS ? blockIdx.x * 64 : blockIdx.x * 256 + wave * 64;
   if (n0 >= N) return;
-  const char* wbase = (const char*)a.w + expert * a.w_stride * T::WBYTES;
-
-  // per-lane row pointers
-  const char* wptr[4];
-  // byte strides between K blocks and between the 16-byte vectors of a lane
-  const long kstride = a.kslab ? 4 * 2048 * T::WBYTES : 128 * T::WBYTES;
-  const int vstride = a.kslab ? 1024 : 16;
+  // Operands are addressed through buffer descriptors: a 32-bit lane offset plus a scalar K-block offset
+  // per load (no 64-bit address arithmetic in the loop; the host checks that one expert's weights, the
+  // activations and their scales each stay below 4 GiB).
+  const rsrc_t wres = make_rsrc((const char*)a.w + expert * a.w_stride * T::WBYTES, (uint32_t)((size_t)N * K * T::WBYTES));
+  const uint32_t kstride = a.kslab ? 4 * 2048 * T::WBYTES : 128 * T::WBYTES;   // bytes between K blocks
+  const uint32_t vstride = a.kslab ? 1024 : 16;                                 // ... between the 16-byte vectors of a lane
+  uint32_t woff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     if (a.kslab) {
-      wptr[i] = wbase + (((size_t)(n0 >> 6) * KB) * 4 + i) * (2048 * T::WBYTES) + lane * 16;
+      woff[i] = (uint32_t)((((size_t)(n0 >> 6) * KB) * 4 + i) * (2048 * T::WBYTES) + lane * 16);
     } else {
       const int n = min(n0 + 16 * i + r16, N - 1);
-      wptr[i] = wbase + ((size_t)n * K + 32 * q) * T::WBYTES;
+      woff[i] = (uint32_t)(((size_t)n * K + 32 * q) * T::WBYTES);
     }
   }
-  const char* aptr[MT];
+  const int arows = GROUPED ? (a.numel + a.topk - 1) / a.topk : a.M;          // rows of the activation matrix
+  const rsrc_t xres = make_rsrc(a.a, (uint32_t)((size_t)arows * K * T::ABYTES));
+  const rsrc_t asres = make_rsrc(a.a_scale, MODE == KC_FP8_BLOCK ? (uint32_t)((size_t)arows * KB * 4) : 0u);
+  uint32_t aoff[MT];
   int arow[MT];
-#pragma unroll
-  for (int j = 0; j < MT; ++j) {
-    int row;
-    if (GROUPED) row = min(tok[16 * j + r16], a.numel - 1) / a.topk;
-    else row = min(m0 + 16 * j + r16, a.M - 1);
-    arow[j] = row;
-    aptr[j] = (const char*)a.a + ((size_t)row * K + 32 * q) * T::ABYTES;
-  }
 
   acc_t acc[4][MT];
 #pragma unroll
@@ -182,21 +184,16 @@ kcontig_gemm_kernel(KcArgs a) {
   const uint16_t* ws16 = (const uint16_t*)a.w_scale + expert * a.ws_stride;
   const int gper = GW ? 128 / a.wgroup : 1;        // scale groups per K block
   const float* wsf = (const float*)a.w_scale + expert * a.ws_stride;
-  auto load_blk = [&](Blk& b, int kb) {
+  const rsrc_t wsres = make_rsrc(wsf, MODE == KC_FP8_BLOCK ? (uint32_t)((size_t)((N + 127) >> 7) * KB * 4) : 0u);
+  const int wsrow = __builtin_amdgcn_readfirstlane((n0 >> 7) * KB);     // n0 is the same in every lane
+  auto load_w = [&](Blk& b, int kb) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int v = 0; v < WV; ++v)
-        b.w[i][v] = __builtin_nontemporal_load((const u4*)(wptr[i] + (size_t)kb * kstride + v * vstride));
-#pragma unroll
-    for (int j = 0; j < MT; ++j)
-#pragma unroll
-      for (int v = 0; v < AV; ++v) b.x[j][v] = *((const u4*)(aptr[j] + (size_t)kb * 128 * T::ABYTES) + v);
-    if (MODE == KC_FP8_BLOCK) {
-#pragma unroll
-      for (int j = 0; j < MT; ++j) b.as[j] = a.a_scale[(size_t)arow[j] * KB + kb];
-      b.ws = wsf[(size_t)(n0 >> 7) * KB + kb];
-    }
+      for (int v = 0; v < WV; ++v)     // streamed once: non-temporal
+        b.w[i][v] = bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(wres, (int)woff[i], (int)(kb * kstride + v * vstride), 2));
+    // one block scale per wavefront and K block: a scalar offset, no lane address
+    if (MODE == KC_FP8_BLOCK) b.ws = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(wsres, 0, (wsrow + kb) * 4, 0));
     if (GW) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -206,6 +203,22 @@ kcontig_gemm_kernel(KcArgs a) {
           b.gs[i][h] = *(const uint2*)(ws16 + (size_t)(kb * gper + min(h, gper - 1)) * N + n);
       }
     }
+  };
+  auto load_x = [&](Blk& b, int kb) {
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < AV; ++v)
+        b.x[j][v] = bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(xres, (int)(aoff[j] + 16 * v), kb * 128 * T::ABYTES, 0));
+    if (MODE == KC_FP8_BLOCK) {
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        b.as[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(asres, arow[j] * KB * 4, kb * 4, 0));
+    }
+  };
+  auto load_blk = [&](Blk& b, int kb) {
+    load_w(b, kb);
+    load_x(b, kb);
   };
 
   auto compute_blk = [&](const Blk& b, int kb) {
@@ -295,10 +308,23 @@ kcontig_gemm_kernel(KcArgs a) {
   {
     constexpr int kstep = KS ? 4 : 1;
     const int kfirst = KS ? wave : 0;
-    if (kfirst < KB) {
+    Blk b0, b1;
+    // the first weights are requested before the slot ids are looked at: they depend on the expert only
+    // (unconditional where K is not split over the wavefronts: behind a branch the wait for the ids
+    // below would have to cover both paths, i.e. wait for these requests too)
+    if (!KS || kfirst < KB) load_w(b0, kfirst);
+    __builtin_amdgcn_sched_barrier(0);               // (keeps the requests above in front of the wait for the ids)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      int row;
+      if (GROUPED) row = min(tok[j], a.numel - 1) / a.topk;
+      else row = min(m0 + 16 * j + r16, a.M - 1);
+      arow[j] = row;
+      aoff[j] = (uint32_t)(((size_t)row * K + 32 * q) * T::ABYTES);
+    }
+    if (!KS || kfirst < KB) {
       const int klast = kfirst + (KB - 1 - kfirst) / kstep * kstep;   // this wavefront's last block
-      Blk b0, b1;
-      load_blk(b0, kfirst);
+      load_x(b0, kfirst);
       int kb = kfirst;
       while (true) {
         load_blk(b1, min(kb + kstep, klast));
@@ -359,13 +385,15 @@ kcontig_gemm_kernel(KcArgs a) {
 
   // ---- epilogue: lane holds row (l % 16) of each row tile and columns
   // n0 + 16 i + 4 q + {0..3}
+  const bool wide = !KS && a.wide_stores;
+  const rsrc_t ores = make_rsrc(a.out, (uint32_t)((size_t)(GROUPED ? a.numel : a.M) * N * 2));
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
     int m;
     bool ok;
     float rw = 1.0f;
     if (GROUPED) {
-      m = tok[16 * j + r16];
+      m = tok[j];
       ok = m < a.numel;
       if (ok && a.topk_weights) rw = a.topk_weights[m];
     } else {
@@ -375,13 +403,15 @@ kcontig_gemm_kernel(KcArgs a) {
     if (!ok) continue;
     float xs = 1.0f;
     if (MODE == KC_INT8 && a.a_scale) xs = a.a_scale[arow[j]];
+    uint32_t held[2] = {0u, 0u};                   // packed outputs of the even column tile of a pair
 #pragma unroll
     for (int i = 0; i < (KS ? 1 : 4); ++i) {
       const int n = n0 + 16 * (KS ? wave : i) + 4 * q;
-      if (n >= N) continue;
+      if (!wide && n >= N) continue;
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
+        if (wide && n >= N) { v[e] = 0.f; continue; }
         if (MODE == KC_INT8) {
           const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + n + e];
           v[e] = ((float)bitcast<i4>(KS ? fin[j] : acc[i][j])[e] * xs) * ws;
@@ -398,7 +428,26 @@ kcontig_gemm_kernel(KcArgs a) {
       u2 o;
       o.x = (uint32_t)Elem<ODT>::from_f32(v[0]) | ((uint32_t)Elem<ODT>::from_f32(v[1]) << 16);
       o.y = (uint32_t)Elem<ODT>::from_f32(v[2]) | ((uint32_t)Elem<ODT>::from_f32(v[3]) << 16);
-      *(u2*)((uint16_t*)a.out + (size_t)m * N + n) = o;
+      if (!wide) {
+        *(u2*)((uint16_t*)a.out + (size_t)m * N + n) = o;
+      } else if ((i & 1) == 0) {
+        held[0] = o.x;
+        held[1] = o.y;
+      } else {
+        // the lanes of a row that hold columns 4 q .. 4 q + 3 of two neighbouring column tiles trade
+        // halves (v_permlane16_swap: lanes 16..31 of the first register with lanes 0..15 of the second,
+        // likewise 48..63 with 32..47): lane q then holds 8 adjacent columns of tile i - 1 + (q & 1) and
+        // a store instruction writes 64 contiguous bytes per row instead of 32
+        const auto lo2 = __builtin_amdgcn_permlane16_swap(held[0], o.x, false, false);
+        const auto hi2 = __builtin_amdgcn_permlane16_swap(held[1], o.y, false, false);
+        const int nw = n0 + 16 * (i - 1 + (q & 1)) + 8 * (q >> 1);
+        // written through (sc0 sc1): the scattered output rows leave the L2 as they are produced instead of
+        // being evicted later in between the weight reads (1-2 % on the DeepSeek-style layer)
+        if (nw < N)
+          __builtin_amdgcn_raw_buffer_store_b128(
+              bitcast<__attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int>((u4){lo2[0], hi2[0], lo2[1], hi2[1]}),
+              ores, (int)(((size_t)m * N + nw) * 2), 0, 17);
+      }
     }
   }
 }
@@ -526,9 +575,12 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
   }
   MQ_REQUIRE(N % 4 == 0, "moe_gemm: N=%d must be a multiple of 4", N);
   MQ_REQUIRE(w_layout == 0 || (w_layout == 1 && N % 64 == 0), "moe_gemm: weight layout %d needs N=%d %% 64 == 0", w_layout, N);
+  MQ_REQUIRE((size_t)N * K * 2 < ((size_t)1 << 32) && ((size_t)numel / topk + 1) * K * 2 < ((size_t)1 << 32),
+             "moe_gemm: one expert's weights and the activations must each stay below 4 GiB (N=%d K=%d, %d slots)", N, K, numel);
   KcArgs g = {};
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = nullptr;
   g.M = numel; g.N = N; g.K = K; g.kslab = w_layout;
+  g.wide_stores = (N % 8 == 0 && ((size_t)out & 15) == 0 && (size_t)numel * N * 2 < ((size_t)1 << 32)) ? 1 : 0;
   g.sorted_ids = sorted_token_ids; g.expert_ids = expert_ids; g.npp = num_tokens_post_pad;
   g.topk_weights = topk_weights; g.numel = numel; g.topk = topk; g.block_size = block_size; g.E = E;
   g.w_stride = (long)N * K;
@@ -577,9 +629,12 @@ extern "C" int mi355q_kcontig_gemm(void* out, const void* a, const void* w, cons
   MQ_REQUIRE(out && a && w, "kcontig_gemm: null pointer");
   MQ_REQUIRE(K % 128 == 0 && N % 4 == 0, "kcontig_gemm: K=%d must be a multiple of 128 and N=%d of 4", K, N);
   MQ_REQUIRE(w_layout == 0 || (w_layout == 1 && N % 64 == 0), "kcontig_gemm: weight layout %d needs N=%d %% 64 == 0", w_layout, N);
+  MQ_REQUIRE((size_t)N * K * 2 < ((size_t)1 << 32) && (size_t)M * K * 2 < ((size_t)1 << 32),
+             "kcontig_gemm: the weights and the activations must each stay below 4 GiB (M=%d N=%d K=%d)", M, N, K);
   KcArgs g = {};
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = bias;
   g.M = M; g.N = N; g.K = K; g.kslab = w_layout;
+  g.wide_stores = (N % 8 == 0 && ((size_t)out & 15) == 0 && (size_t)M * N * 2 < ((size_t)1 << 32)) ? 1 : 0;
   g.numel = M; g.topk = 1; g.block_size = 64;
   int mode;
   if (quant_mode == 1) {

@@ -171,20 +171,6 @@ __device__ __forceinline__ void load_halves(const uint16_t* p, uint32_t* dst) {
   else dst[0] = *p;
 }
 
-// Buffer loads: an offset at or past the descriptor's size reads as zero
-// without touching memory, which makes "no such K block" a branch-free case
-// (callers add 2^31 to the lane offset; every buffer here is below 2 GiB).
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ u4 buf_load16(rsrc_t r, uint32_t off) {
-  return bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
-}
-// streamed once: non-temporal
-__device__ __forceinline__ u4 buf_load16_nt(rsrc_t r, uint32_t off) {
-  return bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 2));
-}
 template <int NT>
 __device__ __forceinline__ void buf_load_halves(rsrc_t r, uint32_t off, uint32_t* dst) {
   if (NT == 8) { u4 v = buf_load16(r, off); dst[0] = v[0]; dst[NT > 2 ? 1 : 0] = v[1]; dst[NT > 4 ? 2 : 0] = v[2]; dst[NT > 6 ? 3 : 0] = v[3]; }
