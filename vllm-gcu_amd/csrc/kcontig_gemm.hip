@@ -120,7 +120,9 @@ kcontig_gemm_kernel(KcArgs a) {
   constexpr bool GW = MODE == KC_W8A16G_F16 || MODE == KC_W8A16G_BF16;    // group-wise weight scales
   constexpr int AV = T::ABYTES * 2;               // 16-byte vectors per lane per K block (activations)
   constexpr int WV = T::WBYTES * 2;               // ... weights
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (the wavefront index is made visibly uniform: K-block offsets that depend on it are scalar operands of
+  // the buffer loads, and a value the compiler cannot prove uniform costs a loop around every load)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, q = lane >> 4;
   const int N = a.N, K = a.K;
   const int KB = K >> 7;
@@ -185,7 +187,7 @@ kcontig_gemm_kernel(KcArgs a) {
   const int gper = GW ? 128 / a.wgroup : 1;        // scale groups per K block
   const float* wsf = (const float*)a.w_scale + expert * a.ws_stride;
   const rsrc_t wsres = make_rsrc(wsf, MODE == KC_FP8_BLOCK ? (uint32_t)((size_t)((N + 127) >> 7) * KB * 4) : 0u);
-  const int wsrow = __builtin_amdgcn_readfirstlane((n0 >> 7) * KB);     // n0 is the same in every lane
+  const int wsrow = (n0 >> 7) * KB;
   auto load_w = [&](Blk& b, int kb) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
