@@ -149,16 +149,26 @@ __device__ __forceinline__ void store_out_row(uint16_t* out, const uint16_t* bia
     if (bias) f += Elem<DT>::to_f32(bias[ncol + t]);
     h[t] = Elem<DT>::from_f32(f);
   }
+  // Written through to memory (sc0 sc1) instead of left dirty in this XCD's L2: the kernel ends a little
+  // sooner (nothing to write back at its end) -- 0.1-0.2 us per launch, 1.8 % of the four-layer decode step.
   if (NT == 1) {
-    *out = h[0];
+    const uint32_t val = h[0];
+    asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(out), "v"(val) : "memory");
   } else {
     constexpr int P = NT >= 2 ? NT / 2 : 1;
     uint32_t o[P];
 #pragma unroll
     for (int t = 0; t < NT / 2; ++t) o[t] = (uint32_t)h[2 * t] | ((uint32_t)h[2 * t + 1] << 16);
-    if (NT == 8) *(u4*)out = (u4){o[0], o[P > 1 ? 1 : 0], o[P > 2 ? 2 : 0], o[P > 3 ? 3 : 0]};
-    else if (NT == 4) *(u2*)out = (u2){o[0], o[P > 1 ? 1 : 0]};
-    else *(uint32_t*)out = o[0];
+    if (NT == 8) {
+      const u4 val = (u4){o[0], o[P > 1 ? 1 : 0], o[P > 2 ? 2 : 0], o[P > 3 ? 3 : 0]};
+      asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(out), "v"(val) : "memory");
+    } else if (NT == 4) {
+      const u2 val = (u2){o[0], o[P > 1 ? 1 : 0]};
+      asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(out), "v"(val) : "memory");
+    } else {
+      const uint32_t val = o[0];
+      asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(out), "v"(val) : "memory");
+    }
   }
 }
 
