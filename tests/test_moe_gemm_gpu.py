@@ -144,9 +144,13 @@ def test_grouped_fp8_block(fmoe, ops, block):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
-def test_grouped_int8_and_fp16_and_w8a16(fmoe, ops):
+@pytest.mark.parametrize("N", [260, 264, 200])
+def test_grouped_int8_and_fp16_and_w8a16(fmoe, ops, N):
+    # widths that end inside a 64-column group: 260 takes the 8-byte output stores (not a multiple of 8),
+    # 264 and 200 the 16-byte ones with a last piece of 8 columns
+    print(f"case grouped int8 / fp16 / w8a16 N={N}", flush=True)
     rng = np.random.default_rng(11)
-    M, E, T, K, N = 33, 4, 2, 256, 260
+    M, E, T, K = 33, 4, 2, 256
     ids_w, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
     # int8 per-token x per-channel
     x = rng.standard_normal((M, K)).astype(np.float16)
