@@ -275,6 +275,10 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
  * with few column tiles: the second expert GEMM of a gated MLP at prefill token counts) split K
  * into fp32 partial tiles and add them up in a second kernel; without it they run unsplit.  The
  * result differs between the two only in the order of the fp32 additions.
+ *
+ * Size limits (the kernels address operands with 32-bit offsets; exceeding one is an error, not a
+ * silent wrap): one expert's weights N * K elements and the activation matrix (numel / topk + 1) * K
+ * elements must each stay below 2^31 elements.
  */
 size_t mi355q_moe_gemm_workspace_bytes(int quant_mode, int numel, int block_size, int max_blocks, int E,
                                        int K, int N);
@@ -288,7 +292,7 @@ int mi355q_moe_gemm(void* out, const void* a, const void* w, const float* a_scal
  * as called by linear_quant (csrc/src/linear_quant.cpp:16-95, fp8 block-scaled
  * C = sum_kb (A_kb B_kb^T) As Bs) and by weight_only_quant
  * (csrc/src/weight_only_quant.cpp:28-101, W8A16).  w is [N, K]; bias [N] in
- * the output dtype or NULL. */
+ * the output dtype or NULL.  N * K and M * K must each stay below 2^31 elements. */
 int mi355q_kcontig_gemm(void* out, const void* a, const void* w, const float* a_scale,
                         const void* w_scale, const void* bias, int quant_mode, int group_size, int M,
                         int K, int N, int act_dtype, int out_dtype, int w_layout, void* stream);
