@@ -99,3 +99,70 @@ def test_w8a8_int8_tile_and_streaming_kernels_replay():
 
         print(f"case graph replay w8a8 M={M}", flush=True)
         _replay_against_eager(run, [x], lambda i: [torch.randn(M, K, generator=gen).half()])
+
+
+def _moe_layer(mode):
+    from vllm_gcu_amd.kernels.modular_experts import TritonExpertsPad
+    from vllm_gcu_amd.kernels.modular_kernel import FusedMoEModularKernel
+    from vllm_gcu_amd.kernels.prepare_finalize import MoEPrepareAndFinalizeNoEP
+    if mode == "w4a16":
+        fe = TritonExpertsPad(use_int4_w4a16=True, block_shape=[0, 128])
+    else:
+        fe = TritonExpertsPad(use_fp8_w8a8=True, block_shape=[128, 128])
+    return FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), fe)
+
+
+@pytest.mark.parametrize("tokens", [16, 200])
+def test_fused_moe_w4a16_layer_replays_with_new_routing(tokens):
+    """A whole W4A16 expert layer (routing, align, two grouped GEMMs, gate, sum) captured once and replayed
+    with new activations and new router logits: the routing -- which blocks exist, which experts they
+    belong to, how many slots are valid -- is read on the device, so every replay must equal eager."""
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    E, T, H, I, g = 8, 2, 512, 1024, 128
+    gen = torch.Generator(device="cpu").manual_seed(tokens)
+
+    def rnd(*shape):
+        return torch.randint(-2 ** 31, 2 ** 31 - 1, shape, dtype=torch.int32, generator=gen).cuda()
+
+    w13, z13 = rnd(E, H // 8, 2 * I), rnd(E, H // g, 2 * I // 8)
+    w2, z2 = rnd(E, I // 8, H), rnd(E, I // g, H // 8)
+    s13 = (torch.rand(E, H // g, 2 * I, generator=gen) * 0.009 + 0.001).half().cuda()
+    s2 = (torch.rand(E, I // g, H, generator=gen) * 0.009 + 0.001).half().cuda()
+    x = torch.randn(tokens, H, generator=gen).half().cuda()
+    logits = torch.randn(tokens, E, generator=gen).cuda()
+    moe = _moe_layer("w4a16")
+
+    def run():
+        tw, ids = ops.fused_topk(x, logits, T, True)
+        return moe(x, w13, w2, tw, ids, w1_scale=s13, w2_scale=s2, w1_zp=z13, w2_zp=z2)
+
+    print(f"case graph replay fused moe w4a16 tokens={tokens}", flush=True)
+    _replay_against_eager(run, [x, logits],
+                          lambda i: [torch.randn(tokens, H, generator=gen).half(), torch.randn(tokens, E, generator=gen) * (1 + 3 * i)])
+
+
+def test_fused_moe_fp8_block_layer_replays_with_new_routing():
+    """The same for a block-scaled fp8 layer with grouped routing (quantisers, K-contiguous grouped GEMMs)."""
+    from vllm_gcu_amd.kernels import fused_moe
+    E, T, H, I, tokens = 32, 4, 512, 256, 48
+    gen = torch.Generator(device="cpu").manual_seed(7)
+
+    def rnd_fp8(*shape):
+        b = torch.randint(0, 256, shape, dtype=torch.uint8, generator=gen)
+        b[(b & 0x7f) == 0x7f] = 0                       # no NaN codes
+        return b.cuda().view(torch.float8_e4m3fn)
+
+    w13, w2 = rnd_fp8(E, 2 * I, H), rnd_fp8(E, H, I)
+    s13 = (torch.rand(E, 2 * I // 128, H // 128, generator=gen) * 1e-3 + 1e-4).cuda()
+    s2 = (torch.rand(E, H // 128, I // 128, generator=gen) * 1e-3 + 1e-4).cuda()
+    x = torch.randn(tokens, H, generator=gen).to(torch.bfloat16).cuda()
+    logits = torch.randn(tokens, E, generator=gen).cuda()
+    moe = _moe_layer("fp8")
+
+    def run():
+        tw, ids = fused_moe.grouped_topk(x, logits, T, True, 4, 2, "softmax", None)
+        return moe(x, w13, w2, tw, ids, w1_scale=s13, w2_scale=s2)
+
+    print("case graph replay fused moe fp8", flush=True)
+    _replay_against_eager(run, [x, logits],
+                          lambda i: [torch.randn(tokens, H, generator=gen).to(torch.bfloat16), torch.randn(tokens, E, generator=gen) * (1 + 2 * i)])
