@@ -440,19 +440,32 @@ def test_config3_full_size_properties_and_sample(ops, rearrange):
     perm = torch.randperm(M, generator=g)
     out_p = moe(x[perm].cuda(), w13d, w2d, tw[perm.cuda()], ids[perm.cuda()], **kw)
     assert torch.equal(out_p, out[perm.cuda()])
-    # one token against the oracle (only its two experts are dequantised on the CPU)
-    tok = 17
-    e_tok = ids[tok].cpu().numpy()
+    # up to sixteen tokens against the oracle: for every expert and slot position the first token routed
+    # there (each expert is dequantised once per GEMM on the CPU)
     two, ido, _ = om.topk_softmax(logits.numpy(), T, True)
     assert np.array_equal(ids.cpu().numpy(), ido)
+    toks = []
+    for e in range(E):
+        for slot in range(T):
+            toks += [int(t) for t in np.nonzero(ido[:, slot] == e)[0][:1]]
+    toks = sorted(set(toks))
+    assert len(toks) >= 8 and set(np.unique(ido[toks])) == set(range(E))
 
-    def expert(wq, zq, sc, e):
-        return ow4.dequantize(ow4.gptq_unpack_weight(wq[e].numpy()), ow4.gptq_unpack_zeros(zq[e].numpy()),
-                              sc[e].numpy(), 128)
+    buf = np.empty(H * 2 * I, np.float32)      # one dense expert matrix, reused: sixteen of them are dequantised
 
-    want = om.fused_experts(x[tok:tok + 1].float().numpy(), lambda e: expert(w13, z13, s13, e),
-                            lambda e: expert(w2, z2, s2, e), two[tok:tok + 1], e_tok[None, :], f16)
-    np.testing.assert_allclose(out[tok:tok + 1].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    def expert(wq, zq, sc, e, rows=512):
+        K, N = wq.shape[1] * 8, wq.shape[2]
+        dense = buf[:K * N].reshape(K, N)
+        wn, zn, sn = wq[e].numpy(), zq[e].numpy(), sc[e].numpy()
+        for k0 in range(0, K, rows):
+            dense[k0:k0 + rows] = ow4.dequantize(ow4.gptq_unpack_weight(wn[k0 // 8:(k0 + rows) // 8]),
+                                                 ow4.gptq_unpack_zeros(zn[k0 // 128:(k0 + rows) // 128]),
+                                                 sn[k0 // 128:(k0 + rows) // 128], 128)
+        return dense
+
+    want = om.fused_experts(x[toks].float().numpy(), lambda e: expert(w13, z13, s13, e),
+                            lambda e: expert(w2, z2, s2, e), two[toks], ido[toks], f16)
+    np.testing.assert_allclose(out[toks].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("block", [16, 32, 64])

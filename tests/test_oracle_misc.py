@@ -284,3 +284,65 @@ def test_fused_add_rms_norm_is_add_then_norm():
     out, z = norm.fused_add_rms_norm(x, r, w, 1e-6, _f16)
     assert np.array_equal(z, _f16(x + r))
     assert np.array_equal(out, norm.rms_norm(z, w, 1e-6, _f16))
+
+
+def test_moe_expert_int8_quant_known_rows_and_scalar_loop():
+    """q[t] = sat_s8(rne(x[t // topk] * rec[expert(t)])), product in float32
+    (oracle/w8a8.py; the reference stores reciprocals, w8a8.py:226-236)."""
+    # hand-written rows: K = 6, two experts
+    x = np.array([[1.0, 2.5, -2.5, 3.5, 1000.0, -1000.0],      # ties at .5 go to even; saturation
+                  [0.0, 0.0, 0.0, 0.0, 0.0, 0.0]], np.float16)  # zero row
+    rec = np.array([[1.0, 1.0, 1.0, 1.0, 1.0, 1.0],
+                    [0.5, 0.2, 0.2, 1.0, 0.127, 0.128]], np.float32)
+    ids = np.array([[0, 1], [1, 0]], np.int32)                  # topk 2
+    q = w8a8.moe_expert_int8_quant(x, rec, ids)
+    assert q.dtype == np.int8 and q.shape == (4, 6)
+    assert q[0].tolist() == [1, 2, -2, 4, 127, -128]            # expert 0: 2.5 -> 2, -2.5 -> -2, 3.5 -> 4
+    # expert 1: the float32 products decide (0.2 is not exact), evaluated one by one
+    want1 = [int(np.clip(np.rint(np.float32(a) * np.float32(b)), -128, 127)) for a, b in zip(x[0], rec[1])]
+    assert q[1].tolist() == want1 and want1[0] == 0 and want1[4] == 127 and want1[5] == -128
+    assert not q[2].any() and not q[3].any()
+    # scalar loop over (token, slot), topk 1 and 2, float64 product where exact -> same rounding
+    rng = np.random.default_rng(11)
+    for topk in (1, 2):
+        M, K, E = 5, 16, 3
+        xr = (rng.integers(-40, 41, size=(M, K)) / 4.0).astype(np.float16)     # quarter steps: exact products
+        rr = (2.0 ** rng.integers(-2, 3, size=(E, K))).astype(np.float32)      # powers of two
+        tid = rng.integers(0, E, size=(M, topk)).astype(np.int32)
+        got = w8a8.moe_expert_int8_quant(xr, rr, tid)
+        for m in range(M):
+            for s in range(topk):
+                e = int(tid[m, s])
+                for k in range(K):
+                    y = float(xr[m, k]) * float(rr[e, k])
+                    r = round(y)                        # Python rounds half to even
+                    assert int(got[m * topk + s, k]) == max(-128, min(127, r))
+    # 1-D ids are one slot per row
+    got = w8a8.moe_expert_int8_quant(x, rec, np.array([1, 0], np.int32))
+    assert got[0].tolist() == want1 and not got[1].any()
+
+
+def test_per_token_quant_fp8_is_group_quant_with_one_group():
+    """dynamic_per_token_scaled_fp8_quant: one scale per row = absmax / 448
+    (csrc/src/dynamic_per_token_scaled_fp8_quant.cpp; FP8_E4M3_MAX native_vllm.h:34)."""
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((4, 96)).astype(np.float32)
+    x[2] = 0.0
+    x[3, 5] = 448.0 * 3
+    q, s = fp8.per_token_quant_fp8(x)
+    assert q.shape == x.shape and s.shape == (4, 1)
+    absmax = np.abs(x).max(axis=-1)
+    assert np.array_equal(s[:, 0], (np.maximum(absmax, np.float32(1e-10)) / np.float32(448.0)).astype(np.float32))
+    # the largest element of each non-zero row lands exactly on +-448 (code 0x7e / 0xfe)
+    for m in (0, 1, 3):
+        k = int(np.abs(x[m]).argmax())
+        assert int(q[m, k]) & 0x7F == 0x7E
+    assert not q[2].any()
+    # equals the group quantiser called with the whole row as its group, and rows are independent
+    q2, s2 = fp8.per_token_group_quant_fp8(x, 96)
+    assert np.array_equal(q, q2) and np.array_equal(s, s2)
+    q1, s1 = fp8.per_token_quant_fp8(x[1:2])
+    assert np.array_equal(q1[0], q[1]) and s1[0, 0] == s[1, 0]
+    # dequantised codes reproduce x within half an e4m3 step (2^-4 relative) of the row maximum
+    back = fp8.from_e4m3fn(q) * s
+    assert np.all(np.abs(back - x) <= absmax[:, None] / 16 + 1e-12)

@@ -198,3 +198,54 @@ def test_dequantize_closed_form_and_gemm_exact_cases():
     # bias
     b = rng.integers(-3, 4, size=N).astype(np.float16)
     assert np.array_equal(w4.w4a16_gemm(x, q, z, s, g, bias=b), out + b.astype(np.float32))
+
+
+# ------------------------------------------------------------------------
+# Golden vectors written from the reference's own rearrange.py
+# (tests/golden/make_rearrange_vectors.py; rearrange.py:6-133)
+# ------------------------------------------------------------------------
+def _golden():
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "rearrange_vectors.npz")
+    return np.load(path, allow_pickle=False)
+
+
+def test_rearrange_gptq_equals_reference_vectors():
+    g = _golden()
+    rw, zf = w4.rearrange_gptq(g["gptq_g128_qweight"], g["gptq_g128_qzeros"], g["gptq_g128_scales"])
+    assert rw.dtype == np.uint8 and np.array_equal(rw, g["gptq_g128_rweight"])
+    assert zf.dtype == np.float16 and np.array_equal(zf.view(np.uint16), g["gptq_g128_zeros"].view(np.uint16))
+    # the first packed zero word is all ones: every nibble 15 wraps to 0 -> z*s == 0
+    assert np.all(g["gptq_g128_zeros"][0, :8] == 0)
+    rw2, z2 = w4.rearrange_gptq(g["gptq_g128_qweight"], None, g["gptq_g128_scales"])
+    assert z2 is None and np.array_equal(rw2, g["gptq_g128_rweight"])
+
+
+def test_rearrange_awq_equals_reference_vectors():
+    g = _golden()
+    qw, qz, sc = g["awq_qweight"], g["awq_qzeros"], g["awq_scales"]
+    rw, zf = w4.rearrange_awq(qw, qz, sc)
+    assert rw.dtype == np.uint8 and np.array_equal(rw, g["awq_fzeros_rweight"])
+    assert zf.dtype == np.float16 and np.array_equal(zf.view(np.uint16), g["awq_fzeros_zeros"].view(np.uint16))
+    rw, zi = w4.rearrange_awq(qw, qz, sc, zeros_in_int8=True)
+    assert rw.dtype == np.int8 and np.array_equal(rw.view(np.uint8), g["awq_fzeros_rweight"])
+    assert zi.dtype == np.int8 and np.array_equal(zi, g["awq_i8zeros_zeros"])
+    rw, zn = w4.rearrange_awq(qw, qz, sc, rearrange_group=64, zeros_in_int8=True, use_w4a8=True)
+    assert zn is None and rw.dtype == np.int8 and np.array_equal(rw, g["awq_w4a8_g64_rweight"])
+
+
+def test_native_pack_zeros_known_word():
+    """Nibble j of word c holds z[g, 8c + j], true value: columns 0..7 -> 0x76543210."""
+    z = np.arange(16, dtype=np.uint8).reshape(1, 16)
+    words = w4.native_pack_zeros(z).view(np.uint32)
+    assert words.shape == (1, 2)
+    assert int(words[0, 0]) == 0x76543210 and int(words[0, 1]) == 0xFEDCBA98
+    # and it differs from the GPTQ exporter's word (which stores z - 1)
+    assert int(w4.gptq_pack_zeros(z).view(np.uint32)[0, 0]) == 0x6543210F
+    # scalar walk on random data
+    rng = np.random.default_rng(3)
+    z = rng.integers(0, 16, size=(3, 24), dtype=np.uint8)
+    words = w4.native_pack_zeros(z).view(np.uint32)
+    for gi in range(3):
+        for n in range(24):
+            assert (int(words[gi, n // 8]) >> (4 * (n % 8))) & 15 == int(z[gi, n])
