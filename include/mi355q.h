@@ -102,7 +102,9 @@ int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
  * holds until the process ends.  A shape whose split-K plan needs more is rejected with an error
  * (use mi355q_w4a16_gemm then).  All calls on one GPU share the array: calls that may overlap in time
  * on one GPU (different streams, different threads) race and must be serialised by the caller.
- * Calls no allocating routine; enqueues one small clearing kernel before a split-K launch. */
+ * Calls no allocating routine; enqueues one small clearing kernel before a split-K launch (after every
+ * argument check).  The first call on a device looks the array's address up (hipGetSymbolAddress):
+ * make one call on each device before capturing a graph that contains this entry point. */
 size_t mi355q_w4a16_noalloc_scratch_bytes(void);
 int mi355q_w4a16_gemm_noalloc(void* out, const void* x, const int32_t* qweight, const void* scales,
                               const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
@@ -268,7 +270,10 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
  * block b < num_tokens_post_pad / block_size with e = expert_ids[b] and every
  * id t < numel in the block,  out[t, :] = a[t / topk, :] @ W[e]^T  (times
  * topk_weights[t] when that pointer is given).  max_blocks = entries of
- * expert_ids.  block_size in {16, 32, 64, 128}.
+ * expert_ids.  block_size in {16, 32, 64, 128}.  sorted_token_ids must hold at least
+ * max_blocks * block_size entries (the kernels load a block's ids before they compare the block
+ * with num_tokens_post_pad).  Rows of ids that appear in no block below num_tokens_post_pad (ids
+ * the alignment dropped) are not written, with or without a workspace.
  *
  * workspace (optional, may be NULL): device scratch of mi355q_moe_gemm_workspace_bytes(...) bytes for
  * the same shape.  With it, W4A16 launches whose grid would leave most of the chip idle (a long K

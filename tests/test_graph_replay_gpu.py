@@ -1,7 +1,8 @@
 """The GEMM launches that keep state between calls -- arrival counters that the last workgroup of a
 split-K exchange resets, partial-sum workspaces shared by every layer, the persistent int8 tile
 kernel's tile stream -- replayed from a captured HIP graph: every replay, with new inputs written
-between replays and eager launches of other shapes in between (they use the same workspace), must
+between replays and eager launches of other shapes in between (on the capture stream, so they use the
+same workspace), must
 give exactly the bits of an eager launch on the same inputs."""
 import pytest
 import torch
@@ -11,28 +12,34 @@ pytestmark = pytest.mark.gpu
 
 def _replay_against_eager(run, inputs, fresh_inputs, between=None, replays=3):
     """run() -> output tensor computed from the tensors in `inputs`; fresh_inputs(i) -> replacement
-    values for them."""
+    values for them.  Everything -- warm-up, capture, replays, the eager launches in between and the
+    eager reference -- runs on ONE side stream, so all of it shares that stream's workspace and
+    arrival counters (the workspace is keyed by device and stream)."""
+    from vllm_gcu_amd.kernels import _runtime as rt
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         run()                                        # warm-up: workspaces are allocated outside the capture
         side.synchronize()
+        ws_at_capture = rt.workspace(torch.device("cuda", torch.cuda.current_device()), 1).data_ptr()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
             out = run()
+        side.synchronize()
+        for i in range(replays):
+            for t, v in zip(inputs, fresh_inputs(i)):
+                t.copy_(v, non_blocking=False)
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            got = out.clone()
+            if between is not None:
+                between()                            # other launches on the same workspace / counters
+            want = run()
+            side.synchronize()
+            assert rt.workspace(torch.device("cuda", torch.cuda.current_device()), 1).data_ptr() == ws_at_capture
+            assert torch.isfinite(got).all()
+            assert torch.equal(got, want), f"replay {i} differs from the eager launch"
     torch.cuda.synchronize()
-    for i in range(replays):
-        for t, v in zip(inputs, fresh_inputs(i)):
-            t.copy_(v)
-        torch.cuda.synchronize()
-        graph.replay()
-        torch.cuda.synchronize()
-        got = out.clone()
-        if between is not None:
-            between()                                # other launches on the same workspace / counters
-        want = run()
-        torch.cuda.synchronize()
-        assert torch.isfinite(got).all()
-        assert torch.equal(got, want), f"replay {i} differs from the eager launch"
 
 
 @pytest.mark.parametrize("M", [16, 32, 128, 512])
@@ -55,6 +62,35 @@ def test_w4a16_split_k_launches_replay(M):
         lambda: ops.w4a16_gemm(x, qw, sc, zp, None, g),
         [x], lambda i: [torch.randn(M, K, generator=gen).half()],
         between=lambda: ops.w4a16_gemm(other_x, other_qw, other_sc, other_zp, None, g))
+
+
+def test_replay_survives_a_larger_eager_plan_on_the_capture_stream():
+    """A graph captured at a decode size holds the workspace's address for its partial tiles and arrival
+    counters.  An eager prefill-sized launch on the same stream afterwards needs a far larger plan; the
+    workspace must neither move nor be freed, and the replays must still equal eager."""
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    K, N, g = 14336, 4096, 128
+    gen = torch.Generator(device="cpu").manual_seed(77)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 8, N), dtype=torch.int32, generator=gen).cuda()
+    zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, generator=gen).cuda()
+    sc = (torch.rand(K // g, N, generator=gen) * 0.009 + 0.001).half().cuda()
+    x = torch.randn(16, K, generator=gen).half().cuda()
+    big = torch.randn(1100, K, generator=gen).half().cuda()       # wide tiles, K split three ways: 54 MB of partials
+    print("case graph replay w4a16 decode graph, prefill eager in between", flush=True)
+    _replay_against_eager(
+        lambda: ops.w4a16_gemm(x, qw, sc, zp, None, g),
+        [x], lambda i: [torch.randn(16, K, generator=gen).half()],
+        between=lambda: ops.w4a16_gemm(big, qw, sc, zp, None, g))
+
+
+def test_workspace_refuses_to_allocate_under_capture(monkeypatch):
+    from vllm_gcu_amd.kernels import _runtime as rt
+    dev = torch.device("cuda", torch.cuda.current_device())
+    rt.workspace(dev, 1)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    held = rt.workspace(dev, 1)                                   # already there: fine under capture
+    with pytest.raises(RuntimeError, match="before capturing"):
+        rt.workspace(dev, held.numel() + 1)
 
 
 def test_grouped_w4a16_split_k_replay():

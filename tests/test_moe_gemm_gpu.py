@@ -613,3 +613,40 @@ def test_grouped_w4a16_split_k_long_k_narrow_n(fmoe, ops, rearrange, dtype):
             want[t] = (x[t].float().numpy() @ ow4.dequantize(q[le], z[le], sd[le].float().numpy(), 128)) * tw[t, 0]
     assert np.isfinite(got).all() and (got[emap[ids[:, 0]] < 0] == 0).all()
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+def test_grouped_split_k_leaves_rows_of_dropped_ids_alone(fmoe, ops, rearrange):
+    """Ids the alignment drops -- experts outside [0, E) and rows past the valid count of the `_pad`
+    operators -- sit in no block, so no split writes their partial tiles.  The split-K reduction must
+    not read those (stale, possibly NaN) partial rows: their output rows keep what they held, as with
+    the unsplit launch."""
+    from vllm_gcu_amd import _lib
+    from vllm_gcu_amd.kernels import _runtime as rt
+    print("case grouped split-K with dropped ids", flush=True)
+    rng = np.random.default_rng(78)
+    M, E, K, N = 300, 4, 4096, 256
+    valid = 260                                            # rows past this count are padding
+    assert _lib.load().mi355q_moe_gemm_workspace_bytes(_lib.Q_W4A16, M, 64, (M + E * 63) // 64, E, K, N) > 0
+    q, z, s = make_int4_experts(rng, E, K, N)
+    w, zp = int4_to_device(rearrange, q, z)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).half()
+    ids = rng.integers(0, E, size=(M, 1)).astype(np.int32)
+    ids[rng.choice(valid, 40, replace=False), 0] = E + 3   # out of range: dropped
+    tw = rng.uniform(0.1, 1.0, size=(M, 1)).astype(np.float32)
+    so, eo, no = fmoe.moe_align_block_size(dev(ids), 64, E, None, torch.tensor([valid], dtype=torch.int32).cuda())
+    # poison the workspace the launch will use, so a read of an unwritten partial row shows
+    ws = rt.workspace(torch.device("cuda", torch.cuda.current_device()), 1)
+    ws[1 << 20:(1 << 20) + 4 * 4 * M * N].view(torch.float32).fill_(float("nan"))
+    cfg = {"BLOCK_SIZE_M": 64}
+    kw = dict(use_fp8_w8a8=False, use_int8_w8a8=False, use_int8_w8a16=False, use_int4_w4a16=True, block_shape=[0, 128])
+    C = torch.full((M, 1, N), 123.0, dtype=torch.float16, device="cuda")
+    fmoe.invoke_fused_moe_kernel(x.cuda(), w, C, None, dev(s), zp, dev(tw), dev(ids), so, eo, no, True, 1, cfg, **kw)
+    torch.cuda.synchronize()
+    got = C.view(M, N).float().cpu().numpy()
+    live = (np.arange(M) < valid) & (ids[:, 0] < E)
+    assert (got[~live] == 123.0).all(), "rows of dropped ids were written"
+    for t in np.nonzero(live)[0][::7]:
+        e = ids[t, 0]
+        want = (x[t].float().numpy() @ ow4.dequantize(q[e], z[e], s[e].astype(np.float32), 128)) * tw[t, 0]
+        np.testing.assert_allclose(got[t], want, rtol=RTOL, atol=ATOL)
+    assert np.isfinite(got).all()

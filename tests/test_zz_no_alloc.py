@@ -70,6 +70,58 @@ def test_noalloc_entry_point_matches_the_workspace_one_on_calls_in_a_row():
     assert torch.equal(a.view(torch.int16), b.view(torch.int16)) and torch.equal(b.view(torch.int16), d.view(torch.int16))
 
 
+def test_noalloc_entry_point_in_a_captured_graph_replays_with_new_inputs():
+    """After one eager call (which looks the scratch array up), the entry point is captured into a HIP
+    graph on a side stream and replayed with new activations each time; other eager no-alloc calls run
+    on the same stream between the replays and leave their contents in the shared array."""
+    from vllm_gcu_amd import _lib
+    from vllm_gcu_amd.kernels import _runtime as rt
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    lib = _lib.load()
+    M, K, N, g = 16, 14336, 4096, 128                       # cross-workgroup split-K: counters + partial tiles
+    q, z, s, x = _case(21, M, K, N)
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    xd, sd = dev(x), dev(s)
+    q2, z2, s2, x2 = _case(22, 8, 8192, 2048)
+    w2, zp2 = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q2)), dev(ow4.gptq_pack_zeros(z2)))
+    x2d, s2d = dev(x2), dev(s2)
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    out2 = torch.empty((8, 2048), dtype=torch.float16, device="cuda")
+    ws = torch.zeros(max(lib.mi355q_w4a16_workspace_bytes(M, K, N), 16), dtype=torch.uint8, device="cuda")
+    ref = torch.empty_like(out)
+
+    def noalloc(o, xx, ww, ss, zz, m, k, n):
+        _lib.check(lib.mi355q_w4a16_gemm_noalloc(o.data_ptr(), xx.data_ptr(), ww.data_ptr(), ss.data_ptr(),
+                                                 zz.data_ptr(), _lib.ZP_PACKED, None, m, k, n, g, _lib.F16,
+                                                 rt.stream_ptr()), "w4a16_gemm_noalloc")
+
+    print("case noalloc captured graph", flush=True)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        noalloc(out, xd, w, sd, zp, M, K, N)                # warm-up outside the capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            noalloc(out, xd, w, sd, zp, M, K, N)
+        side.synchronize()
+        rng = np.random.default_rng(23)
+        for i in range(3):
+            xd.copy_(dev(rng.standard_normal((M, K)).astype(np.float16)))
+            out.fill_(float("nan"))
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            got = out.clone()
+            noalloc(out2, x2d, w2, s2d, zp2, 8, 8192, 2048)  # another shape through the same array
+            _lib.check(lib.mi355q_w4a16_gemm(ref.data_ptr(), xd.data_ptr(), w.data_ptr(), sd.data_ptr(),
+                                             zp.data_ptr(), _lib.ZP_PACKED, None, M, K, N, g, _lib.F16,
+                                             ws.data_ptr(), ws.numel(), rt.stream_ptr()), "w4a16_gemm")
+            side.synchronize()
+            assert torch.isfinite(got).all()
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"replay {i}"
+    torch.cuda.synchronize()
+
+
 def test_noalloc_entry_point_rejects_what_does_not_fit():
     from vllm_gcu_amd import _lib
     from vllm_gcu_amd.kernels import _runtime as rt

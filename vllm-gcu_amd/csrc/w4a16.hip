@@ -129,6 +129,9 @@ extern "C" int mi355q_w4a16_gemm_noalloc(void* out, const void* x, const int32_t
                                          int N, int group_size, int dtype, void* stream) {
   MQ_REQUIRE(M >= 0 && K > 0 && N > 0, "w4a16_gemm_noalloc: bad shape M=%d K=%d N=%d", M, K, N);
   if (M == 0) return 0;
+  // every argument check of the GEMM happens before the first launch (the clear below)
+  MQ_REQUIRE(out && x && qweight && scales, "w4a16_gemm_noalloc: null pointer");
+  MQ_REQUIRE(dtype == MI355Q_F16 || dtype == MI355Q_BF16, "w4a16_gemm_noalloc: dtype %d not supported", dtype);
   MQ_REQUIRE(K % 128 == 0 && N % 128 == 0,
              "w4a16_gemm_noalloc: K=%d and N=%d must be multiples of 128 (slab layout)", K, N);
   const int gs = group_size <= 0 ? K : group_size;

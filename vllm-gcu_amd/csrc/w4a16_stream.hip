@@ -474,11 +474,18 @@ w4a16_stream_kernel(StreamArgs a) {
   // reproducible.  No workgroup barrier: the wavefronts of a workgroup do not
   // wait for each other's trips to memory.
   if (!fin_wave) return;
+  // The hardware order is: partial stores acknowledged (vmcnt(0)) -> counter increment -> partial loads
+  // (issued after the increment has returned).  The compiler must keep that order too: relaxed atomics
+  // to different addresses may legally be reordered, so the increment sits between two signal fences
+  // (compiler-only barriers: no instruction, no cache writeback).
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   int* counter = a.counters + (int)blockIdx.x * W + wave;
   int old = 0;
   if (lane == 0) old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   old = __builtin_amdgcn_readfirstlane(old);
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   if (old != a.splits - 1) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {

@@ -493,6 +493,39 @@ w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* 
   *(uint2*)(out + i) = o;
 }
 
+// The same for a grouped launch: the rows are visited through the aligned id list, so a slot id that the
+// alignment dropped (an expert outside [0, E), a row past the valid count) -- whose partial rows no
+// split wrote -- is left alone, exactly as the unsplit launch leaves it.
+template <int DT>
+__global__ void __launch_bounds__(256)
+w4a16_grouped_reduce_kernel(uint16_t* out, const float* partial, const float* row_weight,
+                            const int32_t* sorted_ids, const int32_t* npp, int numel, int N, int splits) {
+  const int n4 = N >> 2;
+  const long t = (long)blockIdx.x * 256 + threadIdx.x;
+  const long p = t / n4;
+  if (p >= *npp) return;
+  const int id = sorted_ids[p];
+  if (id >= numel || id < 0) return;
+  const long MN = (long)numel * N;
+  const long i = (long)id * N + (t - p * n4) * 4;
+  f4 v = *(const f4*)(partial + i);
+  int s = 1;
+  for (; s + 3 < splits; s += 4) {
+    const f4 p0 = *(const f4*)(partial + (size_t)s * MN + i), p1 = *(const f4*)(partial + (size_t)(s + 1) * MN + i);
+    const f4 p2 = *(const f4*)(partial + (size_t)(s + 2) * MN + i), p3 = *(const f4*)(partial + (size_t)(s + 3) * MN + i);
+    v += p0;
+    v += p1;
+    v += p2;
+    v += p3;
+  }
+  for (; s < splits; ++s) v += *(const f4*)(partial + (size_t)s * MN + i);
+  if (row_weight) v *= row_weight[id];
+  uint2 o;
+  o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
+  o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);
+  *(uint2*)(out + i) = o;
+}
+
 template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32>
 hipError_t launch_wm(const TileArgs& a, int row_blocks, hipStream_t st) {
   constexpr int BM = 16 * MT;
@@ -913,15 +946,16 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   MQ_REQUIRE(e == hipSuccess, "moe_w4a16: cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("moe_w4a16");
   if (splits > 1) {
-    // every slot id below numel sits in exactly one block, so every row of the partial tiles is written
-    const long MN = (long)numel * N;
-    const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
+    // the reduction walks the aligned id list (at most max_blocks * block_size positions, cut at *npp on
+    // the device): rows of ids that the alignment dropped have no partial tiles and are not touched
+    const long threads = (long)max_blocks * block_size * (N / 4);
+    const unsigned blocks = (unsigned)((threads + 255) / 256);
     if (dtype == MI355Q_F16)
-      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, (const uint16_t*)nullptr, topk_weights, MN, N, splits);
+      hipLaunchKernelGGL((w4a16_grouped_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
+                         (const float*)workspace, topk_weights, sorted_ids, npp, numel, N, splits);
     else
-      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, (const uint16_t*)nullptr, topk_weights, MN, N, splits);
+      hipLaunchKernelGGL((w4a16_grouped_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
+                         (const float*)workspace, topk_weights, sorted_ids, npp, numel, N, splits);
     MQ_LAUNCH_CHECK("moe_w4a16(split-K reduce)");
   }
   return 0;

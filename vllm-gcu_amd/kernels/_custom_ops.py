@@ -151,6 +151,9 @@ def _require_trivial_g_idx(g_idx: Optional[torch.Tensor], group_size: int) -> No
     tag = (g_idx.data_ptr(), g_idx._version, int(group_size))
     if getattr(g_idx, "_mi355q_trivial", None) == tag:
         return
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("gptq_gemm_gcu: this g_idx has not been checked yet and the check reads it back to the "
+                           "host; call the operator once with it before capturing a graph")
     K = g_idx.numel()
     gs = int(group_size) if group_size > 0 else K
     want = torch.arange(K, device=g_idx.device, dtype=g_idx.dtype) // gs

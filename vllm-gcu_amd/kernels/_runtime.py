@@ -30,17 +30,34 @@ def ptr(t):
 
 
 _workspaces = {}
+_retired = []          # superseded buffers: a captured graph may still hold their addresses
+# the largest plan of any entry point: two split-K regions of 64 MiB, arrival counters, slack
+WORKSPACE_BYTES = (130 << 20)
 
 
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Zero-initialised scratch for split-K partial tiles and arrival counters.
     One buffer per (device, stream) so launches that may overlap never share
-    it; the kernels restore the counters to zero themselves."""
+    it; the kernels restore the counters to zero themselves.
+
+    The buffer is allocated once at the size of the largest plan, so its
+    address never changes afterwards: a HIP graph captured on the stream keeps
+    pointing at live memory whatever runs eagerly later.  Should a larger
+    request ever arrive, the old buffer is kept alive (never handed back to the
+    allocator) for the same reason.  Allocating or growing while the stream is
+    being captured raises: the allocation and its zero fill would land in the
+    graph's private pool.  Run the operator once on the capture stream first."""
     key = (device.index if device.index is not None else torch.cuda.current_device(),
            torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        size = max(nbytes, 8 << 20)
-        buf = torch.zeros(size, dtype=torch.uint8, device=device)
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                "mi355q: the split-K workspace of this stream would have to be allocated during graph "
+                f"capture ({nbytes} bytes asked, {0 if buf is None else buf.numel()} held); run the "
+                "operator once on the capture stream before capturing")
+        if buf is not None:
+            _retired.append(buf)
+        buf = torch.zeros(max(nbytes, WORKSPACE_BYTES), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
