@@ -161,7 +161,7 @@ def fused_moe_gemm(a_rows: np.ndarray, expert_weight_fn, topk_ids: np.ndarray,
 
 
 def fused_experts(x, w1_fn, w2_fn, topk_weights, topk_ids, act_dtype,
-                  quant_a2=None):
+                  quant_a2=None, return_slots=False):
     """modular_experts.py:81-288 on the CPU: GEMM1 -> cast -> silu_and_mul ->
     cast -> GEMM2 (routed weights applied) -> cast -> sum over slots.
 
@@ -177,4 +177,6 @@ def fused_experts(x, w1_fn, w2_fn, topk_weights, topk_ids, act_dtype,
         c2 = quant_a2(c2)
     c3 = fused_moe_gemm(c2, w2_fn, topk_ids, 1, topk_weights, True)
     c3 = act_dtype(c3).reshape(M, T, -1)
+    if return_slots:                       # also the rounded per-slot terms [M, T, K] that are summed
+        return act_dtype(moe_sum(c3)), c3
     return act_dtype(moe_sum(c3))

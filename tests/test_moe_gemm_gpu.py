@@ -463,9 +463,19 @@ def test_config3_full_size_properties_and_sample(ops, rearrange):
                                                  sn[k0 // 128:(k0 + rows) // 128], 128)
         return dense
 
-    want = om.fused_experts(x[toks].float().numpy(), lambda e: expert(w13, z13, s13, e),
-                            lambda e: expert(w2, z2, s2, e), two[toks], ido[toks], f16)
-    np.testing.assert_allclose(out[toks].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    want, slots = om.fused_experts(x[toks].float().numpy(), lambda e: expert(w13, z13, s13, e),
+                                   lambda e: expert(w2, z2, s2, e), two[toks], ido[toks], f16, return_slots=True)
+    got = out[toks].float().cpu().numpy()
+    # The layer stores each slot's term in fp16 before the sum (modular_experts.py:257-288).  Terms reach
+    # 8..32 here, where fp16 steps are 2^-7..2^-6, and outputs are differences of such terms: a term whose
+    # fp32 value rounds the other way moves the sum by one step of that term however small the sum is.  So
+    # the bound per output is rtol * |want| + atol plus one fp16 step of each of its terms.
+    step = np.where(slots != 0, 2.0 ** (np.floor(np.log2(np.maximum(np.abs(slots), 2.0 ** -14))) - 10), 0.0).sum(axis=1)
+    err = np.abs(got - want)
+    bound = ATOL + RTOL * np.abs(want) + step
+    assert (err <= bound).all(), f"max excess {(err - bound).max()} at {np.unravel_index((err - bound).argmax(), err.shape)}"
+    # and without that allowance all but a handful of the outputs are inside the plain tolerance
+    assert (err > ATOL + RTOL * np.abs(want)).mean() < 1e-3
 
 
 @pytest.mark.parametrize("block", [16, 32, 64])
