@@ -607,7 +607,24 @@ def fp8_dense_bench(ops, dev, stream, iters=12):
                         "frac_hbm": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
                         "TFLOPs": round(2.0 * M * N * K / t / 1e12, 1),
                         "frac_fp8_mfma_peak": round(2.0 * M * N * K / t / 1e12 / 5000.0, 4)}
-    return {"workload": "fp8 block-scaled dense linear K=8192 N=28672, bf16 out", **out}
+    # the same layer with per-token x per-channel scales (cutlass_scaled_mm on fp8 operands)
+    wch = torch.rand(N, 1, device=dev) * 0.019 + 0.001
+    pc = {}
+    for M in (16, 128, 2048):
+        x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+        xq, xs = ops.scaled_fp8_quant(x, None, use_per_token_if_dynamic=True)
+        o = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        fns = [(lambda w=w: torch.ops._C.cutlass_scaled_mm(o, xq, w.t(), xs, wch, None)) for w in ws_]
+        time_graph(fns, iters, 3, stream)
+        t = time_graph(fns, iters, 0, stream) / iters
+        nbytes = N * K + M * K + 4 * M + 4 * N + 2 * M * N
+        pc[f"M{M}"] = {"us": round(t * 1e6, 1), "GBps": round(nbytes / t / 1e9, 1),
+                       "frac_hbm": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
+                       "TFLOPs": round(2.0 * M * N * K / t / 1e12, 1),
+                       "frac_fp8_mfma_peak": round(2.0 * M * N * K / t / 1e12 / 5000.0, 4)}
+    return {"workload": "fp8 block-scaled dense linear K=8192 N=28672, bf16 out", **out,
+            "per_token_per_channel": {"workload": "fp8 per-token x per-channel scaled GEMM (cutlass_scaled_mm), same layer",
+                                      **pc}}
 
 
 def yardsticks(dev, stream, iters=30):

@@ -122,6 +122,22 @@ int mi355q_fp8_block_gemm(void* out, const void* x, const void* w, const float* 
                           const float* w_scale, const void* bias, int M, int N, int K, long ldx,
                           long ldw, long ldo, int out_dtype, void* stream);
 
+/* fp8-e4m3 GEMM with the scales outside the K sum: what cutlass_scaled_mm computes when it is handed
+ * fp8 operands (csrc/src/cutlass_scaled_mm.cpp:12-36 forwards any dtype to topsatenDotBiasQuant with
+ * x_scale 0-d -> [1] and w_scale [N, 1] -> [N]; reached from the non-block branch of
+ * Fp8GCULinearMethod.apply, vllm_gcu/kernels/quantization/fp8.py:68-69),
+ *   out[m, n] = (sum_k x[m, k] * w[n, k]) * x_scale[m or 0] * w_scale[n or 0] (+ bias[n]),   fp32 accumulation.
+ * x is [M, K] fp8 with row stride ldx bytes; w is [N, K] fp8 with row stride ldw bytes, or in the
+ * kslab order when ldw = 0; x_scale f32 [M] when x_scale_per_row else one value; w_scale f32 [N]
+ * when w_scale_per_col else one value; bias in the output dtype (f16 / bf16) or NULL; out row
+ * stride ldo elements.  K %% 128 == 0, N %% 4 == 0.  Up to 64 rows (and for layers with few
+ * 256 x 128 output tiles) the weight-streaming kernel runs and wants dense operands
+ * (ldx = K, ldw = K or 0, ldo = N); above, the MFMA tile kernel (N %% 128 == 0, strides multiples of 16). */
+int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, const float* x_scale,
+                           int x_scale_per_row, const float* w_scale, int w_scale_per_col,
+                           const void* bias, int M, int N, int K, long ldx, long ldw, long ldo,
+                           int out_dtype, void* stream);
+
 /* ---- W8A8 int8 -------------------------------------------------------------
  * Replaces topsatenDotBiasQuant as called by cutlass_scaled_mm
  * (csrc/src/cutlass_scaled_mm.cpp:12-36) and dot_bias_quant

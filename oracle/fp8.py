@@ -9,6 +9,9 @@ Test infrastructure only.
 * ``w8a8_block_fp8_matmul`` (_custom_ops.py:564-579 ->
   csrc/src/linear_quant.cpp:16-95): ``C = sum_kb (A[:, kb] @ B[:, kb].T) *
   As[:, kb] * Bs[nb, kb]``.
+* ``cutlass_scaled_mm`` on fp8 operands (csrc/src/cutlass_scaled_mm.cpp:12-36,
+  reached from the non-block branch of vllm_gcu/kernels/quantization/fp8.py:68-69):
+  ``C = (A @ B.T) * a_scale[m] * b_scale[n] (+ bias)``.
 """
 import numpy as np
 import torch
@@ -107,3 +110,20 @@ def block_fp8_gemm(a_codes, a_scale, b_codes, b_scale, block=(128, 128), bias=No
     if bias is not None:
         res = res + bias.astype(np.float32)[None, :]
     return res
+
+
+def scaled_fp8_mm(a_codes, a_scale, b_codes, b_scale, bias=None):
+    """fp8 x fp8 with the scales outside the K sum: a_codes uint8 [M, K], b_codes uint8 [N, K] (the
+    operator's weight argument is its [K, N] view); a_scale scalar, [1], [M] or [M, 1]; b_scale scalar,
+    [1], [N] or [N, 1] (cutlass_scaled_mm.cpp:23-32 unsqueezes a 0-d x_scale and squeezes an [N, 1]
+    w_scale) -> float32 [M, N] = ``(float32 sum over K) * a_scale * b_scale (+ bias)``, formed as
+    ``(acc * a_scale) * b_scale`` like the int8 epilogue."""
+    a = torch.from_numpy(from_e4m3fn(a_codes))
+    b = torch.from_numpy(from_e4m3fn(b_codes))
+    acc = (a @ b.T).numpy()
+    xs = np.asarray(a_scale, dtype=np.float32).reshape(-1, 1)
+    ws = np.asarray(b_scale, dtype=np.float32).reshape(1, -1)
+    out = (acc * xs).astype(np.float32) * ws
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=np.float32).reshape(1, -1)
+    return out.astype(np.float32)

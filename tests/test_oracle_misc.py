@@ -346,3 +346,35 @@ def test_per_token_quant_fp8_is_group_quant_with_one_group():
     # dequantised codes reproduce x within half an e4m3 step (2^-4 relative) of the row maximum
     back = fp8.from_e4m3fn(q) * s
     assert np.all(np.abs(back - x) <= absmax[:, None] / 16 + 1e-12)
+
+
+def test_scaled_fp8_mm_vs_float64_and_block_identity():
+    """Scales outside the K sum (cutlass_scaled_mm.cpp:12-36 on fp8 operands): float64 brute force, every
+    scale shape, and the identity with the block-scaled GEMM when the block scales do not vary along K
+    and the channel scales do not vary inside a 128-column block."""
+    rng = np.random.default_rng(31)
+    M, K, N = 5, 256, 256
+    a = fp8.to_e4m3fn(np.clip(rng.standard_normal((M, K)) * 3, -448, 448).astype(np.float32))
+    b = fp8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 0.5, -448, 448).astype(np.float32))
+    xs = rng.uniform(0.01, 0.1, size=M).astype(np.float32)
+    ws = rng.uniform(0.001, 0.02, size=N).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tab = fp8.e4m3fn_decode_table()
+    want = (tab[a] @ tab[b].T) * xs[:, None].astype(np.float64) * ws[None, :].astype(np.float64) + bias
+    got = fp8.scaled_fp8_mm(a, xs, b, ws, bias)
+    assert got.dtype == np.float32 and got.shape == (M, N)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+    # scale shapes: [M, 1] / [N, 1] equal the flat ones; scalars broadcast
+    assert np.array_equal(fp8.scaled_fp8_mm(a, xs.reshape(M, 1), b, ws.reshape(N, 1), bias), got)
+    one = fp8.scaled_fp8_mm(a, np.float32(0.5), b, np.array([0.25], np.float32))
+    np.testing.assert_allclose(one, (tab[a] @ tab[b].T) * 0.125, rtol=1e-5, atol=1e-5)
+    # a known small case: codes 0x38 = 1.0, 0x40 = 2.0, 0xb8 = -1.0
+    a1 = np.array([[0x38, 0x40, 0xb8, 0x00]], np.uint8)
+    b1 = np.array([[0x40, 0x40, 0x40, 0x40], [0x38, 0x00, 0x38, 0x7e]], np.uint8)
+    assert fp8.scaled_fp8_mm(a1, 2.0, b1, np.array([1.0, 0.5], np.float32)).tolist() == [[8.0, 0.0]]
+    # block identity (exact here: scales are powers of two, so scaling commutes with the fp32 additions)
+    xs2 = (2.0 ** rng.integers(-4, 1, size=M)).astype(np.float32)
+    wsb = (2.0 ** rng.integers(-6, -2, size=N // 128)).astype(np.float32)
+    blk = fp8.block_fp8_gemm(a, np.repeat(xs2[:, None], K // 128, 1), b, np.repeat(wsb[:, None], K // 128, 1))
+    pc = fp8.scaled_fp8_mm(a, xs2, b, np.repeat(wsb, 128))
+    np.testing.assert_allclose(pc, blk, rtol=2e-6, atol=1e-6)

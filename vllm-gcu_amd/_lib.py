@@ -36,6 +36,8 @@ SIGNATURES = {
                                       c_void_p]),
     "mi355q_fp8_block_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                       c_int, c_long, c_long, c_long, c_int, c_void_p]),
+    "mi355q_fp8_scaled_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                       c_int, c_int, c_long, c_long, c_long, c_int, c_void_p]),
     "mi355q_dynamic_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355q_silu_mul_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_void_p]),
@@ -66,7 +68,7 @@ SIGNATURES = {
 }
 
 # must equal mi355q_abi_version() of the library (csrc/core.hip)
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 

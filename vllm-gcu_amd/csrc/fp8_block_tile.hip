@@ -17,9 +17,16 @@
 // tiles through LDS (4-byte direct-to-LDS copies).  Two wavefronts per SIMD
 // leave each 256 registers: 64 running sums, two sets of x operands, one set
 // of w operands that is re-read tile by tile behind the MFMAs (see `step`).
+//
+// PC variant (per-token x per-channel scales, cutlass_scaled_mm on fp8 operands): the scales live
+// outside the K sum, so every MFMA accumulates straight into the running sum, no scales travel
+// through LDS, and the epilogue multiplies by x_scale[m] (or one value) and w_scale[n] (or one value).
 #include "common.h"
 
 namespace mi355q {
+int kcontig_fp8_pc_launch(void* out, const void* a, const void* w, const float* a_scale, int scale_per_row,
+                          const float* w_scale, int scale_per_col, const void* bias, int M, int K, int N,
+                          int out_dtype, int w_layout, hipStream_t st);
 namespace {
 
 constexpr int FTM = 256, FTN = 128, FTKB = 128;
@@ -29,8 +36,9 @@ struct F8Args {
   void* out;                // [M, N] f16 / bf16, row stride ldo elements
   const uint8_t* x;         // [M, K] fp8, row stride ldx bytes
   const uint8_t* w;         // [N, K] fp8 row-major (row stride ldw) or in the kslab order
-  const float* x_scale;     // [M, K / 128]
-  const float* w_scale;     // [N / 128, K / 128]
+  const float* x_scale;     // [M, K / 128]; PC: [M] or one value
+  const float* w_scale;     // [N / 128, K / 128]; PC: [N] or one value
+  int xs_mul, ws_mul;       // PC: index multipliers of x_scale / w_scale (1 = per token / per channel, 0 = one value)
   const void* bias;         // [N] in the output dtype or null
   int M, N, K;
   long ldx, ldw, ldo;
@@ -50,7 +58,7 @@ __device__ __forceinline__ void dma4(const void* gptr, void* lds_wave_base) {
 
 typedef int i8v __attribute__((ext_vector_type(8)));
 
-template <int DT>
+template <int DT, bool PC>
 __global__ void __launch_bounds__(F8_THREADS, 1)
 fp8_block_gemm_kernel(F8Args a) {
   constexpr int WN = 2, NI = 4, NJ = 4;                 // 4 x 2 wavefronts of 64 x 64
@@ -136,6 +144,8 @@ fp8_block_gemm_kernel(F8Args a) {
       const int p = s - XCOPIES;
       dma16(wtile + (a.w_kslab ? (long)kt * FTKB * 64 : (long)kt * FTKB) + wo[p < WCOPIES ? p : 0],
             xs + X_BYTES + (wave + 8 * p) * 1024);
+    } else if (PC) {
+      // no scales inside the K sum
     } else if (wave < 4) {
       dma4(a.x_scale + xso + kt, xs + X_BYTES + W_BYTES + wave * 256);
     } else if (wave == 4) {
@@ -181,6 +191,7 @@ fp8_block_gemm_kernel(F8Args a) {
     }
   };
   auto read_xs = [&](XOps& f, uint32_t stage_off) {
+    if (PC) return;
     const uint32_t ad = xsaddr + stage_off;
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
@@ -215,8 +226,9 @@ fp8_block_gemm_kernel(F8Args a) {
         const i4 a0 = i < 3 ? w012[i < 3 ? i : 0][0] : w3cur[0], a1 = i < 3 ? w012[i < 3 ? i : 0][1] : w3cur[1];
         const i8v av = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
         const i8v bv = __builtin_shufflevector(cur.bx[0][j], cur.bx[1][j], 0, 1, 2, 3, 4, 5, 6, 7);
-        ring[n & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-        if (n >= 2) {
+        if (PC) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[i][j], 0, 0, 0, 0, 0, 0);
+        else ring[n & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+        if (!PC && n >= 2) {
           const int pn = n - 2;
           acc[pn / NJ][pn % NJ] += sc[pn % NJ] * ring[pn & 3];
         }
@@ -237,8 +249,10 @@ fp8_block_gemm_kernel(F8Args a) {
         __builtin_amdgcn_sched_barrier(0);
         ++n;
       }
+    if (!PC) {
 #pragma unroll
-    for (int pn = NI * NJ - 2; pn < NI * NJ; ++pn) acc[pn / NJ][pn % NJ] += sc[pn % NJ] * ring[pn & 3];
+      for (int pn = NI * NJ - 2; pn < NI * NJ; ++pn) acc[pn / NJ][pn % NJ] += sc[pn % NJ] * ring[pn & 3];
+    }
   };
   static_assert(NI == 4 && NJ == 4 && NSLOT <= 8, "the read and copy schedule is written for 16 MFMAs per K block");
 
@@ -266,8 +280,8 @@ fp8_block_gemm_kernel(F8Args a) {
   };
   auto wait_all_but_last_step = [&]() {
     // copies per step and wavefront: 4 x + 2 w, and one of scales in wavefronts 0..4
-    if (wave <= 4) __builtin_amdgcn_s_waitcnt(0x0f77);  // vmcnt(7)
-    else __builtin_amdgcn_s_waitcnt(0x0f76);            // vmcnt(6)
+    if (!PC && wave <= 4) __builtin_amdgcn_s_waitcnt(0x0f77);  // vmcnt(7)
+    else __builtin_amdgcn_s_waitcnt(0x0f76);                   // vmcnt(6)
   };
 #pragma unroll
   for (int d = 0; d < 3; ++d) {
@@ -277,7 +291,7 @@ fp8_block_gemm_kernel(F8Args a) {
   }
   wait_all_but_last_step();                        // elements 0 and 1 landed
   __builtin_amdgcn_s_barrier();
-  XOps o0, o1;
+  XOps o0 = {}, o1 = {};
   WTile w3a, w3b;
 #pragma unroll
   for (int r = 0; r < 8; ++r) read_x(o0, r >> 2, r & 3, 0);
@@ -331,16 +345,29 @@ fp8_block_gemm_kernel(F8Args a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) bia[i][e] = a.bias ? Elem<DT>::to_f32(((const uint16_t*)a.bias)[n + e]) : 0.0f;
     }
+    float wsc[NI][4];
+    if (PC) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) wsc[i][e] = a.w_scale[(n + e) * a.ws_mul];
+      }
+    }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
       if (m >= M) continue;
+      const float xsc = PC ? a.x_scale[(long)m * a.xs_mul] : 1.0f;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (PC ? (acc[i][j][e] * xsc) * wsc[i][e] : acc[i][j][e]) + bia[i][e];
         u2 o;
-        o.x = (uint32_t)Elem<DT>::from_f32(acc[i][j][0] + bia[i][0]) | ((uint32_t)Elem<DT>::from_f32(acc[i][j][1] + bia[i][1]) << 16);
-        o.y = (uint32_t)Elem<DT>::from_f32(acc[i][j][2] + bia[i][2]) | ((uint32_t)Elem<DT>::from_f32(acc[i][j][3] + bia[i][3]) << 16);
+        o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
+        o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);
         *(u2*)((uint16_t*)a.out + (long)m * a.ldo + n) = o;
       }
     }
@@ -352,19 +379,19 @@ fp8_block_gemm_kernel(F8Args a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
 }
 
-template <int DT>
+template <int DT, bool PC>
 int launch_f8(const F8Args& a, hipStream_t st) {
   const int mtiles = (a.M + FTM - 1) / FTM, ntiles = a.N / FTN;
   F8Args b = a;
   b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
   const size_t shmem = 3 * (size_t)(FTM * FTKB + FTN * FTKB + FTM * 4 + 256);
-  static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT>,
+  static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT, PC>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-  MQ_REQUIRE(attr == hipSuccess, "fp8_block_gemm: cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
+  MQ_REQUIRE(attr == hipSuccess, "fp8 gemm: cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
   int grid = mtiles * ntiles, cus = device_cu_count() / 8 * 8;
   if (cus >= 8 && grid > cus) grid = cus;
-  hipLaunchKernelGGL((fp8_block_gemm_kernel<DT>), dim3(grid), dim3(F8_THREADS), shmem, st, b);
-  MQ_LAUNCH_CHECK("fp8_block_gemm");
+  hipLaunchKernelGGL((fp8_block_gemm_kernel<DT, PC>), dim3(grid), dim3(F8_THREADS), shmem, st, b);
+  MQ_LAUNCH_CHECK("fp8 gemm");
   return 0;
 }
 
@@ -393,6 +420,48 @@ extern "C" int mi355q_fp8_block_gemm(void* out, const void* x, const void* w, co
   a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;
   a.w_kslab = kslab ? 1 : 0;
   a.n_panels_swizzle = 0;
-  if (out_dtype == MI355Q_F16) return launch_f8<MI355Q_F16>(a, as_stream(stream));
-  return launch_f8<MI355Q_BF16>(a, as_stream(stream));
+  a.xs_mul = a.ws_mul = 0;
+  if (out_dtype == MI355Q_F16) return launch_f8<MI355Q_F16, false>(a, as_stream(stream));
+  return launch_f8<MI355Q_BF16, false>(a, as_stream(stream));
+}
+
+// fp8 x fp8 with per-token (or one) activation scale and per-channel (or one) weight scale, fp32
+// accumulation over the whole of K:  out[m, n] = (sum_k x[m, k] w[n, k]) * x_scale[m] * w_scale[n] (+ bias[n])
+extern "C" int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, const float* x_scale,
+                                      int x_scale_per_row, const float* w_scale, int w_scale_per_col,
+                                      const void* bias, int M, int N, int K, long ldx, long ldw, long ldo,
+                                      int out_dtype, void* stream) {
+  MQ_REQUIRE(M >= 0 && N > 0 && K > 0, "fp8_scaled_gemm: bad shape M=%d N=%d K=%d", M, N, K);
+  if (M == 0) return 0;
+  MQ_REQUIRE(out && x && w && x_scale && w_scale, "fp8_scaled_gemm: null pointer");
+  MQ_REQUIRE(K % 128 == 0 && N % 4 == 0, "fp8_scaled_gemm: K=%d must be a multiple of 128 and N=%d of 4", K, N);
+  MQ_REQUIRE(out_dtype == MI355Q_F16 || out_dtype == MI355Q_BF16, "fp8_scaled_gemm: bad out dtype %d", out_dtype);
+  const bool kslab = ldw == 0;
+  MQ_REQUIRE(!kslab || N % 64 == 0, "fp8_scaled_gemm: weights in the kslab order need N=%d %% 64 == 0", N);
+  MQ_REQUIRE(ldx >= K && (kslab || ldw >= K) && ldo >= N,
+             "fp8_scaled_gemm: row strides (%ld, %ld, %ld) must cover K=%d / N=%d", ldx, ldw, ldo, K, N);
+  // the MFMA tile kernel from 65 rows on when its 256 x 128 tiles fill a good part of the chip; below
+  // (and for shapes it does not take) the weight-streaming kernel, which wants dense operands
+  const long tiles = (long)((M + FTM - 1) / FTM) * (N / FTN);
+  const bool tile_ok = N % 128 == 0 && ldx % 16 == 0 && (kslab || ldw % 16 == 0) && ldo % 4 == 0 &&
+                       (size_t)N * K < ((size_t)1 << 32) && (size_t)256 * (size_t)ldx < ((size_t)1 << 32) &&
+                       (size_t)128 * (size_t)(kslab ? K : ldw) < ((size_t)1 << 32);
+  const bool stream_ok = ldx == K && (kslab || ldw == K) && ldo == N && (size_t)N * K * 2 < ((size_t)1 << 32) &&
+                         (size_t)M * K * 2 < ((size_t)1 << 32);
+  if (tile_ok && ((M > 64 && tiles >= 64) || !stream_ok)) {
+    F8Args a;
+    a.out = out; a.x = (const uint8_t*)x; a.w = (const uint8_t*)w; a.x_scale = x_scale; a.w_scale = w_scale;
+    a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;
+    a.w_kslab = kslab ? 1 : 0;
+    a.n_panels_swizzle = 0;
+    a.xs_mul = x_scale_per_row ? 1 : 0;
+    a.ws_mul = w_scale_per_col ? 1 : 0;
+    if (out_dtype == MI355Q_F16) return launch_f8<MI355Q_F16, true>(a, as_stream(stream));
+    return launch_f8<MI355Q_BF16, true>(a, as_stream(stream));
+  }
+  MQ_REQUIRE(stream_ok, "fp8_scaled_gemm: M=%d N=%d K=%d with row strides (%ld, %ld, %ld) fits neither kernel "
+             "(dense operands, or N %% 128 == 0 with strides that are multiples of 16)", M, N, K, ldx, ldw, ldo);
+  // the streaming kernel covers 64 rows (128 on narrow layers) per pass over the weights
+  return kcontig_fp8_pc_launch(out, x, w, x_scale, x_scale_per_row, w_scale, w_scale_per_col, bias, M, K, N, out_dtype,
+                               kslab ? 1 : 0, as_stream(stream));
 }

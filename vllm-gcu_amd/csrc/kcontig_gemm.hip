@@ -27,14 +27,17 @@ namespace mi355q {
 namespace {
 
 enum { KC_FP8_BLOCK = 0, KC_INT8 = 1, KC_F16 = 2, KC_BF16 = 3, KC_W8A16_F16 = 4, KC_W8A16_BF16 = 5,
-       KC_W8A16G_F16 = 6, KC_W8A16G_BF16 = 7 };   // G: group-wise scales [E, K/g, N], g = 64 or 128
+       KC_W8A16G_F16 = 6, KC_W8A16G_BF16 = 7,     // G: group-wise scales [E, K/g, N], g = 64 or 128
+       KC_FP8_PC = 8 };                           // fp8 with per-token x per-channel (or per-tensor) scales
 
 struct KcArgs {
   void* out;                   // [rows_out, N] f16/bf16
   const void* a;               // activations [Ma, K]
   const void* w;               // weights [E, N, K]
-  const float* a_scale;        // fp8: [Ma, K/128]; int8: [Ma]
-  const void* w_scale;         // fp8: f32 [E, ceil(N/128), K/128]; int8: f32 [E, N]; W8A16: act dtype [E, N] or [E, K/g, N]
+  const float* a_scale;        // fp8 block: [Ma, K/128]; int8 / fp8 per token: [Ma] (one value with sc_row = 0)
+  const void* w_scale;         // fp8 block: f32 [E, ceil(N/128), K/128]; int8 / fp8 per channel: f32 [E, N] (one value
+                               // with sc_col = 0); W8A16: act dtype [E, N] or [E, K/g, N]
+  int sc_row, sc_col;          // int8 / fp8 per token x per channel: index multipliers of a_scale / w_scale (1, or 0 = per tensor)
   const void* bias;            // [N] in out dtype, dense mode only
   int M, N, K;
   int kslab;                   // weights are in the kslab layout (N % 64 == 0)
@@ -57,6 +60,10 @@ template <> struct Kc<KC_FP8_BLOCK> {
 template <> struct Kc<KC_INT8> {
   static constexpr int ABYTES = 1, WBYTES = 1;
   typedef i4 acc_t;
+};
+template <> struct Kc<KC_FP8_PC> {
+  static constexpr int ABYTES = 1, WBYTES = 1;
+  typedef f4 acc_t;
 };
 template <> struct Kc<KC_F16> {
   static constexpr int ABYTES = 2, WBYTES = 2;
@@ -243,6 +250,25 @@ kcontig_gemm_kernel(KcArgs a) {
           const float sc = b.as[j] * b.ws;
           acc[i][j] = bitcast<acc_t>(bitcast<f4>(acc[i][j]) + sc * part);
         }
+    } else if (MODE == KC_FP8_PC) {
+      // scales live outside the K sum: the products of all K blocks go into one fp32 accumulator
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          f4 sum = bitcast<f4>(acc[i][j]);
+#pragma unroll
+          for (int v = 0; v < 2; ++v) {
+            const u4 wv = b.w[i][v], xv = b.x[j][v];
+            long w0 = (long)((unsigned long)wv[0] | ((unsigned long)wv[1] << 32));
+            long w1 = (long)((unsigned long)wv[2] | ((unsigned long)wv[3] << 32));
+            long x0 = (long)((unsigned long)xv[0] | ((unsigned long)xv[1] << 32));
+            long x1 = (long)((unsigned long)xv[2] | ((unsigned long)xv[3] << 32));
+            sum = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, x0, sum, 0, 0, 0);
+            sum = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, x1, sum, 0, 0, 0);
+          }
+          acc[i][j] = bitcast<acc_t>(sum);
+        }
     } else if (MODE == KC_INT8) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -404,7 +430,7 @@ kcontig_gemm_kernel(KcArgs a) {
     }
     if (!ok) continue;
     float xs = 1.0f;
-    if (MODE == KC_INT8 && a.a_scale) xs = a.a_scale[arow[j]];
+    if ((MODE == KC_INT8 || MODE == KC_FP8_PC) && a.a_scale) xs = a.a_scale[arow[j] * a.sc_row];
     uint32_t held[2] = {0u, 0u};                   // packed outputs of the even column tile of a pair
 #pragma unroll
     for (int i = 0; i < (KS ? 1 : 4); ++i) {
@@ -415,8 +441,11 @@ kcontig_gemm_kernel(KcArgs a) {
       for (int e = 0; e < 4; ++e) {
         if (wide && n >= N) { v[e] = 0.f; continue; }
         if (MODE == KC_INT8) {
-          const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + n + e];
+          const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + (n + e) * a.sc_col];
           v[e] = ((float)bitcast<i4>(KS ? fin[j] : acc[i][j])[e] * xs) * ws;
+        } else if (MODE == KC_FP8_PC) {
+          const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + (n + e) * a.sc_col];
+          v[e] = (bitcast<f4>(KS ? fin[j] : acc[i][j])[e] * xs) * ws;
         } else if ((W8H || W8B) && !GW) {
           const uint16_t raw = ((const uint16_t*)a.w_scale)[expert * a.ws_stride + n + e];
           const float ws = W8H ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw);
@@ -479,14 +508,14 @@ void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
   if constexpr (!GROUPED) {
     // too few workgroups to fill the chip: split K inside the workgroup
     // (64-row launches only for one-byte weights x one-byte activations: the others run out of registers)
-    if ((mt <= 2 || MODE == KC_FP8_BLOCK || MODE == KC_INT8) &&
+    if ((mt <= 2 || MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8) &&
         (a.N + 255) / 256 * row_blocks < 2 * device_cu_count()) {
       dim3 gks((a.N + 63) / 64, row_blocks);
       if (mt == 1) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true>), gks, block, 0, st, a);
       else if (mt == 2) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true>), gks, block, 0, st, a);
-      else if constexpr (MODE == KC_FP8_BLOCK || MODE == KC_INT8) {
+      else if constexpr (MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8) {
         if (mt == 4) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true>), gks, block, 0, st, a);
-        else if constexpr (MODE == KC_FP8_BLOCK)
+        else if constexpr (MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC)
           hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 8, false, true>), gks, block, 0, st, a);
       }
       return;
@@ -505,6 +534,8 @@ int launch_mode(const KcArgs& a, int mode, int odt, int mt, int row_blocks, hipS
   if (mode == M_ && odt == O_) { launch_mt<M_, O_, GROUPED>(a, mt, row_blocks, st); return 0; }
   KC_CASE(KC_FP8_BLOCK, MI355Q_BF16)
   KC_CASE(KC_FP8_BLOCK, MI355Q_F16)
+  KC_CASE(KC_FP8_PC, MI355Q_BF16)
+  KC_CASE(KC_FP8_PC, MI355Q_F16)
   KC_CASE(KC_INT8, MI355Q_F16)
   KC_CASE(KC_INT8, MI355Q_BF16)
   KC_CASE(KC_F16, MI355Q_F16)
@@ -529,6 +560,27 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                          int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
 size_t w4a16_grouped_workspace_bytes(int numel, int block_size, int max_blocks, int E, int K, int N);
+
+// fp8 x fp8 with scales outside the K sum (per token or one value; per output channel or one value), M <= 128:
+// the weight-streaming kernel.  Arguments are checked by the caller (mi355q_fp8_scaled_gemm).
+int kcontig_fp8_pc_launch(void* out, const void* a, const void* w, const float* a_scale, int scale_per_row,
+                          const float* w_scale, int scale_per_col, const void* bias, int M, int K, int N,
+                          int out_dtype, int w_layout, hipStream_t st) {
+  KcArgs g = {};
+  g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = bias;
+  g.M = M; g.N = N; g.K = K; g.kslab = w_layout;
+  g.sc_row = scale_per_row ? 1 : 0;
+  g.sc_col = scale_per_col ? 1 : 0;
+  g.wide_stores = (N % 8 == 0 && ((size_t)out & 15) == 0 && (size_t)M * N * 2 < ((size_t)1 << 32)) ? 1 : 0;
+  g.numel = M; g.topk = 1; g.block_size = 64;
+  int mt = pick_mt(M < 64 ? M : 64);
+  if (M > 64 && M <= 128 && (N + 255) / 256 < 2 * device_cu_count()) mt = 8;   // one 128-row block: weights streamed once
+  const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
+  int rc = launch_mode<false>(g, KC_FP8_PC, out_dtype, mt, row_blocks, st);
+  if (rc) return rc;
+  MQ_LAUNCH_CHECK("fp8_scaled_gemm");
+  return 0;
+}
 
 }  // namespace mi355q
 
@@ -582,6 +634,7 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
   KcArgs g = {};
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = nullptr;
   g.M = numel; g.N = N; g.K = K; g.kslab = w_layout;
+  g.sc_row = g.sc_col = 1;
   g.wide_stores = (N % 8 == 0 && ((size_t)out & 15) == 0 && (size_t)numel * N * 2 < ((size_t)1 << 32)) ? 1 : 0;
   g.sorted_ids = sorted_token_ids; g.expert_ids = expert_ids; g.npp = num_tokens_post_pad;
   g.topk_weights = topk_weights; g.numel = numel; g.topk = topk; g.block_size = block_size; g.E = E;
@@ -636,6 +689,7 @@ extern "C" int mi355q_kcontig_gemm(void* out, const void* a, const void* w, cons
   KcArgs g = {};
   g.out = out; g.a = a; g.w = w; g.a_scale = a_scale; g.w_scale = w_scale; g.bias = bias;
   g.M = M; g.N = N; g.K = K; g.kslab = w_layout;
+  g.sc_row = g.sc_col = 1;
   g.wide_stores = (N % 8 == 0 && ((size_t)out & 15) == 0 && (size_t)M * N * 2 < ((size_t)1 << 32)) ? 1 : 0;
   g.numel = M; g.topk = 1; g.block_size = 64;
   int mode;

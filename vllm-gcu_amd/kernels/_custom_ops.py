@@ -300,8 +300,61 @@ def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
                   x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.stream_ptr())
 
 
+def _scaled_fp8_mm(out, x, weight, x_scale, w_scale, bias):
+    """fp8-e4m3fn operands through ``cutlass_scaled_mm`` (cutlass_scaled_mm.cpp:12-36 forwards any dtype;
+    the non-block branch of the fp8 linear method ends here, kernels/quantization/fp8.py:68-69):
+    ``out = (x @ weight) * x_scale * w_scale (+ bias)`` with ``x_scale`` one value or one per row and
+    ``w_scale`` one value or one per output channel, fp32 accumulation."""
+    rt.require_gpu(out, x, weight, x_scale, w_scale, bias)
+    if x.numel() == 0:
+        return
+    if weight.dtype != torch.float8_e4m3fn or weight.dim() != 2:
+        raise RuntimeError(f"fp8 scaled matmul needs a 2-D float8_e4m3fn weight, got {weight.dtype} {tuple(weight.shape)}")
+    if out.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"fp8 scaled matmul writes float16 or bfloat16, got {out.dtype}")
+    if x_scale is None or w_scale is None:
+        raise RuntimeError("fp8 scaled matmul needs both scales")
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or x2.stride(0) % 16 != 0:
+        x2 = x2.contiguous()
+    M, K = x2.shape
+    if weight.shape[0] != K:
+        raise RuntimeError(f"weight is {tuple(weight.shape)} but activations have K={K}")
+    N = weight.shape[1]
+    out2 = out.reshape(-1, N)
+    if out2.data_ptr() != out.data_ptr() or out2.stride(-1) != 1:
+        raise RuntimeError("output must be a dense [.., N] tensor")
+    # the operator's weight argument is the [K, N] view of an [N, K] K-contiguous tensor (or kslab bytes)
+    if rearrange.is_kslab(weight):
+        w, ldw = weight, 0
+    elif weight.stride(0) == 1 and weight.stride(1) >= K:
+        w, ldw = weight, weight.stride(1)
+        if _AUTO_KSLAB and ldw == K and rearrange.kslab_eligible(weight.t()):
+            w, ldw = _converted(weight, lambda t: rearrange.to_kslab(t.t())), 0
+    else:
+        w = _converted(weight, lambda t: t.t().contiguous())
+        ldw = w.stride(0)
+    xs = x_scale.to(torch.float32).reshape(-1).contiguous()
+    ws = w_scale.to(torch.float32).reshape(-1).contiguous()
+    if xs.numel() not in (1, M):
+        raise RuntimeError(f"x_scale has {xs.numel()} entries for M={M}")
+    if ws.numel() not in (1, N):
+        raise RuntimeError(f"w_scale has {ws.numel()} entries for N={N}")
+    if bias is not None:
+        bias = bias.to(out.dtype).contiguous()
+        if bias.numel() != N:
+            raise RuntimeError(f"bias has {bias.numel()} entries for N={N}")
+    with torch.cuda.device(x.device):
+        _lib.call("mi355q_fp8_scaled_gemm", out2.data_ptr(), x2.data_ptr(), w.data_ptr(), xs.data_ptr(),
+                  int(xs.numel() > 1), ws.data_ptr(), int(ws.numel() > 1), rt.ptr(bias), M, N, K,
+                  x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.stream_ptr())
+
+
 def _cutlass_scaled_mm_impl(out, x, weight, x_scale, w_scale, bias):
-    _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias)
+    if x.dtype == torch.float8_e4m3fn:
+        _scaled_fp8_mm(out, x, weight, x_scale, w_scale, bias)
+    else:
+        _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias)
 
 
 def _dot_bias_quant_impl(out, lhs, rhs, scale, bias):

@@ -1,7 +1,12 @@
-"""fp8-e4m3fn block-scaled linear / MoE methods on MI355X.
+"""fp8-e4m3fn linear / MoE methods on MI355X.
 
 Mirrors ``Fp8GCULinearMethod`` / ``Fp8GCUMoEMethod`` and
 ``apply_w8a8_block_fp8_linear`` (vllm_gcu/kernels/quantization/fp8.py:49-205).
+Block-quantised checkpoints (128 x 128 weight scales) take ``linear_quant``;
+checkpoints without ``weight_block_size`` -- per-tensor or per-channel weight
+scales -- take the branch the reference leaves to upstream's
+``Fp8LinearMethod.apply`` (fp8.py:68-69): quantise the activations (static
+scale, or one scale per token) and call ``cutlass_scaled_mm`` on fp8 operands.
 """
 from typing import List, Optional
 
@@ -39,8 +44,11 @@ def apply_w8a8_block_fp8_linear(input: torch.Tensor, weight: torch.Tensor, block
 
 @register_gcu_quantization_config("fp8_gcu")
 class Fp8GCUConfig:
-    def __init__(self, weight_block_size=(128, 128)):
-        self.weight_block_size = list(weight_block_size)
+    def __init__(self, weight_block_size=(128, 128), activation_scheme: str = "dynamic"):
+        self.weight_block_size = None if weight_block_size is None else list(weight_block_size)
+        if activation_scheme not in ("dynamic", "static"):
+            raise ValueError(f"fp8: unsupported activation scheme {activation_scheme!r}")
+        self.activation_scheme = activation_scheme
 
     @classmethod
     def get_name(cls) -> str:
@@ -48,25 +56,31 @@ class Fp8GCUConfig:
 
     @classmethod
     def from_config(cls, config):
-        return cls(config.get("weight_block_size", [128, 128]))
+        # upstream Fp8Config.from_config: no "weight_block_size" key means per-tensor / per-channel scales.
+        # (An empty dict keeps this class's default of 128 x 128 blocks.)
+        if not config:
+            return cls()
+        return cls(config.get("weight_block_size", None), config.get("activation_scheme", "dynamic"))
 
     def get_quant_method(self, layer=None, prefix: str = "", moe: bool = False):
         return Fp8GCUMoEMethod(self) if moe else Fp8GCULinearMethod(self)
 
 
 class Fp8GCULinearMethod:
-    """Weights ``weight`` fp8 [N, K] and ``weight_scale_inv`` f32 [N/128, K/128]."""
+    """Block-quantised: ``weight`` fp8 [N, K] and ``weight_scale_inv`` f32 [N/128, K/128].
+    Otherwise: ``weight`` fp8 [N, K], ``weight_scale`` f32 with one value per logical shard (merged
+    projections) or per output channel, and ``input_scale`` (static scheme) or none (dynamic)."""
 
-    def __init__(self, quant_config: Fp8GCUConfig):
+    def __init__(self, quant_config):
         self.quant_config = quant_config
-        self.block_quant = quant_config.weight_block_size is not None
+        self.block_quant = getattr(quant_config, "weight_block_size", None) is not None
 
     def create_weights(self, layer, input_size_per_partition: int, output_partition_sizes: List[int],
                        input_size: int, output_size: int, params_dtype: torch.dtype, **extra_weight_attrs):
-        """Block-quantised checkpoint tensors as upstream vLLM 0.9.2's ``Fp8LinearMethod.create_weights``
-        registers them (the reference inherits it, fp8.py:49-70): ``weight`` fp8 ``[N, K]``,
-        ``weight_scale_inv`` f32 ``[ceil(N / 128), ceil(K / 128)]``, no static input scale."""
-        bn, bk = self.quant_config.weight_block_size
+        """Checkpoint tensors as upstream vLLM 0.9.2's ``Fp8LinearMethod.create_weights`` registers them (the
+        reference inherits it, fp8.py:49-70).  Block-quantised: ``weight`` fp8 ``[N, K]``, ``weight_scale_inv``
+        f32 ``[ceil(N / 128), ceil(K / 128)]``, no static input scale.  Per-tensor: ``weight_scale`` f32 with one
+        entry per logical shard, and with the static scheme ``input_scale`` likewise."""
         N, K = sum(output_partition_sizes), input_size_per_partition
 
         def reg(name, t):
@@ -75,24 +89,61 @@ class Fp8GCULinearMethod:
                 setattr(p, k, v)
             layer.register_parameter(name, p)
         reg("weight", torch.empty(N, K, dtype=torch.float8_e4m3fn))
-        reg("weight_scale_inv", torch.empty(-(-N // bn), -(-K // bk), dtype=torch.float32))
-        layer.input_scale = None
+        layer.logical_widths = list(output_partition_sizes)
         layer.orig_dtype = params_dtype
+        if self.block_quant:
+            bn, bk = self.quant_config.weight_block_size
+            reg("weight_scale_inv", torch.empty(-(-N // bn), -(-K // bk), dtype=torch.float32))
+            layer.input_scale = None
+            return
+        shards = len(output_partition_sizes)
+        reg("weight_scale", torch.full((shards,), torch.finfo(torch.float32).min, dtype=torch.float32))
+        if getattr(self.quant_config, "activation_scheme", "dynamic") == "static":
+            reg("input_scale", torch.full((shards,), torch.finfo(torch.float32).min, dtype=torch.float32))
+        else:
+            layer.input_scale = None
 
     def process_weights_after_loading(self, layer) -> None:
         # the reference keeps the checkpoint tensors as they are (fp8.py:72-166);
         # here the weight bytes are re-ordered once for contiguous wavefront loads
+        if not self.block_quant:
+            N = layer.weight.shape[0]
+            ws = layer.weight_scale.data.to(torch.float32).reshape(-1)
+            widths = getattr(layer, "logical_widths", None)
+            if ws.numel() not in (1, N):
+                # one scale per logical shard of a merged projection.  Upstream re-quantises every shard to
+                # the largest scale; the GEMM here takes a scale per output channel, so each shard keeps its
+                # own scale and its own fp8 codes: nothing is rounded twice.
+                if not widths or len(widths) != ws.numel() or sum(widths) != N:
+                    raise RuntimeError(f"fp8: {ws.numel()} weight scales do not match the shards {widths} of {N} rows")
+                ws = torch.repeat_interleave(ws, torch.tensor(widths, device=ws.device))
+            layer.weight_scale = torch.nn.Parameter(ws.contiguous(), requires_grad=False)
+            xs = getattr(layer, "input_scale", None)
+            if xs is not None:
+                # a static activation scale is one number per layer: the largest of the shards' (upstream)
+                layer.input_scale = torch.nn.Parameter(xs.data.to(torch.float32).max().reshape(1), requires_grad=False)
         rearrange.kslab_parameters_(layer, ("weight",))
 
     def apply(self, layer, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
               x_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
         if not self.block_quant:
-            raise NotImplementedError("per-tensor fp8 linear is not built; block-quantised only")
+            return self._apply_scaled_mm(layer, x, bias)
         return apply_w8a8_block_fp8_linear(input=x, weight=layer.weight,
                                            block_size=self.quant_config.weight_block_size,
                                            weight_scale=layer.weight_scale_inv,
                                            input_scale=getattr(layer, "input_scale", None) if x_scale is None else x_scale,
                                            bias=bias)
+
+    def _apply_scaled_mm(self, layer, x, bias):
+        """Upstream's ``Fp8LinearOp.apply`` on this build's operators: static scheme -> ``static_scaled_fp8_quant``
+        with the layer's one input scale; dynamic -> one scale per token
+        (``dynamic_per_token_scaled_fp8_quant``; the reference's per-tensor dynamic quantiser is an empty
+        body, csrc/src/dynamic_scaled_fp8_quant.cpp:21-22); then ``cutlass_scaled_mm`` with the ``[K, N]``
+        view of the weight and its per-tensor or per-channel scales."""
+        x2 = x.reshape(-1, x.shape[-1])
+        q, xs = ops.scaled_fp8_quant(x2, getattr(layer, "input_scale", None), use_per_token_if_dynamic=True)
+        out = ops.cutlass_scaled_mm(q, layer.weight.t(), xs, layer.weight_scale, x.dtype, bias)
+        return out.view(*x.shape[:-1], layer.weight.shape[0])
 
 
 class Fp8GCUMoEMethod:
