@@ -58,9 +58,11 @@ def per_token_quant_int8_gcu(x: torch.Tensor):
     return x_q, scales
 
 
-def install() -> None:
+def install():
     """Replace, in an importable vLLM 0.9.2, the attributes the reference replaces
-    (moe_layer.py:73-79, utils.py:17-22).  Raises ImportError when vLLM is absent."""
+    (moe_layer.py:73-79, utils.py:17-22) and register the quantization configs, methods and kernels
+    (``vllm_registration.register_with_vllm``; returns its dictionary of registered classes).
+    Raises ImportError when vLLM is absent."""
     import importlib
     try:
         fm = importlib.import_module("vllm.model_executor.layers.fused_moe")
@@ -70,7 +72,11 @@ def install() -> None:
     except ImportError as e:
         raise ImportError("install() wires the kernels into vLLM 0.9.2, which is not importable here") from e
 
-    class FusedMoE(fml.FusedMoE):
+    upstream_layer = getattr(fml.FusedMoE, "_mi355q_base", fml.FusedMoE)      # a second install() re-wraps the original
+
+    class FusedMoE(upstream_layer):
+        _mi355q_base = upstream_layer
+
         def forward_impl(self, hidden_states: torch.Tensor, router_logits: torch.Tensor):
             set_shared_experts(self)
             return super().forward_impl(hidden_states, router_logits)
@@ -82,3 +88,6 @@ def install() -> None:
     f8u.per_token_group_quant_fp8 = ops.per_token_group_quant_fp8
     fmu.per_token_group_quant_fp8 = ops.per_token_group_quant_fp8
     fmu.per_token_quant_int8 = per_token_quant_int8_gcu
+    # quantization configs, HF-name overrides, v2 weight loaders, scaled-mm kernel list
+    from .vllm_registration import register_with_vllm
+    return register_with_vllm()
