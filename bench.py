@@ -39,11 +39,24 @@ INT8_PEAK_TOPS = 5000.0
 # copy of --calibrate-copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per
 # unit).  Keyed by (M, --split-k); other settings were not profiled.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {(16, 0): 34022694}
-# when and on which build the figure above was taken; it must be re-measured (profiles/ names the
-# commands) whenever the streaming kernel's work split changes
-MEASURED_TRAFFIC_PROVENANCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (commands and per-layer figures in "
-                               "profiles/w4a16_stream_kernel_llama3_8b_m16.txt), re-measured after the last change to the "
-                               "streaming kernel; work split unchanged since")
+# the build the figure was taken on, and the work split (tiles per workgroup, K splits) it belongs to: the
+# line carries `traffic` only while the library still plans the four layers that way (a different split
+# moves the traffic: re-measure with the commands in profiles/w4a16_stream_kernel_llama3_8b_m16.txt)
+MEASURED_TRAFFIC_COMMIT = "1cb0412"
+MEASURED_TRAFFIC_PLAN = {"qkv": (2, 1), "o": (1, 1), "gate_up": (8, 1), "down": (4, 4)}
+
+
+def stream_plans(M):
+    """(tiles per workgroup, K splits) the library takes for the four layers at M rows on this device."""
+    import ctypes
+    from vllm_gcu_amd import _lib
+    lib = _lib.load()
+    out = {}
+    for name, K, N in LLAMA3_8B:
+        nt, sp = ctypes.c_int(0), ctypes.c_int(0)
+        _lib.check(lib.mi355q_w4a16_stream_plan(M, K, N, GROUP, ctypes.byref(nt), ctypes.byref(sp)), "stream_plan")
+        out[name] = (nt.value, sp.value)
+    return out
 
 
 def w4a16_bytes(M, K, N, g=GROUP):
@@ -275,11 +288,23 @@ def main():
     launch_us = ms_per_step * 1e3 / launches
     achieved = step_bytes / launches / (launch_us * 1e-6) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((M, args.split_k))
+    plans = stream_plans(M) if M <= 64 else {}
+    provenance = None
+    if traffic is not None:
+        if plans == MEASURED_TRAFFIC_PLAN:
+            provenance = {"measured_on_commit": MEASURED_TRAFFIC_COMMIT, "work_split": {k: list(v) for k, v in plans.items()},
+                          "how": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, commands and per-layer figures in "
+                                 "profiles/w4a16_stream_kernel_llama3_8b_m16.txt; the streaming kernel's loads and "
+                                 "work split are unchanged since that commit"}
+        else:
+            print(f"bench.py: the library plans {plans}, the traffic figure was measured on {MEASURED_TRAFFIC_PLAN}: "
+                  "traffic left out, re-measure it", file=sys.stderr)
+            traffic = None
     roofline = {"bound": "hbm", "kernel": "w4a16_stream_kernel", "launches_per_step": launches,
                 "avg_launch_us": round(launch_us, 3), "algorithmic_bytes_per_launch": step_bytes // launches,
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                "traffic_provenance": MEASURED_TRAFFIC_PROVENANCE if traffic else None}
+                "traffic_provenance": provenance}
     if M > 64:
         # --m above the decode range: the launches are the MFMA tile kernel and the bound is the fp16 matrix peak
         step_flops = sum(2.0 * M * K * N for _, K, N in LLAMA3_8B)
@@ -375,11 +400,13 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40, cpu=False):
     w_nk = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g).to(dev)
     ws = (torch.rand(N, generator=g) * 0.019 + 0.001).float().to(dev)
     out = torch.empty(M, N, dtype=torch.float16, device=dev)
-    wt = w_nk.t()
+    # three weight copies in turn (3 x 235 MB against a 256 MB last-level cache), as the decode legs do
+    wts = [w_nk.t(), w_nk.roll(1, 0).t(), w_nk.roll(2, 0).t()]
     # long warm-up: the core clock settles (it drops under sustained MFMA load and
     # recovers part of the way) only after some tens of launches
     # (several launches per graph: a graph of one short kernel would time the replay gap with it)
-    t = time_graph([lambda: torch.ops._C.cutlass_scaled_mm(out, xq, wt, xs, ws, None)] * 5, iters, warmup, stream) / iters
+    t = time_graph([(lambda wt=wt: torch.ops._C.cutlass_scaled_mm(out, xq, wt, xs, ws, None)) for wt in wts] * 2,
+                   iters, warmup, stream) / iters
     tq = time_graph([lambda: ops.scaled_int8_quant(x)] * 10, iters, 10, stream) / iters
     ops_ = 2.0 * M * K * N
     # decode: 16 tokens against the same layer, weights as the linear method keeps them after
@@ -391,7 +418,8 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40, cpu=False):
     fns = [(lambda w=w: torch.ops._C.cutlass_scaled_mm(outd, xq[:Md], w.t(), xs[:Md], ws, None)) for w in ksl]
     td = time_graph(fns * 2, iters, 6, stream) / iters
     res_cpu = cpu_baseline_w8a8(x, w_nk, ws) if cpu else None
-    return {"workload": "W8A8 int8 GEMM M=2048 K=8192 N=28672, fused per-token x per-channel scales, fp16 out",
+    return {"workload": "W8A8 int8 GEMM M=2048 K=8192 N=28672, fused per-token x per-channel scales, fp16 out, "
+                        "three weight copies in turn",
             "gemm_us": round(t * 1e6, 1), "TOPs": round(ops_ / t / 1e12, 1),
             "frac_int8_mfma_peak": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
             "roofline": {"bound": "mfma", "kernel": "w8a8_int8_gemm_kernel", "avg_launch_us": round(t * 1e6, 1),
@@ -473,7 +501,7 @@ def cpu_baseline_moe_fp8(x, tw, ids, w13, s13, w2, s2, tokens=2):
                       f"experts' weights"}
 
 
-def moe_bench(ops, dev, stream, which, iters=10, tokens=None, cpu=False):
+def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False):
     """BASELINE configs[3] (Mixtral-8x7B layer, W4A16) and configs[4]
     (DeepSeek-V3-style layer, fp8 block-scaled): routing + the whole
     fused-experts sequence, one layer."""
@@ -528,13 +556,21 @@ def moe_bench(ops, dev, stream, which, iters=10, tokens=None, cpu=False):
     else:
         M, H, E, I, T = 256, 7168, 256, 2048, 8
 
-        def rnd_fp8(*shape):
-            b = torch.randint(0, 256, shape, dtype=torch.uint8, device=dev)
-            b[(b & 0x7f) == 0x7f] = 0                       # no NaN codes
-            return b.view(torch.float8_e4m3fn)
-        w13, w2 = rnd_fp8(E, 2 * I, H), rnd_fp8(E, H, I)
-        s13 = torch.rand(E, 2 * I // 128, H // 128, device=dev) * 1e-4 + 1e-5
-        s2 = torch.rand(E, H // 128, I // 128, device=dev) * 1e-4 + 1e-5
+        def block_fp8(n, k):
+            """[E, n, k] weights ~ N(0, 0.02) quantised to fp8-e4m3 with one fp32 scale per 128 x 128 block
+            (scale = block absmax / 448), as BASELINE configs[4] states; one expert at a time on the device."""
+            codes = torch.empty((E, n, k), dtype=torch.float8_e4m3fn, device=dev)
+            scales = torch.empty((E, n // 128, k // 128), dtype=torch.float32, device=dev)
+            gg = torch.Generator(device=dev).manual_seed(n + k)
+            for e in range(E):
+                w = torch.randn(n, k, device=dev, generator=gg) * 0.02
+                blk = w.view(n // 128, 128, k // 128, 128)
+                sc = blk.abs().amax(dim=(1, 3)).clamp_min(1e-12) / 448.0
+                codes[e] = (blk / sc[:, None, :, None]).view(n, k).to(torch.float8_e4m3fn)
+                scales[e] = sc
+            return codes, scales
+        w13, s13 = block_fp8(2 * I, H)
+        w2, s2 = block_fp8(H, I)
         x = torch.randn(M, H, generator=g).to(torch.bfloat16).to(dev)
         logits = torch.randn(M, E, generator=g).to(dev)
         moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad(use_fp8_w8a8=True, block_shape=[128, 128]))
@@ -548,8 +584,10 @@ def moe_bench(ops, dev, stream, which, iters=10, tokens=None, cpu=False):
         flops = 2.0 * M * T * (H * 2 * I + I * H)
         bytes_ = hit * (2 * I * H + H * I + 4 * (2 * I // 128 * H // 128 + H // 128 * I // 128)) \
             + M * H + M * H // 128 * 4 + M * H * 2
-        name = f"fused MoE fp8 block-scaled, DeepSeek-V3-style layer: 256 tok, hidden 7168, 256 experts ({hit} hit), inter 2048, top-8"
-    t = time_graph([step], iters, 2, stream) / iters
+        name = (f"fused MoE fp8 block-scaled, DeepSeek-V3-style layer: 256 tok, hidden 7168, 256 experts ({hit} hit), inter 2048, "
+                "top-8; weights ~ N(0, 0.02) quantised per 128 x 128 block")
+    time_graph([step], 5, 3, stream)
+    t = time_graph([step], iters, 0, stream) / iters
     res = {"workload": name, "us": round(t * 1e6, 1), "compulsory_bytes": int(bytes_),
            "GBps": round(bytes_ / t / 1e9, 1), "frac_hbm": round(bytes_ / t / 1e9 / HBM_PEAK_GBPS, 4),
            "TFLOPs": round(flops / t / 1e12, 1),

@@ -94,6 +94,11 @@ int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          int dtype, void* workspace, size_t workspace_bytes,
                          int split_k, int family, void* stream);
 
+/* No counterpart in the reference (the vendor GEMM chooses its own launch).  The work split the streaming
+ * kernel takes for M <= 64 rows of a shape on the current device: 16-column tiles per workgroup (1, 2, 4
+ * or 8) and the number of K ranges that separate workgroups sum through the workspace. */
+int mi355q_w4a16_stream_plan(int M, int K, int N, int group_size, int* tiles_per_workgroup, int* k_splits);
+
 /* No counterpart in the reference.  mi355q_w4a16_gemm for callers that cannot allocate device memory
  * or pass a workspace (code under HIP graph capture, serving loops and harnesses that forbid
  * allocation): same arguments without the workspace, same kernels, bit-identical results.  The

@@ -28,6 +28,7 @@ SIGNATURES = {
     "mi355q_w4a16_gemm_ex": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_int,
                                      c_int, c_void_p]),
+    "mi355q_w4a16_stream_plan": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_w4a16_noalloc_scratch_bytes": (c_size_t, []),
     "mi355q_w4a16_gemm_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                           c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -38,6 +38,28 @@ extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
   return s > tt ? s : tt;
 }
 
+namespace mi355q {
+struct StreamPlan { int nt, splits; };
+StreamPlan w4a16_stream_auto_plan(int M, int K, int N, int gs);
+}  // namespace mi355q
+
+// the work split the streaming (decode) kernel takes for a shape: tiles of 16 columns per workgroup and
+// K splits across workgroups (what a caller sizes the workspace for, and what a profile was taken on)
+extern "C" int mi355q_w4a16_stream_plan(int M, int K, int N, int group_size, int* tiles_per_workgroup,
+                                        int* k_splits) {
+  MQ_REQUIRE(M > 0 && K > 0 && N > 0 && K % 128 == 0 && N % 128 == 0, "w4a16_stream_plan: bad shape M=%d K=%d N=%d", M, K, N);
+  MQ_REQUIRE(tiles_per_workgroup && k_splits, "w4a16_stream_plan: null pointer");
+  const int gs = group_size <= 0 ? K : group_size;
+  const StreamPlan p = w4a16_stream_auto_plan(M > 64 ? 64 : M, K, N, gs);
+  const int G = K / 128;
+  int splits = p.splits > G ? G : p.splits;
+  if (splits > 32) splits = 32;
+  while (splits > 1 && ((G + splits - 1) / splits) * (splits - 1) >= G) --splits;
+  *tiles_per_workgroup = p.nt;
+  *k_splits = splits;
+  return 0;
+}
+
 extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                                     const void* scales, const void* zeros, int zeros_kind,
                                     const void* bias, int M, int K, int N, int group_size,
