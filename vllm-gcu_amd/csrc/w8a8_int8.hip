@@ -35,6 +35,7 @@ struct I8Args {
   const void* bias;         // [N] in out dtype (or f32 when bias_f32) or null
   int M, N, K;
   long ldx, ldw, ldo;
+  long ldacc;               // row stride of acc_out (elements)
   int x_scale_per_row, w_scale_per_col, bias_f32;
   int n_panels_swizzle;     // non-zero: XCD-aware tile order
   int w_kslab;              // w is in the kslab order (see include/mi355q.h) instead of row-major
@@ -362,7 +363,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
-        if (a.acc_out && n < N) *(i4*)(a.acc_out + (long)m * N + n) = acc[i][j];
+        if (a.acc_out && n < N) *(i4*)(a.acc_out + (long)m * a.ldacc + n) = acc[i][j];
         if (DT != MI355Q_F32 && wide && (i & 1) == 0 && i + 1 < NI) {
           typedef Elem<DT == MI355Q_F32 ? MI355Q_F16 : DT> E;
           float v0[4], v1[4];
@@ -543,18 +544,63 @@ int launch_tile(const I8Args& a, hipStream_t st) {
   return 0;
 }
 
-// Tile width: the one that wastes fewer tile slots in the last round of
-// workgroups over the CUs (time ~ rounds x tile width).
+// Columns [n0, n1) of the problem as a launch of its own (n0 a multiple of 128): the operand, scale,
+// bias and output pointers move to the first column, the row strides stay.
+template <int DT, int WM, int WN, int NI, int NJ>
+int launch_columns(const I8Args& a, int n0, int n1, hipStream_t st) {
+  I8Args b = a;
+  b.N = n1 - n0;
+  b.w = a.w + (size_t)n0 * (size_t)(a.w_kslab ? a.K : a.ldw);       // 64 kslab columns are K * 64 bytes too
+  if (a.w_scale && a.w_scale_per_col) b.w_scale = a.w_scale + n0;
+  if (a.bias) b.bias = (const char*)a.bias + (size_t)n0 * ((a.bias_f32 || DT == MI355Q_F32) ? 4 : 2);
+  b.out = (char*)a.out + (size_t)n0 * (DT == MI355Q_F32 ? 4 : 2);
+  if (a.acc_out) b.acc_out = a.acc_out + n0;
+  return launch_tile<DT, WM, WN, NI, NJ>(b, st);
+}
+
+// Tile width.  One workgroup per CU works through the output tiles in rounds; a last round that is
+// only part full idles the rest of the chip for a whole tile time.  Measured per round of 256 CUs on
+// K = 8192 (256 rows x TN columns per CU): TN = 256: 101 us, 224: 98.8 us, 128: 55 us -- the widest
+// tile is the cheapest per column.  So: as many FULL rounds of 256-wide tiles as the columns give, and
+// the remaining columns as a second launch with the width that wastes least (M 2048, N 28672: three
+// rounds of 256 and one of 128 instead of four of 224: 395 -> 387 us; under the profiler the two
+// launches last 315-337 us and 65-70 us, i.e. a round costs a little more when three follow each other
+// than the single-round figures above say).  A single width is kept where it is as good.
 template <int DT>
 int launch_gemm(const I8Args& a, hipStream_t st) {
   const long cus = device_cu_count(), mtiles = (a.M + TM - 1) / TM;
+  auto rounds = [&](long cols, long w) { return (mtiles * ((cols + w - 1) / w) + cus - 1) / cus; };
+  const double c256 = 1.0, c224 = 0.978, c128 = 0.545;            // cost of one round, relative
   const long t256 = mtiles * ((a.N + 255) / 256), t224 = mtiles * ((a.N + 223) / 224);
-  const long cost256 = (t256 + cus - 1) / cus * 256, cost224 = (t224 + cus - 1) / cus * 224;
   // a single row of tiles that leaves most CUs idle: tiles half as wide (the launch is bound by
   // the weight stream, which then comes in over twice as many CUs)
   const long t128 = mtiles * ((a.N + 127) / 128);
-  if (mtiles == 1 && (t224 < cost224 ? t224 : t256) * 3 <= cus * 2 && t128 > t224) return launch_tile<DT, 4, 2, 4, 4>(a, st);
-  if (cost224 < cost256) return launch_tile<DT, 4, 2, 7, 4>(a, st);
+  const long r224 = rounds(a.N, 224), r256 = rounds(a.N, 256);
+  if (mtiles == 1 && (t224 < r224 * 224 ? t224 : t256) * 3 <= cus * 2 && t128 > t224) return launch_tile<DT, 4, 2, 4, 4>(a, st);
+  double best = r224 * c224 < r256 * c256 ? r224 * c224 : r256 * c256;
+  int split = 0, tail_w = 0;
+  const long full = t256 / cus;                       // whole rounds of 256-wide tiles
+  if (full >= 1 && cus % mtiles == 0) {
+    const long ncols = full * (cus / mtiles) * 256;   // columns they cover
+    if (ncols < a.N) {
+      const long rest = a.N - ncols;
+      const double tails[3] = {rounds(rest, 128) * c128, rounds(rest, 224) * c224, rounds(rest, 256) * c256};
+      const int widths[3] = {128, 224, 256};
+      for (int i = 0; i < 3; ++i)
+        if (full * c256 + tails[i] < best - 0.05) {   // (a second launch has to pay for itself)
+          best = full * c256 + tails[i];
+          split = (int)ncols;
+          tail_w = widths[i];
+        }
+    }
+  }
+  if (split) {
+    if (int rc = launch_columns<DT, 2, 4, 4, 8>(a, 0, split, st)) return rc;
+    if (tail_w == 128) return launch_columns<DT, 4, 2, 4, 4>(a, split, a.N, st);
+    if (tail_w == 224) return launch_columns<DT, 4, 2, 7, 4>(a, split, a.N, st);
+    return launch_columns<DT, 2, 4, 4, 8>(a, split, a.N, st);
+  }
+  if (r224 * c224 < r256 * c256) return launch_tile<DT, 4, 2, 7, 4>(a, st);
   return launch_tile<DT, 2, 4, 4, 8>(a, st);
 }
 
@@ -581,7 +627,7 @@ extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* 
   MQ_REQUIRE(out_dtype >= MI355Q_F16 && out_dtype <= MI355Q_F32, "w8a8_int8_gemm: bad out dtype %d", out_dtype);
   I8Args a;
   a.out = out; a.acc_out = acc_out; a.x = x; a.w = w; a.x_scale = x_scale; a.w_scale = w_scale;
-  a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;
+  a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo; a.ldacc = N;
   a.x_scale_per_row = x_scale_per_row; a.w_scale_per_col = w_scale_per_col; a.bias_f32 = bias_f32;
   a.n_panels_swizzle = 0;
   a.w_kslab = kslab ? 1 : 0;
