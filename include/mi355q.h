@@ -87,7 +87,9 @@ int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight,
 /* tuning hook used by the benchmark.  split_k: bits 0..7 force the split-K
  * factor, bits 8..15 the tiles (of 16 columns) per workgroup of the streaming
  * kernel (1, 2, 4 or 8); 0 in a field = automatic.  family: 0 = auto,
- * 1 = streaming, 2 = LDS/MFMA. */
+ * 1 = streaming, 2 = MFMA tiles of 64 rows (32 x 64 below 129 rows on narrow
+ * layers), 3 = MFMA workgroups of up to 128 rows fed through a ring of LDS
+ * stages (fp16, group sizes that are multiples of 128). */
 int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          const void* scales, const void* zeros, int zeros_kind,
                          const void* bias, int M, int K, int N, int group_size,

@@ -367,6 +367,58 @@ def test_narrow_tiles_mid_rows(ops, rearrange, M, dtype):
     assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, 128, torch.float16)).to(torch.float16))
 
 
+# ------------------------------------------------ 128-row ring kernel (family 3) ----
+@pytest.mark.parametrize("M,K,N,g,split", [(128, 512, 256, 128, 1), (100, 1024, 384, 128, 1), (17, 512, 128, 128, 1),
+                                           (64, 2048, 512, 256, 0), (128, 4096, 512, 128, 0), (128, 1536, 256, 128, 3),
+                                           (48, 4096, 256, 128, 4), (130, 1024, 256, 128, 1), (300, 1024, 640, 128, 0),
+                                           (2048, 2048, 384, 128, 0)])
+def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split):
+    """The kernel that owns up to 128 rows per workgroup and streams K through a ring of LDS stages
+    (fp16; B operands are (q - z) * s rounded to fp16): ragged M, a half-empty last column tile, several
+    row blocks, K split with the separate reduction, groups of 256, bias; run-to-run identical; exact
+    inputs bit for bit (every scale a power of two, so the fp16 weights are exact)."""
+    print(f"case ring M={M} K={K} N={N} g={g} split={split}", flush=True)
+    q, z, s, x = make_case(M + K, M, K, N, g)
+    bias = np.random.default_rng(9).standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=3, split_k=split)
+    assert torch.equal(got, run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=3, split_k=split))
+    np.testing.assert_allclose(got.float().cpu().numpy(), oracle(q, z, s, x, g, torch.float16, bias=bias), rtol=RTOL, atol=ATOL)
+    q, z, s, x = make_case(5, M, K, N, g, exact=True)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=3, split_k=split)
+    assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16))
+
+
+@pytest.mark.parametrize("M", [32, 64, 128, 200])
+def test_ring_gemm_zero_kinds(ops, rearrange, M):
+    """No zero-points (z = 8) and the reference's pre-scaled fp16 zero-points, where the kernel forms
+    q * s - zs in one fused multiply-add: the oracle of that form is dequantize_prescaled_zeros."""
+    K, N, g = 1024, 384, 128
+    print(f"case ring zero kinds M={M}", flush=True)
+    q, z, s, x = make_case(M + 1, M, K, N, g)
+    w, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
+    xs = to_act(x, torch.float16).cuda()
+    out = ops.w4a16_gemm(xs, w, to_act(s, torch.float16).cuda(), None, None, g, family=3)
+    np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, None, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)
+    s16 = s.astype(np.float16)
+    zs = (z.astype(np.float32) * s16.astype(np.float32)).astype(np.float16)
+    out = ops.w4a16_gemm(xs, w, dev(s16), dev(zs), None, g, family=3)
+    want = to_act(x, torch.float16).float().numpy() @ ow4.dequantize_prescaled_zeros(q, zs, s16, g)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_ring_gemm_is_fp16_only_and_tile_family_still_forced(ops, rearrange):
+    M, K, N, g = 160, 512, 256, 128
+    q, z, s, x = make_case(8, M, K, N, g)
+    with pytest.raises(RuntimeError, match="fp16"):
+        run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, family=3)
+    # family 2 keeps meaning the 64-row tile kernel; both agree with the oracle
+    a = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=2).float().cpu().numpy()
+    b = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=3).float().cpu().numpy()
+    want = oracle(q, z, s, x, g, torch.float16)
+    np.testing.assert_allclose(a, want, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(b, want, rtol=RTOL, atol=ATOL)
+
+
 def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):
     M, K, N, g = 150, 256, 128, 64
     q, z, s, x = make_case(5, M, K, N, g)

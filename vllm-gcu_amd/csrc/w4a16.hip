@@ -13,8 +13,12 @@ size_t w4a16_stream_workspace_bytes(int M, int N);
 size_t w4a16_stream_plan_workspace_bytes(int M, int K, int N, int gs);
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
-                      int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
+                      int group_size, int dtype, void* workspace, size_t workspace_bytes, bool allow_ring,
+                      hipStream_t st);
 size_t w4a16_tile_workspace_bytes(int M, int K, int N);
+int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
+                     int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
+                     void* workspace, size_t workspace_bytes, int splits, hipStream_t st);
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -79,7 +83,8 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
   MQ_REQUIRE(zeros_kind >= MI355Q_ZP_NONE && zeros_kind <= MI355Q_ZP_PRESCALED,
              "w4a16_gemm: unknown zeros_kind %d", zeros_kind);
   MQ_REQUIRE(zeros_kind == MI355Q_ZP_NONE || zeros, "w4a16_gemm: zeros pointer missing");
-  MQ_REQUIRE(family >= 0 && family <= 2, "w4a16_gemm: unknown kernel family %d", family);
+  MQ_REQUIRE(family >= 0 && family <= 3, "w4a16_gemm: unknown kernel family %d", family);
+  const int caller_family = family;       // 0: the library chooses, also between the two MFMA kernels
   if (family == 0) family = auto_family(M, group_size, zeros_kind, dtype);
   MQ_REQUIRE(family != 2 || group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
@@ -99,9 +104,13 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
     return 0;
   }
   const bool ws_ok = workspace && workspace_bytes > TILE_WS_OFFSET;
+  if (family == 3)
+    return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
+                            ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,
+                            ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, split_k & 0xff, as_stream(stream));
   return w4a16_tile_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
                            ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,
-                           ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, as_stream(stream));
+                           ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, caller_family == 0, as_stream(stream));
 }
 
 extern "C" int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight, const void* scales,

@@ -1,0 +1,413 @@
+// W4A16 MFMA GEMM for a few dozen to 128 rows on gfx950: every weight is read from HBM once.
+//
+// At these heights a layer is neither a pure stream (the matrix pipes matter) nor a tile problem (each
+// weight tile meets one block of rows only, so nothing is ever re-read from the L2 and the latency of
+// HBM is in the open).  One workgroup per CU owns all rows of a block (16 MT, up to 128) of 256 columns
+// and walks K (or its share of K) in blocks of 128.  Everything a K block needs -- the activation rows,
+// the packed weights, the group scales and zero-points -- is copied from global memory straight into a
+// ring of LDS stages (global_load_lds, 16 B per lane, no staging registers) several K blocks ahead; the
+// ring is the latency cover that a second workgroup per CU provides in the tile kernel.  Each of the
+// eight wavefronts (two per SIMD: one wavefront alone issues an instruction every five or six clocks,
+// too few for the matrix pipe) dequantises the weights of its 32 columns once per K block into MFMA B
+// operands, scaled: (q - z) * s rounded to fp16, which is the dequantised weight the operator is
+// defined on -- and feeds them to all row tiles, accumulating in place.  No weight is dequantised twice.
+//
+// The copies are issued from inline assembly, so the compiler does not know of them: it schedules and
+// waits for the LDS reads itself (lgkmcnt), and the waits for the copies (vmcnt) are written by hand.
+// No load that the compiler can see is in flight while a copy is (prologue and epilogue drain first).
+#include "common.h"
+
+namespace mi355q {
+
+int w4a16_splitk_reduce_launch(void* out, const float* partial, const void* bias, int M, int N, int splits,
+                               int dtype, hipStream_t st);
+
+namespace {
+
+struct MidArgs {
+  uint16_t* out;
+  const uint16_t* x;
+  const u4* qw;
+  const uint16_t* scales;
+  const void* zeros;
+  const uint16_t* bias;
+  int M, K, N;
+  int kper;                   // K blocks per split (blockIdx.z)
+  uint32_t gpk, gpk_magic;    // K blocks per group and ceil(2^32 / gpk)
+  float* partial;             // split K: fp32 tiles [split][M][N]; null: write the output
+};
+
+template <int MT>
+struct MidCfg {
+  static constexpr int BM = 16 * MT;
+  static constexpr int A_BYTES = BM * 256;            // 128 halves per row
+  static constexpr int W_OFF = A_BYTES;               // 8 wavefronts x 2 column tiles x 1 KiB
+  static constexpr int SZ_OFF = A_BYTES + 16384;      // 8 wavefronts x (256 B of scales + 256 B of zero-points)
+  static constexpr int STAGE = A_BYTES + 16384 + 4096;
+  static constexpr int D = MT >= 8 ? 3 : MT >= 4 ? 4 : 5;   // stages in the ring
+  static constexpr int XC = MT >= 2 ? MT / 2 : 1;     // activation copies (4 rows each) per wavefront and stage
+};
+
+// 64 lanes x 16 B from saddr + voff into LDS at lds_addr + 16 * lane
+__device__ __forceinline__ void dma16(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(sbase), "s"(lds_addr)
+               : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+struct MidDq {
+  uint32_t magic, mlo, mhi;
+};
+
+// Pair p (0..3) of one packed word -> two of the 8 weights of an MFMA K step, (q - z) * s in fp16,
+// as the 32-bit word p of the B operand.  zlo = 1024 + z, zhi = 64 + z (PRESCALED: 1024 and 64, and
+// zs = z * s is subtracted after the scaling).  Three or four instructions: the K loop deals them out
+// between the matrix instructions instead of dequantising an operand in one burst.
+template <int ZK>
+__device__ __forceinline__ uint32_t mid_dequant_pair(uint32_t w, int p, _Float16 zlo1, _Float16 zhi1, _Float16 s1,
+                                                     _Float16 zs1, const MidDq& k) {
+  const h2 zlo = {zlo1, zlo1}, zhi = {zhi1, zhi1}, ss = {s1, s1}, zs = {zs1, zs1};
+  const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const uint32_t ws = (p & 2) ? w >> 8 : w;
+  h2 r;
+  if (p & 1) {
+    const h2 a = bitcast<h2>((ws & k.mhi) | k.magic);  // 1024 + 16 q
+    r = __builtin_elementwise_fma(a, sixteenth, -zhi);
+  } else {
+    const h2 a = bitcast<h2>((ws & k.mlo) | k.magic);  // 1024 + q
+    r = a - zlo;
+  }
+  if (ZK == MI355Q_ZP_PRESCALED) r = __builtin_elementwise_fma(r, ss, -zs);
+  else r *= ss;
+  return bitcast<uint32_t>(r);
+}
+
+template <int ZK, int MT>
+__global__ void __launch_bounds__(512, 1)
+w4a16_mid_kernel(MidArgs a) {
+  typedef MidCfg<MT> C;
+  constexpr int D = C::D, STAGE = C::STAGE, XC = C::XC;
+  constexpr bool HASZ = ZK != MI355Q_ZP_NONE;
+  constexpr int NSLOT = XC + 3;                       // copy slots per wavefront and stage (the last: scales + zeros)
+  constexpr int NC = XC + 3 + (HASZ ? 1 : 0);         // copy instructions per wavefront and stage
+  static_assert((D - 1) * NC <= 63, "vmcnt is a 6-bit counter");
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, kq = lane >> 4;
+  const int N = a.N, K = a.K, M = a.M, G = K >> 7;
+  const int m0 = blockIdx.y * C::BM;
+  // N may end in the middle of the 256-column tile: the two wavefronts of the missing slab work on the
+  // previous one and skip the epilogue
+  const bool live = (blockIdx.x * 2 + (wave >> 2)) < (N >> 7);
+  const int slab = live ? blockIdx.x * 2 + (wave >> 2) : (N >> 7) - 1;
+  const int t0 = (wave & 3) * 2;
+  const int ncol = 128 * slab + 8 * c + t0;           // first of this lane's 2 adjacent columns
+  const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
+  const uint32_t lds_base =
+      __builtin_amdgcn_readfirstlane((uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds);
+
+  // ---- copies.  Activations: one copy moves 4 rows of 256 B; lane = 16 * row + position, and position p
+  // of row r receives the row's 16-byte chunk p ^ (r & 15), which keeps the MFMA operand reads (16 rows x
+  // one chunk index per quarter wavefront) on 16 different bank groups.  Wavefront v copies row groups
+  // v, v + 8, ...; rows past M re-read the last row (their results are never stored).
+  uint32_t xo[XC];
+#pragma unroll
+  for (int p = 0; p < XC; ++p) {
+    const int r = 4 * (wave + 8 * p) + (lane >> 4);
+    const int row = min(m0 + r, M - 1);
+    xo[p] = ((uint32_t)row * (uint32_t)K + 8u * (uint32_t)((lane & 15) ^ (r & 15))) * 2u;
+  }
+  const uint32_t lane16 = (uint32_t)lane * 16u;
+  const uint32_t zlane = ZK == MI355Q_ZP_PACKED ? (uint32_t)(lane & 3) * 16u : lane16;
+  const char* const xg = (const char*)a.x;
+  const char* const wg = (const char*)a.qw + ((size_t)slab * G * 8 + t0) * 1024;
+  const char* const sg = (const char*)a.scales + 256 * slab;
+  const char* const zg = (const char*)a.zeros + (ZK == MI355Q_ZP_PACKED ? 64 : 256) * slab;
+  const uint32_t zrow = ZK == MI355Q_ZP_PACKED ? (uint32_t)N / 2u : (uint32_t)N * 2u;
+  // The workgroups of one split start together and stay roughly in step, and K block g of every
+  // activation row lies a multiple of 8 KiB (Llama shapes) from that of the next: all of them would ask
+  // the same few L2 channels for the same bytes at the same time.  Each column tile therefore walks its K
+  // range from a different starting block (and wraps round): iteration i is K block gb + (rot + i) % nk.
+  const int nk = ge - gb;
+  const int rot = (int)(blockIdx.x % (unsigned)nk);
+  auto copy_slot = [&](int s, int slot, int i) {
+    const uint32_t sb = lds_base + (uint32_t)(slot * STAGE);
+    int gq = rot + min(i, nk - 1);                    // past the end: a re-read into a stage nobody reads
+    gq = gb + (gq >= nk ? gq - nk : gq);
+    if (s < XC) {
+      dma16(xo[s < XC ? s : 0], xg + (size_t)gq * 256, sb + (uint32_t)((wave + 8 * s) * 1024));
+    } else if (s < XC + 2) {
+      const int t = s - XC;
+      dma16(lane16, wg + (size_t)gq * 8192 + t * 1024, sb + (uint32_t)(C::W_OFF + wave * 2048 + t * 1024));
+    } else {
+      const uint32_t qrow = a.gpk_magic ? (uint32_t)(((uint64_t)(uint32_t)gq * a.gpk_magic) >> 32) : (uint32_t)gq;
+      if (lane < 16) {
+        dma16(lane16, sg + (size_t)qrow * N * 2, sb + (uint32_t)(C::SZ_OFF + wave * 512));
+        if (HASZ) dma16(zlane, zg + (size_t)qrow * zrow, sb + (uint32_t)(C::SZ_OFF + wave * 512 + 256));
+      }
+    }
+  };
+
+  // ---- LDS reads (plain loads: the compiler places the waits)
+  const uint32_t a_lane = (uint32_t)(c * 256);
+  uint32_t a_pos[4];
+#pragma unroll
+  for (int st = 0; st < 4; ++st) a_pos[st] = a_lane + (uint32_t)(((4 * st + kq) ^ c) * 16);
+  auto read_a = [&](int slot, int mt, int st) {
+    return bitcast<h8>(*(const u4*)(lds + slot * STAGE + a_pos[st] + mt * 4096));
+  };
+  auto read_w = [&](u4 (&w)[2], int slot) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) w[t] = *(const u4*)(lds + slot * STAGE + C::W_OFF + wave * 2048 + t * 1024 + lane * 16);
+  };
+  struct Sz { uint32_t s; uint32_t zs; uint32_t z; };
+  auto read_sz = [&](Sz& q, int slot) {
+    const unsigned char* p = lds + slot * STAGE + C::SZ_OFF + wave * 512;
+    q.s = *(const uint32_t*)(p + (8 * c + t0) * 2);
+    if (ZK == MI355Q_ZP_PACKED) q.z = *(const uint32_t*)(p + 256 + c * 4) >> (4 * t0);
+    if (ZK == MI355Q_ZP_PRESCALED) q.zs = *(const uint32_t*)(p + 256 + (8 * c + t0) * 2);
+  };
+  // per column tile: scale, 1024 + z, 64 + z, z * s
+  _Float16 sc[2], zlo[2], zhi[2], zsc[2];
+  auto prep = [&](const Sz& q) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const uint32_t sw = q.s;
+      sc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+      if (ZK == MI355Q_ZP_PRESCALED) {
+        const uint32_t zw = q.zs;
+        zsc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu)));
+        zlo[t] = (_Float16)1024.0f;
+        zhi[t] = (_Float16)64.0f;
+      } else {
+        // fp16 bit patterns directly: 1024 + z = 0x6400 | z, 64 + z = 0x5400 | z << 4
+        const uint32_t z = ZK == MI355Q_ZP_PACKED ? (q.z >> (4 * t)) & 15u : 8u;
+        zlo[t] = bitcast<_Float16>((uint16_t)(0x6400u | z));
+        zhi[t] = bitcast<_Float16>((uint16_t)(0x5400u | (z << 4)));
+        zsc[t] = (_Float16)0.0f;
+      }
+    }
+  };
+  MidDq dqk = {0x64006400u, 0x000f000fu, 0x00f000f0u};
+  asm volatile("" : "+v"(dqk.magic));
+  asm volatile("" : "+s"(dqk.mlo));
+  asm volatile("" : "+s"(dqk.mhi));
+
+  f4 acc[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  // ---- prologue: the whole ring is requested, the first stage awaited
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+#pragma unroll
+    for (int s = 0; s < NSLOT; ++s) copy_slot(s, d, d);
+  wait_vmcnt<(D - 1) * NC>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  u4 w0[2], w1[2];
+  Sz sz;
+  h8 av[2][MT];
+  u4 bv[2][2];
+  read_w(w0, 0);
+  read_sz(sz, 0);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) av[0][mt] = read_a(0, mt, 0);
+  prep(sz);
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int p = 0; p < 4; ++p) bv[0][t][p] = mid_dequant_pair<ZK>(w0[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
+
+  constexpr int PPG = 8 / MT;                         // operand words (of 2 tiles x 4) dequantised per row-tile group
+  constexpr int CPG = (NSLOT + MT - 1) / MT;          // copy slots issued per row-tile group
+  int slot = 0;
+  // One K block: four K steps of MT groups of two matrix instructions.  While step st multiplies, the
+  // A operands of step st + 1 are read and its B operands dequantised, one operand and 8 / MT words per group.  In step 2 the
+  // wavefront's own copies of the next stage are awaited and its packed weights and scales read; at the
+  // top of step 3 every LDS read of this stage has been issued and awaited, so after the barrier there the
+  // stage is refilled with K block g + D while the first operands of block g + 1 are fetched.
+  auto kblock = [&](int i, u4 (&wc)[2], u4 (&wn)[2]) {
+    const int nslot = slot + 1 == D ? 0 : slot + 1;
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      const int cur = st & 1, nxt = cur ^ 1;
+      if (st == 2) {
+        wait_vmcnt<(D - 2) * NC>();
+        read_w(wn, nslot);
+        read_sz(sz, nslot);
+      }
+      if (st == 3) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        prep(sz);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        // a matrix instruction occupies its pipe for four issue slots: the other work of the group goes
+        // into the slots behind each of the two
+        acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][0]), acc[mt][0], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        av[nxt][mt] = st < 3 ? read_a(slot, mt, st + 1) : read_a(nslot, mt, 0);
+        if (st == 3) {
+#pragma unroll
+          for (int s = mt * CPG; s < (mt + 1) * CPG && s < NSLOT; ++s) copy_slot(s, slot, i + D);
+        }
+#pragma unroll
+        for (int q = mt * PPG; q < mt * PPG + (PPG + 1) / 2; ++q) {
+          const int t = q >> 2, p = q & 3;
+          bv[nxt][t][p] = mid_dequant_pair<ZK>(st < 3 ? wc[t][st + 1] : wn[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][1]), acc[mt][1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = mt * PPG + (PPG + 1) / 2; q < (mt + 1) * PPG; ++q) {
+          const int t = q >> 2, p = q & 3;
+          bv[nxt][t][p] = mid_dequant_pair<ZK>(st < 3 ? wc[t][st + 1] : wn[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    slot = nslot;
+  };
+  for (int i = 0;; i += 2) {
+    kblock(i, w0, w1);
+    if (i + 1 >= nk) break;
+    kblock(i + 1, w1, w0);
+    if (i + 2 >= nk) break;
+  }
+  // no copy may still be writing LDS when the workgroup retires, and none may be in flight next to the
+  // loads below
+  wait_vmcnt<0>();
+
+  // ---- epilogue through LDS (the ring is free now): a lane holds 2 adjacent columns of 4 rows per
+  // row tile, which as stores would touch 8 bytes in every 32; written to an fp32 tile in LDS and read
+  // back row by row, every store instruction writes one whole row of the 256-column tile.
+  constexpr int EP = 1024 + 16;                        // bytes per tile row in LDS
+  static_assert(C::BM * EP <= D * STAGE, "the output tile fits in the ring");
+  __syncthreads();                                     // every wavefront has left the K loop
+  {
+    unsigned char* base = lds + (128 * (wave >> 2) + 8 * c + t0) * 4;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *(f2*)(base + (mt * 16 + 4 * kq + i) * EP) = (f2){acc[mt][0][i], acc[mt][1][i]};
+  }
+  __syncthreads();
+  const int col = blockIdx.x * 256 + 4 * lane;         // this lane's 4 columns of every row
+  if (col >= N) return;
+  f4 bs = {0.f, 0.f, 0.f, 0.f};
+  if (a.bias && !a.partial) {
+    const uint2 bw = *(const uint2*)(a.bias + col);
+    bs = (f4){Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x >> 16)),
+              Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y >> 16))};
+  }
+#pragma unroll
+  for (int p = 0; p < 2 * MT; ++p) {
+    const int r = wave + 8 * p, m = m0 + r;
+    if (m >= M) break;
+    const f4 v = *(const f4*)(lds + r * EP + lane * 16);
+    if (a.partial) {
+      *(f4*)(a.partial + ((size_t)blockIdx.z * M + m) * N + col) = v;
+    } else {
+      uint2 o;
+      o.x = (uint32_t)Elem<MI355Q_F16>::from_f32(v[0] + bs[0]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[1] + bs[1]) << 16);
+      o.y = (uint32_t)Elem<MI355Q_F16>::from_f32(v[2] + bs[2]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[3] + bs[3]) << 16);
+      *(uint2*)(a.out + (size_t)m * N + col) = o;
+    }
+  }
+}
+
+template <int ZK, int MT>
+int launch_mid(const MidArgs& a, int row_blocks, int splits, hipStream_t st) {
+  typedef MidCfg<MT> C;
+  const size_t shmem = (size_t)C::D * C::STAGE;
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_mid_kernel<ZK, MT>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  MQ_REQUIRE(attr == hipSuccess, "w4a16_gemm(mid): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
+  dim3 grid((a.N + 255) / 256, row_blocks, splits);
+  hipLaunchKernelGGL((w4a16_mid_kernel<ZK, MT>), grid, dim3(512), shmem, st, a);
+  MQ_LAUNCH_CHECK("w4a16_gemm(mid)");
+  return 0;
+}
+
+template <int ZK>
+int launch_mid_mt(const MidArgs& a, int mt, int row_blocks, int splits, hipStream_t st) {
+  if (mt <= 2) return launch_mid<ZK, 2>(a, row_blocks, splits, st);
+  if (mt <= 4) return launch_mid<ZK, 4>(a, row_blocks, splits, st);
+  return launch_mid<ZK, 8>(a, row_blocks, splits, st);
+}
+
+}  // namespace
+
+// Row tiles of 16 per workgroup for M rows: the smallest of 2, 4, 8 that holds them all, 8 beyond.
+static int mid_rows_mt(int M) { return M <= 32 ? 2 : M <= 64 ? 4 : 8; }
+
+// K splits: as many as still fit the chip in one round (one workgroup per CU), each at least four K
+// blocks long and the partial tiles within 64 MiB.
+int w4a16_mid_splits(int M, int K, int N) {
+  const int mt = mid_rows_mt(M), G = K / 128;
+  const long wgs = (long)((M + 16 * mt - 1) / (16 * mt)) * ((N + 255) / 256);
+  const long cus = device_cu_count();
+  long s = cus / wgs;
+  if (s > G / 4) s = G / 4;
+  while (s > 1 && (size_t)s * M * N * sizeof(float) > ((size_t)64 << 20)) --s;
+  if (s < 1) s = 1;
+  const int kper = (int)((G + s - 1) / s);
+  return (G + kper - 1) / kper;
+}
+
+size_t w4a16_mid_workspace_bytes(int M, int K, int N) {
+  const int s = w4a16_mid_splits(M, K, N);
+  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+
+// fp16 activations, group sizes that are multiples of 128.  `splits` 0: the plan above.
+int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
+                     int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
+                     void* workspace, size_t workspace_bytes, int splits, hipStream_t st) {
+  MQ_REQUIRE(dtype == MI355Q_F16 && group_size % 128 == 0,
+             "w4a16_gemm(mid): fp16 and group sizes that are multiples of 128 only (dtype %d, group %d)", dtype, group_size);
+  MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
+  const int G = K / 128;
+  if (splits <= 0) splits = w4a16_mid_splits(M, K, N);
+  if (splits > G) splits = G;
+  if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * M * N * sizeof(float))) splits = 1;
+  MidArgs a = {};
+  a.out = (uint16_t*)out;
+  a.x = (const uint16_t*)x;
+  a.qw = (const u4*)qweight;
+  a.scales = (const uint16_t*)scales;
+  a.zeros = zeros;
+  a.bias = (const uint16_t*)bias;
+  a.M = M; a.K = K; a.N = N;
+  a.kper = (G + splits - 1) / splits;
+  splits = (G + a.kper - 1) / a.kper;                  // no empty splits
+  a.gpk = (uint32_t)group_size / 128u;
+  a.gpk_magic = a.gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + a.gpk - 1) / a.gpk) : 0u;
+  a.partial = splits > 1 ? (float*)workspace : nullptr;
+  const int mt = mid_rows_mt(M);
+  const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
+  int rc;
+  if (zeros_kind == MI355Q_ZP_NONE) rc = launch_mid_mt<MI355Q_ZP_NONE>(a, mt, row_blocks, splits, st);
+  else if (zeros_kind == MI355Q_ZP_PACKED) rc = launch_mid_mt<MI355Q_ZP_PACKED>(a, mt, row_blocks, splits, st);
+  else rc = launch_mid_mt<MI355Q_ZP_PRESCALED>(a, mt, row_blocks, splits, st);
+  if (rc) return rc;
+  if (splits > 1) return w4a16_splitk_reduce_launch(out, (const float*)workspace, bias, M, N, splits, dtype, st);
+  return 0;
+}
+
+}  // namespace mi355q

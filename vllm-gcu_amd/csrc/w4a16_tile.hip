@@ -763,6 +763,21 @@ hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStrea
 
 }  // namespace
 
+// sum of the fp32 partial tiles of a dense split-K launch into the output (+ bias), in split order
+int w4a16_splitk_reduce_launch(void* out, const float* partial, const void* bias, int M, int N, int splits,
+                               int dtype, hipStream_t st) {
+  const long MN = (long)M * N;
+  const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
+  if (dtype == MI355Q_F16)
+    hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out, partial,
+                       (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
+  else
+    hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out, partial,
+                       (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
+  MQ_LAUNCH_CHECK("w4a16_gemm(split-K reduce)");
+  return 0;
+}
+
 // split-K plan for grids that leave most of the chip idle: as many splits as
 // bring the grid to about one workgroup per CU, at least 4 K blocks each, and
 // partial tiles of at most TILE_SPLITK_BYTES in total
@@ -812,18 +827,58 @@ static int tile_narrow_splits(int M, int K, int N) {
   if (s > K / 128 / 4) s = K / 128 / 4;
   return s < 1 ? 1 : (int)s;
 }
+int w4a16_mid_splits(int M, int K, int N);
+int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
+                     int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
+                     void* workspace, size_t workspace_bytes, int splits, hipStream_t st);
+
+// Above 128 rows two kernels can take a dense fp16 layer: the 64-row tiles of this file, two workgroups
+// per CU, or the 128-row workgroups with the LDS ring (w4a16_mid.hip), one per CU.  A full round of either
+// covers the same rows; the ring kernel's is about a tenth shorter, but which of them leaves the
+// emptier last round depends on the shape.  Both are priced in microseconds per K block from what was
+// measured on Llama-shaped layers (full rounds: 2.05 for a pair of 64-row tiles sharing a CU, 1.85 for
+// a 128-row workgroup; a last round that leaves workgroups alone on their CUs: 1.2, respectively 1.6
+// when at most half the CUs are busy), plus a reduction launch when K is split.  The ring kernel is
+// taken when it is priced 5 % or more below the tiles: over 112 measured (shape, M) points that rule
+// is within 4 % of the better kernel everywhere and 0.2 % on average.
+static double tile_time_model(int M, int K, int N) {
+  const long cus = device_cu_count(), G = K / 128;
+  const int s = tile_splits(M, K, N);
+  const long wgs = (long)((M + 63) / 64) * ((N + BN - 1) / BN) * s, kper = (G + s - 1) / s;
+  const long full = wgs / (2 * cus), rest = wgs - full * 2 * cus;
+  return (double)kper * (full * 2.05 + (rest == 0 ? 0.0 : rest <= cus ? 1.2 : 2.05)) + (s > 1 ? 6.0 : 0.0) + 5.0;
+}
+static double mid_time_model(int M, int K, int N) {
+  const long cus = device_cu_count(), G = K / 128;
+  const int s = w4a16_mid_splits(M, K, N);
+  const long wgs = (long)((M + 127) / 128) * ((N + 255) / 256) * s, kper = (G + s - 1) / s;
+  const long full = wgs / cus, rest = wgs - full * cus;
+  return (double)kper * (full * 1.85 + (rest == 0 ? 0.0 : rest * 2 <= cus ? 1.6 : 1.85)) + (s > 1 ? 6.0 : 0.0) + 6.0;
+}
+static bool tile_prefers_ring(int M, int K, int N) {
+  return M > 128 && mid_time_model(M, K, N) < 0.95 * tile_time_model(M, K, N);
+}
+
 size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
+  // (the choice between the kernels also depends on the dtype and the group size, which this
+  // function does not see: room for whichever plan is larger)
   const int narrow = tile_narrow_splits(M, K, N);
   const int s = narrow ? narrow : tile_splits(M, K, N);
-  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+  const int sr = tile_prefers_ring(M, K, N) ? w4a16_mid_splits(M, K, N) : 1;
+  const int m = s > sr ? s : sr;
+  return m > 1 ? (size_t)m * M * N * sizeof(float) : 0;
 }
 
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
-                      int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
+                      int group_size, int dtype, void* workspace, size_t workspace_bytes, bool allow_ring,
+                      hipStream_t st) {
   MQ_REQUIRE(group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
+  if (allow_ring && dtype == MI355Q_F16 && tile_prefers_ring(M, K, N))
+    return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
+                            workspace_bytes, 0, st);
   TileArgs a = {};
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;
@@ -858,17 +913,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                               : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
   MQ_REQUIRE(e == hipSuccess, "w4a16_gemm(tile): cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("w4a16_gemm(tile)");
-  if (splits > 1) {
-    const long MN = (long)M * N;
-    const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
-    if (dtype == MI355Q_F16)
-      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
-    else
-      hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
-    MQ_LAUNCH_CHECK("w4a16_gemm(split-K reduce)");
-  }
+  if (splits > 1) return w4a16_splitk_reduce_launch(out, (const float*)workspace, bias, M, N, splits, dtype, st);
   return 0;
 }
 
