@@ -23,7 +23,7 @@ def rounder(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("rows,K", [(1, 128), (7, 4096), (33, 7168), (3, 8)])
+@pytest.mark.parametrize("rows,K", [(1, 128), (7, 4096), (33, 7168), (3, 8), (5, 8192), (4, 8200), (3, 16384)])
 def test_rms_norm_and_fused_add_vs_oracle(ops, dtype, rows, K):
     print(f"case rms_norm {dtype} rows={rows} K={K}", flush=True)
     rng = np.random.default_rng(rows * 131 + K)
@@ -36,9 +36,12 @@ def test_rms_norm_and_fused_add_vs_oracle(ops, dtype, rows, K):
     torch.ops._C.rms_norm(out, xd, wd, 1e-6)
     want = onorm.rms_norm(x, w, 1e-6, act)
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
-    # at most one unit in the last place of the activation type apart (rsqrt vs 1 / sqrt)
+    # at most one unit in the last place of the activation type apart (rsqrt vs 1 / sqrt); a flip of the
+    # first rounding (x * rs) times a weight up to 1.5 can land two units away, seen on rows of 8200
     ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
-    assert np.all(np.abs(out.float().cpu().numpy() - want) <= ulp * np.maximum(np.abs(want), 2.0 ** -14) * 1.01)
+    diff = np.abs(out.float().cpu().numpy() - want)
+    assert np.all(diff <= 2 * ulp * np.maximum(np.abs(want), 2.0 ** -14) * 1.01)
+    assert np.mean(diff > ulp * np.maximum(np.abs(want), 2.0 ** -14) * 1.01) < 1e-3
     xin, res = xd.clone(), rd.clone()
     torch.ops._C.fused_add_rms_norm(xin, res, wd, 1e-6)
     want_o, want_z = onorm.fused_add_rms_norm(x, r, w, 1e-6, act)

@@ -318,10 +318,115 @@ rms_norm_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* resid
   }
 }
 
+// The same operator for rows of up to 8192 elements: the row (and the weight vector) is loaded once,
+// up to four 16-byte pieces per lane with all loads in flight together, and both passes run from
+// registers -- the loop version above waits for one piece at a time and reads the row twice.  Same
+// arithmetic in the same order per element; the sum of squares adds the lane's pieces in the same
+// order too, so the results are bit-identical.
+template <int DT, bool ADD, int QM>
+__global__ void __launch_bounds__(256)
+rms_norm_row_kernel(void* out, float* out_scales, const uint16_t* x, uint16_t* residual, const uint16_t* weight,
+                    const float* scale, float eps, int K, int gs) {
+  const long row = blockIdx.x;
+  const int chunks = K / 8;
+  const uint16_t* xr = x + row * K;
+  uint16_t* rr = ADD ? residual + row * K : nullptr;
+  __shared__ float red[4];
+  u4 xv[4], rv[4], wv[4];
+  bool live[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c0 = threadIdx.x + 256 * i;
+    live[i] = c0 < chunks;
+    const int c = live[i] ? c0 : 0;
+    xv[i] = *(const u4*)(xr + 8 * c);
+    if (ADD) rv[i] = *(const u4*)(rr + 8 * c);
+    wv[i] = *(const u4*)(weight + 8 * c);
+  }
+  float v[4][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    unpack8<DT>(xv[i], v[i]);
+    if (ADD) {
+      float r[8];
+      unpack8<DT>(rv[i], r);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = round_act<DT>(v[i][e] + r[e]);
+      if (live[i]) *(u4*)(rr + 8 * (threadIdx.x + 256 * i)) = pack8<DT>(v[i]);
+    }
+    if (live[i]) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+    }
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = (red[0] + red[1]) + (red[2] + red[3]);
+  const float rs = rsqrtf(ss / (float)K + eps);
+  float qs = 1.f;
+  if (QM == 1) qs = *scale;
+  if (QM == 3) qs = round_act<DT>(1.0f / *scale);
+  const int lpg = QM == 2 ? gs / 8 : 1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (256 * i >= chunks) break;                       // (uniform: every lane stays for the group shuffles)
+    const int c = threadIdx.x + 256 * i;
+    float w[8];
+    unpack8<DT>(wv[i], w);
+    float* y = v[i];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = round_act<DT>(round_act<DT>(y[e] * rs) * w[e]);
+    if (QM == 0) {
+      if (live[i]) *(u4*)((uint16_t*)out + row * K + 8 * c) = pack8<DT>(y);
+    } else if (QM == 1) {
+      float q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(y[e] / qs);
+      if (live[i]) *(u2*)((uint8_t*)out + row * K + 8 * c) = to_fp8x8(q);
+    } else if (QM == 2) {
+      float mx = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(y[e]));
+      if (!live[i]) mx = 0.f;
+      mx = lane_group_max(mx, lpg);
+      const float sg = fmaxf(mx, 1e-10f) / FP8_MAX;
+      const SharedDivisor by_sg(sg);
+      float q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(by_sg.div(y[e]));
+      if (live[i]) {
+        *(u2*)((uint8_t*)out + row * K + 8 * c) = to_fp8x8(q);
+        if ((c % lpg) == 0) out_scales[row * (K / gs) + c / lpg] = sg;
+      }
+    } else {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float a = fminf(fmaxf(__builtin_rintf(y[e] * qs), -128.f), 127.f);
+        float b = fminf(fmaxf(__builtin_rintf(y[4 + e] * qs), -128.f), 127.f);
+        lo |= ((uint32_t)(int)a & 0xffu) << (8 * e);
+        hi |= ((uint32_t)(int)b & 0xffu) << (8 * e);
+      }
+      if (live[i]) *(u2*)((uint8_t*)out + row * K + 8 * c) = (u2){lo, hi};
+    }
+  }
+}
+
 template <int DT, bool ADD>
 void launch_rms(int qm, long rows, hipStream_t st, void* out, float* out_scales, const uint16_t* x,
                 uint16_t* residual, const uint16_t* weight, const float* scale, float eps, int K, int gs) {
   const dim3 grid((unsigned)rows);
+  if (K <= 8192) {
+    switch (qm) {
+      case 0: hipLaunchKernelGGL((rms_norm_row_kernel<DT, ADD, 0>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+      case 1: hipLaunchKernelGGL((rms_norm_row_kernel<DT, ADD, 1>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+      case 2: hipLaunchKernelGGL((rms_norm_row_kernel<DT, ADD, 2>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+      default: hipLaunchKernelGGL((rms_norm_row_kernel<DT, ADD, 3>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
+    }
+    return;
+  }
   switch (qm) {
     case 0: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 0>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
     case 1: hipLaunchKernelGGL((rms_norm_kernel<DT, ADD, 1>), grid, dim3(256), 0, st, out, out_scales, x, residual, weight, scale, eps, K, gs); break;
