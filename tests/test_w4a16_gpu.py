@@ -372,12 +372,15 @@ def test_narrow_tiles_mid_rows(ops, rearrange, M, dtype):
                                            (64, 2048, 512, 256, 0), (128, 4096, 512, 128, 0), (128, 1536, 256, 128, 3),
                                            (48, 4096, 256, 128, 4), (130, 1024, 256, 128, 1), (300, 1024, 640, 128, 0),
                                            (2048, 2048, 384, 128, 0)])
-def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split):
+@pytest.mark.parametrize("tw", [2, 1])
+def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split, tw):
     """The kernel that owns up to 128 rows per workgroup and streams K through a ring of LDS stages
-    (fp16; B operands are (q - z) * s rounded to fp16): ragged M, a half-empty last column tile, several
-    row blocks, K split with the separate reduction, groups of 256, bias; run-to-run identical; exact
-    inputs bit for bit (every scale a power of two, so the fp16 weights are exact)."""
-    print(f"case ring M={M} K={K} N={N} g={g} split={split}", flush=True)
+    (fp16; B operands are (q - z) * s rounded to fp16), with two 16-column tiles per wavefront
+    (workgroups of 256 columns) and with one (128 columns): ragged M, a half-empty last column tile,
+    several row blocks, K split with the separate reduction, groups of 256, bias; run-to-run
+    identical; exact inputs bit for bit (every scale a power of two, so the fp16 weights are exact)."""
+    print(f"case ring M={M} K={K} N={N} g={g} split={split} tiles per wavefront={tw}", flush=True)
+    split |= tw << 8
     q, z, s, x = make_case(M + K, M, K, N, g)
     bias = np.random.default_rng(9).standard_normal(N).astype(np.float32)
     got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=3, split_k=split)
@@ -388,8 +391,9 @@ def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split):
     assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16))
 
 
+@pytest.mark.parametrize("tw", [2, 1])
 @pytest.mark.parametrize("M", [32, 64, 128, 200])
-def test_ring_gemm_zero_kinds(ops, rearrange, M):
+def test_ring_gemm_zero_kinds(ops, rearrange, M, tw):
     """No zero-points (z = 8) and the reference's pre-scaled fp16 zero-points, where the kernel forms
     q * s - zs in one fused multiply-add: the oracle of that form is dequantize_prescaled_zeros."""
     K, N, g = 1024, 384, 128
@@ -397,13 +401,29 @@ def test_ring_gemm_zero_kinds(ops, rearrange, M):
     q, z, s, x = make_case(M + 1, M, K, N, g)
     w, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
     xs = to_act(x, torch.float16).cuda()
-    out = ops.w4a16_gemm(xs, w, to_act(s, torch.float16).cuda(), None, None, g, family=3)
+    out = ops.w4a16_gemm(xs, w, to_act(s, torch.float16).cuda(), None, None, g, family=3, split_k=tw << 8)
     np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, None, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)
     s16 = s.astype(np.float16)
     zs = (z.astype(np.float32) * s16.astype(np.float32)).astype(np.float16)
-    out = ops.w4a16_gemm(xs, w, dev(s16), dev(zs), None, g, family=3)
+    out = ops.w4a16_gemm(xs, w, dev(s16), dev(zs), None, g, family=3, split_k=tw << 8)
     want = to_act(x, torch.float16).float().numpy() @ ow4.dequantize_prescaled_zeros(q, zs, s16, g)
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_mid_rows_take_the_ring_kernel_where_k_is_long(ops, rearrange):
+    """33..128 rows on a layer whose workgroups walk ten K blocks or more: the dispatcher takes the ring
+    kernel with 128-column workgroups and splits K four ways here (64 column tiles on 256 CUs).  Sampled
+    columns against the oracle, the forced 64-row tile kernel beside it, run-to-run identical."""
+    M, K, N, g = 96, 5120, 8192, 128
+    print(f"case ring auto M={M} K={K} N={N}", flush=True)
+    q, z, s, x = make_case(21, M, K, N, g)
+    bias = np.random.default_rng(3).standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias)
+    assert torch.equal(got, run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias))
+    want = oracle(q, z, s, x, g, torch.float16, bias=bias)
+    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    tile = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=2)
+    np.testing.assert_allclose(tile.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
 def test_ring_gemm_is_fp16_only_and_tile_family_still_forced(ops, rearrange):

@@ -18,7 +18,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
 size_t w4a16_tile_workspace_bytes(int M, int K, int N);
 int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
-                     void* workspace, size_t workspace_bytes, int splits, hipStream_t st);
+                     void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st);
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -107,7 +107,7 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
   if (family == 3)
     return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
                             ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,
-                            ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, split_k & 0xff, as_stream(stream));
+                            ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, split_k & 0xff, (split_k >> 8) & 0xff, as_stream(stream));
   return w4a16_tile_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
                            ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,
                            ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0, caller_family == 0, as_stream(stream));

@@ -1,16 +1,18 @@
-// W4A16 MFMA GEMM for a few dozen to 128 rows on gfx950: every weight is read from HBM once.
+// W4A16 MFMA GEMM in which every operand reaches the CU through a ring of LDS stages (fp16).
 //
-// At these heights a layer is neither a pure stream (the matrix pipes matter) nor a tile problem (each
-// weight tile meets one block of rows only, so nothing is ever re-read from the L2 and the latency of
-// HBM is in the open).  One workgroup per CU owns all rows of a block (16 MT, up to 128) of 256 columns
-// and walks K (or its share of K) in blocks of 128.  Everything a K block needs -- the activation rows,
-// the packed weights, the group scales and zero-points -- is copied from global memory straight into a
-// ring of LDS stages (global_load_lds, 16 B per lane, no staging registers) several K blocks ahead; the
-// ring is the latency cover that a second workgroup per CU provides in the tile kernel.  Each of the
-// eight wavefronts (two per SIMD: one wavefront alone issues an instruction every five or six clocks,
-// too few for the matrix pipe) dequantises the weights of its 32 columns once per K block into MFMA B
-// operands, scaled: (q - z) * s rounded to fp16, which is the dequantised weight the operator is
-// defined on -- and feeds them to all row tiles, accumulating in place.  No weight is dequantised twice.
+// One workgroup per CU owns all rows of a block (16 MT, up to 128) of 256 or 128 columns and walks K
+// (or its share of K) in blocks of 128.  Everything a K block needs -- the activation rows, the packed
+// weights, the group scales and zero-points -- is copied from global memory straight into a ring of LDS
+// stages (global_load_lds, 16 B per lane, no staging registers) several K blocks ahead; the ring is the
+// latency cover that a second workgroup per CU provides in the 64-row tile kernel.  Each of the eight
+// wavefronts (two per SIMD: one wavefront alone issues an instruction every five or six clocks, too
+// few for the matrix pipe) owns all row tiles of TW = 2 or 1 of the 16-column tiles: no weight is
+// dequantised twice.  B operands are scaled, (q - z) * s rounded to fp16 -- the dequantised weight the
+// operator is defined on -- so the matrix instructions accumulate in place.
+//
+// Two uses: above 128 rows (TW = 2, workgroups of 256 columns, row blocks in blockIdx.y) where a round
+// model prices it below the 64-row tiles, and from 33 to 128 rows (TW = 1, workgroups of 128 columns:
+// twice the workgroups, so K needs half the splits) where a workgroup walks ten K blocks or more.
 //
 // The copies are issued from inline assembly, so the compiler does not know of them: it schedules and
 // waits for the LDS reads itself (lgkmcnt), and the waits for the copies (vmcnt) are written by hand.
@@ -37,14 +39,17 @@ struct MidArgs {
   float* partial;             // split K: fp32 tiles [split][M][N]; null: write the output
 };
 
-template <int MT>
+// TW: 16-column tiles per wavefront -- 2: a workgroup of 256 columns; 1: of 128 columns (one slab), for
+// launches of up to 128 rows, where 256-column workgroups are too few to fill the chip without splitting K
+template <int MT, int TW>
 struct MidCfg {
   static constexpr int BM = 16 * MT;
+  static constexpr int BNW = 128 * TW;                // columns per workgroup
   static constexpr int A_BYTES = BM * 256;            // 128 halves per row
-  static constexpr int W_OFF = A_BYTES;               // 8 wavefronts x 2 column tiles x 1 KiB
-  static constexpr int SZ_OFF = A_BYTES + 16384;      // 8 wavefronts x (256 B of scales + 256 B of zero-points)
-  static constexpr int STAGE = A_BYTES + 16384 + 4096;
-  static constexpr int D = MT >= 8 ? 3 : MT >= 4 ? 4 : 5;   // stages in the ring
+  static constexpr int W_OFF = A_BYTES;               // 8 wavefronts x TW column tiles x 1 KiB
+  static constexpr int SZ_OFF = A_BYTES + 8192 * TW;  // 8 wavefronts x (256 B of scales + 256 B of zero-points)
+  static constexpr int STAGE = A_BYTES + 8192 * TW + 4096;
+  static constexpr int D = (160 * 1024 - 1024) / STAGE < 6 ? (160 * 1024 - 1024) / STAGE : 6;   // stages in the ring
   static constexpr int XC = MT >= 2 ? MT / 2 : 1;     // activation copies (4 rows each) per wavefront and stage
 };
 
@@ -88,14 +93,14 @@ __device__ __forceinline__ uint32_t mid_dequant_pair(uint32_t w, int p, _Float16
   return bitcast<uint32_t>(r);
 }
 
-template <int ZK, int MT>
+template <int ZK, int MT, int TW>
 __global__ void __launch_bounds__(512, 1)
 w4a16_mid_kernel(MidArgs a) {
-  typedef MidCfg<MT> C;
+  typedef MidCfg<MT, TW> C;
   constexpr int D = C::D, STAGE = C::STAGE, XC = C::XC;
   constexpr bool HASZ = ZK != MI355Q_ZP_NONE;
-  constexpr int NSLOT = XC + 3;                       // copy slots per wavefront and stage (the last: scales + zeros)
-  constexpr int NC = XC + 3 + (HASZ ? 1 : 0);         // copy instructions per wavefront and stage
+  constexpr int NSLOT = XC + TW + 1;                  // copy slots per wavefront and stage (the last: scales + zeros)
+  constexpr int NC = XC + TW + 1 + (HASZ ? 1 : 0);    // copy instructions per wavefront and stage
   static_assert((D - 1) * NC <= 63, "vmcnt is a 6-bit counter");
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -103,12 +108,12 @@ w4a16_mid_kernel(MidArgs a) {
   const int c = lane & 15, kq = lane >> 4;
   const int N = a.N, K = a.K, M = a.M, G = K >> 7;
   const int m0 = blockIdx.y * C::BM;
-  // N may end in the middle of the 256-column tile: the two wavefronts of the missing slab work on the
-  // previous one and skip the epilogue
-  const bool live = (blockIdx.x * 2 + (wave >> 2)) < (N >> 7);
-  const int slab = live ? blockIdx.x * 2 + (wave >> 2) : (N >> 7) - 1;
-  const int t0 = (wave & 3) * 2;
-  const int ncol = 128 * slab + 8 * c + t0;           // first of this lane's 2 adjacent columns
+  // N may end in the middle of a 256-column tile: the wavefronts of the missing slab work on the
+  // previous one and their columns are never stored
+  const int wslab = TW == 2 ? wave >> 2 : 0;          // slab of the workgroup this wavefront works on
+  const bool live = (blockIdx.x * TW + wslab) < (N >> 7);
+  const int slab = live ? blockIdx.x * TW + wslab : (N >> 7) - 1;
+  const int t0 = TW == 2 ? (wave & 3) * 2 : wave;     // first of this wavefront's TW tiles of the slab
   const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
   const uint32_t lds_base =
       __builtin_amdgcn_readfirstlane((uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds);
@@ -143,9 +148,9 @@ w4a16_mid_kernel(MidArgs a) {
     gq = gb + (gq >= nk ? gq - nk : gq);
     if (s < XC) {
       dma16(xo[s < XC ? s : 0], xg + (size_t)gq * 256, sb + (uint32_t)((wave + 8 * s) * 1024));
-    } else if (s < XC + 2) {
+    } else if (s < XC + TW) {
       const int t = s - XC;
-      dma16(lane16, wg + (size_t)gq * 8192 + t * 1024, sb + (uint32_t)(C::W_OFF + wave * 2048 + t * 1024));
+      dma16(lane16, wg + (size_t)gq * 8192 + t * 1024, sb + (uint32_t)(C::W_OFF + wave * 1024 * TW + t * 1024));
     } else {
       const uint32_t qrow = a.gpk_magic ? (uint32_t)(((uint64_t)(uint32_t)gq * a.gpk_magic) >> 32) : (uint32_t)gq;
       if (lane < 16) {
@@ -163,22 +168,24 @@ w4a16_mid_kernel(MidArgs a) {
   auto read_a = [&](int slot, int mt, int st) {
     return bitcast<h8>(*(const u4*)(lds + slot * STAGE + a_pos[st] + mt * 4096));
   };
-  auto read_w = [&](u4 (&w)[2], int slot) {
+  auto read_w = [&](u4 (&w)[TW], int slot) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) w[t] = *(const u4*)(lds + slot * STAGE + C::W_OFF + wave * 2048 + t * 1024 + lane * 16);
+    for (int t = 0; t < TW; ++t) w[t] = *(const u4*)(lds + slot * STAGE + C::W_OFF + wave * 1024 * TW + t * 1024 + lane * 16);
   };
   struct Sz { uint32_t s; uint32_t zs; uint32_t z; };
   auto read_sz = [&](Sz& q, int slot) {
     const unsigned char* p = lds + slot * STAGE + C::SZ_OFF + wave * 512;
-    q.s = *(const uint32_t*)(p + (8 * c + t0) * 2);
+    // (one tile per wavefront: t0 may be odd, the 32-bit read starts at the even column below it)
+    const int te = t0 & ~1;
+    q.s = *(const uint32_t*)(p + (8 * c + te) * 2) >> (16 * (t0 & 1));
     if (ZK == MI355Q_ZP_PACKED) q.z = *(const uint32_t*)(p + 256 + c * 4) >> (4 * t0);
-    if (ZK == MI355Q_ZP_PRESCALED) q.zs = *(const uint32_t*)(p + 256 + (8 * c + t0) * 2);
+    if (ZK == MI355Q_ZP_PRESCALED) q.zs = *(const uint32_t*)(p + 256 + (8 * c + te) * 2) >> (16 * (t0 & 1));
   };
   // per column tile: scale, 1024 + z, 64 + z, z * s
-  _Float16 sc[2], zlo[2], zhi[2], zsc[2];
+  _Float16 sc[TW], zlo[TW], zhi[TW], zsc[TW];
   auto prep = [&](const Sz& q) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < TW; ++t) {
       const uint32_t sw = q.s;
       sc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
       if (ZK == MI355Q_ZP_PRESCALED) {
@@ -200,11 +207,11 @@ w4a16_mid_kernel(MidArgs a) {
   asm volatile("" : "+s"(dqk.mlo));
   asm volatile("" : "+s"(dqk.mhi));
 
-  f4 acc[MT][2];
+  f4 acc[MT][TW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < 2; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < TW; ++t) acc[mt][t] = (f4){0.f, 0.f, 0.f, 0.f};
 
   // ---- prologue: the whole ring is requested, the first stage awaited
 #pragma unroll
@@ -214,21 +221,21 @@ w4a16_mid_kernel(MidArgs a) {
   wait_vmcnt<(D - 1) * NC>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  u4 w0[2], w1[2];
+  u4 w0[TW], w1[TW];
   Sz sz;
   h8 av[2][MT];
-  u4 bv[2][2];
+  u4 bv[2][TW];
   read_w(w0, 0);
   read_sz(sz, 0);
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) av[0][mt] = read_a(0, mt, 0);
   prep(sz);
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+  for (int t = 0; t < TW; ++t)
 #pragma unroll
     for (int p = 0; p < 4; ++p) bv[0][t][p] = mid_dequant_pair<ZK>(w0[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
 
-  constexpr int PPG = 8 / MT;                         // operand words (of 2 tiles x 4) dequantised per row-tile group
+  constexpr int NP = 4 * TW;                          // operand words dequantised per K step, dealt out over the MT groups
   constexpr int CPG = (NSLOT + MT - 1) / MT;          // copy slots issued per row-tile group
   int slot = 0;
   // One K block: four K steps of MT groups of two matrix instructions.  While step st multiplies, the
@@ -236,7 +243,7 @@ w4a16_mid_kernel(MidArgs a) {
   // wavefront's own copies of the next stage are awaited and its packed weights and scales read; at the
   // top of step 3 every LDS read of this stage has been issued and awaited, so after the barrier there the
   // stage is refilled with K block g + D while the first operands of block g + 1 are fetched.
-  auto kblock = [&](int i, u4 (&wc)[2], u4 (&wn)[2]) {
+  auto kblock = [&](int i, u4 (&wc)[TW], u4 (&wn)[TW]) {
     const int nslot = slot + 1 == D ? 0 : slot + 1;
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
@@ -256,7 +263,7 @@ w4a16_mid_kernel(MidArgs a) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         // a matrix instruction occupies its pipe for four issue slots: the other work of the group goes
-        // into the slots behind each of the two
+        // into the slots behind it
         acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][0]), acc[mt][0], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         av[nxt][mt] = st < 3 ? read_a(slot, mt, st + 1) : read_a(nslot, mt, 0);
@@ -265,19 +272,16 @@ w4a16_mid_kernel(MidArgs a) {
           for (int s = mt * CPG; s < (mt + 1) * CPG && s < NSLOT; ++s) copy_slot(s, slot, i + D);
         }
 #pragma unroll
-        for (int q = mt * PPG; q < mt * PPG + (PPG + 1) / 2; ++q) {
+        for (int q = 0; q < NP; ++q) {
+          if (q * MT / NP != mt) continue;             // word q belongs to group q * MT / NP
           const int t = q >> 2, p = q & 3;
           bv[nxt][t][p] = mid_dequant_pair<ZK>(st < 3 ? wc[t][st + 1] : wn[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
         }
         __builtin_amdgcn_sched_barrier(0);
-        acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][1]), acc[mt][1], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int q = mt * PPG + (PPG + 1) / 2; q < (mt + 1) * PPG; ++q) {
-          const int t = q >> 2, p = q & 3;
-          bv[nxt][t][p] = mid_dequant_pair<ZK>(st < 3 ? wc[t][st + 1] : wn[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
+        if (TW == 2) {
+          acc[mt][TW - 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][TW - 1]), acc[mt][TW - 1], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
     }
     slot = nslot;
@@ -295,19 +299,23 @@ w4a16_mid_kernel(MidArgs a) {
   // ---- epilogue through LDS (the ring is free now): a lane holds 2 adjacent columns of 4 rows per
   // row tile, which as stores would touch 8 bytes in every 32; written to an fp32 tile in LDS and read
   // back row by row, every store instruction writes one whole row of the 256-column tile.
-  constexpr int EP = 1024 + 16;                        // bytes per tile row in LDS
+  constexpr int EP = C::BNW * 4 + 16;                  // bytes per tile row in LDS
   static_assert(C::BM * EP <= D * STAGE, "the output tile fits in the ring");
   __syncthreads();                                     // every wavefront has left the K loop
   {
-    unsigned char* base = lds + (128 * (wave >> 2) + 8 * c + t0) * 4;
+    unsigned char* base = lds + (128 * wslab + 8 * c + t0) * 4;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        *(f2*)(base + (mt * 16 + 4 * kq + i) * EP) = (f2){acc[mt][0][i], acc[mt][1][i]};
+      for (int i = 0; i < 4; ++i) {
+        if (TW == 2) *(f2*)(base + (mt * 16 + 4 * kq + i) * EP) = (f2){acc[mt][0][i], acc[mt][TW - 1][i]};
+        else *(float*)(base + (mt * 16 + 4 * kq + i) * EP) = acc[mt][0][i];
+      }
   }
   __syncthreads();
-  const int col = blockIdx.x * 256 + 4 * lane;         // this lane's 4 columns of every row
+  // 4 columns per lane: a wavefront instruction covers one 256-column row or two 128-column rows
+  constexpr int LPR = C::BNW / 4, RPI = 64 / LPR;      // lanes per row, rows per instruction
+  const int col = blockIdx.x * C::BNW + 4 * (lane % LPR);
   if (col >= N) return;
   f4 bs = {0.f, 0.f, 0.f, 0.f};
   if (a.bias && !a.partial) {
@@ -316,10 +324,10 @@ w4a16_mid_kernel(MidArgs a) {
               Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y >> 16))};
   }
 #pragma unroll
-  for (int p = 0; p < 2 * MT; ++p) {
-    const int r = wave + 8 * p, m = m0 + r;
+  for (int p = 0; p < 2 * MT / RPI; ++p) {
+    const int r = RPI * (wave + 8 * p) + lane / LPR, m = m0 + r;
     if (m >= M) break;
-    const f4 v = *(const f4*)(lds + r * EP + lane * 16);
+    const f4 v = *(const f4*)(lds + r * EP + (lane % LPR) * 16);
     if (a.partial) {
       *(f4*)(a.partial + ((size_t)blockIdx.z * M + m) * N + col) = v;
     } else {
@@ -331,24 +339,29 @@ w4a16_mid_kernel(MidArgs a) {
   }
 }
 
-template <int ZK, int MT>
+template <int ZK, int MT, int TW>
 int launch_mid(const MidArgs& a, int row_blocks, int splits, hipStream_t st) {
-  typedef MidCfg<MT> C;
+  typedef MidCfg<MT, TW> C;
   const size_t shmem = (size_t)C::D * C::STAGE;
-  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_mid_kernel<ZK, MT>,
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_mid_kernel<ZK, MT, TW>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   MQ_REQUIRE(attr == hipSuccess, "w4a16_gemm(mid): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
-  dim3 grid((a.N + 255) / 256, row_blocks, splits);
-  hipLaunchKernelGGL((w4a16_mid_kernel<ZK, MT>), grid, dim3(512), shmem, st, a);
+  dim3 grid((a.N + C::BNW - 1) / C::BNW, row_blocks, splits);
+  hipLaunchKernelGGL((w4a16_mid_kernel<ZK, MT, TW>), grid, dim3(512), shmem, st, a);
   MQ_LAUNCH_CHECK("w4a16_gemm(mid)");
   return 0;
 }
 
 template <int ZK>
-int launch_mid_mt(const MidArgs& a, int mt, int row_blocks, int splits, hipStream_t st) {
-  if (mt <= 2) return launch_mid<ZK, 2>(a, row_blocks, splits, st);
-  if (mt <= 4) return launch_mid<ZK, 4>(a, row_blocks, splits, st);
-  return launch_mid<ZK, 8>(a, row_blocks, splits, st);
+int launch_mid_mt(const MidArgs& a, int mt, int tw, int row_blocks, int splits, hipStream_t st) {
+  if (tw == 1) {
+    if (mt <= 2) return launch_mid<ZK, 2, 1>(a, row_blocks, splits, st);
+    if (mt <= 4) return launch_mid<ZK, 4, 1>(a, row_blocks, splits, st);
+    return launch_mid<ZK, 8, 1>(a, row_blocks, splits, st);
+  }
+  if (mt <= 2) return launch_mid<ZK, 2, 2>(a, row_blocks, splits, st);
+  if (mt <= 4) return launch_mid<ZK, 4, 2>(a, row_blocks, splits, st);
+  return launch_mid<ZK, 8, 2>(a, row_blocks, splits, st);
 }
 
 }  // namespace
@@ -358,9 +371,9 @@ static int mid_rows_mt(int M) { return M <= 32 ? 2 : M <= 64 ? 4 : 8; }
 
 // K splits: as many as still fit the chip in one round (one workgroup per CU), each at least four K
 // blocks long and the partial tiles within 64 MiB.
-int w4a16_mid_splits(int M, int K, int N) {
-  const int mt = mid_rows_mt(M), G = K / 128;
-  const long wgs = (long)((M + 16 * mt - 1) / (16 * mt)) * ((N + 255) / 256);
+int w4a16_mid_splits(int M, int K, int N, int tw) {
+  const int mt = mid_rows_mt(M), G = K / 128, bn = 128 * tw;
+  const long wgs = (long)((M + 16 * mt - 1) / (16 * mt)) * ((N + bn - 1) / bn);
   const long cus = device_cu_count();
   long s = cus / wgs;
   if (s > G / 4) s = G / 4;
@@ -371,19 +384,20 @@ int w4a16_mid_splits(int M, int K, int N) {
 }
 
 size_t w4a16_mid_workspace_bytes(int M, int K, int N) {
-  const int s = w4a16_mid_splits(M, K, N);
+  const int s = w4a16_mid_splits(M, K, N, 2);
   return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
 }
 
 // fp16 activations, group sizes that are multiples of 128.  `splits` 0: the plan above.
 int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
-                     void* workspace, size_t workspace_bytes, int splits, hipStream_t st) {
+                     void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st) {
   MQ_REQUIRE(dtype == MI355Q_F16 && group_size % 128 == 0,
              "w4a16_gemm(mid): fp16 and group sizes that are multiples of 128 only (dtype %d, group %d)", dtype, group_size);
   MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
   const int G = K / 128;
-  if (splits <= 0) splits = w4a16_mid_splits(M, K, N);
+  if (tw != 1) tw = 2;
+  if (splits <= 0) splits = w4a16_mid_splits(M, K, N, tw);
   if (splits > G) splits = G;
   if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * M * N * sizeof(float))) splits = 1;
   MidArgs a = {};
@@ -402,9 +416,9 @@ int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const voi
   const int mt = mid_rows_mt(M);
   const int row_blocks = (M + 16 * mt - 1) / (16 * mt);
   int rc;
-  if (zeros_kind == MI355Q_ZP_NONE) rc = launch_mid_mt<MI355Q_ZP_NONE>(a, mt, row_blocks, splits, st);
-  else if (zeros_kind == MI355Q_ZP_PACKED) rc = launch_mid_mt<MI355Q_ZP_PACKED>(a, mt, row_blocks, splits, st);
-  else rc = launch_mid_mt<MI355Q_ZP_PRESCALED>(a, mt, row_blocks, splits, st);
+  if (zeros_kind == MI355Q_ZP_NONE) rc = launch_mid_mt<MI355Q_ZP_NONE>(a, mt, tw, row_blocks, splits, st);
+  else if (zeros_kind == MI355Q_ZP_PACKED) rc = launch_mid_mt<MI355Q_ZP_PACKED>(a, mt, tw, row_blocks, splits, st);
+  else rc = launch_mid_mt<MI355Q_ZP_PRESCALED>(a, mt, tw, row_blocks, splits, st);
   if (rc) return rc;
   if (splits > 1) return w4a16_splitk_reduce_launch(out, (const float*)workspace, bias, M, N, splits, dtype, st);
   return 0;

@@ -827,10 +827,10 @@ static int tile_narrow_splits(int M, int K, int N) {
   if (s > K / 128 / 4) s = K / 128 / 4;
   return s < 1 ? 1 : (int)s;
 }
-int w4a16_mid_splits(int M, int K, int N);
+int w4a16_mid_splits(int M, int K, int N, int tw);
 int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
-                     void* workspace, size_t workspace_bytes, int splits, hipStream_t st);
+                     void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st);
 
 // Above 128 rows two kernels can take a dense fp16 layer: the 64-row tiles of this file, two workgroups
 // per CU, or the 128-row workgroups with the LDS ring (w4a16_mid.hip), one per CU.  A full round of either
@@ -850,7 +850,7 @@ static double tile_time_model(int M, int K, int N) {
 }
 static double mid_time_model(int M, int K, int N) {
   const long cus = device_cu_count(), G = K / 128;
-  const int s = w4a16_mid_splits(M, K, N);
+  const int s = w4a16_mid_splits(M, K, N, 2);
   const long wgs = (long)((M + 127) / 128) * ((N + 255) / 256) * s, kper = (G + s - 1) / s;
   const long full = wgs / cus, rest = wgs - full * cus;
   return (double)kper * (full * 1.85 + (rest == 0 ? 0.0 : rest * 2 <= cus ? 1.6 : 1.85)) + (s > 1 ? 6.0 : 0.0) + 6.0;
@@ -858,13 +858,34 @@ static double mid_time_model(int M, int K, int N) {
 static bool tile_prefers_ring(int M, int K, int N) {
   return M > 128 && mid_time_model(M, K, N) < 0.95 * tile_time_model(M, K, N);
 }
+// 33..128 rows: the ring kernel with one 16-column tile per wavefront (workgroups of 128 columns), K
+// split so that the grid stays within one workgroup per CU.  Returns the split count, 0 = not taken.
+// It pays where a workgroup walks ten K blocks or more (the ring has to fill before the first
+// matrix instruction): K 14336 x N 4096 at M = 64 / 128: 24.0 / 29.4 -> 19.6 / 29.2 us, 8192 x 8192:
+// 24.9 / 36.7 -> 20.6 / 30.0 us, 4096 x 28672: 29.9 / 39.3 -> 26.6 / 38.4 us; with fewer blocks per
+// workgroup (K 4096 on layers up to 6144 wide) the narrow tiles stay ahead, and up to 64 rows on a
+// layer of 200 column tiles or more the 64-row tiles do (K 8192 x N 28672, M = 48: 41.9 against 46.2 us).
+static int ring_small_splits(int M, int K, int N) {
+  if (M <= 32 || M > 128) return 0;
+  const long cus = device_cu_count(), ctiles = N / 128, G = K / 128;
+  if (ctiles >= 200 && M <= 64) return 0;
+  long s = cus / ctiles;
+  if (s > G / 8) s = G / 8;
+  while (s > 1 && (size_t)s * M * N * sizeof(float) > TILE_SPLITK_BYTES) --s;
+  if (s < 1) s = 1;
+  const long kper = (G + s - 1) / s;
+  if (kper < 10) return 0;
+  return (int)((G + kper - 1) / kper);
+}
 
 size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
   // (the choice between the kernels also depends on the dtype and the group size, which this
   // function does not see: room for whichever plan is larger)
   const int narrow = tile_narrow_splits(M, K, N);
   const int s = narrow ? narrow : tile_splits(M, K, N);
-  const int sr = tile_prefers_ring(M, K, N) ? w4a16_mid_splits(M, K, N) : 1;
+  int sr = tile_prefers_ring(M, K, N) ? w4a16_mid_splits(M, K, N, 2) : 1;
+  const int ss = ring_small_splits(M, K, N);
+  if (ss > sr) sr = ss;
   const int m = s > sr ? s : sr;
   return m > 1 ? (size_t)m * M * N * sizeof(float) : 0;
 }
@@ -878,7 +899,12 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
   if (allow_ring && dtype == MI355Q_F16 && tile_prefers_ring(M, K, N))
     return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
-                            workspace_bytes, 0, st);
+                            workspace_bytes, 0, 2, st);
+  if (allow_ring && dtype == MI355Q_F16) {
+    if (const int ss = ring_small_splits(M, K, N))
+      return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
+                              workspace_bytes, ss, 1, st);
+  }
   TileArgs a = {};
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;
