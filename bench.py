@@ -202,6 +202,9 @@ def main():
     ap.add_argument("--extras", action="store_true",
                     help="also the decode-sized MoE layer, the w4a8 experts, norm + quant and the fp8 dense linear")
     ap.add_argument("--split-k", type=int, default=0)
+    ap.add_argument("--family", type=int, default=0,
+                    help="W4A16 kernel of the headline leg: 0 the library's choice, 1 streaming, 2 MFMA tiles of 64 rows, "
+                         "3 the 128-row ring kernel")
     ap.add_argument("--no-w8a8", action="store_true", help="skip the W8A8 int8 GEMM leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run a 256 MiB device copy at the end (reference reading for rocprofv3 --pmc)")
@@ -227,7 +230,7 @@ def main():
 
     def layer_call(name, K, c):
         qw, zp, sc = layers[name][c]
-        return ops.w4a16_gemm(xs[K], qw, sc, zp, None, GROUP, split_k=args.split_k)
+        return ops.w4a16_gemm(xs[K], qw, sc, zp, None, GROUP, split_k=args.split_k, family=args.family)
 
     def make_step(c):
         def step():
@@ -306,10 +309,11 @@ def main():
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                 "traffic_provenance": provenance}
     if M > 64:
-        # --m above the decode range: the launches are the MFMA tile kernel and the bound is the fp16 matrix peak
+        # --m above the decode range: the launches are the MFMA kernels (64-row tiles or the 128-row ring kernel,
+        # chosen per layer) and the bound is the fp16 matrix peak
         step_flops = sum(2.0 * M * K * N for _, K, N in LLAMA3_8B)
         tf = step_flops / launches / (launch_us * 1e-6) / 1e12
-        roofline = {"bound": "mfma", "kernel": "w4a16_tile_kernel", "launches_per_step": launches,
+        roofline = {"bound": "mfma", "kernel": "w4a16_mid_kernel / w4a16_tile_kernel", "launches_per_step": launches,
                     "avg_launch_us": round(launch_us, 3), "algorithmic_flops_per_launch": step_flops / launches,
                     "achieved": round(tf, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(tf / 2500.0, 4),
                     "traffic": None}
@@ -425,7 +429,10 @@ def w8a8_gemm_bench(ops, dev, stream, iters=30, warmup=40, cpu=False):
             "roofline": {"bound": "mfma", "kernel": "w8a8_int8_gemm_kernel", "avg_launch_us": round(t * 1e6, 1),
                          "algorithmic_ops_per_launch": ops_, "achieved": round(ops_ / t / 1e12, 1),
                          "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops_ / t / 1e12 / INT8_PEAK_TOPS, 4),
-                         "timed_launches": iters, "warmup_launches": warmup},
+                         "timed_launches": iters, "warmup_launches": warmup,
+                         "note": "one GEMM = two launches of the kernel at this shape (three full rounds of 256 x 256 "
+                                 "tiles, then the remaining columns as one round of 256 x 128 tiles); avg_launch_us is "
+                                 "the pair"},
             "cpu_baseline": res_cpu,
             "dynamic_quant_us": round(tq * 1e6, 1),
             "dynamic_quant_GBps": round((2 * M * K + M * K + 4 * M) / tq / 1e9, 1),
