@@ -90,7 +90,8 @@ int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight,
  * 1 = streaming, 2 = MFMA tiles of 64 rows (32 x 64 below 129 rows on narrow
  * layers), 3 = MFMA workgroups of up to 128 rows fed through a ring of LDS
  * stages (fp16, group sizes that are multiples of 128; there bits 8..15 of
- * split_k = 1 select workgroups of 128 columns instead of 256). */
+ * split_k = 1 or 4 select workgroups of 128 or 512 columns instead of
+ * 256). */
 int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          const void* scales, const void* zeros, int zeros_kind,
                          const void* bias, int M, int K, int N, int group_size,

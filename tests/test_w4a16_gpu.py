@@ -372,11 +372,12 @@ def test_narrow_tiles_mid_rows(ops, rearrange, M, dtype):
                                            (64, 2048, 512, 256, 0), (128, 4096, 512, 128, 0), (128, 1536, 256, 128, 3),
                                            (48, 4096, 256, 128, 4), (130, 1024, 256, 128, 1), (300, 1024, 640, 128, 0),
                                            (2048, 2048, 384, 128, 0)])
-@pytest.mark.parametrize("tw", [2, 1])
+@pytest.mark.parametrize("tw", [2, 1, 4])
 def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split, tw):
     """The kernel that owns up to 128 rows per workgroup and streams K through a ring of LDS stages
     (fp16; B operands are (q - z) * s rounded to fp16), with two 16-column tiles per wavefront
-    (workgroups of 256 columns) and with one (128 columns): ragged M, a half-empty last column tile,
+    (workgroups of 256 columns), with one (128 columns) and with four (512 columns, always 128 rows
+    per workgroup): ragged M, a half-empty last column tile and workgroups with whole slabs past N,
     several row blocks, K split with the separate reduction, groups of 256, bias; run-to-run
     identical; exact inputs bit for bit (every scale a power of two, so the fp16 weights are exact)."""
     print(f"case ring M={M} K={K} N={N} g={g} split={split} tiles per wavefront={tw}", flush=True)
@@ -391,7 +392,7 @@ def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split, tw):
     assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, g, torch.float16)).to(torch.float16))
 
 
-@pytest.mark.parametrize("tw", [2, 1])
+@pytest.mark.parametrize("tw", [2, 1, 4])
 @pytest.mark.parametrize("M", [32, 64, 128, 200])
 def test_ring_gemm_zero_kinds(ops, rearrange, M, tw):
     """No zero-points (z = 8) and the reference's pre-scaled fp16 zero-points, where the kernel forms
@@ -423,6 +424,22 @@ def test_mid_rows_take_the_ring_kernel_where_k_is_long(ops, rearrange):
     want = oracle(q, z, s, x, g, torch.float16, bias=bias)
     np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
     tile = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, bias=bias, family=2)
+    np.testing.assert_allclose(tile.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_even_rounds_take_the_512_column_ring_workgroups(ops, rearrange):
+    """1024 rows x 16384 columns is exactly one round of 128 x 512 workgroups on 256 CUs and two rounds of
+    either other kernel: the dispatcher takes the 512-column ring workgroups, so its result is bit for
+    bit that of the forced launch; against the oracle, and the 64-row tiles beside it."""
+    M, K, N, g = 1024, 512, 16384, 128
+    print(f"case ring 512 columns auto M={M} K={K} N={N}", flush=True)
+    q, z, s, x = make_case(33, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16)
+    forced = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=3, split_k=4 << 8)
+    assert torch.equal(got, forced)
+    want = oracle(q, z, s, x, g, torch.float16)
+    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    tile = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=2)
     np.testing.assert_allclose(tile.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 

@@ -1,18 +1,23 @@
 // W4A16 MFMA GEMM in which every operand reaches the CU through a ring of LDS stages (fp16).
 //
-// One workgroup per CU owns all rows of a block (16 MT, up to 128) of 256 or 128 columns and walks K
+// One workgroup per CU owns all rows of a block (16 MT, up to 128) of 512, 256 or 128 columns and walks K
 // (or its share of K) in blocks of 128.  Everything a K block needs -- the activation rows, the packed
 // weights, the group scales and zero-points -- is copied from global memory straight into a ring of LDS
 // stages (global_load_lds, 16 B per lane, no staging registers) several K blocks ahead; the ring is the
 // latency cover that a second workgroup per CU provides in the 64-row tile kernel.  Each of the eight
 // wavefronts (two per SIMD: one wavefront alone issues an instruction every five or six clocks, too
-// few for the matrix pipe) owns all row tiles of TW = 2 or 1 of the 16-column tiles: no weight is
+// few for the matrix pipe) owns all row tiles of TW = 4, 2 or 1 of the 16-column tiles: no weight is
 // dequantised twice.  B operands are scaled, (q - z) * s rounded to fp16 -- the dequantised weight the
 // operator is defined on -- so the matrix instructions accumulate in place.
 //
-// Two uses: above 128 rows (TW = 2, workgroups of 256 columns, row blocks in blockIdx.y) where a round
-// model prices it below the 64-row tiles, and from 33 to 128 rows (TW = 1, workgroups of 128 columns:
-// twice the workgroups, so K needs half the splits) where a workgroup walks ten K blocks or more.
+// Three uses: above 128 rows (TW = 2 or 4, workgroups of 256 or 512 columns, row blocks in blockIdx.y)
+// where a round model prices it below the 64-row tiles, and from 33 to 128 rows (TW = 1, workgroups of
+// 128 columns: twice the workgroups, so K needs half the splits) where a workgroup walks ten K blocks
+// or more.  With TW = 4 an activation operand read from LDS feeds four matrix instructions instead of
+// two -- the LDS reads per matrix instruction fall from 0.75 to 0.5 and the copies per column from a
+// 128-row block of activations per 256 columns to one per 512 -- at the price of a ring of two stages
+// instead of three and of registers: the 128 accumulators of the 8 x 4 tiles leave room for a ring of
+// four activation operands and one set of packed weights, read twice per K block.
 //
 // The copies are issued from inline assembly, so the compiler does not know of them: it schedules and
 // waits for the LDS reads itself (lgkmcnt), and the waits for the copies (vmcnt) are written by hand.
@@ -39,8 +44,9 @@ struct MidArgs {
   float* partial;             // split K: fp32 tiles [split][M][N]; null: write the output
 };
 
-// TW: 16-column tiles per wavefront -- 2: a workgroup of 256 columns; 1: of 128 columns (one slab), for
-// launches of up to 128 rows, where 256-column workgroups are too few to fill the chip without splitting K
+// TW: 16-column tiles per wavefront -- 2: a workgroup of 256 columns; 4: of 512 columns (128 rows only);
+// 1: of 128 columns (one slab), for launches of up to 128 rows, where 256-column workgroups are too few
+// to fill the chip without splitting K
 template <int MT, int TW>
 struct MidCfg {
   static constexpr int BM = 16 * MT;
@@ -55,6 +61,8 @@ struct MidCfg {
 
 // 64 lanes x 16 B from saddr + voff into LDS at lds_addr + 16 * lane
 __device__ __forceinline__ void dma16(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+  // (uniform by construction; inside a divergent region the compiler may otherwise keep it in a vector register)
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(voff), "s"(sbase), "s"(lds_addr)
@@ -110,10 +118,10 @@ w4a16_mid_kernel(MidArgs a) {
   const int m0 = blockIdx.y * C::BM;
   // N may end in the middle of a 256-column tile: the wavefronts of the missing slab work on the
   // previous one and their columns are never stored
-  const int wslab = TW == 2 ? wave >> 2 : 0;          // slab of the workgroup this wavefront works on
+  const int wslab = TW == 4 ? wave >> 1 : TW == 2 ? wave >> 2 : 0;   // slab of the workgroup this wavefront works on
   const bool live = (blockIdx.x * TW + wslab) < (N >> 7);
   const int slab = live ? blockIdx.x * TW + wslab : (N >> 7) - 1;
-  const int t0 = TW == 2 ? (wave & 3) * 2 : wave;     // first of this wavefront's TW tiles of the slab
+  const int t0 = TW == 4 ? (wave & 1) * 4 : TW == 2 ? (wave & 3) * 2 : wave;   // first of this wavefront's TW tiles of the slab
   const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
   const uint32_t lds_base =
       __builtin_amdgcn_readfirstlane((uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds);
@@ -172,24 +180,28 @@ w4a16_mid_kernel(MidArgs a) {
 #pragma unroll
     for (int t = 0; t < TW; ++t) w[t] = *(const u4*)(lds + slot * STAGE + C::W_OFF + wave * 1024 * TW + t * 1024 + lane * 16);
   };
-  struct Sz { uint32_t s; uint32_t zs; uint32_t z; };
+  struct Sz { uint2 s; uint2 zs; uint32_t z; };
   auto read_sz = [&](Sz& q, int slot) {
     const unsigned char* p = lds + slot * STAGE + C::SZ_OFF + wave * 512;
     // (one tile per wavefront: t0 may be odd, the 32-bit read starts at the even column below it)
     const int te = t0 & ~1;
-    q.s = *(const uint32_t*)(p + (8 * c + te) * 2) >> (16 * (t0 & 1));
+    if (TW == 4) q.s = *(const uint2*)(p + (8 * c + t0) * 2);
+    else q.s.x = *(const uint32_t*)(p + (8 * c + te) * 2) >> (16 * (t0 & 1));
     if (ZK == MI355Q_ZP_PACKED) q.z = *(const uint32_t*)(p + 256 + c * 4) >> (4 * t0);
-    if (ZK == MI355Q_ZP_PRESCALED) q.zs = *(const uint32_t*)(p + 256 + (8 * c + te) * 2) >> (16 * (t0 & 1));
+    if (ZK == MI355Q_ZP_PRESCALED) {
+      if (TW == 4) q.zs = *(const uint2*)(p + 256 + (8 * c + t0) * 2);
+      else q.zs.x = *(const uint32_t*)(p + 256 + (8 * c + te) * 2) >> (16 * (t0 & 1));
+    }
   };
   // per column tile: scale, 1024 + z, 64 + z, z * s
   _Float16 sc[TW], zlo[TW], zhi[TW], zsc[TW];
   auto prep = [&](const Sz& q) {
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
-      const uint32_t sw = q.s;
+      const uint32_t sw = t < 2 ? q.s.x : q.s.y;
       sc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
       if (ZK == MI355Q_ZP_PRESCALED) {
-        const uint32_t zw = q.zs;
+        const uint32_t zw = t < 2 ? q.zs.x : q.zs.y;
         zsc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu)));
         zlo[t] = (_Float16)1024.0f;
         zhi[t] = (_Float16)64.0f;
@@ -221,14 +233,22 @@ w4a16_mid_kernel(MidArgs a) {
   wait_vmcnt<(D - 1) * NC>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  u4 w0[TW], w1[TW];
+  // A operands travel through a small ring of registers: group j (K step j / MT, row tile j % MT) uses
+  // entry j % R and requests the operand of group j + PF.  A whole K step ahead where the registers
+  // allow (R = 2 MT entries); with four column tiles per wavefront the 128 accumulator registers leave
+  // room for a ring of four, three groups (twelve matrix instructions) ahead -- and for one set of
+  // packed weights instead of two, re-read when its last word has been dequantised.
+  constexpr int PF = TW == 4 ? 3 : MT, R = TW == 4 ? 4 : 2 * MT;
+  constexpr bool WDB = TW != 4;                        // two sets of packed weights that swap roles per K block
+  static_assert((4 * MT) % R == 0, "the ring index of a group is the same in every K block");
+  u4 w0[TW], w1[WDB ? TW : 1];
   Sz sz;
-  h8 av[2][MT];
+  h8 av[R];
   u4 bv[2][TW];
   read_w(w0, 0);
   read_sz(sz, 0);
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) av[0][mt] = read_a(0, mt, 0);
+  for (int j = 0; j < PF; ++j) av[j % R] = read_a(0, j % MT, j / MT);
   prep(sz);
 #pragma unroll
   for (int t = 0; t < TW; ++t)
@@ -236,50 +256,59 @@ w4a16_mid_kernel(MidArgs a) {
     for (int p = 0; p < 4; ++p) bv[0][t][p] = mid_dequant_pair<ZK>(w0[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
 
   constexpr int NP = 4 * TW;                          // operand words dequantised per K step, dealt out over the MT groups
-  constexpr int CPG = (NSLOT + MT - 1) / MT;          // copy slots issued per row-tile group
+  constexpr int JX = 4 * MT - PF;                     // first group whose request goes to the next stage
+  constexpr int CPG = (NSLOT + PF - 1) / PF;          // copy slots issued per group from there on
   int slot = 0;
-  // One K block: four K steps of MT groups of two matrix instructions.  While step st multiplies, the
-  // A operands of step st + 1 are read and its B operands dequantised, one operand and 8 / MT words per group.  In step 2 the
-  // wavefront's own copies of the next stage are awaited and its packed weights and scales read; at the
-  // top of step 3 every LDS read of this stage has been issued and awaited, so after the barrier there the
-  // stage is refilled with K block g + D while the first operands of block g + 1 are fetched.
-  auto kblock = [&](int i, u4 (&wc)[TW], u4 (&wn)[TW]) {
+  // One K block: four K steps of MT groups of TW matrix instructions, with the group's other work dealt
+  // out behind them (a matrix instruction occupies its pipe for four issue slots).  While step st
+  // multiplies, the B operands of step st + 1 are dequantised.  In step 2 the wavefront's own copies of
+  // the next stage are awaited and its scales (and, with two weight sets, packed weights) read.  Before
+  // group JX every LDS read of this stage has been issued and awaited: after the barrier there the stage
+  // is refilled with K block i + D while the first A operands of block i + 1 are requested.
+  auto kblock = [&](int i, u4 (&wc)[TW], u4 (&wn)[TW]) __attribute__((always_inline)) {
     const int nslot = slot + 1 == D ? 0 : slot + 1;
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
       const int cur = st & 1, nxt = cur ^ 1;
       if (st == 2) {
         wait_vmcnt<(D - 2) * NC>();
-        read_w(wn, nslot);
+        if (WDB) read_w(wn, nslot);
         read_sz(sz, nslot);
       }
       if (st == 3) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
+        if (!WDB) read_w(wn, nslot);                  // (its own copies: no barrier needed; wc and wn are one array)
         prep(sz);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        // a matrix instruction occupies its pipe for four issue slots: the other work of the group goes
-        // into the slots behind it
-        acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][0]), acc[mt][0], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        av[nxt][mt] = st < 3 ? read_a(slot, mt, st + 1) : read_a(nslot, mt, 0);
-        if (st == 3) {
-#pragma unroll
-          for (int s = mt * CPG; s < (mt + 1) * CPG && s < NSLOT; ++s) copy_slot(s, slot, i + D);
+        const int j = st * MT + mt, jn = j + PF;
+        if (j == JX) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int q = 0; q < NP; ++q) {
-          if (q * MT / NP != mt) continue;             // word q belongs to group q * MT / NP
-          const int t = q >> 2, p = q & 3;
-          bv[nxt][t][p] = mid_dequant_pair<ZK>(st < 3 ? wc[t][st + 1] : wn[t][0], p, zlo[t], zhi[t], sc[t], zsc[t], dqk);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (TW == 2) {
-          acc[mt][TW - 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[cur][mt], bitcast<h8>(bv[cur][TW - 1]), acc[mt][TW - 1], 0, 0, 0);
+        for (int t = 0; t < TW; ++t) {
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[j % R], bitcast<h8>(bv[cur][t]), acc[mt][t], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (t == 0) {
+            av[jn % R] = jn < 4 * MT ? read_a(slot, jn % MT, jn / MT) : read_a(nslot, (jn - 4 * MT) % MT, (jn - 4 * MT) / MT);
+            if (j >= JX) {
+#pragma unroll
+              for (int sl = (j - JX) * CPG; sl < (j - JX + 1) * CPG && sl < NSLOT; ++sl) copy_slot(sl, slot, i + D);
+            }
+          }
+          // the operand words of this group (word q belongs to group q * MT / NP), dealt out over its TW slices
+          int k = 0;
+#pragma unroll
+          for (int q = 0; q < NP; ++q) {
+            if (q * MT / NP != mt) continue;
+            if (k++ % TW != (TW == 1 ? 0 : (t + 1) % TW)) continue;
+            const int tt = q >> 2, p = q & 3;
+            bv[nxt][tt][p] = mid_dequant_pair<ZK>(st < 3 ? wc[tt][st + 1] : wn[tt][0], p, zlo[tt], zhi[tt], sc[tt], zsc[tt], dqk);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -287,54 +316,73 @@ w4a16_mid_kernel(MidArgs a) {
     slot = nslot;
   };
   for (int i = 0;; i += 2) {
-    kblock(i, w0, w1);
+    if (WDB) kblock(i, w0, (u4(&)[TW])w1);
+    else kblock(i, w0, w0);
     if (i + 1 >= nk) break;
-    kblock(i + 1, w1, w0);
+    if (WDB) kblock(i + 1, (u4(&)[TW])w1, w0);
+    else kblock(i + 1, w0, w0);
     if (i + 2 >= nk) break;
   }
   // no copy may still be writing LDS when the workgroup retires, and none may be in flight next to the
   // loads below
   wait_vmcnt<0>();
 
-  // ---- epilogue through LDS (the ring is free now): a lane holds 2 adjacent columns of 4 rows per
-  // row tile, which as stores would touch 8 bytes in every 32; written to an fp32 tile in LDS and read
-  // back row by row, every store instruction writes one whole row of the 256-column tile.
+  // ---- epilogue through LDS (the ring is free now): a lane holds TW adjacent columns of 4 rows per row
+  // tile, which as stores would touch a few bytes in every 32; written to an fp32 tile in LDS and read
+  // back row by row, every store instruction writes whole rows of the workgroup's columns.  (512 columns:
+  // the tile goes through in two halves of 64 rows.)
   constexpr int EP = C::BNW * 4 + 16;                  // bytes per tile row in LDS
-  static_assert(C::BM * EP <= D * STAGE, "the output tile fits in the ring");
-  __syncthreads();                                     // every wavefront has left the K loop
-  {
-    unsigned char* base = lds + (128 * wslab + 8 * c + t0) * 4;
+  constexpr int HALVES = TW == 4 ? 2 : 1, MTH = MT / HALVES;
+  static_assert(16 * MTH * EP <= D * STAGE, "the output tile fits in the ring");
+  // 4 columns per lane: a wavefront instruction covers part of a row, one row or two rows
+  constexpr int LPR = C::BNW / 4;                      // lanes per row
+  constexpr int RPI = LPR >= 64 ? 1 : 64 / LPR, IPR = LPR >= 64 ? LPR / 64 : 1;   // rows per instruction, instructions per row
+  f4 bs[IPR];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+  for (int q = 0; q < IPR; ++q) {
+    bs[q] = (f4){0.f, 0.f, 0.f, 0.f};
+    const int col = blockIdx.x * C::BNW + 4 * (lane % LPR) + 256 * q;
+    if (a.bias && !a.partial && col < N) {
+      const uint2 bw = *(const uint2*)(a.bias + col);
+      bs[q] = (f4){Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x >> 16)),
+                   Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y >> 16))};
+    }
+  }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (TW == 2) *(f2*)(base + (mt * 16 + 4 * kq + i) * EP) = (f2){acc[mt][0][i], acc[mt][TW - 1][i]};
-        else *(float*)(base + (mt * 16 + 4 * kq + i) * EP) = acc[mt][0][i];
+  for (int h = 0; h < HALVES; ++h) {
+    __syncthreads();                                   // every wavefront has left the K loop (or the half before)
+    {
+      unsigned char* base = lds + (128 * wslab + 8 * c + t0) * 4;
+#pragma unroll
+      for (int mh = 0; mh < MTH; ++mh)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int mt = h * MTH + mh;
+          unsigned char* q = base + (mh * 16 + 4 * kq + i) * EP;
+          if (TW == 4) *(f4*)q = (f4){acc[mt][0][i], acc[mt][1 % TW][i], acc[mt][2 % TW][i], acc[mt][3 % TW][i]};
+          else if (TW == 2) *(f2*)q = (f2){acc[mt][0][i], acc[mt][TW - 1][i]};
+          else *(float*)q = acc[mt][0][i];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 2 * MTH / RPI; ++p) {
+      const int r = RPI * (wave + 8 * p) + (LPR >= 64 ? 0 : lane / LPR), m = m0 + h * 16 * MTH + r;
+      if (m >= M) break;
+#pragma unroll
+      for (int q = 0; q < IPR; ++q) {
+        const int col = blockIdx.x * C::BNW + 4 * (lane % LPR) + 256 * q;
+        if (col >= N) continue;
+        const f4 v = *(const f4*)(lds + r * EP + (lane % LPR) * 16 + 1024 * q);
+        if (a.partial) {
+          *(f4*)(a.partial + ((size_t)blockIdx.z * M + m) * N + col) = v;
+        } else {
+          uint2 o;
+          o.x = (uint32_t)Elem<MI355Q_F16>::from_f32(v[0] + bs[q][0]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[1] + bs[q][1]) << 16);
+          o.y = (uint32_t)Elem<MI355Q_F16>::from_f32(v[2] + bs[q][2]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[3] + bs[q][3]) << 16);
+          *(uint2*)(a.out + (size_t)m * N + col) = o;
+        }
       }
-  }
-  __syncthreads();
-  // 4 columns per lane: a wavefront instruction covers one 256-column row or two 128-column rows
-  constexpr int LPR = C::BNW / 4, RPI = 64 / LPR;      // lanes per row, rows per instruction
-  const int col = blockIdx.x * C::BNW + 4 * (lane % LPR);
-  if (col >= N) return;
-  f4 bs = {0.f, 0.f, 0.f, 0.f};
-  if (a.bias && !a.partial) {
-    const uint2 bw = *(const uint2*)(a.bias + col);
-    bs = (f4){Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x >> 16)),
-              Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y >> 16))};
-  }
-#pragma unroll
-  for (int p = 0; p < 2 * MT / RPI; ++p) {
-    const int r = RPI * (wave + 8 * p) + lane / LPR, m = m0 + r;
-    if (m >= M) break;
-    const f4 v = *(const f4*)(lds + r * EP + (lane % LPR) * 16);
-    if (a.partial) {
-      *(f4*)(a.partial + ((size_t)blockIdx.z * M + m) * N + col) = v;
-    } else {
-      uint2 o;
-      o.x = (uint32_t)Elem<MI355Q_F16>::from_f32(v[0] + bs[0]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[1] + bs[1]) << 16);
-      o.y = (uint32_t)Elem<MI355Q_F16>::from_f32(v[2] + bs[2]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[3] + bs[3]) << 16);
-      *(uint2*)(a.out + (size_t)m * N + col) = o;
     }
   }
 }
@@ -354,6 +402,7 @@ int launch_mid(const MidArgs& a, int row_blocks, int splits, hipStream_t st) {
 
 template <int ZK>
 int launch_mid_mt(const MidArgs& a, int mt, int tw, int row_blocks, int splits, hipStream_t st) {
+  if (tw == 4) return launch_mid<ZK, 8, 4>(a, row_blocks, splits, st);
   if (tw == 1) {
     if (mt <= 2) return launch_mid<ZK, 2, 1>(a, row_blocks, splits, st);
     if (mt <= 4) return launch_mid<ZK, 4, 1>(a, row_blocks, splits, st);
@@ -396,7 +445,7 @@ int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const voi
              "w4a16_gemm(mid): fp16 and group sizes that are multiples of 128 only (dtype %d, group %d)", dtype, group_size);
   MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
   const int G = K / 128;
-  if (tw != 1) tw = 2;
+  if (tw != 1 && tw != 4) tw = 2;
   if (splits <= 0) splits = w4a16_mid_splits(M, K, N, tw);
   if (splits > G) splits = G;
   if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * M * N * sizeof(float))) splits = 1;

@@ -832,31 +832,43 @@ int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const voi
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
                      void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st);
 
-// Above 128 rows two kernels can take a dense fp16 layer: the 64-row tiles of this file, two workgroups
-// per CU, or the 128-row workgroups with the LDS ring (w4a16_mid.hip), one per CU.  A full round of either
-// covers the same rows; the ring kernel's is about a tenth shorter, but which of them leaves the
-// emptier last round depends on the shape.  Both are priced in microseconds per K block from what was
-// measured on Llama-shaped layers (full rounds: 2.05 for a pair of 64-row tiles sharing a CU, 1.85 for
-// a 128-row workgroup; a last round that leaves workgroups alone on their CUs: 1.2, respectively 1.6
-// when at most half the CUs are busy), plus a reduction launch when K is split.  The ring kernel is
-// taken when it is priced 5 % or more below the tiles: over 112 measured (shape, M) points that rule
-// is within 4 % of the better kernel everywhere and 0.2 % on average.
+// Above 128 rows three kernels can take a dense fp16 layer: the 64-row tiles of this file, two workgroups
+// per CU, or the 128-row workgroups with the LDS ring (w4a16_mid.hip), one per CU, 256 or 512 columns
+// wide.  A full round of the 512-column workgroups covers twice the columns in about 1.7 times the time
+// of the other two, so it wins wherever the rounds come out even, and loses where its coarser grid
+// leaves a nearly empty last round or where K would have to be split to fill the chip.  All three are
+// priced in microseconds per K block from what was measured, with weights cold in the caches, on 120
+// (shape, M) points of ten Llama- and Qwen-shaped layers, M = 129..8192: full rounds 2.15 for a pair
+// of 64-row tiles sharing a CU (1.0 for a last round that leaves each workgroup alone on its CU), 2.05
+// and 3.55 for the ring workgroups, whose last round costs 1.25 respectively 1.8 when nearly empty and
+// grows linearly with the share of the CUs it occupies; plus a reduction launch when K is split.
+// Taking the cheapest by these prices is within 0.6 % of the best of the three on average over those
+// points (11 % at worst) and 4.5 % faster than the 64-row tiles alone (always the best: 5.1 %).
 static double tile_time_model(int M, int K, int N) {
   const long cus = device_cu_count(), G = K / 128;
   const int s = tile_splits(M, K, N);
   const long wgs = (long)((M + 63) / 64) * ((N + BN - 1) / BN) * s, kper = (G + s - 1) / s;
   const long full = wgs / (2 * cus), rest = wgs - full * 2 * cus;
-  return (double)kper * (full * 2.05 + (rest == 0 ? 0.0 : rest <= cus ? 1.2 : 2.05)) + (s > 1 ? 6.0 : 0.0) + 5.0;
+  return (double)kper * (full * 2.15 + (rest == 0 ? 0.0 : rest <= cus ? 1.0 : 2.15)) + (s > 1 ? 6.0 : 0.0) + 5.0;
 }
-static double mid_time_model(int M, int K, int N) {
+static double mid_time_model(int M, int K, int N, int tw) {
   const long cus = device_cu_count(), G = K / 128;
-  const int s = w4a16_mid_splits(M, K, N, 2);
-  const long wgs = (long)((M + 127) / 128) * ((N + 255) / 256) * s, kper = (G + s - 1) / s;
+  const int s = w4a16_mid_splits(M, K, N, tw);
+  const long wgs = (long)((M + 127) / 128) * ((N + 128 * tw - 1) / (128 * tw)) * s, kper = (G + s - 1) / s;
   const long full = wgs / cus, rest = wgs - full * cus;
-  return (double)kper * (full * 1.85 + (rest == 0 ? 0.0 : rest * 2 <= cus ? 1.6 : 1.85)) + (s > 1 ? 6.0 : 0.0) + 6.0;
+  const double cf = tw == 4 ? 3.55 : 2.05, ca = tw == 4 ? 1.8 : 1.25;
+  return (double)kper * (full * cf + (rest == 0 ? 0.0 : ca + (cf - ca) * (double)rest / (double)cus)) +
+         (s > 1 ? 6.0 : 0.0) + 6.0;
 }
-static bool tile_prefers_ring(int M, int K, int N) {
-  return M > 128 && mid_time_model(M, K, N) < 0.95 * tile_time_model(M, K, N);
+// 0: the 64-row tiles; 2 / 4: the ring kernel with that many column tiles per wavefront
+static int tile_ring_plan(int M, int K, int N) {
+  if (M <= 128) return 0;
+  double best = tile_time_model(M, K, N);
+  int plan = 0;
+  const double t2 = mid_time_model(M, K, N, 2);
+  if (t2 < best) { best = t2; plan = 2; }
+  if (w4a16_mid_splits(M, K, N, 4) == 1 && mid_time_model(M, K, N, 4) < best) plan = 4;
+  return plan;
 }
 // 33..128 rows: the ring kernel with one 16-column tile per wavefront (workgroups of 128 columns), K
 // split so that the grid stays within one workgroup per CU.  Returns the split count, 0 = not taken.
@@ -883,7 +895,8 @@ size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
   // function does not see: room for whichever plan is larger)
   const int narrow = tile_narrow_splits(M, K, N);
   const int s = narrow ? narrow : tile_splits(M, K, N);
-  int sr = tile_prefers_ring(M, K, N) ? w4a16_mid_splits(M, K, N, 2) : 1;
+  // (the 512-column ring workgroups are only taken where they need no split)
+  int sr = tile_ring_plan(M, K, N) == 2 ? w4a16_mid_splits(M, K, N, 2) : 1;
   const int ss = ring_small_splits(M, K, N);
   if (ss > sr) sr = ss;
   const int m = s > sr ? s : sr;
@@ -897,10 +910,10 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   MQ_REQUIRE(group_size % 128 == 0,
              "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
   MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
-  if (allow_ring && dtype == MI355Q_F16 && tile_prefers_ring(M, K, N))
-    return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
-                            workspace_bytes, 0, 2, st);
   if (allow_ring && dtype == MI355Q_F16) {
+    if (const int tw = tile_ring_plan(M, K, N))
+      return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
+                              workspace, workspace_bytes, 0, tw, st);
     if (const int ss = ring_small_splits(M, K, N))
       return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
                               workspace_bytes, ss, 1, st);
