@@ -91,14 +91,21 @@ template <> struct TileMma<MI355Q_BF16> {
   static __device__ __forceinline__ f4 run(vec a, vec b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
-  // small integers held exactly in fp16 -> the same integers in bf16
-  static __device__ __forceinline__ uint32_t cvt(h2 r) {
-    uint32_t lo = bitcast<uint32_t>((float)r.x), hi = bitcast<uint32_t>((float)r.y);
-    return __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+  // The fp16 patterns 1024 + q and 1024 + 16 q, minus 1024 + z respectively times 1 / 16 minus 64 + z, in one
+  // mixed-precision fused multiply-add per weight (fp16 sources, exact fp32 result q - z), then one packed
+  // conversion per pair: the small integer is exact in bf16 too.  Four instructions per pair.
+  static __device__ __forceinline__ uint32_t pair(h2 a, float m, _Float16 z) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    const bf2 r = {(__bf16)__builtin_fmaf((float)a.x, m, -(float)z), (__bf16)__builtin_fmaf((float)a.y, m, -(float)z)};
+    return bitcast<uint32_t>(r);
   }
   static __device__ __forceinline__ vec dequant(uint32_t w, h2 zz, const DqConst& k) {
-    h8 v = TileMma<MI355Q_F16>::dequant(w, zz, k);
-    u4 r = {cvt((h2){v[0], v[1]}), cvt((h2){v[2], v[3]}), cvt((h2){v[4], v[5]}), cvt((h2){v[6], v[7]})};
+    float one = 1.0f, sixteenth = 0.0625f;
+    asm volatile("" : "+s"(one));                     // (as a literal the multiplication folds away and the
+    asm volatile("" : "+s"(sixteenth));               //  conversion becomes an instruction of its own)
+    const uint32_t w8 = w >> 8;
+    const u4 r = {pair(bitcast<h2>((w & k.mlo) | k.magic), one, zz.x), pair(bitcast<h2>((w & k.mhi) | k.magic), sixteenth, zz.y),
+                  pair(bitcast<h2>((w8 & k.mlo) | k.magic), one, zz.x), pair(bitcast<h2>((w8 & k.mhi) | k.magic), sixteenth, zz.y)};
     return bitcast<vec>(r);
   }
 };
@@ -232,7 +239,8 @@ w4a16_tile_kernel(TileArgs a) {
 
   const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
   // The pipelined loop needs nearly the whole register file; it is used where it fits
-  // (fp16, 128-row tiles), the plain loop elsewhere.
+  // (fp16, 128-row tiles), the plain loop elsewhere (bf16 with packed zero-points spills 30-56 registers
+  // into the K loop there: gate_up at M = 2048 646 us against 560 us on the plain loop).
   constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED && !SF32;
   // (a grouped block with at most a quarter of its row tiles holding real slots takes the plain loop,
   // which skips the others: the pipelined loop has no room for branches -- guarding its matrix
