@@ -72,10 +72,12 @@ int mi355q_w4_unpack(const int32_t* packed, uint8_t* dst, int batch, int K, int 
  * (csrc/src/gptq_gemm_gcu.cpp:27-48, csrc/src/awq_gemm_gcu.cpp:27-47):
  *   out[M, N] = x[M, K] @ ((q - z) * s)[K, N] (+ bias[N]),  fp32 accumulate.
  * x, out, scales, bias share `dtype` (F16 or BF16); qweight is the slab
- * layout; scales [K/g, N]; group_size a multiple of 32 dividing K (or -1 for
- * one group).  M <= 64 runs the split-K streaming kernel, larger M the
- * LDS-staged MFMA kernel (which splits K over two kernels when its grid would
- * leave most of the chip idle).  `workspace` must hold
+ * layout; scales [K/g, N]; group_size a multiple of 32 dividing K that divides
+ * 128 or is a multiple of it (or -1 for one group).  M <= 64 runs the split-K
+ * streaming kernel, larger M the LDS-staged MFMA kernels (groups of 32, 64 and
+ * multiples of 128; other sizes go through the streaming kernel 32 rows at a
+ * time), which split K over two kernels when their grid would leave most of
+ * the chip idle.  `workspace` must hold
  * mi355q_w4a16_workspace_bytes() bytes, be zero-filled once before first use,
  * and must not be shared by launches that may overlap in time. */
 size_t mi355q_w4a16_workspace_bytes(int M, int K, int N);
@@ -277,7 +279,7 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
 
 /* ---- fused-MoE grouped GEMM and K-contiguous skinny GEMMs -------------------
  * quant_mode: 0 = W4A16 (slab-layout int4 per expert [E, K/8, N], scales
- * [E, K/g, N], zeros per zeros_kind), 1 = fp8-e4m3fn with 128x128 block scales
+ * [E, K/g, N], zeros per zeros_kind; g = 32, 64 or a multiple of 128), 1 = fp8-e4m3fn with 128x128 block scales
  * (w [E, N, K], a_scale f32 [Ma, K/128], w_scale f32 [E, ceil(N/128), K/128]),
  * 2 = int8 (a_scale f32 [Ma] or NULL, w_scale f32 [E, N]), 3 = unquantised
  * f16/bf16 (w [E, N, K]), 4 = W8A16 (w int8 [E, N, K], w_scale in the activation

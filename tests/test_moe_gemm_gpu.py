@@ -66,29 +66,33 @@ def run_grouped(fmoe, A, B, C, A_scale, B_scale, B_zp, tw, ids, E, block, mul, t
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("g", [128, 64, 32])
 @pytest.mark.parametrize("block", [16, 32, 64, 128])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_grouped_w4a16_both_gemms(fmoe, rearrange, block, dtype):
-    print(f"case grouped w4a16 block={block} {dtype}", flush=True)
+def test_grouped_w4a16_both_gemms(fmoe, rearrange, block, dtype, g):
+    """Both expert GEMM forms on every align block size, with quantisation groups of 128, 64 and 32
+    (groups of 128 on blocks of 16 / 32 slots: the grouped streaming kernel; everything else: the MFMA
+    kernel, whose plain loop carries two or four groups per K block)."""
+    print(f"case grouped w4a16 block={block} {dtype} g={g}", flush=True)
     rng = np.random.default_rng(block)
     M, E, T, K, N = 37, 4, 2, 256, 384
-    q, z, s = make_int4_experts(rng, E, K, N)
+    q, z, s = make_int4_experts(rng, E, K, N, g)
     w, zp = int4_to_device(rearrange, q, z)
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
     sd = torch.from_numpy(s).to(dtype)
     tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
-    wf = lambda e: ow4.dequantize(q[e], z[e], sd[e].float().numpy(), 128)
+    wf = lambda e: ow4.dequantize(q[e], z[e], sd[e].float().numpy(), g)
     # GEMM 1 form: A is [M, K], output row t reads A[t // topk], no routed weight
     C = torch.full((M, T, N), 7.0, dtype=dtype, device="cuda")
     run_grouped(fmoe, x.cuda(), w, C, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, False, T,
-                use_int4_w4a16=True, block_shape=[0, 128])
+                use_int4_w4a16=True, block_shape=[0, g])
     want = om.fused_moe_gemm(x.float().numpy(), wf, ids, T)
     np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
     # GEMM 2 form: A is [M * topk, K], topk = 1, routed weights applied
     x2 = torch.from_numpy(rng.standard_normal((M * T, K)).astype(np.float32)).to(dtype)
     C2 = torch.empty((M, T, N), dtype=dtype, device="cuda")
     run_grouped(fmoe, x2.cuda(), w, C2, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, True, 1,
-                use_int4_w4a16=True, block_shape=[0, 128])
+                use_int4_w4a16=True, block_shape=[0, g])
     want2 = om.fused_moe_gemm(x2.float().numpy(), wf, ids, 1, tw, True)
     np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
 

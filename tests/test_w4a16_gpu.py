@@ -457,10 +457,57 @@ def test_ring_gemm_is_fp16_only_and_tile_family_still_forced(ops, rearrange):
 
 
 def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):
+    """Groups of 64 on the streaming kernel when it is forced (32 rows per launch) and through the
+    library's own choice (the MFMA kernel from 65 rows on)."""
     M, K, N, g = 150, 256, 128, 64
     q, z, s, x = make_case(5, M, K, N, g)
+    want = oracle(q, z, s, x, g, torch.float16)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=1).float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
     got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).float().cpu().numpy()
-    np.testing.assert_allclose(got, oracle(q, z, s, x, g, torch.float16), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("g", [64, 32])
+@pytest.mark.parametrize("M,K,N", [(65, 512, 256, ), (100, 1024, 384), (300, 2048, 640), (1100, 8192, 256), (2048, 1024, 1024)])
+def test_tile_gemm_groups_of_64_and_32(ops, rearrange, M, K, N, g, dtype):
+    """Group sizes below a K block on the MFMA kernel (two or four groups per K block of 128, each with a
+    partial tile, scale and zero-point of its own): ragged M, a half-empty last column tile, a shape
+    that splits K (1100 x 8192 x 256), bias; the streaming kernel on the same data beside it; run-to-run
+    identical; exact inputs bit for bit."""
+    print(f"case small groups M={M} K={K} N={N} g={g} {dtype}", flush=True)
+    q, z, s, x = make_case(M + g, M, K, N, g)
+    bias = np.random.default_rng(4).standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias)
+    assert torch.equal(got, run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias))
+    want = oracle(q, z, s, x, g, dtype, bias=bias)
+    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    forced = run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias, family=2)
+    assert torch.equal(got, forced)
+    if M <= 300:
+        stream = run_gemm(ops, rearrange, q, z, s, x, g, dtype, bias=bias, family=1)
+        np.testing.assert_allclose(stream.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    q, z, s, x = make_case(5, M, K, N, g, exact=True)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, dtype, family=2)
+    assert torch.equal(got.cpu(), torch.from_numpy(oracle(q, z, s, x, g, dtype)).to(dtype))
+
+
+@pytest.mark.parametrize("g", [64, 32])
+def test_tile_gemm_small_groups_zero_kinds(ops, rearrange, g):
+    """No zero-points and pre-scaled 16-bit zero-points with groups of 64 and 32 on the MFMA kernel."""
+    M, K, N = 200, 1024, 384
+    print(f"case small groups zero kinds g={g}", flush=True)
+    q, z, s, x = make_case(M + 1, M, K, N, g)
+    w, _ = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), None)
+    for dtype in (torch.float16, torch.bfloat16):
+        xs, sd = to_act(x, dtype).cuda(), to_act(s, dtype).cuda()
+        out = ops.w4a16_gemm(xs, w, sd, None, None, g)
+        np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, None, s, x, g, dtype), rtol=RTOL, atol=ATOL)
+        sf = to_act(s, dtype).float().numpy()
+        zs = to_act(z.astype(np.float32) * sf, dtype)
+        out = ops.w4a16_gemm(xs, w, sd, zs.cuda(), None, g)
+        np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, z, s, x, g, dtype), rtol=RTOL, atol=ATOL)
 
 
 def test_operand_shapes_are_checked_on_the_host(ops, rearrange):

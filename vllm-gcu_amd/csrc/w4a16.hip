@@ -26,10 +26,13 @@ using namespace mi355q;
 static constexpr size_t TILE_WS_OFFSET = (size_t)1 << 20;
 
 // streaming kernel up to 32 rows; 33..64 rows: the MFMA kernel where its pipelined loop exists
-// (fp16, integer zero-points; measured equal or up to 22 % faster there), else streaming again
+// (fp16, integer zero-points; measured equal or up to 22 % faster there), else streaming again.
+// Groups of 64 and 32: the streaming kernel takes 32 rows per launch, so from 65 rows on the MFMA
+// kernel's plain loop with two or four groups per K block takes over.
 static int auto_family(int M, int group_size, int zeros_kind, int dtype) {
+  if (group_size % 128 != 0) return ((group_size == 64 || group_size == 32) && M > 64) ? 2 : 1;
   const bool piped = dtype == MI355Q_F16 && zeros_kind != MI355Q_ZP_PRESCALED;
-  return (group_size % 128 != 0 || M <= 32 || (M <= 64 && !piped)) ? 1 : 2;
+  return (M <= 32 || (M <= 64 && !piped)) ? 1 : 2;
 }
 
 extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
@@ -86,8 +89,8 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
   MQ_REQUIRE(family >= 0 && family <= 3, "w4a16_gemm: unknown kernel family %d", family);
   const int caller_family = family;       // 0: the library chooses, also between the two MFMA kernels
   if (family == 0) family = auto_family(M, group_size, zeros_kind, dtype);
-  MQ_REQUIRE(family != 2 || group_size % 128 == 0,
-             "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
+  MQ_REQUIRE(family != 2 || group_size % 128 == 0 || group_size == 64 || group_size == 32,
+             "w4a16_gemm: the MFMA kernel needs a group size of 32, 64 or a multiple of 128, got %d", group_size);
   if (family == 1) {
     // the streaming kernel covers 64 rows per launch (32 with group sizes
     // below 128, whose four scale rows per K block leave no registers for

@@ -115,7 +115,9 @@ template <> struct TileMma<MI355Q_BF16> {
 // columns.  WM = 2: eight wavefronts, the upper four take the upper half of
 // the rows (both halves dequantise the same weights, but two wavefronts per
 // SIMD keep the matrix pipe fed while one of them waits or dequantises).
-template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false>
+// GPB = quantisation groups per K block of 128: 1 for group sizes that are multiples of 128, 2 / 4 for
+// groups of 64 / 32 (plain loop only: each group's steps accumulate into a partial tile of their own).
+template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false, int GPB = 1>
 __global__ void __launch_bounds__(256 * WM, WM == 1 ? 2 : 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
@@ -224,6 +226,10 @@ w4a16_tile_kernel(TileArgs a) {
   f4 sreg32;
   uint32_t zreg = 0x88888888u;
   uint2 zsreg = {0u, 0u};
+  // groups 1 .. GPB - 1 of the K block (group sizes below 128)
+  uint2 sregx[GPB > 1 ? GPB - 1 : 1];
+  uint32_t zregx[GPB > 1 ? GPB - 1 : 1];
+  uint2 zsregx[GPB > 1 ? GPB - 1 : 1];
   auto load_w = [&](u4 (&w)[4], int g) {
     const u4* p = wbase + (size_t)g * 512;
 #pragma unroll
@@ -235,13 +241,22 @@ w4a16_tile_kernel(TileArgs a) {
     else sreg = *(const uint2*)(scales + (size_t)qrow * N + ncol);
     if (ZK == MI355Q_ZP_PACKED) zreg = ((const uint32_t*)zeros)[(size_t)qrow * (N >> 3) + (ncol >> 3)] >> (4 * t0);
     if (ZK == MI355Q_ZP_PRESCALED) zsreg = *(const uint2*)((const uint16_t*)zeros + (size_t)qrow * N + ncol);
+    if constexpr (GPB > 1) {
+#pragma unroll
+      for (int sg = 1; sg < GPB; ++sg) {
+        const size_t r = (size_t)(qrow + sg);
+        sregx[sg - 1] = *(const uint2*)(scales + r * N + ncol);
+        if (ZK == MI355Q_ZP_PACKED) zregx[sg - 1] = ((const uint32_t*)zeros)[r * (N >> 3) + (ncol >> 3)] >> (4 * t0);
+        if (ZK == MI355Q_ZP_PRESCALED) zsregx[sg - 1] = *(const uint2*)((const uint16_t*)zeros + r * N + ncol);
+      }
+    }
   };
 
   const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
   // The pipelined loop needs nearly the whole register file; it is used where it fits
   // (fp16, 128-row tiles), the plain loop elsewhere (bf16 with packed zero-points spills 30-56 registers
   // into the K loop there: gate_up at M = 2048 646 us against 560 us on the plain loop).
-  constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED && !SF32;
+  constexpr bool PIPE = MTW == 4 && DT == MI355Q_F16 && ZK != MI355Q_ZP_PRESCALED && !SF32 && GPB == 1;
   // (a grouped block with at most a quarter of its row tiles holding real slots takes the plain loop,
   // which skips the others: the pipelined loop has no room for branches -- guarding its matrix
   // instructions cost 17 % on full blocks -- and beats the plain loop once two of four tiles are live;
@@ -376,22 +391,27 @@ w4a16_tile_kernel(TileArgs a) {
       u4 wcur[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) wcur[t] = wreg[t];
-      float sc[4];
-      h2 zz[4];
+      float sc[GPB][4];
+      h2 zz[GPB][4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const uint32_t sw = (t < 2) ? sreg.x : sreg.y;
-        sc[t] = SF32 ? sreg32[t] : Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
-        float zf;
-        if (ZK == MI355Q_ZP_PRESCALED) {
-          const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
-          // the loader pre-multiplied an integer zero-point by the scale
-          // (z * s rounded to the activation type): recover the integer
-          zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[t]);
-        } else {
-          zf = (float)((zreg >> (4 * t)) & 15u);
+      for (int sg = 0; sg < GPB; ++sg) {
+        const uint2 sv = sg == 0 ? sreg : sregx[sg > 0 ? sg - 1 : 0], zsv = sg == 0 ? zsreg : zsregx[sg > 0 ? sg - 1 : 0];
+        const uint32_t zv = sg == 0 ? zreg : zregx[sg > 0 ? sg - 1 : 0];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t sw = (t < 2) ? sv.x : sv.y;
+          sc[sg][t] = SF32 ? sreg32[t] : Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+          float zf;
+          if (ZK == MI355Q_ZP_PRESCALED) {
+            const uint32_t zw = (t < 2) ? zsv.x : zsv.y;
+            // the loader pre-multiplied an integer zero-point by the scale
+            // (z * s rounded to the activation type): recover the integer
+            zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[sg][t]);
+          } else {
+            zf = (float)((zv >> (4 * t)) & 15u);
+          }
+          zz[sg][t] = (h2){(_Float16)(1024.0f + zf), (_Float16)(64.0f + zf)};
         }
-        zz[t] = (h2){(_Float16)(1024.0f + zf), (_Float16)(64.0f + zf)};
       }
       const int gn = min(g + 1, ge - 1);
       load_a(gn);
@@ -404,23 +424,26 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
       for (int s = 0; s < 4; ++s)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zz[t], dqk);
+        for (int t = 0; t < 4; ++t) bv[s][t] = MM::dequant(wcur[t][s], zz[s * GPB / 4][t], dqk);
 
       const unsigned char* abase = lds + buf + (wmh * MTW * 16 + c) * A_ROW + kq * 16;
 #pragma unroll
       for (int mt = 0; mt < MTW; ++mt) {
         if (!tile_live(mt)) continue;
-        f4 part[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
+        for (int sg = 0; sg < GPB; ++sg) {
+          f4 part[4];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const vec av = bitcast<vec>(*(const u4*)(abase + mt * 16 * A_ROW + s * 64));
+          for (int t = 0; t < 4; ++t) part[t] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int t = 0; t < 4; ++t) part[t] = MM::run(av, bv[s][t], part[t]);
+          for (int s = sg * (4 / GPB); s < (sg + 1) * (4 / GPB); ++s) {
+            const vec av = bitcast<vec>(*(const u4*)(abase + mt * 16 * A_ROW + s * 64));
+#pragma unroll
+            for (int t = 0; t < 4; ++t) part[t] = MM::run(av, bv[s][t], part[t]);
+          }
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[mt][t] += sc[sg][t] * part[t];
         }
-#pragma unroll
-        for (int t = 0; t < 4; ++t) acc[mt][t] += sc[t] * part[t];
       }
       // the other buffer was last read one iteration ago: every wavefront has
       // passed the barrier below since, so it can be overwritten now
@@ -545,6 +568,31 @@ hipError_t launch_wm(const TileArgs& a, int row_blocks, hipStream_t st) {
   if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, SF32>), grid, block, shmem, st, a);
   return hipSuccess;
+}
+
+// group sizes of 64 and 32 (two and four groups per K block): dense 64-row tiles, MoE blocks of 64 and 128 slots
+template <int DT, int ZK, int MT, bool GROUPED, int GPB>
+hipError_t launch_small_groups_one(const TileArgs& a, int row_blocks, hipStream_t st) {
+  constexpr int WM = MT >= 8 ? 2 : 1;
+  const int G = a.K >> 7;
+  dim3 grid((a.N + BN - 1) / BN, row_blocks, (G + a.kper - 1) / a.kper), block(256 * WM);
+  const size_t shmem = 2 * 16 * MT * A_ROW;
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, false, GPB>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  if (attr != hipSuccess) return attr;
+  hipLaunchKernelGGL((w4a16_tile_kernel<DT, ZK, MT, GROUPED, WM, false, GPB>), grid, block, shmem, st, a);
+  return hipSuccess;
+}
+template <int DT, int MT, bool GROUPED>
+hipError_t launch_small_groups(const TileArgs& a, int zk, int gpb, int row_blocks, hipStream_t st) {
+  if (gpb == 2) {
+    if (zk == MI355Q_ZP_NONE) return launch_small_groups_one<DT, MI355Q_ZP_NONE, MT, GROUPED, 2>(a, row_blocks, st);
+    if (zk == MI355Q_ZP_PACKED) return launch_small_groups_one<DT, MI355Q_ZP_PACKED, MT, GROUPED, 2>(a, row_blocks, st);
+    return launch_small_groups_one<DT, MI355Q_ZP_PRESCALED, MT, GROUPED, 2>(a, row_blocks, st);
+  }
+  if (zk == MI355Q_ZP_NONE) return launch_small_groups_one<DT, MI355Q_ZP_NONE, MT, GROUPED, 4>(a, row_blocks, st);
+  if (zk == MI355Q_ZP_PACKED) return launch_small_groups_one<DT, MI355Q_ZP_PACKED, MT, GROUPED, 4>(a, row_blocks, st);
+  return launch_small_groups_one<DT, MI355Q_ZP_PRESCALED, MT, GROUPED, 4>(a, row_blocks, st);
 }
 
 template <int DT, int ZK, int MT, bool GROUPED, bool SF32 = false>
@@ -915,10 +963,12 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
                       int group_size, int dtype, void* workspace, size_t workspace_bytes, bool allow_ring,
                       hipStream_t st) {
-  MQ_REQUIRE(group_size % 128 == 0,
-             "w4a16_gemm: the MFMA kernel needs group_size %% 128 == 0, got %d", group_size);
+  // groups of 64 and 32: two and four groups per K block, 64-row tiles with the plain loop only
+  const bool small_groups = group_size == 64 || group_size == 32;
+  MQ_REQUIRE(group_size % 128 == 0 || small_groups,
+             "w4a16_gemm: the MFMA kernel needs a group size of 32, 64 or a multiple of 128, got %d", group_size);
   MQ_REQUIRE((size_t)M * K * 2 < ((size_t)1 << 32), "w4a16_gemm: activation matrix %d x %d is 4 GiB or more", M, K);
-  if (allow_ring && dtype == MI355Q_F16) {
+  if (allow_ring && dtype == MI355Q_F16 && !small_groups) {
     if (const int tw = tile_ring_plan(M, K, N))
       return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
                               workspace, workspace_bytes, 0, tw, st);
@@ -938,7 +988,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   int ntw = 4;
   const int G = K / 128;
   int splits = tile_splits(M, K, N);
-  const int narrow = tile_narrow_splits(M, K, N);
+  const int narrow = small_groups ? 0 : tile_narrow_splits(M, K, N);
   if (narrow) {
     mt = 2;
     ntw = 1;
@@ -952,7 +1002,10 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   hipError_t e;
   const uint32_t gpk = (uint32_t)group_size / 128u;
   a.gpk_magic = gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + gpk - 1) / gpk) : 0u;
-  if (ntw < 4)
+  if (small_groups)
+    e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 4, false>(a, zeros_kind, 128 / group_size, row_blocks, st)
+                              : launch_small_groups<MI355Q_BF16, 4, false>(a, zeros_kind, 128 / group_size, row_blocks, st);
+  else if (ntw < 4)
     e = (dtype == MI355Q_F16) ? launch_narrow<MI355Q_F16>(a, zeros_kind, row_blocks, st)
                               : launch_narrow<MI355Q_BF16>(a, zeros_kind, row_blocks, st);
   else
@@ -999,14 +1052,18 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
                          const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp,
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                          int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
-  MQ_REQUIRE(group_size % 128 == 0, "moe_w4a16: group_size=%d must be a multiple of 128", group_size);
+  // groups of 64 and 32: the plain loop of the MFMA kernel at every block size
+  const bool small_groups = group_size == 64 || group_size == 32;
+  MQ_REQUIRE(group_size % 128 == 0 || (small_groups && !scales_f32 && !out_scale),
+             "moe_w4a16: group_size=%d must be 32, 64 or a multiple of 128 (a multiple of 128 with fp32 scales)", group_size);
   MQ_REQUIRE((size_t)(numel / (topk > 0 ? topk : 1)) * K * 2 < ((size_t)1 << 32),
              "moe_w4a16: activation matrix of %d rows x %d is 4 GiB or more", numel / (topk > 0 ? topk : 1), K);
   MQ_REQUIRE(block_size == 16 || block_size == 32 || block_size == 64 || block_size == 128,
              "moe_w4a16: block_size=%d must be 16, 32, 64 or 128", block_size);
   // blocks of 16 or 32 slots (decode-sized token counts): the layer is bound by the experts' weights,
   // which the streaming kernel reads faster than the MFMA tile kernel with one or two row tiles
-  if (block_size <= 32 && !scales_f32 && !out_scale)
+  // (the grouped streaming kernel takes groups that are multiples of 128 only)
+  if (block_size <= 32 && !scales_f32 && !out_scale && !small_groups)
     return w4a16_stream_grouped_launch(out, x, qweight, scales, zeros, zeros_kind, topk_weights, sorted_ids,
                                        expert_ids, npp, numel, topk, block_size, max_blocks, E, K, N, group_size,
                                        dtype, st);
@@ -1032,9 +1089,25 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   a.w_stride = (long)(K / 8) * N / 4;              // u4 elements per expert
   a.s_stride = (long)(K / group_size) * N;
   a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
-  hipError_t e = (dtype == MI355Q_F16)
-                     ? launch_mt<MI355Q_F16, true>(a, zeros_kind, block_size / 16, max_blocks, st)
-                     : launch_mt<MI355Q_BF16, true>(a, zeros_kind, block_size / 16, max_blocks, st);
+  hipError_t e;
+  if (small_groups) {
+    const int gpb = 128 / group_size;
+    if (block_size == 16)
+      e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 1, true>(a, zeros_kind, gpb, max_blocks, st)
+                                : launch_small_groups<MI355Q_BF16, 1, true>(a, zeros_kind, gpb, max_blocks, st);
+    else if (block_size == 32)
+      e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 2, true>(a, zeros_kind, gpb, max_blocks, st)
+                                : launch_small_groups<MI355Q_BF16, 2, true>(a, zeros_kind, gpb, max_blocks, st);
+    else if (block_size == 64)
+      e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 4, true>(a, zeros_kind, gpb, max_blocks, st)
+                                : launch_small_groups<MI355Q_BF16, 4, true>(a, zeros_kind, gpb, max_blocks, st);
+    else
+      e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 8, true>(a, zeros_kind, gpb, max_blocks, st)
+                                : launch_small_groups<MI355Q_BF16, 8, true>(a, zeros_kind, gpb, max_blocks, st);
+  } else {
+    e = (dtype == MI355Q_F16) ? launch_mt<MI355Q_F16, true>(a, zeros_kind, block_size / 16, max_blocks, st)
+                              : launch_mt<MI355Q_BF16, true>(a, zeros_kind, block_size / 16, max_blocks, st);
+  }
   MQ_REQUIRE(e == hipSuccess, "moe_w4a16: cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("moe_w4a16");
   if (splits > 1) {
