@@ -510,6 +510,58 @@ def test_tile_gemm_small_groups_zero_kinds(ops, rearrange, g):
         np.testing.assert_allclose(out.float().cpu().numpy(), oracle(q, z, s, x, g, dtype), rtol=RTOL, atol=ATOL)
 
 
+def _random_cases():
+    rng = np.random.default_rng(2024)
+    cases = []
+    for i in range(28):
+        g = int(rng.choice([128, 128, 128, 64, 32, 256, -1]))
+        K = 128 * int(rng.integers(1, 33))
+        if g == 256:
+            K = 256 * max(1, K // 256)
+        N = 128 * int(rng.integers(1, 25))
+        M = int(rng.choice([rng.integers(1, 33), rng.integers(33, 129), rng.integers(129, 700), rng.integers(700, 2600)]))
+        cases.append((i, M, K, N, g, ["f16", "bf16"][int(rng.integers(0, 2))], int(rng.integers(0, 3)), bool(rng.integers(0, 2))))
+    # wide enough for the 512-column ring workgroups and for several rounds of every kernel
+    cases += [(100, 2048, 1024, 8192, 128, "f16", 1, True), (101, 1536, 512, 12288, 128, "f16", 0, False),
+              (102, 1300, 2048, 4096, 128, "bf16", 1, True), (103, 640, 1024, 16384, 64, "f16", 1, False)]
+    return cases
+
+
+@pytest.mark.parametrize("seed,M,K,N,g,dt,zk,with_bias", _random_cases())
+def test_random_shapes_through_the_library_s_own_choice(ops, rearrange, seed, M, K, N, g, dt, zk, with_bias):
+    """Seeded random shapes, group sizes, types, zero-point kinds and bias through mi355q_w4a16_gemm as a
+    caller uses it (no family forced): whichever kernel and split the dispatcher takes, the result is the
+    oracle's within the tolerance and run-to-run identical."""
+    dtype = torch.float16 if dt == "f16" else torch.bfloat16
+    print(f"case random {seed}: M={M} K={K} N={N} g={g} {dt} zeros kind {zk} bias {with_bias}", flush=True)
+    q, z, s, x = make_case(1000 + seed, M, K, N, g)
+    bias = np.random.default_rng(seed).standard_normal(N).astype(np.float32) if with_bias else None
+    gg = K if g == -1 else g
+    w, zp = rearrange.rearrange_uint4_int32_gptq(dev(ow4.gptq_pack_weight(q)), dev(ow4.gptq_pack_zeros(z)))
+    xs, sd = to_act(x, dtype).cuda(), to_act(s, dtype).cuda()
+    bd = None if bias is None else to_act(bias, dtype).cuda()
+    if zk == 0:                                      # symmetric: no zero-points, z = 8
+        zeros, want = None, oracle(q, None, s, x, gg, dtype, bias=bias)
+    elif zk == 1:                                    # packed integer zero-points
+        zeros, want = zp, oracle(q, z, s, x, gg, dtype, bias=bias)
+    else:                                            # z * s rounded to the activation type
+        sf = to_act(s, dtype).float().numpy()
+        zs = to_act(z.astype(np.float32) * sf, dtype)
+        zeros, want = zs.cuda(), oracle(q, z, s, x, gg, dtype, bias=bias)
+    got = ops.w4a16_gemm(xs, w, sd, zeros, bd, g)
+    again = ops.w4a16_gemm(xs, w, sd, zeros, bd, g)
+    assert torch.equal(got, again)
+    got = got.float().cpu().numpy()
+    if zk == 2 and not np.allclose(got, want, rtol=RTOL, atol=ATOL):
+        # the streaming and ring kernels take the pre-scaled value as it is, q * s - zs, where the tile kernel
+        # recovers the integer zero-point: the two readings differ by the rounding of z * s times the sum of
+        # a group's activations, which a group of many hundred rows in bf16 makes visible
+        want = to_act(x, dtype).float().numpy() @ ow4.dequantize_prescaled_zeros(q, zs.float().numpy(), sf, gg)
+        if bias is not None:
+            want = want + to_act(bias, dtype).float().numpy()[None, :]
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
 def test_operand_shapes_are_checked_on_the_host(ops, rearrange):
     """The kernels index scales, zero-points and bias by (group row, column) without bounds checks, so
     the wrapper refuses operands whose sizes do not fit K / group_size x N before anything is launched."""
