@@ -363,6 +363,8 @@ def main():
         out["norm_quant"] = glue_bench(ops, dev, stream)
         torch.cuda.empty_cache()
         out["fp8_dense"] = fp8_dense_bench(ops, dev, stream)
+        torch.cuda.empty_cache()
+        out["w4a16_variants"] = variants_bench(ops, dev, stream)
     if args.calibrate_copy:
         # a plain copy of known size: its FETCH_SIZE / WRITE_SIZE readings scale
         # the counters of the profiled kernels to bytes
@@ -735,6 +737,32 @@ def yardsticks(dev, stream, iters=30):
         res["vendor_int8_mm"] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1), "TOPs": round(2.0 * M * K * N / t / 1e12, 1)}
     except RuntimeError as e:
         res["vendor_int8_mm"] = {"error": str(e)[:120]}
+    return res
+
+
+def variants_bench(ops, dev, stream):
+    """W4A16 away from the headline's type and group size: bf16 activations, and quantisation groups of 64
+    and 32, on two Llama-3-8B layers at prefill heights (weights rotated past the last-level cache)."""
+    import torch
+    res = []
+    for name, K, N in (("gate_up", 4096, 28672), ("down", 14336, 4096)):
+        copies = max(2, -(-2 * 256 * 2**20 // (K * N // 2)) + 1)
+        gen = torch.Generator(device="cpu").manual_seed(11)
+        qws = [torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, generator=gen).to(dev) for _ in range(copies)]
+        for dt, g in ((torch.float16, 128), (torch.bfloat16, 128), (torch.float16, 64), (torch.float16, 32)):
+            zp = torch.randint(-2**31, 2**31 - 1, (K // g, N // 8), dtype=torch.int32, generator=gen).to(dev)
+            sc = (torch.rand(K // g, N, generator=gen) * 0.009 + 0.001).to(dt).to(dev)
+            for M in (128, 2048):
+                x = torch.randn(M, K, dtype=dt, device=dev)
+                fns = [(lambda qw=qw: ops.w4a16_gemm(x, qw, sc, zp, None, g)) for qw in qws]
+                n = 30
+                t = time_graph(fns, n, 6, stream) / n
+                fl = 2.0 * M * K * N
+                res.append({"layer": name, "M": M, "dtype": str(dt).split(".")[-1], "group_size": g,
+                            "us": round(t * 1e6, 1), "TFLOPs": round(fl / t / 1e12, 1),
+                            "frac_fp16_mfma": round(fl / t / 1e12 / FP16_PEAK_TFLOPS, 4)})
+        del qws
+        torch.cuda.empty_cache()
     return res
 
 
