@@ -299,10 +299,25 @@ w8a8_int8_gemm_kernel(I8Args a) {
   if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f7c);     // vmcnt(12): element 0 landed
   else __builtin_amdgcn_s_waitcnt(0x0f70);
   __builtin_amdgcn_s_barrier();
+  int st = 0;                                      // stage of the current K tile
+  // One row tile in all (M <= 256) and none of its rows in this wavefront's share: the wavefront only
+  // copies.  It keeps the workgroup's barriers and its own copy slots, and leaves the matrix pipe and
+  // the LDS read port of its SIMD to the wavefront that has rows (65 .. 128 rows: half the wavefronts).
+  if (mtiles == 1 && wm * (16 * NJ) >= M) {
+    for (; tile < total_tiles; tile += gdim) {
+      for (int T = 0; T < nt; ++T) {
+        wait_landed();
+        __builtin_amdgcn_s_barrier();
+        issue(st, ahead_k0(T, STAGES));
+        st = st + 1 == STAGES ? 0 : st + 1;
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);            // vmcnt(0)
+    return;
+  }
   Frag f0, f1;
   read_frag(f0, 0, 0);
   lds_wait(f0);
-  int st = 0;                                      // stage of the current K tile
   for (; tile < total_tiles; tile += gdim) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
