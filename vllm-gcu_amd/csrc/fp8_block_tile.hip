@@ -302,6 +302,23 @@ fp8_block_gemm_kernel(F8Args a) {
   lds_wait(o0, w3a);
   __builtin_amdgcn_s_barrier();                    // nobody still reads element 0 when step 0 overwrites its stage
   int st = 0;                                      // stage of the current element
+  // One row tile in all (M <= 256) and none of its rows in this wavefront's share: the wavefront only
+  // copies.  It keeps the workgroup's barriers and its own copy slots, and leaves the matrix pipe and
+  // the LDS read port of its SIMD to the wavefront that has rows (65 .. 128 rows: half the wavefronts).
+  if (mtiles == 1 && wm * (16 * NJ) >= M) {
+    for (; tile < total_tiles; tile += gdim) {
+      for (int T = 0; T < nt; ++T) {
+        const int kt = ahead_kt(T, 3);
+#pragma unroll
+        for (int s = 0; s < NSLOT; ++s) copy_slot(s, st, kt);
+        wait_all_but_last_step();
+        __builtin_amdgcn_s_barrier();
+        st = st == 2 ? 0 : st + 1;
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);            // vmcnt(0)
+    return;
+  }
   for (; tile < total_tiles; tile += gdim) {
     int m0, n0;
     tile_origin(tile, m0, n0);
@@ -448,7 +465,8 @@ extern "C" int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, c
                        (size_t)128 * (size_t)(kslab ? K : ldw) < ((size_t)1 << 32);
   const bool stream_ok = ldx == K && (kslab || ldw == K) && ldo == N && (size_t)N * K * 2 < ((size_t)1 << 32) &&
                          (size_t)M * K * 2 < ((size_t)1 << 32);
-  if (tile_ok && ((M > 64 && tiles >= 64) || !stream_ok)) {
+  // (from 41 rows on layers of 128 tiles or more: the wavefronts without rows only copy there)
+  if (tile_ok && ((M > 64 && tiles >= 64) || (M > 40 && tiles >= 128) || !stream_ok)) {
     F8Args a;
     a.out = out; a.x = (const uint8_t*)x; a.w = (const uint8_t*)w; a.x_scale = x_scale; a.w_scale = w_scale;
     a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;

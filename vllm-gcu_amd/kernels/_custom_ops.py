@@ -285,7 +285,10 @@ def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
             bias = bias.to(torch.float32)
             bias_f32 = 1
         bias = bias.contiguous()
-    if ldw == 0 and M <= _INT8_STREAM_MAX_M and acc_out is None and ws_col and (xs is None or xs_row or M == 1) \
+    # (49..64 rows on a layer of 128 column tiles or more go to the MFMA kernel, whose wavefronts without rows
+    # only copy: K 8192 x N 28672 at M = 56 / 64: 52.5 / 55.5 -> 49.4 / 49.1 us)
+    stream_rows = _INT8_STREAM_MAX_M * 3 // 4 if N >= 128 * 128 and N % 128 == 0 else _INT8_STREAM_MAX_M
+    if ldw == 0 and M <= stream_rows and acc_out is None and ws_col and (xs is None or xs_row or M == 1) \
             and not bias_f32 and out.dtype in (torch.float16, torch.bfloat16) and x2.is_contiguous() \
             and out2.stride(0) == N:
         # decode-sized M on kslab weights: the weight-streaming kernel (same int32 sums, same
@@ -1186,7 +1189,10 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
         raise RuntimeError("linear_quant: operands must be float8_e4m3fn")
     M, N, K = lhs.numel() // lhs.shape[-1], rhs.shape[0], lhs.shape[-1]
     tiles = -(-M // 256) * (N // 128)               # 256 x 128 output tiles, one workgroup each
-    if M > _FP8_TILE_MIN_M and tiles >= _FP8_TILE_MIN_TILES and N % 128 == 0 and K % 128 == 0 \
+    # (from 41 rows on a layer of 128 tiles or more: the tile kernel's wavefronts without rows only copy,
+    # K 8192 x N 28672 at M = 48 / 64: 59.6 / 68.4 -> 52.9 / 55.1 us; 112 tiles: the streamer stays ahead)
+    if ((M > _FP8_TILE_MIN_M and tiles >= _FP8_TILE_MIN_TILES) or (M > _FP8_TILE_MIN_M * 5 // 8 and tiles >= 2 * _FP8_TILE_MIN_TILES)) \
+            and N % 128 == 0 and K % 128 == 0 \
             and out.dtype in (torch.float16, torch.bfloat16) \
             and rhs.dim() == 2 and rhs.is_contiguous() and out.is_contiguous():
         # prefill-sized M: the MFMA tile kernel (the weight-streaming kernel re-reads the weights per 64 rows)
