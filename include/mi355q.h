@@ -167,6 +167,20 @@ int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* x, const in
                           const float* x_scale, int x_scale_per_row, const float* w_scale,
                           int w_scale_per_col, const void* bias, int bias_f32, int M, int N, int K,
                           long ldx, long ldw, long ldo, int out_dtype, void* stream);
+/* The same with a workspace (no counterpart in the reference: the vendor GEMM chooses its own launch).
+ * A layer with few 256 x 128 output tiles (N of 4096 .. 10240 at up to a few hundred rows) leaves
+ * most of the chip idle behind a long K; with mi355q_w8a8_int8_workspace_bytes(M, N, K) bytes of
+ * workspace (0 = this shape is not split) K is cut into ranges that run side by side, and a second
+ * launch adds their int32 sums and applies the scales and the bias: integer sums, so the result --
+ * acc_out included -- is bit for bit that of the call without workspace.  The workspace follows the
+ * rules of mi355q_w4a16_gemm's (its first MiB is left alone, so one buffer serves both); without
+ * one, or with a smaller one, the unsplit launch runs. */
+size_t mi355q_w8a8_int8_workspace_bytes(int M, int N, int K);
+int mi355q_w8a8_int8_gemm_ws(void* out, int32_t* acc_out, const int8_t* x, const int8_t* w,
+                             const float* x_scale, int x_scale_per_row, const float* w_scale,
+                             int w_scale_per_col, const void* bias, int bias_f32, int M, int N, int K,
+                             long ldx, long ldw, long ldo, int out_dtype, void* workspace,
+                             size_t workspace_bytes, void* stream);
 /* Replaces topsvllmDynamicScaledInt8Quant (csrc/src/dynamic_scaled_int8_quant.cpp:12-19):
  * per row scale = absmax / 127 (fp32 [M]), q = sat_s8(rne(x * (127 / absmax))).
  * valid_rows (optional device int32[1]) limits the rows processed. */

@@ -103,6 +103,42 @@ def test_int8_gemm_kslab_weights(ops, M, K, N):
         np.testing.assert_allclose(a.float().cpu().numpy(), wantf, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("M,K,N,splits", [(128, 4096, 1024, 4), (200, 8192, 512, 8), (700, 2048, 1024, 2),
+                                            (64, 14336, 4096, 8), (1000, 3072, 768, 3)])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_int8_gemm_split_k_is_bit_identical(ops, M, K, N, splits, out_dtype):
+    """Few output tiles behind a long K: the operator cuts K into ranges that run side by side (int32
+    partial sums in the stream's workspace, a second launch adds them and applies scales and bias).
+    Integer sums: outputs and raw accumulators equal those of the entry point without workspace bit
+    for bit, and the accumulators equal the oracle's."""
+    from vllm_gcu_amd import _lib
+    from vllm_gcu_amd.kernels import _runtime as rt
+    print(f"case i8 split K {M}x{K}x{N} {out_dtype}", flush=True)
+    lib = _lib.load()
+    need = lib.mi355q_w8a8_int8_workspace_bytes(M, N, K)
+    assert need == (1 << 20) + splits * M * N * 4              # the plan this test was written for
+    rng = np.random.default_rng(M + K + N)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    xs = rng.uniform(0.001, 0.01, size=(M, 1)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(out_dtype).cuda()
+    xd, wd, xsd, wsd = dev(x), dev(w_nk), dev(xs).reshape(-1), dev(ws)
+    got = ops.cutlass_scaled_mm(xd, wd.t(), dev(xs), wsd, out_dtype, bias)
+    acc = ops.int8_gemm_accumulators(xd, wd.t())
+    assert np.array_equal(acc.cpu().numpy(), o8.int8_gemm_i32(x, np.ascontiguousarray(w_nk.T)))
+    ref = torch.empty(M, N, dtype=out_dtype, device="cuda")
+    ref_acc = torch.empty(M, N, dtype=torch.int32, device="cuda")
+    with torch.cuda.device(0):
+        _lib.call("mi355q_w8a8_int8_gemm", ref.data_ptr(), ref_acc.data_ptr(), xd.data_ptr(), wd.data_ptr(),
+                  xsd.data_ptr(), 1, wsd.data_ptr(), 1, bias.data_ptr(), 0, M, N, K, K, K, N,
+                  rt.dtype_code(out_dtype), rt.stream_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(acc, ref_acc)
+    assert torch.equal(got, ref)
+    assert torch.equal(got, ops.cutlass_scaled_mm(xd, wd.t(), dev(xs), wsd, out_dtype, bias))
+
+
 @pytest.mark.parametrize("M,N", [(2305, 2048), (4200, 1792), (2049, 4096)])
 def test_int8_gemm_more_than_eight_row_tiles(ops, M, N):
     # above 2048 rows the XCD-aware tile order walks the row tiles in chunks of eight (with a

@@ -35,6 +35,10 @@ SIGNATURES = {
     "mi355q_w8a8_int8_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                       c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_int,
                                       c_void_p]),
+    "mi355q_w8a8_int8_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "mi355q_w8a8_int8_gemm_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                         c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_int,
+                                         c_void_p, c_size_t, c_void_p]),
     "mi355q_fp8_block_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                       c_int, c_long, c_long, c_long, c_int, c_void_p]),
     "mi355q_fp8_scaled_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
@@ -69,7 +73,7 @@ SIGNATURES = {
 }
 
 # must equal mi355q_abi_version() of the library (csrc/core.hip)
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 

@@ -61,6 +61,20 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   return bitcast<uint16_t>((__bf16)f);
 }
 
+// Epilogue of the scaled integer / fp8 GEMMs, (sum * x_scale) * w_scale (+ bias), with every operation
+// rounded on its own: left to the compiler's contraction rules the multiply-add pairs fuse in some
+// kernels (and in some paths of one kernel) and not in others, and kernels that must agree bit for bit
+// -- the tile kernels, the weight-streaming kernels, the split-K epilogue -- would differ in the last place.
+__device__ __forceinline__ float scaled_sum(float sum, float x_scale, float w_scale) {
+#pragma clang fp contract(off)
+  const float t = sum * x_scale;
+  return t * w_scale;
+}
+__device__ __forceinline__ float plus_bias(float v, float bias) {
+#pragma clang fp contract(off)
+  return v + bias;
+}
+
 template <int DT> struct Elem;            // activation element traits
 template <> struct Elem<MI355Q_F16> {
   typedef _Float16 type;

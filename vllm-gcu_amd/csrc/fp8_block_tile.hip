@@ -381,7 +381,7 @@ fp8_block_gemm_kernel(F8Args a) {
         const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = (PC ? (acc[i][j][e] * xsc) * wsc[i][e] : acc[i][j][e]) + bia[i][e];
+        for (int e = 0; e < 4; ++e) v[e] = plus_bias(PC ? scaled_sum(acc[i][j][e], xsc, wsc[i][e]) : acc[i][j][e], bia[i][e]);
         u2 o;
         o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
         o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);

@@ -442,10 +442,10 @@ kcontig_gemm_kernel(KcArgs a) {
         if (wide && n >= N) { v[e] = 0.f; continue; }
         if (MODE == KC_INT8) {
           const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + (n + e) * a.sc_col];
-          v[e] = ((float)bitcast<i4>(KS ? fin[j] : acc[i][j])[e] * xs) * ws;
+          v[e] = scaled_sum((float)bitcast<i4>(KS ? fin[j] : acc[i][j])[e], xs, ws);
         } else if (MODE == KC_FP8_PC) {
           const float ws = ((const float*)a.w_scale)[expert * a.ws_stride + (n + e) * a.sc_col];
-          v[e] = (bitcast<f4>(KS ? fin[j] : acc[i][j])[e] * xs) * ws;
+          v[e] = scaled_sum(bitcast<f4>(KS ? fin[j] : acc[i][j])[e], xs, ws);
         } else if ((W8H || W8B) && !GW) {
           const uint16_t raw = ((const uint16_t*)a.w_scale)[expert * a.ws_stride + n + e];
           const float ws = W8H ? Elem<MI355Q_F16>::to_f32(raw) : Elem<MI355Q_BF16>::to_f32(raw);
@@ -454,7 +454,7 @@ kcontig_gemm_kernel(KcArgs a) {
           v[e] = bitcast<f4>(KS ? fin[j] : acc[i][j])[e];
         }
         v[e] *= rw;
-        if (!GROUPED && a.bias) v[e] += Elem<ODT>::to_f32(((const uint16_t*)a.bias)[n + e]);
+        if (!GROUPED && a.bias) v[e] = plus_bias(v[e], Elem<ODT>::to_f32(((const uint16_t*)a.bias)[n + e]));
       }
       u2 o;
       o.x = (uint32_t)Elem<ODT>::from_f32(v[0]) | ((uint32_t)Elem<ODT>::from_f32(v[1]) << 16);

@@ -40,6 +40,8 @@ struct I8Args {
   int n_panels_swizzle;     // non-zero: XCD-aware tile order
   int w_kslab;              // w is in the kslab order (see include/mi355q.h) instead of row-major
   int wide_stores;          // N, ldo and the output address allow 16-byte stores of 8 adjacent 16-bit outputs
+  int ksplits;              // > 1: every output tile is worked on by `ksplits` workgroups, each a K range of its own,
+  int32_t* partial;         //      which leave their int32 sums in partial[split][M][N]; the epilogue is a second launch
 };
 
 template <int DT>
@@ -93,10 +95,15 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // of the same weight panels.
   const int mtiles = (M + TM - 1) / TM;
   const int ntiles_n = (N + TN - 1) / TN;
-  const int total_tiles = mtiles * ntiles_n;
+  const int ksplits = a.ksplits > 1 ? a.ksplits : 1;
+  const int total_tiles = mtiles * ntiles_n * ksplits;   // (split K: tile ids count (output tile, K range) pairs)
   auto tile_origin = [&](int tile, int& m0, int& n0) {
     int tm, tn;
-    if (a.n_panels_swizzle) {
+    if (ksplits > 1) {
+      const int t = tile / ksplits;
+      tm = t % mtiles;
+      tn = t / mtiles;
+    } else if (a.n_panels_swizzle) {
       // XCD x takes the weight panels tn = x, x + 8, ...; it sweeps them for a chunk of 8 row tiles
       // (2048 rows of x: what its L2 can keep warm next to a panel) before the next chunk
       const int x = tile & 7, j = tile >> 3;
@@ -155,8 +162,10 @@ w8a8_int8_gemm_kernel(I8Args a) {
         wo[p] = (uint32_t)((min(n0 + r, N - 1) - n0) * a.ldw + 16 * cchunk);
       }
     }
-    xtile = a.x + (long)m0 * a.ldx;
-    wtile = a.w_kslab ? a.w : a.w + (long)n0 * a.ldw;
+    // (split K: the tile's K range starts kbeg bytes into every row; 64 kslab rows interleave their K tiles)
+    const long kbeg = ksplits > 1 ? (long)(tile % ksplits) * (K / ksplits) : 0;
+    xtile = a.x + (long)m0 * a.ldx + kbeg;
+    wtile = a.w_kslab ? a.w + kbeg * 64 : a.w + (long)n0 * a.ldw + kbeg;
   };
   // copy slot s of this wavefront: slots 0 .. XCOPIES-1 are its x row groups,
   // the rest its w row groups (the last one only exists for some wavefronts)
@@ -274,7 +283,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // output tile arrive while the epilogue of this one runs; past the last
   // output tile the copies re-read its last K tile into a stage nobody reads.
   static_assert(STAGES == 2 || (WCOPIES * 8 == WGROUPS && NSLOT == 6), "the three-stage wait counts six copies per wavefront and element");
-  const int nt = K / TKB;
+  const int nt = K / TKB / ksplits;                // K tiles per (output tile, K range)
   // (kept in a register: read through the dispatch packet it is fetched again in every iteration)
   const int gdim = __builtin_amdgcn_readfirstlane((int)gridDim.x);
   int tile = blockIdx.x;
@@ -342,6 +351,24 @@ w8a8_int8_gemm_kernel(I8Args a) {
     // would each wait out a full memory round trip.
     int m0, n0;
     tile_origin(tile, m0, n0);
+    if (ksplits > 1) {
+      // split K: the int32 sums of this K range, nothing else; scales and bias are the second launch's
+      int32_t* const part = a.partial + (long)(tile % ksplits) * M * N;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+          if (n < N) *(i4*)(part + (long)m * N + n) = acc[i][j];
+        }
+      }
+      if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f70);
+      read_frag(f0, st, 0);
+      lds_wait(f0);
+      continue;
+    }
     float xsc[NJ];
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -371,8 +398,8 @@ w8a8_int8_gemm_kernel(I8Args a) {
       auto scaled = [&](int i, float* v) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          v[e] = ((float)acc[i][j][e] * xsc[j]) * wsc[i][e];
-          if (a.bias) v[e] += bia[i][e];
+          v[e] = scaled_sum((float)acc[i][j][e], xsc[j], wsc[i][e]);
+          if (a.bias) v[e] = plus_bias(v[e], bia[i][e]);
         }
       };
 #pragma unroll
@@ -544,7 +571,8 @@ int launch_tile(const I8Args& a, hipStream_t st) {
   constexpr int TN = WN * NI * 16;
   const int mtiles = (a.M + TM - 1) / TM, ntiles = (a.N + TN - 1) / TN;
   I8Args b = a;
-  b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
+  const int ks = a.ksplits > 1 ? a.ksplits : 1;
+  b.n_panels_swizzle = (ntiles % 8 == 0 && ks == 1) ? 1 : 0;
   const size_t stage = (size_t)(TM + TN) * TKB;
   const size_t shmem = (3 * stage <= 160 * 1024 ? 3 : 2) * stage;   // 144 KiB (three stages), 120 or 128 KiB (two)
   static hipError_t attr = hipFuncSetAttribute((const void*)w8a8_int8_gemm_kernel<DT, WM, WN, NI, NJ>,
@@ -552,7 +580,7 @@ int launch_tile(const I8Args& a, hipStream_t st) {
   MQ_REQUIRE(attr == hipSuccess, "w8a8_int8_gemm: cannot reserve %zu bytes of LDS: %s", shmem,
              hipGetErrorString(attr));
   // one workgroup per CU (a multiple of 8, so tile id mod 8 stays the XCD)
-  int grid = mtiles * ntiles, cus = device_cu_count() / 8 * 8;
+  int grid = mtiles * ntiles * ks, cus = device_cu_count() / 8 * 8;
   if (cus >= 8 && grid > cus) grid = cus;
   hipLaunchKernelGGL((w8a8_int8_gemm_kernel<DT, WM, WN, NI, NJ>), dim3(grid), dim3(GEMM_THREADS), shmem, st, b);
   MQ_LAUNCH_CHECK("w8a8_int8_gemm");
@@ -571,6 +599,60 @@ int launch_columns(const I8Args& a, int n0, int n1, hipStream_t st) {
   b.out = (char*)a.out + (size_t)n0 * (DT == MI355Q_F32 ? 4 : 2);
   if (a.acc_out) b.acc_out = a.acc_out + n0;
   return launch_tile<DT, WM, WN, NI, NJ>(b, st);
+}
+
+// ---- split K -----------------------------------------------------------------------------------
+// A layer with few output tiles (N 4096 .. 10240 at a few hundred rows) leaves most CUs without a
+// tile while the others walk a long K.  The sums are integers, so K can be cut into ranges whose
+// int32 sums add up exactly: the result is bit for bit that of the unsplit launch.  Second launch:
+// sum of the ranges, then the epilogue of the GEMM kernel in its order of operations.
+template <int DT>
+__global__ void __launch_bounds__(256)
+w8a8_splitk_epilogue_kernel(I8Args a) {
+  const long q = (long)blockIdx.x * 256 + threadIdx.x;     // 4 adjacent columns of one row
+  const int nq = a.N / 4;
+  if (q >= (long)a.M * nq) return;
+  const int m = (int)(q / nq), n = (int)(q % nq) * 4;
+  i4 acc = {0, 0, 0, 0};
+  for (int s = 0; s < a.ksplits; ++s) acc += *(const i4*)(a.partial + ((long)s * a.M + m) * a.N + n);
+  if (a.acc_out) *(i4*)(a.acc_out + (long)m * a.ldacc + n) = acc;
+  const float xsc = a.x_scale ? a.x_scale[a.x_scale_per_row ? m : 0] : 1.0f;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float wsc = a.w_scale ? a.w_scale[a.w_scale_per_col ? n + e : 0] : 1.0f;
+    v[e] = scaled_sum((float)acc[e], xsc, wsc);
+    if (a.bias) v[e] = plus_bias(v[e], load_bias<DT>(a.bias, a.bias_f32, n + e));
+  }
+  store4<DT>(a.out, (long)m * a.ldo + n, v);
+}
+
+constexpr size_t I8_SPLITK_BYTES = (size_t)64 << 20;
+constexpr size_t I8_WS_OFFSET = (size_t)1 << 20;     // the first MiB of a workspace belongs to the W4A16 arrival counters
+
+// K ranges for a shape: as many as put about one 256 x 128 tile on every CU, each at least eight K
+// tiles long, a divisor of the K tile count, partial sums within 64 MiB.  1: no split.
+int int8_ksplits(int M, int N, int K) {
+  const long cus = device_cu_count(), tiles = (long)((M + TM - 1) / TM) * ((N + 127) / 128);
+  const int nt = K / TKB;
+  if (N % 4 != 0 || tiles * 2 > cus) return 1;
+  long s = cus / tiles;
+  if (s > 8) s = 8;
+  if (s > nt / 8) s = nt / 8;
+  while (s > 1 && (nt % s != 0 || (size_t)s * M * N * sizeof(int32_t) > I8_SPLITK_BYTES)) --s;
+  return s < 1 ? 1 : (int)s;
+}
+
+template <int DT>
+int launch_gemm_splitk(const I8Args& a, int splits, void* workspace, hipStream_t st) {
+  I8Args b = a;
+  b.ksplits = splits;
+  b.partial = (int32_t*)((char*)workspace + I8_WS_OFFSET);
+  if (int rc = launch_tile<DT, 4, 2, 4, 4>(b, st)) return rc;
+  const long quads = (long)a.M * (a.N / 4);
+  hipLaunchKernelGGL((w8a8_splitk_epilogue_kernel<DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, b);
+  MQ_LAUNCH_CHECK("w8a8_int8_gemm(split-K epilogue)");
+  return 0;
 }
 
 // Tile width.  One workgroup per CU works through the output tiles in rounds; a last round that is
@@ -624,10 +706,25 @@ int launch_gemm(const I8Args& a, hipStream_t st) {
 
 using namespace mi355q;
 
+extern "C" size_t mi355q_w8a8_int8_workspace_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  const int s = int8_ksplits(M, N, K);
+  return s > 1 ? I8_WS_OFFSET + (size_t)s * M * N * sizeof(int32_t) : 0;
+}
+
 extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* x, const int8_t* w,
                                      const float* x_scale, int x_scale_per_row, const float* w_scale,
                                      int w_scale_per_col, const void* bias, int bias_f32, int M, int N,
                                      int K, long ldx, long ldw, long ldo, int out_dtype, void* stream) {
+  return mi355q_w8a8_int8_gemm_ws(out, acc_out, x, w, x_scale, x_scale_per_row, w_scale, w_scale_per_col, bias, bias_f32,
+                                  M, N, K, ldx, ldw, ldo, out_dtype, nullptr, 0, stream);
+}
+
+extern "C" int mi355q_w8a8_int8_gemm_ws(void* out, int32_t* acc_out, const int8_t* x, const int8_t* w,
+                                        const float* x_scale, int x_scale_per_row, const float* w_scale,
+                                        int w_scale_per_col, const void* bias, int bias_f32, int M, int N,
+                                        int K, long ldx, long ldw, long ldo, int out_dtype, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
   MQ_REQUIRE(M >= 0 && N > 0 && K > 0, "w8a8_int8_gemm: bad shape M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
   MQ_REQUIRE(out && x && w, "w8a8_int8_gemm: null pointer");
@@ -647,6 +744,14 @@ extern "C" int mi355q_w8a8_int8_gemm(void* out, int32_t* acc_out, const int8_t* 
   a.n_panels_swizzle = 0;
   a.w_kslab = kslab ? 1 : 0;
   a.wide_stores = (N % 8 == 0 && ldo % 8 == 0 && ((size_t)out & 15) == 0) ? 1 : 0;
+  a.ksplits = 1;
+  a.partial = nullptr;
+  const int splits = int8_ksplits(M, N, K);
+  if (splits > 1 && workspace && workspace_bytes >= I8_WS_OFFSET + (size_t)splits * M * N * sizeof(int32_t)) {
+    if (out_dtype == MI355Q_F16) return launch_gemm_splitk<MI355Q_F16>(a, splits, workspace, as_stream(stream));
+    if (out_dtype == MI355Q_BF16) return launch_gemm_splitk<MI355Q_BF16>(a, splits, workspace, as_stream(stream));
+    return launch_gemm_splitk<MI355Q_F32>(a, splits, workspace, as_stream(stream));
+  }
   if (out_dtype == MI355Q_F16) return launch_gemm<MI355Q_F16>(a, as_stream(stream));
   if (out_dtype == MI355Q_BF16) return launch_gemm<MI355Q_BF16>(a, as_stream(stream));
   return launch_gemm<MI355Q_F32>(a, as_stream(stream));

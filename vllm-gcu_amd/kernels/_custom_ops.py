@@ -229,6 +229,27 @@ def _gptq_gemm_gcu_fake(a, b_q_weight, b_gptq_qzeros, b_gptq_scales, b_g_idx, bi
 _INT8_STREAM_MAX_M = 64      # measured on MI355X (K 8192, N 28672): 40-51 us against 90 us for the MFMA tile kernel
 
 
+def _int8_stream_rows(K: int, N: int) -> int:
+    """Up to how many rows the weight-streaming kernel takes a kslab layer (measured on MI355X, us,
+    streaming / MFMA tile kernel).  The tile kernel's wavefronts without rows only copy, and on layers of
+    at most 128 column tiles it cuts K into ranges that fill the chip:
+    a long K behind a narrow N (down projections) is its case from a handful of rows on --
+    28672 x 8192: M = 16 52.7 / 48.2, M = 64 82.6 / 50.7; 14336 x 4096: M = 16 25.2 / 19.7, M = 64 42.1 / 21.0;
+    square layers from about 40 rows -- 8192 x 8192: M = 32 20.2 / 20.6, M = 48 23.8 / 21.3;
+    wide layers (128 column tiles or more, no split) from 49 -- 8192 x 28672: M = 48 49.4 / 49.9, M = 64 55.3 / 50.8;
+    a short K in front of a wide N stays with the streaming kernel -- 4096 x 14336: M = 64 18.1 / 21.4."""
+    top = _INT8_STREAM_MAX_M
+    if N % 128 != 0:
+        return top
+    if N >= 128 * 128:
+        return top * 3 // 4
+    if K >= 2 * N:
+        return top // 8
+    if K >= N:
+        return top * 5 // 8
+    return top
+
+
 def _int8_weight_nk(weight: torch.Tensor):
     """-> (tensor whose memory is [N, K] K-contiguous, row stride in bytes).
 
@@ -285,9 +306,7 @@ def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
             bias = bias.to(torch.float32)
             bias_f32 = 1
         bias = bias.contiguous()
-    # (49..64 rows on a layer of 128 column tiles or more go to the MFMA kernel, whose wavefronts without rows
-    # only copy: K 8192 x N 28672 at M = 56 / 64: 52.5 / 55.5 -> 49.4 / 49.1 us)
-    stream_rows = _INT8_STREAM_MAX_M * 3 // 4 if N >= 128 * 128 and N % 128 == 0 else _INT8_STREAM_MAX_M
+    stream_rows = _int8_stream_rows(K, N)
     if ldw == 0 and M <= stream_rows and acc_out is None and ws_col and (xs is None or xs_row or M == 1) \
             and not bias_f32 and out.dtype in (torch.float16, torch.bfloat16) and x2.is_contiguous() \
             and out2.stride(0) == N:
@@ -298,9 +317,13 @@ def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
                       rt.ptr(bias), _lib.Q_INT8, 0, M, K, N, _lib.F16, rt.dtype_code(out.dtype), 1, rt.stream_ptr())
         return
     with torch.cuda.device(x.device):
-        _lib.call("mi355q_w8a8_int8_gemm", out2.data_ptr(), rt.ptr(acc_out), x2.data_ptr(), w.data_ptr(),
+        # (few output tiles behind a long K: K ranges side by side through the stream's workspace, bit-identical)
+        need = _lib.load().mi355q_w8a8_int8_workspace_bytes(M, N, K)
+        wsp = rt.workspace(x.device, need) if need else None
+        _lib.call("mi355q_w8a8_int8_gemm_ws", out2.data_ptr(), rt.ptr(acc_out), x2.data_ptr(), w.data_ptr(),
                   rt.ptr(xs), xs_row, rt.ptr(ws), ws_col, rt.ptr(bias), bias_f32, M, N, K,
-                  x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.stream_ptr())
+                  x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.ptr(wsp),
+                  0 if wsp is None else wsp.numel(), rt.stream_ptr())
 
 
 def _scaled_fp8_mm(out, x, weight, x_scale, w_scale, bias):
