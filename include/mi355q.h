@@ -148,6 +148,24 @@ int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, const float*
                            int x_scale_per_row, const float* w_scale, int w_scale_per_col,
                            const void* bias, int M, int N, int K, long ldx, long ldw, long ldo,
                            int out_dtype, void* stream);
+/* The two fp8 GEMMs with a workspace (no counterpart in the reference: the vendor GEMM chooses its own
+ * launch).  A layer with few 256 x 128 output tiles behind a long K leaves most of the chip idle; with
+ * mi355q_fp8_gemm_workspace_bytes(M, N, K) bytes (0 = this shape is not split; below 65 rows it is not 0
+ * only where the split launch is ahead of the weight-streaming kernel) K is cut into ranges of
+ * whole K blocks that run side by side, and a second launch adds their fp32 sums in range order and
+ * applies bias (and, for the scaled GEMM, the scales): run-to-run identical, and equal to the unsplit
+ * launch up to the order of the fp32 additions.  The workspace follows the rules of
+ * mi355q_w4a16_gemm's (its first MiB is left alone); without one, or with a smaller one, the unsplit
+ * launch (or, for the scaled GEMM on few tiles, the streaming kernel) runs. */
+size_t mi355q_fp8_gemm_workspace_bytes(int M, int N, int K);
+int mi355q_fp8_block_gemm_ws(void* out, const void* x, const void* w, const float* x_scale,
+                             const float* w_scale, const void* bias, int M, int N, int K, long ldx,
+                             long ldw, long ldo, int out_dtype, void* workspace, size_t workspace_bytes,
+                             void* stream);
+int mi355q_fp8_scaled_gemm_ws(void* out, const void* x, const void* w, const float* x_scale,
+                              int x_scale_per_row, const float* w_scale, int w_scale_per_col,
+                              const void* bias, int M, int N, int K, long ldx, long ldw, long ldo,
+                              int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- W8A8 int8 -------------------------------------------------------------
  * Replaces topsatenDotBiasQuant as called by cutlass_scaled_mm

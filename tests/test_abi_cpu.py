@@ -27,7 +27,7 @@ def test_header_symbols_exported_and_bound():
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     for n in _lib.SIGNATURES:
         assert n in names, f"{n} bound in _lib.py but not declared in mi355q.h"
-    assert lib.mi355q_abi_version() == _lib.ABI_VERSION == 4
+    assert lib.mi355q_abi_version() == _lib.ABI_VERSION == 5
 
 
 def test_argument_errors_are_reported_without_gpu():

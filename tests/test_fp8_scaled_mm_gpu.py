@@ -113,6 +113,54 @@ def test_equals_block_scaled_gemm_when_block_scales_are_constant():
         assert (pc.float() - blk.float()).abs().max().item() <= 2 ** -7 * max(1.0, float(np.abs(want).max()))
 
 
+@pytest.mark.parametrize("M,K,N", [(128, 4096, 1024), (300, 8192, 512), (700, 2048, 1024), (65, 7168, 1536),
+                                   (17, 7168, 1536), (25, 7168, 4096), (49, 4096, 1024)])
+@pytest.mark.parametrize("kslab", [False, True])
+def test_few_tiles_behind_a_long_k_are_split_into_k_ranges(M, K, N, kslab):
+    """Both fp8 tile kernels on layers with few 256 x 128 tiles: K ranges run side by side, their fp32 sums
+    go through the stream's workspace and a second launch adds them in range order and applies bias and
+    scales.  Against the oracle, run-to-run identical, and within fp32 accuracy of the entry points
+    without workspace (same products, another order of additions)."""
+    from vllm_gcu_amd import _lib
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    from vllm_gcu_amd.kernels import _runtime as rt
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print(f"case fp8 split K M={M} K={K} N={N} kslab={kslab}", flush=True)
+    lib = _lib.load()
+    assert lib.mi355q_fp8_gemm_workspace_bytes(M, N, K) > (1 << 20)        # a split plan exists for this shape
+    if M < 64:                                                              # ... and none one row below its first height
+        assert lib.mi355q_fp8_gemm_workspace_bytes(M - 1, N, K) == 0
+    rng = np.random.default_rng(M + K + N)
+    xq, xs, w, ws = _operands(rng, M, K, N)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.bfloat16).cuda()
+    xd = dev(xq).view(torch.float8_e4m3fn)
+    wd = dev(w).view(torch.float8_e4m3fn)
+    wk = rearrange.to_kslab(wd) if kslab else wd
+    # per-token x per-channel scales
+    got = ops.cutlass_scaled_mm(xd, wk.t(), dev(xs).reshape(M, 1), dev(ws).reshape(N, 1), torch.bfloat16, bias)
+    assert torch.equal(got, ops.cutlass_scaled_mm(xd, wk.t(), dev(xs).reshape(M, 1), dev(ws).reshape(N, 1), torch.bfloat16, bias))
+    want = of8.scaled_fp8_mm(xq, xs, w, ws, bias.float().cpu().numpy())
+    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    ref = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    xsd, wsd = dev(xs), dev(ws)
+    with torch.cuda.device(0):
+        _lib.call("mi355q_fp8_scaled_gemm", ref.data_ptr(), xd.data_ptr(), wk.data_ptr(), xsd.data_ptr(), 1,
+                  wsd.data_ptr(), 1, bias.data_ptr(), M, N, K, K, 0 if kslab else K, N, rt.dtype_code(torch.bfloat16),
+                  rt.stream_ptr())
+    torch.cuda.synchronize()
+    assert (got.float() - ref.float()).abs().max().item() <= 2 ** -7 * max(1.0, float(np.abs(want).max()))
+    # 128 x 128 block scales
+    xsb = rng.uniform(0.01, 0.05, size=(M, K // 128)).astype(np.float32)
+    wsb = rng.uniform(0.01, 0.05, size=(N // 128, K // 128)).astype(np.float32)
+    blk = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(blk, xd, wk, bias, dev(xsb), dev(wsb))
+    blk2 = torch.empty_like(blk)
+    torch.ops._C.linear_quant(blk2, xd, wk, bias, dev(xsb), dev(wsb))
+    assert torch.equal(blk, blk2)
+    wantb = of8.block_fp8_gemm(xq, xsb, w, wsb, bias=bias.float().cpu().numpy())
+    np.testing.assert_allclose(blk.float().cpu().numpy(), wantb, rtol=RTOL, atol=RTOL * max(1.0, float(np.abs(wantb).max())))
+
+
 @pytest.mark.parametrize("M", [1, 16, 128, 2048])
 def test_full_size_layer_sampled(M):
     """K = 8192, N = 28672 (one Llama-3-70B MLP projection): sampled rows and columns against the oracle, the whole

@@ -43,6 +43,11 @@ SIGNATURES = {
                                       c_int, c_long, c_long, c_long, c_int, c_void_p]),
     "mi355q_fp8_scaled_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                        c_int, c_int, c_long, c_long, c_long, c_int, c_void_p]),
+    "mi355q_fp8_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "mi355q_fp8_block_gemm_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                         c_int, c_long, c_long, c_long, c_int, c_void_p, c_size_t, c_void_p]),
+    "mi355q_fp8_scaled_gemm_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                          c_int, c_int, c_long, c_long, c_long, c_int, c_void_p, c_size_t, c_void_p]),
     "mi355q_dynamic_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi355q_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355q_silu_mul_static_int8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_void_p]),
@@ -73,7 +78,7 @@ SIGNATURES = {
 }
 
 # must equal mi355q_abi_version() of the library (csrc/core.hip)
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib = None
 

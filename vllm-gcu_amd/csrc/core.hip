@@ -34,4 +34,4 @@ int device_cu_count() {
 extern "C" const char* mi355q_last_error(void) { return mi355q::g_err; }
 // bumped whenever an entry point changes its arguments: the Python binding refuses a library of another version
 // (a stale build would be called with shifted arguments)
-extern "C" int mi355q_abi_version(void) { return 4; }
+extern "C" int mi355q_abi_version(void) { return 5; }

@@ -44,6 +44,8 @@ struct F8Args {
   long ldx, ldw, ldo;
   int w_kslab;
   int n_panels_swizzle;
+  int ksplits;              // > 1: every output tile is worked on by `ksplits` workgroups, each a range of K blocks,
+  float* partial;           //      which leave their fp32 sums in partial[split][M][N]; the epilogue is a second launch
 };
 
 __device__ __forceinline__ void dma16(const void* gptr, void* lds_wave_base) {
@@ -74,10 +76,15 @@ fp8_block_gemm_kernel(F8Args a) {
 
   const int mtiles = (M + FTM - 1) / FTM;
   const int ntiles_n = N / FTN;
-  const int total_tiles = mtiles * ntiles_n;
+  const int ksplits = a.ksplits > 1 ? a.ksplits : 1;
+  const int total_tiles = mtiles * ntiles_n * ksplits;   // (split K: tile ids count (output tile, K range) pairs)
   auto tile_origin = [&](int tile, int& m0, int& n0) {
     int tm, tn;
-    if (a.n_panels_swizzle) {
+    if (ksplits > 1) {
+      const int t = tile / ksplits;
+      tm = t % mtiles;
+      tn = t / mtiles;
+    } else if (a.n_panels_swizzle) {
       // XCD x takes the weight panels tn = x, x + 8, ...; it sweeps them for a chunk of 8 row tiles
       // (2048 rows of x: what its L2 can keep warm next to a panel) before the next chunk
       const int x = tile & 7, j = tile >> 3;
@@ -130,10 +137,12 @@ fp8_block_gemm_kernel(F8Args a) {
       }
     }
     // activation scales: wavefronts 0..3 copy 64 rows each (index in floats)
-    xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB;
-    wsbase = (n0 >> 7) * KB;                       // wavefront 4 copies the tile's weight scale
-    xtile = a.x + (long)m0 * a.ldx;
-    wtile = a.w_kslab ? a.w : a.w + (long)n0 * a.ldw;
+    // (split K: the tile's range starts kb0 K blocks into every row; 64 kslab rows interleave their K blocks)
+    const int kb0 = ksplits > 1 ? (tile % ksplits) * (KB / ksplits) : 0;
+    xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB + (uint32_t)kb0;
+    wsbase = (n0 >> 7) * KB + kb0;                 // wavefront 4 copies the tile's weight scale
+    xtile = a.x + (long)m0 * a.ldx + (long)kb0 * FTKB;
+    wtile = a.w_kslab ? a.w + (long)kb0 * FTKB * 64 : a.w + (long)n0 * a.ldw + (long)kb0 * FTKB;
   };
   constexpr int NSLOT = XCOPIES + WCOPIES + 1;
   auto copy_slot = [&](int s, int stage, int kt) {
@@ -262,7 +271,7 @@ fp8_block_gemm_kernel(F8Args a) {
   // finished reading g before the barrier that opened the step).  The step ends when this
   // wavefront's copies of element g + 2 have landed -- those of g + 3 stay in flight -- and a
   // barrier makes that true for everybody's.
-  const int nt = KB;
+  const int nt = KB / ksplits;                     // K blocks per (output tile, K range)
   // (kept in a register: read through the dispatch packet it is fetched again in every iteration)
   const int gdim = __builtin_amdgcn_readfirstlane((int)gridDim.x);
   int tile = blockIdx.x;
@@ -355,6 +364,20 @@ fp8_block_gemm_kernel(F8Args a) {
 
     // ---- epilogue: lane holds, per (w tile i, x tile j), output row m = .. + l16 and columns
     // n = .. + 4 kq + {0..3}
+    if (ksplits > 1) {
+      // split K: the fp32 sums of this K range, nothing else; bias (and the scales that live outside the
+      // K sum) are the second launch's
+      float* const part = a.partial + (long)(tile % ksplits) * M * N;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int m = m0 + wm * (16 * NJ) + j * 16 + l16;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) *(f4*)(part + (long)m * N + n0 + wn * (16 * NI) + i * 16 + 4 * kq) = acc[i][j];
+      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0), as below
+      continue;
+    }
     float bia[NI][4];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
@@ -396,16 +419,94 @@ fp8_block_gemm_kernel(F8Args a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);              // vmcnt(0)
 }
 
+// Second launch of a split: the ranges' sums added in range order (run-to-run identical), then the epilogue.
+template <int DT, bool PC>
+__global__ void __launch_bounds__(256)
+fp8_splitk_epilogue_kernel(F8Args a) {
+  const long q = (long)blockIdx.x * 256 + threadIdx.x;     // 4 adjacent columns of one row
+  const int nq = a.N / 4;
+  if (q >= (long)a.M * nq) return;
+  const int m = (int)(q / nq), n = (int)(q % nq) * 4;
+  f4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < a.ksplits; ++s) acc += *(const f4*)(a.partial + ((long)s * a.M + m) * a.N + n);
+  const float xsc = PC ? a.x_scale[(long)m * a.xs_mul] : 1.0f;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float b = a.bias ? Elem<DT>::to_f32(((const uint16_t*)a.bias)[n + e]) : 0.0f;
+    v[e] = plus_bias(PC ? scaled_sum(acc[e], xsc, a.w_scale[(n + e) * a.ws_mul]) : acc[e], b);
+  }
+  u2 o;
+  o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
+  o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);
+  *(u2*)((uint16_t*)a.out + (long)m * a.ldo + n) = o;
+}
+
+constexpr size_t F8_SPLITK_BYTES = (size_t)64 << 20;
+constexpr size_t F8_WS_OFFSET = (size_t)1 << 20;     // the first MiB of a workspace belongs to the W4A16 arrival counters
+
+// K ranges for a shape: as many as put about one 256 x 128 tile on every CU, each at least eight K
+// blocks long, a divisor of the K block count, partial sums within 64 MiB.  1: no split.
+int fp8_ksplits(int M, int N, int K) {
+  const long cus = device_cu_count(), tiles = (long)((M + FTM - 1) / FTM) * (N / FTN);
+  const int nt = K / FTKB;
+  if (N % FTN != 0 || tiles < 1 || tiles * 2 > cus) return 1;
+  long s = cus / tiles;
+  if (s > 8) s = 8;
+  if (s > nt / 8) s = nt / 8;
+  while (s > 1 && (nt % s != 0 || (size_t)s * M * N * sizeof(float) > F8_SPLITK_BYTES)) --s;
+  return s < 1 ? 1 : (int)s;
+}
+
+template <int DT, bool PC>
+int launch_f8(const F8Args& a, hipStream_t st);
+
+template <int DT, bool PC>
+int launch_f8_splitk(const F8Args& a, int splits, void* workspace, hipStream_t st) {
+  F8Args b = a;
+  b.ksplits = splits;
+  b.partial = (float*)((char*)workspace + F8_WS_OFFSET);
+  if (int rc = launch_f8<DT, PC>(b, st)) return rc;
+  const long quads = (long)a.M * (a.N / 4);
+  hipLaunchKernelGGL((fp8_splitk_epilogue_kernel<DT, PC>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, b);
+  MQ_LAUNCH_CHECK("fp8 gemm (split-K epilogue)");
+  return 0;
+}
+
+// Rows from which the tile kernel with K ranges side by side is ahead of the weight-streaming kernel,
+// whose time grows with the rows while the split tile kernel's hardly does (measured, us at 16 / 32 /
+// 48 / 64 rows, streaming against split: K 16384 N 7168 33/41/52/62 against 33/33/33/35; K 7168 N 4096
+// 16/20/26/30 against 16/17/17/18; K 8192 N 8192 21/24/29/34 against 23/24/24/24; K 4096 N 4096
+// 10/13/17/20 against 15/15/16/17; K 2048 N 7168 7/9/11/12 against 14/15/15/16).
+int fp8_split_min_rows(int N, int K, int splits) {
+  if (splits < 4) return 64;
+  if (K >= 7168) return K >= 2 * N ? 16 : (N <= 4096 ? 24 : 32);
+  if (K >= 4096) return 48;
+  return 64;
+}
+
+// with a workspace that holds the plan's partial sums: K ranges side by side; else the plain launch
+template <int DT, bool PC>
+int launch_f8_auto(F8Args& a, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  a.ksplits = 1;
+  a.partial = nullptr;
+  const int splits = fp8_ksplits(a.M, a.N, a.K);
+  if (splits > 1 && workspace && workspace_bytes >= F8_WS_OFFSET + (size_t)splits * a.M * a.N * sizeof(float))
+    return launch_f8_splitk<DT, PC>(a, splits, workspace, st);
+  return launch_f8<DT, PC>(a, st);
+}
+
 template <int DT, bool PC>
 int launch_f8(const F8Args& a, hipStream_t st) {
   const int mtiles = (a.M + FTM - 1) / FTM, ntiles = a.N / FTN;
   F8Args b = a;
-  b.n_panels_swizzle = (ntiles % 8 == 0) ? 1 : 0;
+  const int ks = a.ksplits > 1 ? a.ksplits : 1;
+  b.n_panels_swizzle = (ntiles % 8 == 0 && ks == 1) ? 1 : 0;
   const size_t shmem = 3 * (size_t)(FTM * FTKB + FTN * FTKB + FTM * 4 + 256);
   static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT, PC>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
   MQ_REQUIRE(attr == hipSuccess, "fp8 gemm: cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
-  int grid = mtiles * ntiles, cus = device_cu_count() / 8 * 8;
+  int grid = mtiles * ntiles * ks, cus = device_cu_count() / 8 * 8;
   if (cus >= 8 && grid > cus) grid = cus;
   hipLaunchKernelGGL((fp8_block_gemm_kernel<DT, PC>), dim3(grid), dim3(F8_THREADS), shmem, st, b);
   MQ_LAUNCH_CHECK("fp8 gemm");
@@ -417,9 +518,22 @@ int launch_f8(const F8Args& a, hipStream_t st) {
 
 using namespace mi355q;
 
+extern "C" size_t mi355q_fp8_gemm_workspace_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  const int s = fp8_ksplits(M, N, K);
+  return s > 1 && M > fp8_split_min_rows(N, K, s) ? F8_WS_OFFSET + (size_t)s * M * N * sizeof(float) : 0;
+}
+
 extern "C" int mi355q_fp8_block_gemm(void* out, const void* x, const void* w, const float* x_scale,
                                      const float* w_scale, const void* bias, int M, int N, int K, long ldx,
                                      long ldw, long ldo, int out_dtype, void* stream) {
+  return mi355q_fp8_block_gemm_ws(out, x, w, x_scale, w_scale, bias, M, N, K, ldx, ldw, ldo, out_dtype, nullptr, 0, stream);
+}
+
+extern "C" int mi355q_fp8_block_gemm_ws(void* out, const void* x, const void* w, const float* x_scale,
+                                        const float* w_scale, const void* bias, int M, int N, int K, long ldx,
+                                        long ldw, long ldo, int out_dtype, void* workspace, size_t workspace_bytes,
+                                        void* stream) {
   MQ_REQUIRE(M >= 0 && N > 0 && K > 0, "fp8_block_gemm: bad shape M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
   MQ_REQUIRE(out && x && w && x_scale && w_scale, "fp8_block_gemm: null pointer");
@@ -438,8 +552,8 @@ extern "C" int mi355q_fp8_block_gemm(void* out, const void* x, const void* w, co
   a.w_kslab = kslab ? 1 : 0;
   a.n_panels_swizzle = 0;
   a.xs_mul = a.ws_mul = 0;
-  if (out_dtype == MI355Q_F16) return launch_f8<MI355Q_F16, false>(a, as_stream(stream));
-  return launch_f8<MI355Q_BF16, false>(a, as_stream(stream));
+  if (out_dtype == MI355Q_F16) return launch_f8_auto<MI355Q_F16, false>(a, workspace, workspace_bytes, as_stream(stream));
+  return launch_f8_auto<MI355Q_BF16, false>(a, workspace, workspace_bytes, as_stream(stream));
 }
 
 // fp8 x fp8 with per-token (or one) activation scale and per-channel (or one) weight scale, fp32
@@ -448,6 +562,14 @@ extern "C" int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, c
                                       int x_scale_per_row, const float* w_scale, int w_scale_per_col,
                                       const void* bias, int M, int N, int K, long ldx, long ldw, long ldo,
                                       int out_dtype, void* stream) {
+  return mi355q_fp8_scaled_gemm_ws(out, x, w, x_scale, x_scale_per_row, w_scale, w_scale_per_col, bias, M, N, K, ldx, ldw,
+                                   ldo, out_dtype, nullptr, 0, stream);
+}
+
+extern "C" int mi355q_fp8_scaled_gemm_ws(void* out, const void* x, const void* w, const float* x_scale,
+                                         int x_scale_per_row, const float* w_scale, int w_scale_per_col,
+                                         const void* bias, int M, int N, int K, long ldx, long ldw, long ldo,
+                                         int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   MQ_REQUIRE(M >= 0 && N > 0 && K > 0, "fp8_scaled_gemm: bad shape M=%d N=%d K=%d", M, N, K);
   if (M == 0) return 0;
   MQ_REQUIRE(out && x && w && x_scale && w_scale, "fp8_scaled_gemm: null pointer");
@@ -466,7 +588,10 @@ extern "C" int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, c
   const bool stream_ok = ldx == K && (kslab || ldw == K) && ldo == N && (size_t)N * K * 2 < ((size_t)1 << 32) &&
                          (size_t)M * K * 2 < ((size_t)1 << 32);
   // (from 41 rows on layers of 128 tiles or more: the wavefronts without rows only copy there)
-  if (tile_ok && ((M > 64 && tiles >= 64) || (M > 40 && tiles >= 128) || !stream_ok)) {
+  // (and, with a workspace, wherever the split plan asks for one: K ranges side by side fill the chip)
+  const size_t split_bytes = mi355q_fp8_gemm_workspace_bytes(M, N, K);
+  const bool split_ok = tile_ok && workspace && split_bytes > 0 && workspace_bytes >= split_bytes;
+  if (tile_ok && ((M > 64 && tiles >= 64) || (M > 40 && tiles >= 128) || split_ok || !stream_ok)) {
     F8Args a;
     a.out = out; a.x = (const uint8_t*)x; a.w = (const uint8_t*)w; a.x_scale = x_scale; a.w_scale = w_scale;
     a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;
@@ -474,8 +599,8 @@ extern "C" int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, c
     a.n_panels_swizzle = 0;
     a.xs_mul = x_scale_per_row ? 1 : 0;
     a.ws_mul = w_scale_per_col ? 1 : 0;
-    if (out_dtype == MI355Q_F16) return launch_f8<MI355Q_F16, true>(a, as_stream(stream));
-    return launch_f8<MI355Q_BF16, true>(a, as_stream(stream));
+    if (out_dtype == MI355Q_F16) return launch_f8_auto<MI355Q_F16, true>(a, workspace, workspace_bytes, as_stream(stream));
+    return launch_f8_auto<MI355Q_BF16, true>(a, workspace, workspace_bytes, as_stream(stream));
   }
   MQ_REQUIRE(stream_ok, "fp8_scaled_gemm: M=%d N=%d K=%d with row strides (%ld, %ld, %ld) fits neither kernel "
              "(dense operands, or N %% 128 == 0 with strides that are multiples of 16)", M, N, K, ldx, ldw, ldo);

@@ -371,9 +371,13 @@ def _scaled_fp8_mm(out, x, weight, x_scale, w_scale, bias):
         if bias.numel() != N:
             raise RuntimeError(f"bias has {bias.numel()} entries for N={N}")
     with torch.cuda.device(x.device):
-        _lib.call("mi355q_fp8_scaled_gemm", out2.data_ptr(), x2.data_ptr(), w.data_ptr(), xs.data_ptr(),
+        # (few output tiles behind a long K: K ranges side by side through the stream's workspace)
+        need = _lib.load().mi355q_fp8_gemm_workspace_bytes(M, N, K)
+        wsp = rt.workspace(x.device, need) if need else None
+        _lib.call("mi355q_fp8_scaled_gemm_ws", out2.data_ptr(), x2.data_ptr(), w.data_ptr(), xs.data_ptr(),
                   int(xs.numel() > 1), ws.data_ptr(), int(ws.numel() > 1), rt.ptr(bias), M, N, K,
-                  x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.stream_ptr())
+                  x2.stride(0), ldw, out2.stride(0), rt.dtype_code(out.dtype), rt.ptr(wsp),
+                  0 if wsp is None else wsp.numel(), rt.stream_ptr())
 
 
 def _cutlass_scaled_mm_impl(out, x, weight, x_scale, w_scale, bias):
@@ -1214,7 +1218,12 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
     tiles = -(-M // 256) * (N // 128)               # 256 x 128 output tiles, one workgroup each
     # (from 41 rows on a layer of 128 tiles or more: the tile kernel's wavefronts without rows only copy,
     # K 8192 x N 28672 at M = 48 / 64: 59.6 / 68.4 -> 52.9 / 55.1 us; 112 tiles: the streamer stays ahead)
-    if ((M > _FP8_TILE_MIN_M and tiles >= _FP8_TILE_MIN_TILES) or (M > _FP8_TILE_MIN_M * 5 // 8 and tiles >= 2 * _FP8_TILE_MIN_TILES)) \
+    # (and, whatever the tile count, where the library plans K ranges side by side that fill the chip:
+    # from 65 rows, and from 17 / 25 / 33 / 49 rows on where K is long, see fp8_split_min_rows)
+    need = _lib.load().mi355q_fp8_gemm_workspace_bytes(M, N, K) \
+        if M > _FP8_TILE_MIN_M // 4 and N % 128 == 0 and K % 128 == 0 else 0
+    if (need or (M > _FP8_TILE_MIN_M and tiles >= _FP8_TILE_MIN_TILES)
+            or (M > _FP8_TILE_MIN_M * 5 // 8 and tiles >= 2 * _FP8_TILE_MIN_TILES)) \
             and N % 128 == 0 and K % 128 == 0 \
             and out.dtype in (torch.float16, torch.bfloat16) \
             and rhs.dim() == 2 and rhs.is_contiguous() and out.is_contiguous():
@@ -1229,9 +1238,10 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
                                f"M={M} N={N} K={K} with 128 x 128 blocks")
         b = None if bias is None else bias.to(out.dtype).contiguous()
         with torch.cuda.device(lhs.device):
-            _lib.call("mi355q_fp8_block_gemm", out.data_ptr(), a2.data_ptr(), rhs.data_ptr(), xs.data_ptr(),
+            wsp = rt.workspace(lhs.device, need) if need else None
+            _lib.call("mi355q_fp8_block_gemm_ws", out.data_ptr(), a2.data_ptr(), rhs.data_ptr(), xs.data_ptr(),
                       ws.data_ptr(), rt.ptr(b), M, N, K, K, 0 if rearrange.is_kslab(rhs) else K, N,
-                      rt.dtype_code(out.dtype), rt.stream_ptr())
+                      rt.dtype_code(out.dtype), rt.ptr(wsp), 0 if wsp is None else wsp.numel(), rt.stream_ptr())
         return
     _kcontig(out, lhs, rhs, lhs_scale.to(torch.float32).reshape(-1, lhs_scale.shape[-1]).contiguous(),
              rhs_scale.to(torch.float32).contiguous(), bias, _lib.Q_FP8_BLOCK, 128)
