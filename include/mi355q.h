@@ -77,7 +77,11 @@ int mi355q_w4_unpack(const int32_t* packed, uint8_t* dst, int batch, int K, int 
  * streaming kernel, larger M the LDS-staged MFMA kernels (groups of 32, 64 and
  * multiples of 128; other sizes go through the streaming kernel 32 rows at a
  * time), which split K over two kernels when their grid would leave most of
- * the chip idle.  `workspace` must hold
+ * the chip idle.  bf16 activations of 129 rows or more on outputs of two million
+ * elements or more are first stored in the workspace as fp16 rows, each times a
+ * power of two of its own (exact), and take the fp16 kernels; with a workspace
+ * too small for that the bf16 kernel runs (same tolerance, other bits).
+ * `workspace` must hold
  * mi355q_w4a16_workspace_bytes() bytes, be zero-filled once before first use,
  * and must not be shared by launches that may overlap in time. */
 size_t mi355q_w4a16_workspace_bytes(int M, int K, int N);
@@ -107,7 +111,9 @@ int mi355q_w4a16_stream_plan(int M, int K, int N, int group_size, int* tiles_per
 
 /* No counterpart in the reference.  mi355q_w4a16_gemm for callers that cannot allocate device memory
  * or pass a workspace (code under HIP graph capture, serving loops and harnesses that forbid
- * allocation): same arguments without the workspace, same kernels, bit-identical results.  The
+ * allocation): same arguments without the workspace, same kernels, bit-identical results (but for
+ * bf16 inputs tall enough for mi355q_w4a16_gemm to stage them as fp16 rows in its workspace: the
+ * fixed array has no room for that, the bf16 kernel runs here -- same tolerance, other bits).  The
  * split-K partial tiles and arrival counters live in a fixed array of
  * mi355q_w4a16_noalloc_scratch_bytes() = 32 MiB of device memory that every GPU running the library
  * holds until the process ends.  A shape whose split-K plan needs more is rejected with an error

@@ -456,6 +456,49 @@ def test_ring_gemm_is_fp16_only_and_tile_family_still_forced(ops, rearrange):
     np.testing.assert_allclose(b, want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("M,K,N,zeros", [(129, 512, 16384, True), (300, 4096, 7168, True), (640, 1024, 3328, False),
+                                         (2400, 14336, 1024, True), (256, 16512, 8192, True)])
+def test_bf16_rows_staged_as_fp16_for_the_pipelined_loop(ops, rearrange, M, K, N, zeros):
+    """bf16 from 129 rows on, the library's own choice with the operator's workspace: each row times a
+    power of two of its own becomes fp16 in the workspace (exact), the fp16 loop multiplies it with the
+    exact integers q - z, the epilogue undoes the power of two.  Rows of magnitudes from 2^-100 to 2^100,
+    a row of zeros and a row that holds an infinity; each row is compared at its own magnitude.  The
+    fourth case is taller than the staging area (2400 x 14336 x 2 bytes > 64 MiB): two row chunks; the
+    last has rows too long to stay in registers between the two passes of the conversion."""
+    from vllm_gcu_amd import _lib
+    g = 128
+    print(f"case bf16 staged M={M} K={K} N={N} zeros={zeros}", flush=True)
+    assert _lib.load().mi355q_w4a16_workspace_bytes(M, K, N) > (65 << 20)     # room for the staging area is asked for
+    q, z, s, x = make_case(M * 3 + K, M, K, N, g)
+    if not zeros:
+        z[:] = 8
+    rng = np.random.default_rng(M)
+    mag = (2.0 ** rng.integers(-100, 101, size=M)).astype(np.float32)
+    mag[:4] = [1.0, 2.0 ** 100, 2.0 ** -100, 2.0 ** 15]
+    x = x * mag[:, None]
+    x[5] = 0.0
+    x[7, K // 2] = np.inf
+    bias = rng.standard_normal(N).astype(np.float32) * 0.0 if M != 300 else rng.standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, bias=bias).float().cpu().numpy()
+    plain = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, bias=bias, family=2).float().cpu().numpy()
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle(q, z, s, x, g, torch.bfloat16, bias=bias)
+    assert not np.isfinite(got[7]).any() and not np.isfinite(plain[7]).any()
+    rows = np.array([m for m in range(M) if m != 7])
+    assert np.isfinite(got[rows]).all()
+    if M == 300:                      # (with a bias the rows cannot be rescaled: unit magnitudes there)
+        rows = rows[(mag[rows] >= 0.5) & (mag[rows] <= 2.0)]
+        mag = np.ones_like(mag)
+    np.testing.assert_allclose(got[rows] / mag[rows, None], want[rows] / mag[rows, None], rtol=RTOL, atol=ATOL)
+    # and against the bf16 loop (same products, fp32 sums in another order, one bf16 rounding each)
+    np.testing.assert_allclose(got[rows] / mag[rows, None], plain[rows] / mag[rows, None], rtol=2 ** -7, atol=1e-3)
+    np.testing.assert_array_equal(got[5], np.float32(torch.from_numpy(bias).to(torch.bfloat16).float().numpy()))
+    # every partial sum representable: bit for bit the oracle
+    q, z, s, x = make_case(11, M, K, N, g, exact=True)
+    want = torch.from_numpy(oracle(q, z, s, x, g, torch.bfloat16)).to(torch.bfloat16)
+    assert torch.equal(run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16).cpu(), want)
+
+
 def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):
     """Groups of 64 on the streaming kernel when it is forced (32 rows per launch) and through the
     library's own choice (the MFMA kernel from 65 rows on)."""

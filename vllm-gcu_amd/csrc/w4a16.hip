@@ -16,6 +16,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                       int group_size, int dtype, void* workspace, size_t workspace_bytes, bool allow_ring,
                       hipStream_t st);
 size_t w4a16_tile_workspace_bytes(int M, int K, int N);
+size_t w4a16_bf16_stage_workspace_bytes(int M, int K);
 int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
                      void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st);
@@ -41,7 +42,11 @@ extern "C" size_t mi355q_w4a16_workspace_bytes(int M, int K, int N) {
   // the split-K partials of the MFMA kernel live behind the first MiB, which
   // holds the streaming kernel's arrival counters (they must stay zero)
   const size_t t = M > 32 ? w4a16_tile_workspace_bytes(M, K, N) : 0;
-  const size_t tt = t ? t + TILE_WS_OFFSET : 0;
+  size_t tt = t ? t + TILE_WS_OFFSET : 0;
+  // (this function does not see the dtype: room for the area that bf16 activations are staged in as
+  // fp16 rows, behind the split-K partials -- a smaller workspace only means the bf16 loop runs instead)
+  const size_t stage = w4a16_bf16_stage_workspace_bytes(M, K);
+  if (stage && stage + TILE_WS_OFFSET > tt) tt = stage + TILE_WS_OFFSET;
   return s > tt ? s : tt;
 }
 

@@ -30,6 +30,7 @@ struct TileArgs {
   const uint16_t* scales;       // group scales in the activation type, or
   const float* scales_f32;      // ... in fp32 (SF32 kernels; the other pointer is unused)
   const float* out_scale;       // optional device scalar multiplied into every output
+  const float* row_scale;       // [M] per-row multiplier of the output (IOBF kernels: bf16 rows staged as fp16)
   const void* zeros;
   const uint16_t* bias;
   int M, K, N, gs;
@@ -117,11 +118,16 @@ template <> struct TileMma<MI355Q_BF16> {
 // SIMD keep the matrix pipe fed while one of them waits or dequantises).
 // GPB = quantisation groups per K block of 128: 1 for group sizes that are multiples of 128, 2 / 4 for
 // groups of 64 / 32 (plain loop only: each group's steps accumulate into a partial tile of their own).
-template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false, int GPB = 1>
+// IOBF (with DT = fp16, dense): the activations are bf16 rows that a pass before this kernel scaled by a
+// power of two each and stored as fp16 (exact: eight mantissa bits into eleven); scales, pre-scaled
+// zero-points, bias and output are bf16, and the epilogue multiplies each row by its power of two.
+template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false, int GPB = 1, bool IOBF = false>
 __global__ void __launch_bounds__(256 * WM, WM == 1 ? 2 : 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
   typedef typename MM::vec vec;
+  static_assert(!IOBF || (DT == MI355Q_F16 && !GROUPED), "bf16 in and out around the fp16 loop: dense only");
+  typedef Elem<IOBF ? MI355Q_BF16 : DT> IO;       // the type of scales, pre-scaled zero-points, bias and output
   static_assert(MT % WM == 0, "row tiles split evenly over the wavefront rows");
   constexpr int BM = 16 * MT;
   constexpr int MTW = MT / WM;                    // row tiles per wavefront
@@ -280,7 +286,7 @@ w4a16_tile_kernel(TileArgs a) {
     uint2 sc, scp;
     auto scale_of = [&](uint2 sv, int t) {
       const uint32_t sw = (t < 2) ? sv.x : sv.y;
-      return Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+      return IO::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
     };
     h2 zz[4];
     auto prep = [&]() {
@@ -291,7 +297,7 @@ w4a16_tile_kernel(TileArgs a) {
           const uint32_t zw = (t < 2) ? zsreg.x : zsreg.y;
           // the loader pre-multiplied an integer zero-point by the scale
           // (z * s rounded to the activation type): recover the integer
-          const float zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / scale_of(sc, t));
+          const float zf = __builtin_rintf(IO::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / scale_of(sc, t));
           zz[t] = (h2){(_Float16)(1024.0f + zf), (_Float16)(64.0f + zf)};
         } else {
           // fp16 bit patterns directly: 1024 + z = 0x6400 | z, 64 + z = 0x5400 | z << 4
@@ -400,13 +406,13 @@ w4a16_tile_kernel(TileArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const uint32_t sw = (t < 2) ? sv.x : sv.y;
-          sc[sg][t] = SF32 ? sreg32[t] : Elem<DT>::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+          sc[sg][t] = SF32 ? sreg32[t] : IO::to_f32((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
           float zf;
           if (ZK == MI355Q_ZP_PRESCALED) {
             const uint32_t zw = (t < 2) ? zsv.x : zsv.y;
             // the loader pre-multiplied an integer zero-point by the scale
             // (z * s rounded to the activation type): recover the integer
-            zf = __builtin_rintf(Elem<DT>::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[sg][t]);
+            zf = __builtin_rintf(IO::to_f32((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu))) / sc[sg][t]);
           } else {
             zf = (float)((zv >> (4 * t)) & 15u);
           }
@@ -458,7 +464,7 @@ w4a16_tile_kernel(TileArgs a) {
   float bs[4] = {0.f, 0.f, 0.f, 0.f};
   if (a.bias) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) bs[t] = Elem<DT>::to_f32(a.bias[ncol + t]);
+    for (int t = 0; t < 4; ++t) bs[t] = IO::to_f32(a.bias[ncol + t]);
   }
 #pragma unroll
   for (int mt = 0; mt < MTW; ++mt)
@@ -474,6 +480,7 @@ w4a16_tile_kernel(TileArgs a) {
       } else {
         m = m0 + (wmh * MTW + mt) * 16 + 4 * kq + i;
         ok = m < M;
+        if (IOBF && ok && !a.partial) rw *= a.row_scale[m];
       }
       if (a.partial) {
         if (ok) {
@@ -482,10 +489,10 @@ w4a16_tile_kernel(TileArgs a) {
         }
       } else if (ok) {
         uint2 o;
-        o.x = (uint32_t)Elem<DT>::from_f32(acc[mt][0][i] * rw + bs[0]) |
-              ((uint32_t)Elem<DT>::from_f32(acc[mt][1][i] * rw + bs[1]) << 16);
-        o.y = (uint32_t)Elem<DT>::from_f32(acc[mt][2][i] * rw + bs[2]) |
-              ((uint32_t)Elem<DT>::from_f32(acc[mt][3][i] * rw + bs[3]) << 16);
+        o.x = (uint32_t)IO::from_f32(acc[mt][0][i] * rw + bs[0]) |
+              ((uint32_t)IO::from_f32(acc[mt][1][i] * rw + bs[1]) << 16);
+        o.y = (uint32_t)IO::from_f32(acc[mt][2][i] * rw + bs[2]) |
+              ((uint32_t)IO::from_f32(acc[mt][3][i] * rw + bs[3]) << 16);
         *(uint2*)(a.out + (size_t)m * N + ncol) = o;
       }
     }
@@ -817,21 +824,123 @@ hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStrea
   }
 }
 
+// bf16 activations staged as fp16 rows: 64-row tiles on the pipelined fp16 loop, bf16 in and out
+hipError_t launch_iobf(const TileArgs& a, int zk, int row_blocks, hipStream_t st) {
+  const int G = a.K >> 7;
+  dim3 grid((a.N + BN - 1) / BN, row_blocks, (G + a.kper - 1) / a.kper), block(256);
+  const size_t shmem = 2 * 64 * A_ROW;
+  if (zk == MI355Q_ZP_NONE) {
+    static hipError_t attr = hipFuncSetAttribute(
+        (const void*)w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_NONE, 4, false, 1, false, 1, true>,
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL((w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_NONE, 4, false, 1, false, 1, true>), grid, block, shmem, st, a);
+  } else {
+    static hipError_t attr = hipFuncSetAttribute(
+        (const void*)w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_PACKED, 4, false, 1, false, 1, true>,
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL((w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_PACKED, 4, false, 1, false, 1, true>), grid, block, shmem, st, a);
+  }
+  return hipSuccess;
+}
+
+// One workgroup per row of bf16 activations: the row's largest magnitude fixes a power of two 2^e that
+// brings it into [2^14, 2^15); the row times 2^-e is stored as fp16 and 2^e as the row's output
+// multiplier.  Exact for every element within 2^28 of the row's largest (eight mantissa bits fit in
+// eleven, the scaling is a power of two); smaller ones lose at most 2^-40 of that largest magnitude in
+// fp16's subnormal range.  A row that holds an infinity or a NaN is stored unscaled (they stay what
+// they are; its finite elements beyond the fp16 range become infinities).
+// HELD: the row stays in registers between the two passes (K up to 16384); else it is read twice.
+template <bool HELD>
+__global__ void __launch_bounds__(256)
+bf16_rows_to_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ x16, float* __restrict__ row_scale, int K) {
+  __shared__ uint32_t wmax[4];
+  const int tid = threadIdx.x;
+  const u4* row = (const u4*)(x + (size_t)blockIdx.x * K);
+  u4* orow = (u4*)(x16 + (size_t)blockIdx.x * K);
+  const int chunks = K >> 3;                        // 16-byte pieces of eight elements
+  uint32_t mx = 0;
+  u4 held[HELD ? 8 : 1];
+  if (HELD) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) held[r] = tid + 256 * r < chunks ? row[tid + 256 * r] : (u4){0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = held[r][j] & 0x7fffu, hi = (held[r][j] >> 16) & 0x7fffu;
+        mx = mx > lo ? mx : lo;
+        mx = mx > hi ? mx : hi;
+      }
+  } else {
+    for (int i = tid; i < chunks; i += 256) {
+      const u4 v = row[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = v[j] & 0x7fffu, hi = (v[j] >> 16) & 0x7fffu;
+        mx = mx > lo ? mx : lo;
+        mx = mx > hi ? mx : hi;
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)mx, o, 64);
+    mx = mx > other ? mx : other;
+  }
+  if ((tid & 63) == 0) wmax[tid >> 6] = mx;
+  __syncthreads();
+  mx = wmax[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) mx = mx > wmax[w] ? mx : wmax[w];
+  const int expo = (int)(mx >> 7);                  // biased exponent of the largest magnitude
+  int e = 0;
+  if (mx != 0 && expo != 255) {
+    e = (expo > 0 ? expo : 1) - 127 - 14;
+    if (e < -126) e = -126;
+  }
+  const float down = bitcast<float>((uint32_t)(127 - e) << 23);
+  if (tid == 0) row_scale[blockIdx.x] = bitcast<float>((uint32_t)(127 + e) << 23);
+  auto convert = [&](u4 v) {
+    u4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const _Float16 lo = (_Float16)(bitcast<float>(v[j] << 16) * down);
+      const _Float16 hi = (_Float16)(bitcast<float>(v[j] & 0xffff0000u) * down);
+      o[j] = (uint32_t)bitcast<uint16_t>(lo) | ((uint32_t)bitcast<uint16_t>(hi) << 16);
+    }
+    return o;
+  };
+  if (HELD) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      if (tid + 256 * r < chunks) orow[tid + 256 * r] = convert(held[r]);
+  } else {
+    for (int i = tid; i < chunks; i += 256) orow[i] = convert(row[i]);     // (second read of the row: from the cache)
+  }
+}
+
 }  // namespace
 
-// sum of the fp32 partial tiles of a dense split-K launch into the output (+ bias), in split order
-int w4a16_splitk_reduce_launch(void* out, const float* partial, const void* bias, int M, int N, int splits,
-                               int dtype, hipStream_t st) {
+// sum of the fp32 partial tiles of a dense split-K launch into the output (+ bias), in split order;
+// row_weight (optional): a multiplier per output row, applied to the sum before the bias
+static int splitk_reduce_rows_launch(void* out, const float* partial, const void* bias, int M, int N, int splits,
+                                     int dtype, hipStream_t st, const float* row_weight) {
   const long MN = (long)M * N;
   const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
   if (dtype == MI355Q_F16)
     hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out, partial,
-                       (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
+                       (const uint16_t*)bias, row_weight, MN, N, splits);
   else
     hipLaunchKernelGGL((w4a16_splitk_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out, partial,
-                       (const uint16_t*)bias, (const float*)nullptr, MN, N, splits);
+                       (const uint16_t*)bias, row_weight, MN, N, splits);
   MQ_LAUNCH_CHECK("w4a16_gemm(split-K reduce)");
   return 0;
+}
+int w4a16_splitk_reduce_launch(void* out, const float* partial, const void* bias, int M, int N, int splits,
+                               int dtype, hipStream_t st) {
+  return splitk_reduce_rows_launch(out, partial, bias, M, N, splits, dtype, st, nullptr);
 }
 
 // split-K plan for grids that leave most of the chip idle: as many splits as
@@ -959,6 +1068,29 @@ size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
   return m > 1 ? (size_t)m * M * N * sizeof(float) : 0;
 }
 
+// bf16 activations staged as fp16: where the staging area sits in the workspace (behind the split-K
+// partial tiles), how many rows it holds at most, and from how many rows on it pays
+constexpr size_t BF16_STAGE_OFFSET = TILE_SPLITK_BYTES;
+constexpr size_t BF16_STAGE_SCALE_BYTES = (size_t)64 << 10;          // one multiplier per staged row
+constexpr size_t BF16_STAGE_BYTES = (size_t)64 << 20;
+constexpr int BF16_STAGE_MIN_M = 129;
+// (measured, us, staged against the bf16 loop: K 4096 x N 28672 at M = 129 / 2048 / 8192: 68 / 477 / 1812
+// against 85 / 578 / 2202; K 4096 x N 6144 at 256 / 512 / 2048: 34 / 49 / 119 against 35 / 55 / 136; K 4096 x
+// N 4096 at 512 / 1024 / 4096: 38 / 53 / 151 against 39 / 58 / 170; K 14336 x N 4096 at 512 / 2048: 85 / 258
+// against 91 / 299: the conversion pass costs 5-25 us, so the output has to have about two million elements)
+static bool bf16_stage_pays(int M, int N) { return M >= BF16_STAGE_MIN_M && (long)M * N >= (1L << 21); }
+
+size_t w4a16_bf16_stage_workspace_bytes(int M, int K) {
+  if (M < BF16_STAGE_MIN_M) return 0;
+  const size_t rows = (size_t)M * K * 2;
+  return BF16_STAGE_OFFSET + BF16_STAGE_SCALE_BYTES + (rows < BF16_STAGE_BYTES ? rows : BF16_STAGE_BYTES);
+}
+
+static int tile_launch_dense(void* out, const void* x, const int32_t* qweight, const void* scales,
+                             const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
+                             int group_size, int dtype, void* workspace, size_t workspace_bytes,
+                             const float* row_scale, hipStream_t st);
+
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
                       int group_size, int dtype, void* workspace, size_t workspace_bytes, bool allow_ring,
@@ -976,7 +1108,48 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
       return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
                               workspace_bytes, ss, 1, st);
   }
+  // bf16 with a workspace that has the staging area: the rows become fp16 times a power of two each
+  // and take the pipelined fp16 loop, whose B operands are the exact integers q - z (the bf16 loop
+  // has no room for that pipeline: it spills); taller inputs than the area holds go in row chunks
+  if (allow_ring && dtype == MI355Q_BF16 && !small_groups && zeros_kind != MI355Q_ZP_PRESCALED &&
+      bf16_stage_pays(M, N) && workspace && workspace_bytes > BF16_STAGE_OFFSET + BF16_STAGE_SCALE_BYTES) {
+    size_t room = workspace_bytes - BF16_STAGE_OFFSET - BF16_STAGE_SCALE_BYTES;
+    if (room > BF16_STAGE_BYTES) room = BF16_STAGE_BYTES;
+    long rows_max = (long)(room / ((size_t)K * 2));
+    if (rows_max > (long)(BF16_STAGE_SCALE_BYTES / sizeof(float))) rows_max = BF16_STAGE_SCALE_BYTES / sizeof(float);
+    rows_max &= ~63L;
+    if (rows_max >= 256 || rows_max >= M) {
+      const long chunks = (M + rows_max - 1) / rows_max;
+      const long per = (((M + chunks - 1) / chunks) + 63) & ~63L;
+      float* rs = (float*)((char*)workspace + BF16_STAGE_OFFSET);
+      uint16_t* x16 = (uint16_t*)((char*)workspace + BF16_STAGE_OFFSET + BF16_STAGE_SCALE_BYTES);
+      for (long m0 = 0; m0 < M; m0 += per) {
+        const int mc = (int)(M - m0 < per ? M - m0 : per);
+        if (K <= 16384)
+          hipLaunchKernelGGL(bf16_rows_to_f16_kernel<true>, dim3(mc), dim3(256), 0, st, (const uint16_t*)x + (size_t)m0 * K, x16, rs, K);
+        else
+          hipLaunchKernelGGL(bf16_rows_to_f16_kernel<false>, dim3(mc), dim3(256), 0, st, (const uint16_t*)x + (size_t)m0 * K, x16, rs, K);
+        MQ_LAUNCH_CHECK("w4a16_gemm(bf16 rows to fp16)");
+        if (int rc = tile_launch_dense((uint16_t*)out + (size_t)m0 * N, x16, qweight, scales, zeros, zeros_kind, bias, mc, K, N,
+                                       group_size, dtype, workspace, BF16_STAGE_OFFSET, rs, st))
+          return rc;
+      }
+      return 0;
+    }
+  }
+  return tile_launch_dense(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
+                           workspace_bytes, nullptr, st);
+}
+
+// 64-row tiles (or the narrow tiles) for one dense problem; row_scale: bf16 rows staged as fp16 (x points
+// at the staged rows, dtype stays bf16 for scales, bias and output)
+static int tile_launch_dense(void* out, const void* x, const int32_t* qweight, const void* scales,
+                             const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
+                             int group_size, int dtype, void* workspace, size_t workspace_bytes,
+                             const float* row_scale, hipStream_t st) {
+  const bool small_groups = group_size == 64 || group_size == 32;
   TileArgs a = {};
+  a.row_scale = row_scale;
   a.out = (uint16_t*)out;
   a.x = (const uint16_t*)x;
   a.qw = (const u4*)qweight;
@@ -988,7 +1161,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   int ntw = 4;
   const int G = K / 128;
   int splits = tile_splits(M, K, N);
-  const int narrow = small_groups ? 0 : tile_narrow_splits(M, K, N);
+  const int narrow = (small_groups || row_scale) ? 0 : tile_narrow_splits(M, K, N);
   if (narrow) {
     mt = 2;
     ntw = 1;
@@ -1002,7 +1175,9 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
   hipError_t e;
   const uint32_t gpk = (uint32_t)group_size / 128u;
   a.gpk_magic = gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + gpk - 1) / gpk) : 0u;
-  if (small_groups)
+  if (row_scale)
+    e = launch_iobf(a, zeros_kind, row_blocks, st);
+  else if (small_groups)
     e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 4, false>(a, zeros_kind, 128 / group_size, row_blocks, st)
                               : launch_small_groups<MI355Q_BF16, 4, false>(a, zeros_kind, 128 / group_size, row_blocks, st);
   else if (ntw < 4)
@@ -1013,7 +1188,7 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                               : launch_mt<MI355Q_BF16, false>(a, zeros_kind, mt, row_blocks, st);
   MQ_REQUIRE(e == hipSuccess, "w4a16_gemm(tile): cannot reserve LDS: %s", hipGetErrorString(e));
   MQ_LAUNCH_CHECK("w4a16_gemm(tile)");
-  if (splits > 1) return w4a16_splitk_reduce_launch(out, (const float*)workspace, bias, M, N, splits, dtype, st);
+  if (splits > 1) return splitk_reduce_rows_launch(out, (const float*)workspace, bias, M, N, splits, dtype, st, row_scale);
   return 0;
 }
 
