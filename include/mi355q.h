@@ -79,8 +79,9 @@ int mi355q_w4_unpack(const int32_t* packed, uint8_t* dst, int batch, int K, int 
  * time), which split K over two kernels when their grid would leave most of
  * the chip idle.  bf16 activations of 129 rows or more on outputs of two million
  * elements or more are first stored in the workspace as fp16 rows, each times a
- * power of two of its own (exact), and take the fp16 kernels; with a workspace
- * too small for that the bf16 kernel runs (same tolerance, other bits).
+ * power of two of its own (exact), and take the fp16 kernels (group sizes that
+ * are multiples of 128, zero-points not pre-scaled); with a workspace too small
+ * for that the bf16 kernel runs (same tolerance, other bits).
  * `workspace` must hold
  * mi355q_w4a16_workspace_bytes() bytes, be zero-filled once before first use,
  * and must not be shared by launches that may overlap in time. */
@@ -97,7 +98,8 @@ int mi355q_w4a16_gemm(void* out, const void* x, const int32_t* qweight,
  * layers), 3 = MFMA workgroups of up to 128 rows fed through a ring of LDS
  * stages (fp16, group sizes that are multiples of 128; there bits 8..15 of
  * split_k = 1 or 4 select workgroups of 128 or 512 columns instead of
- * 256). */
+ * 256; bf16 above 64 rows with the full workspace: the rows staged as
+ * fp16, workgroups of 256 or 512 columns). */
 int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qweight,
                          const void* scales, const void* zeros, int zeros_kind,
                          const void* bias, int M, int K, int N, int group_size,

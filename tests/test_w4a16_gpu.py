@@ -446,8 +446,9 @@ def test_even_rounds_take_the_512_column_ring_workgroups(ops, rearrange):
 def test_ring_gemm_is_fp16_only_and_tile_family_still_forced(ops, rearrange):
     M, K, N, g = 160, 512, 256, 128
     q, z, s, x = make_case(8, M, K, N, g)
+    # (bf16 reaches the ring kernels as staged fp16 rows, above 64 rows only)
     with pytest.raises(RuntimeError, match="fp16"):
-        run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, family=3)
+        run_gemm(ops, rearrange, q, z, s, x[:48], g, torch.bfloat16, family=3)
     # family 2 keeps meaning the 64-row tile kernel; both agree with the oracle
     a = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=2).float().cpu().numpy()
     b = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16, family=3).float().cpu().numpy()
@@ -497,6 +498,69 @@ def test_bf16_rows_staged_as_fp16_for_the_pipelined_loop(ops, rearrange, M, K, N
     q, z, s, x = make_case(11, M, K, N, g, exact=True)
     want = torch.from_numpy(oracle(q, z, s, x, g, torch.bfloat16)).to(torch.bfloat16)
     assert torch.equal(run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16).cpu(), want)
+
+
+def test_bf16_staging_area_at_the_front_of_the_workspace_for_tall_inputs(ops, rearrange):
+    """4800 x 14336 bf16 is 138 MB as fp16 rows: no launch of that height splits K, so the staging area takes
+    the place of the partial tiles at the front of the workspace and the rows go in two chunks of 2400.
+    Sampled rows against the oracle, everything against the bf16 loop."""
+    M, K, N, g = 4800, 14336, 2048, 128
+    print(f"case bf16 staged tall M={M} K={K} N={N}", flush=True)
+    q, z, s, x = make_case(77, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16)
+    assert torch.equal(got, run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16))
+    plain = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, family=2)
+    np.testing.assert_allclose(got.float().cpu().numpy(), plain.float().cpu().numpy(), rtol=2 ** -6, atol=2e-2)
+    rows = np.array([0, 1, 63, 64, 2399, 2400, 2401, 3000, 4736, 4799])
+    want = oracle(q, z, s, x[rows], g, torch.bfloat16)
+    np.testing.assert_allclose(got[torch.from_numpy(rows).cuda()].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("tw", [2, 4])
+@pytest.mark.parametrize("M,K,N,zeros", [(65, 256, 512, True), (300, 1024, 1024, True), (1000, 2048, 640, False)])
+def test_bf16_rows_staged_as_fp16_on_the_ring_kernels(ops, rearrange, M, K, N, zeros, tw):
+    """The ring kernels (forced: family 3) on bf16 rows staged as fp16: the bf16 scales become fp16 times
+    one power of two for the whole array, taken from the largest of them; row and scale powers of two
+    are undone exactly in the epilogue.  Rows from 2^-60 to 2^60, columns whose scales lie up to 2^-12
+    below the largest; every output is compared at the magnitude of its row and column."""
+    g = 128
+    print(f"case bf16 staged ring M={M} K={K} N={N} zeros={zeros} tw={tw}", flush=True)
+    q, z, s, x = make_case(M + K + tw, M, K, N, g)
+    if not zeros:
+        z[:] = 8
+    rng = np.random.default_rng(M + tw)
+    rmag = (2.0 ** rng.integers(-60, 61, size=M)).astype(np.float32)
+    cmag = (2.0 ** -rng.integers(0, 13, size=N).astype(np.float32)).astype(np.float32)
+    cmag[0] = 1.0
+    x = x * rmag[:, None]
+    s = s * cmag[None, :] * np.float32(2.0 ** 9)
+    x[3] = 0.0
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, family=3, split_k=tw << 8).float().cpu().numpy()
+    want = oracle(q, z, s, x, g, torch.bfloat16)
+    assert np.isfinite(got).all() and (got[3] == 0).all()
+    norm = rmag[:, None] * cmag[None, :] * np.float32(2.0 ** 9)
+    np.testing.assert_allclose(got / norm, want / norm, rtol=RTOL, atol=ATOL)
+    # a bias, at unit magnitudes
+    q, z, s, x = make_case(M + 1, M, K, N, g)
+    bias = rng.standard_normal(N).astype(np.float32)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, bias=bias, family=3, split_k=tw << 8)
+    np.testing.assert_allclose(got.float().cpu().numpy(), oracle(q, z, s, x, g, torch.bfloat16, bias=bias), rtol=RTOL, atol=ATOL)
+    # every product and partial sum representable: bit for bit the oracle
+    q, z, s, x = make_case(13, M, K, N, g, exact=True)
+    want = torch.from_numpy(oracle(q, z, s, x, g, torch.bfloat16)).to(torch.bfloat16)
+    assert torch.equal(run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, family=3, split_k=tw << 8).cpu(), want)
+
+
+def test_bf16_even_rounds_take_the_512_column_ring_workgroups(ops, rearrange):
+    """The shape that the fp16 path gives to the 512-column ring workgroups (one round of 128 x 512 on 256
+    CUs) takes them for bf16 too: the library's own choice is bit for bit the forced launch."""
+    M, K, N, g = 1024, 512, 16384, 128
+    print(f"case bf16 ring 512 columns auto M={M} K={K} N={N}", flush=True)
+    q, z, s, x = make_case(34, M, K, N, g)
+    got = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16)
+    forced = run_gemm(ops, rearrange, q, z, s, x, g, torch.bfloat16, family=3, split_k=4 << 8)
+    assert torch.equal(got, forced)
+    np.testing.assert_allclose(got.float().cpu().numpy(), oracle(q, z, s, x, g, torch.bfloat16), rtol=RTOL, atol=ATOL)
 
 
 def test_large_m_small_group_goes_through_stream_chunks(ops, rearrange):

@@ -17,6 +17,9 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                       hipStream_t st);
 size_t w4a16_tile_workspace_bytes(int M, int K, int N);
 size_t w4a16_bf16_stage_workspace_bytes(int M, int K);
+int w4a16_bf16_staged_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
+                             int zeros_kind, const void* bias, int M, int K, int N, int group_size, void* workspace,
+                             size_t workspace_bytes, int force_tw, hipStream_t st);
 int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
                      void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st);
@@ -112,6 +115,19 @@ extern "C" int mi355q_w4a16_gemm_ex(void* out, const void* x, const int32_t* qwe
     return 0;
   }
   const bool ws_ok = workspace && workspace_bytes > TILE_WS_OFFSET;
+  if (family == 3 && dtype == MI355Q_BF16) {
+    // bf16 rows staged as fp16 in the workspace, ring workgroups of 256 (or, bits 8..15 = 4, 512) columns
+    const int rc = w4a16_bf16_staged_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size,
+                                            ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,
+                                            ws_ok ? workspace_bytes - TILE_WS_OFFSET : 0,
+                                            ((split_k >> 8) & 0xff) == 4 ? 4 : 2, as_stream(stream));
+    MQ_REQUIRE(rc != -12345,
+               "w4a16_gemm: the ring kernels are fp16 kernels; bf16 rows reach them through a workspace of "
+               "mi355q_w4a16_workspace_bytes() bytes, above 64 rows, with group sizes that are multiples of 128 and "
+               "zero-points that are not pre-scaled (M %d, group %d, zero-point kind %d, %zu bytes of workspace)",
+               M, group_size, zeros_kind, workspace_bytes);
+    return rc;
+  }
   if (family == 3)
     return w4a16_mid_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype,
                             ws_ok ? (char*)workspace + TILE_WS_OFFSET : nullptr,

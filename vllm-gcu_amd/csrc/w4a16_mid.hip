@@ -42,6 +42,9 @@ struct MidArgs {
   int kper;                   // K blocks per split (blockIdx.z)
   uint32_t gpk, gpk_magic;    // K blocks per group and ceil(2^32 / gpk)
   float* partial;             // split K: fp32 tiles [split][M][N]; null: write the output
+  // IOBF kernels (bf16 rows staged as fp16 times a power of two each; scales, bias and output bf16):
+  const float* row_scale;     // [M] the power of two each staged row has to be multiplied back by
+  const uint32_t* scale_max;  // [64] largest scale magnitude (bf16 bits) of 64 slices of the scales array
 };
 
 // TW: 16-column tiles per wavefront -- 2: a workgroup of 256 columns; 4: of 512 columns (128 rows only);
@@ -101,9 +104,15 @@ __device__ __forceinline__ uint32_t mid_dequant_pair(uint32_t w, int p, _Float16
   return bitcast<uint32_t>(r);
 }
 
-template <int ZK, int MT, int TW>
+// IOBF: the activations are bf16 rows that a pass before this kernel stored as fp16 times a power of
+// two each; the scales are bf16 and become fp16 here, times one power of two for the whole array that
+// brings the largest of them into [2^10, 2^11) -- (q - z) s stays below fp16's largest number and a
+// scale 2^24 below the largest one still keeps all its bits; the epilogue undoes both powers of two
+// exactly (one ldexp per output) and rounds to bf16.
+template <int ZK, int MT, int TW, bool IOBF = false>
 __global__ void __launch_bounds__(512, 1)
 w4a16_mid_kernel(MidArgs a) {
+  static_assert(!IOBF || ZK != MI355Q_ZP_PRESCALED, "pre-scaled zero-points stay with the bf16 kernel");
   typedef MidCfg<MT, TW> C;
   constexpr int D = C::D, STAGE = C::STAGE, XC = C::XC;
   constexpr bool HASZ = ZK != MI355Q_ZP_NONE;
@@ -125,6 +134,18 @@ w4a16_mid_kernel(MidArgs a) {
   const int gb = (int)blockIdx.z * a.kper, ge = min(G, gb + a.kper);
   const uint32_t lds_base =
       __builtin_amdgcn_readfirstlane((uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds);
+  int sshift = 0;                                     // IOBF: scales are multiplied by 2^sshift
+  if (IOBF) {
+    uint32_t mx = a.scale_max[lane];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)mx, o, 64);
+      mx = mx > other ? mx : other;
+    }
+    const int expo = (int)(mx >> 7);
+    if (mx != 0 && expo != 255) sshift = 10 - ((expo > 0 ? expo : 1) - 127);
+    sshift = __builtin_amdgcn_readfirstlane(sshift);
+  }
 
   // ---- copies.  Activations: one copy moves 4 rows of 256 B; lane = 16 * row + position, and position p
   // of row r receives the row's 16-byte chunk p ^ (r & 15), which keeps the MFMA operand reads (16 rows x
@@ -199,7 +220,8 @@ w4a16_mid_kernel(MidArgs a) {
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
       const uint32_t sw = t < 2 ? q.s.x : q.s.y;
-      sc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
+      if (IOBF) sc[t] = (_Float16)__builtin_ldexpf(bitcast<float>((t & 1) ? (sw & 0xffff0000u) : (sw << 16)), sshift);
+      else sc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (sw >> 16) : (sw & 0xffffu)));
       if (ZK == MI355Q_ZP_PRESCALED) {
         const uint32_t zw = t < 2 ? q.zs.x : q.zs.y;
         zsc[t] = bitcast<_Float16>((uint16_t)((t & 1) ? (zw >> 16) : (zw & 0xffffu)));
@@ -337,6 +359,7 @@ w4a16_mid_kernel(MidArgs a) {
   // 4 columns per lane: a wavefront instruction covers part of a row, one row or two rows
   constexpr int LPR = C::BNW / 4;                      // lanes per row
   constexpr int RPI = LPR >= 64 ? 1 : 64 / LPR, IPR = LPR >= 64 ? LPR / 64 : 1;   // rows per instruction, instructions per row
+  typedef Elem<IOBF ? MI355Q_BF16 : MI355Q_F16> IO;
   f4 bs[IPR];
 #pragma unroll
   for (int q = 0; q < IPR; ++q) {
@@ -344,8 +367,8 @@ w4a16_mid_kernel(MidArgs a) {
     const int col = blockIdx.x * C::BNW + 4 * (lane % LPR) + 256 * q;
     if (a.bias && !a.partial && col < N) {
       const uint2 bw = *(const uint2*)(a.bias + col);
-      bs[q] = (f4){Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.x >> 16)),
-                   Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y & 0xffffu)), Elem<MI355Q_F16>::to_f32((uint16_t)(bw.y >> 16))};
+      bs[q] = (f4){IO::to_f32((uint16_t)(bw.x & 0xffffu)), IO::to_f32((uint16_t)(bw.x >> 16)),
+                   IO::to_f32((uint16_t)(bw.y & 0xffffu)), IO::to_f32((uint16_t)(bw.y >> 16))};
     }
   }
 #pragma unroll
@@ -369,17 +392,24 @@ w4a16_mid_kernel(MidArgs a) {
     for (int p = 0; p < 2 * MTH / RPI; ++p) {
       const int r = RPI * (wave + 8 * p) + (LPR >= 64 ? 0 : lane / LPR), m = m0 + h * 16 * MTH + r;
       if (m >= M) break;
+      // IOBF: the row's power of two and the scales' in one exponent
+      int back = 0;
+      if (IOBF) back = (int)((bitcast<uint32_t>(a.row_scale[m]) >> 23) & 255u) - 127 - sshift;
 #pragma unroll
       for (int q = 0; q < IPR; ++q) {
         const int col = blockIdx.x * C::BNW + 4 * (lane % LPR) + 256 * q;
         if (col >= N) continue;
-        const f4 v = *(const f4*)(lds + r * EP + (lane % LPR) * 16 + 1024 * q);
+        f4 v = *(const f4*)(lds + r * EP + (lane % LPR) * 16 + 1024 * q);
+        if (IOBF) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = __builtin_ldexpf(v[e], back);
+        }
         if (a.partial) {
           *(f4*)(a.partial + ((size_t)blockIdx.z * M + m) * N + col) = v;
         } else {
           uint2 o;
-          o.x = (uint32_t)Elem<MI355Q_F16>::from_f32(v[0] + bs[q][0]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[1] + bs[q][1]) << 16);
-          o.y = (uint32_t)Elem<MI355Q_F16>::from_f32(v[2] + bs[q][2]) | ((uint32_t)Elem<MI355Q_F16>::from_f32(v[3] + bs[q][3]) << 16);
+          o.x = (uint32_t)IO::from_f32(v[0] + bs[q][0]) | ((uint32_t)IO::from_f32(v[1] + bs[q][1]) << 16);
+          o.y = (uint32_t)IO::from_f32(v[2] + bs[q][2]) | ((uint32_t)IO::from_f32(v[3] + bs[q][3]) << 16);
           *(uint2*)(a.out + (size_t)m * N + col) = o;
         }
       }
@@ -397,6 +427,20 @@ int launch_mid(const MidArgs& a, int row_blocks, int splits, hipStream_t st) {
   dim3 grid((a.N + C::BNW - 1) / C::BNW, row_blocks, splits);
   hipLaunchKernelGGL((w4a16_mid_kernel<ZK, MT, TW>), grid, dim3(512), shmem, st, a);
   MQ_LAUNCH_CHECK("w4a16_gemm(mid)");
+  return 0;
+}
+
+// bf16 rows staged as fp16: 128-row workgroups of 256 or 512 columns, no K split
+template <int ZK, int TW>
+int launch_mid_iobf(const MidArgs& a, int row_blocks, hipStream_t st) {
+  typedef MidCfg<8, TW> C;
+  const size_t shmem = (size_t)C::D * C::STAGE;
+  static hipError_t attr = hipFuncSetAttribute((const void*)w4a16_mid_kernel<ZK, 8, TW, true>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  MQ_REQUIRE(attr == hipSuccess, "w4a16_gemm(mid): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
+  dim3 grid((a.N + C::BNW - 1) / C::BNW, row_blocks, 1);
+  hipLaunchKernelGGL((w4a16_mid_kernel<ZK, 8, TW, true>), grid, dim3(512), shmem, st, a);
+  MQ_LAUNCH_CHECK("w4a16_gemm(mid, bf16 staged)");
   return 0;
 }
 
@@ -471,6 +515,33 @@ int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const voi
   if (rc) return rc;
   if (splits > 1) return w4a16_splitk_reduce_launch(out, (const float*)workspace, bias, M, N, splits, dtype, st);
   return 0;
+}
+
+// The same kernels on bf16 rows that the caller staged as fp16 (x16, one power of two per row in
+// row_scale); scales, bias and output are bf16, scale_max holds the largest scale magnitude of 64 slices
+// of the scales array.  128-row workgroups of 256 (tw 2) or 512 (tw 4) columns, K unsplit.
+int w4a16_mid_launch_staged(void* out, const void* x16, const int32_t* qweight, const void* scales, const void* zeros,
+                            int zeros_kind, const void* bias, int M, int K, int N, int group_size,
+                            const float* row_scale, const uint32_t* scale_max, int tw, hipStream_t st) {
+  MQ_REQUIRE(group_size % 128 == 0 && zeros_kind != MI355Q_ZP_PRESCALED && row_scale && scale_max && M > 64,
+             "w4a16_gemm(mid, bf16 staged): group %d, zero-point kind %d, M %d not covered", group_size, zeros_kind, M);
+  MidArgs a = {};
+  a.out = (uint16_t*)out;
+  a.x = (const uint16_t*)x16;
+  a.qw = (const u4*)qweight;
+  a.scales = (const uint16_t*)scales;
+  a.zeros = zeros;
+  a.bias = (const uint16_t*)bias;
+  a.M = M; a.K = K; a.N = N;
+  a.kper = K / 128;
+  a.gpk = (uint32_t)group_size / 128u;
+  a.gpk_magic = a.gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + a.gpk - 1) / a.gpk) : 0u;
+  a.row_scale = row_scale;
+  a.scale_max = scale_max;
+  const int row_blocks = (M + 127) / 128;
+  if (zeros_kind == MI355Q_ZP_NONE)
+    return tw == 4 ? launch_mid_iobf<MI355Q_ZP_NONE, 4>(a, row_blocks, st) : launch_mid_iobf<MI355Q_ZP_NONE, 2>(a, row_blocks, st);
+  return tw == 4 ? launch_mid_iobf<MI355Q_ZP_PACKED, 4>(a, row_blocks, st) : launch_mid_iobf<MI355Q_ZP_PACKED, 2>(a, row_blocks, st);
 }
 
 }  // namespace mi355q

@@ -852,11 +852,41 @@ hipError_t launch_iobf(const TileArgs& a, int zk, int row_blocks, hipStream_t st
 // fp16's subnormal range.  A row that holds an infinity or a NaN is stored unscaled (they stay what
 // they are; its finite elements beyond the fp16 range become infinities).
 // HELD: the row stays in registers between the two passes (K up to 16384); else it is read twice.
+// Workgroups past the rows (64 of them, when scale_max is given) each scan a 64th of the bf16 group
+// scales for the largest magnitude, which the ring kernels turn into one power of two for all scales.
 template <bool HELD>
 __global__ void __launch_bounds__(256)
-bf16_rows_to_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ x16, float* __restrict__ row_scale, int K) {
+bf16_rows_to_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ x16, float* __restrict__ row_scale, int K,
+                        int rows, const u4* __restrict__ scales, long scale_chunks, uint32_t* __restrict__ scale_max) {
   __shared__ uint32_t wmax[4];
   const int tid = threadIdx.x;
+  if ((int)blockIdx.x >= rows) {
+    const long per = (scale_chunks + 63) / 64, b = (long)blockIdx.x - rows;
+    const long end = (b + 1) * per < scale_chunks ? (b + 1) * per : scale_chunks;
+    uint32_t mx = 0;
+    for (long i = b * per + tid; i < end; i += 256) {
+      const u4 v = scales[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = v[j] & 0x7fffu, hi = (v[j] >> 16) & 0x7fffu;
+        mx = mx > lo ? mx : lo;
+        mx = mx > hi ? mx : hi;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)mx, o, 64);
+      mx = mx > other ? mx : other;
+    }
+    if ((tid & 63) == 0) wmax[tid >> 6] = mx;
+    __syncthreads();
+    if (tid == 0) {
+      mx = wmax[0];
+      for (int w = 1; w < 4; ++w) mx = mx > wmax[w] ? mx : wmax[w];
+      scale_max[b] = mx;
+    }
+    return;
+  }
   const u4* row = (const u4*)(x + (size_t)blockIdx.x * K);
   u4* orow = (u4*)(x16 + (size_t)blockIdx.x * K);
   const int chunks = K >> 3;                        // 16-byte pieces of eight elements
@@ -996,6 +1026,9 @@ int w4a16_mid_splits(int M, int K, int N, int tw);
 int w4a16_mid_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
                      int zeros_kind, const void* bias, int M, int K, int N, int group_size, int dtype,
                      void* workspace, size_t workspace_bytes, int splits, int tw, hipStream_t st);
+int w4a16_mid_launch_staged(void* out, const void* x16, const int32_t* qweight, const void* scales, const void* zeros,
+                            int zeros_kind, const void* bias, int M, int K, int N, int group_size,
+                            const float* row_scale, const uint32_t* scale_max, int tw, hipStream_t st);
 
 // Above 128 rows three kernels can take a dense fp16 layer: the 64-row tiles of this file, two workgroups
 // per CU, or the 128-row workgroups with the LDS ring (w4a16_mid.hip), one per CU, 256 or 512 columns
@@ -1091,6 +1124,78 @@ static int tile_launch_dense(void* out, const void* x, const int32_t* qweight, c
                              int group_size, int dtype, void* workspace, size_t workspace_bytes,
                              const float* row_scale, hipStream_t st);
 
+// bf16 activations through the fp16 kernels.  The rows are stored in the staging area of the workspace
+// as fp16 times a power of two each (exact); the pipelined 64-row tile loop multiplies them with the
+// exact integers q - z, the ring kernels with (q - z) s in fp16, as for fp16 activations; inputs taller
+// than the area go in row chunks.  force_tw: -1 the kernels the fp16 path would take for the chunk
+// (ring workgroups where their rounds are priced lower and K stays unsplit), 0 the 64-row tiles,
+// 2 / 4 ring workgroups of 256 / 512 columns.  BF16_STAGE_NOT_TAKEN: group size, zero-point kind or
+// workspace do not allow it, nothing was launched.
+constexpr int BF16_STAGE_NOT_TAKEN = -12345;
+int w4a16_bf16_staged_launch(void* out, const void* x, const int32_t* qweight, const void* scales, const void* zeros,
+                             int zeros_kind, const void* bias, int M, int K, int N, int group_size, void* workspace,
+                             size_t workspace_bytes, int force_tw, hipStream_t st) {
+  if (group_size % 128 != 0 || zeros_kind == MI355Q_ZP_PRESCALED || M <= 64 || !workspace ||
+      workspace_bytes <= BF16_STAGE_OFFSET + BF16_STAGE_SCALE_BYTES)
+    return BF16_STAGE_NOT_TAKEN;
+  // Rows per chunk for a staging area that starts `off` bytes into the workspace
+  auto rows_per_chunk = [&](size_t off) -> long {
+    const size_t room = workspace_bytes - off - BF16_STAGE_SCALE_BYTES;
+    long rows_max = (long)(room / ((size_t)K * 2));
+    // (the last 64 words of the multiplier area hold the scale maxima for the ring kernels)
+    if (rows_max > (long)(BF16_STAGE_SCALE_BYTES / sizeof(float)) - 64) rows_max = BF16_STAGE_SCALE_BYTES / sizeof(float) - 64;
+    rows_max &= ~63L;
+    if (rows_max < 256 && rows_max < M) return 0;
+    const long chunks = (M + rows_max - 1) / rows_max;
+    return (((M + chunks - 1) / chunks) + 63) & ~63L;
+  };
+  // The area lies behind the split-K partial tiles -- or, where no chunk's launch splits K (tall
+  // inputs: exactly those that would otherwise need many chunks), at the front of the workspace
+  size_t off = 0;
+  long per = rows_per_chunk(0);
+  if (per > 0) {
+    const int last = (int)(M % per ? M % per : per);
+    if (tile_splits((int)(per < M ? per : M), K, N) != 1 || tile_splits(last, K, N) != 1) per = 0;
+  }
+  if (per == 0) {
+    off = BF16_STAGE_OFFSET;
+    per = rows_per_chunk(off);
+    if (per == 0) return BF16_STAGE_NOT_TAKEN;
+  }
+  float* rs = (float*)((char*)workspace + off);
+  uint32_t* smax = (uint32_t*)rs + BF16_STAGE_SCALE_BYTES / sizeof(float) - 64;
+  uint16_t* x16 = (uint16_t*)((char*)workspace + off + BF16_STAGE_SCALE_BYTES);
+  const long scale_chunks = (long)(K / group_size) * N / 8;
+  bool scanned = false;
+  for (long m0 = 0; m0 < M; m0 += per) {
+    const int mc = (int)(M - m0 < per ? M - m0 : per);
+    int tw = force_tw;
+    if (tw < 0) {
+      tw = tile_ring_plan(mc, K, N);
+      if (tw == 2 && w4a16_mid_splits(mc, K, N, 2) != 1) tw = 0;
+    }
+    if (mc <= 64) tw = 0;                          // (a short last chunk: the ring kernels here are the 128-row ones)
+    const bool scan = tw && !scanned;
+    scanned |= scan;
+    if (K <= 16384)
+      hipLaunchKernelGGL(bf16_rows_to_f16_kernel<true>, dim3(mc + (scan ? 64 : 0)), dim3(256), 0, st,
+                         (const uint16_t*)x + (size_t)m0 * K, x16, rs, K, mc, (const u4*)scales, scale_chunks, smax);
+    else
+      hipLaunchKernelGGL(bf16_rows_to_f16_kernel<false>, dim3(mc + (scan ? 64 : 0)), dim3(256), 0, st,
+                         (const uint16_t*)x + (size_t)m0 * K, x16, rs, K, mc, (const u4*)scales, scale_chunks, smax);
+    MQ_LAUNCH_CHECK("w4a16_gemm(bf16 rows to fp16)");
+    int rc;
+    if (tw)
+      rc = w4a16_mid_launch_staged((uint16_t*)out + (size_t)m0 * N, x16, qweight, scales, zeros, zeros_kind, bias, mc, K, N,
+                                   group_size, rs, smax, tw, st);
+    else
+      rc = tile_launch_dense((uint16_t*)out + (size_t)m0 * N, x16, qweight, scales, zeros, zeros_kind, bias, mc, K, N,
+                             group_size, MI355Q_BF16, workspace, off, rs, st);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
 int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
                       const void* zeros, int zeros_kind, const void* bias, int M, int K, int N,
                       int group_size, int dtype, void* workspace, size_t workspace_bytes, bool allow_ring,
@@ -1109,33 +1214,11 @@ int w4a16_tile_launch(void* out, const void* x, const int32_t* qweight, const vo
                               workspace_bytes, ss, 1, st);
   }
   // bf16 with a workspace that has the staging area: the rows become fp16 times a power of two each
-  // and take the pipelined fp16 loop, whose B operands are the exact integers q - z (the bf16 loop
-  // has no room for that pipeline: it spills); taller inputs than the area holds go in row chunks
-  if (allow_ring && dtype == MI355Q_BF16 && !small_groups && zeros_kind != MI355Q_ZP_PRESCALED &&
-      bf16_stage_pays(M, N) && workspace && workspace_bytes > BF16_STAGE_OFFSET + BF16_STAGE_SCALE_BYTES) {
-    size_t room = workspace_bytes - BF16_STAGE_OFFSET - BF16_STAGE_SCALE_BYTES;
-    if (room > BF16_STAGE_BYTES) room = BF16_STAGE_BYTES;
-    long rows_max = (long)(room / ((size_t)K * 2));
-    if (rows_max > (long)(BF16_STAGE_SCALE_BYTES / sizeof(float))) rows_max = BF16_STAGE_SCALE_BYTES / sizeof(float);
-    rows_max &= ~63L;
-    if (rows_max >= 256 || rows_max >= M) {
-      const long chunks = (M + rows_max - 1) / rows_max;
-      const long per = (((M + chunks - 1) / chunks) + 63) & ~63L;
-      float* rs = (float*)((char*)workspace + BF16_STAGE_OFFSET);
-      uint16_t* x16 = (uint16_t*)((char*)workspace + BF16_STAGE_OFFSET + BF16_STAGE_SCALE_BYTES);
-      for (long m0 = 0; m0 < M; m0 += per) {
-        const int mc = (int)(M - m0 < per ? M - m0 : per);
-        if (K <= 16384)
-          hipLaunchKernelGGL(bf16_rows_to_f16_kernel<true>, dim3(mc), dim3(256), 0, st, (const uint16_t*)x + (size_t)m0 * K, x16, rs, K);
-        else
-          hipLaunchKernelGGL(bf16_rows_to_f16_kernel<false>, dim3(mc), dim3(256), 0, st, (const uint16_t*)x + (size_t)m0 * K, x16, rs, K);
-        MQ_LAUNCH_CHECK("w4a16_gemm(bf16 rows to fp16)");
-        if (int rc = tile_launch_dense((uint16_t*)out + (size_t)m0 * N, x16, qweight, scales, zeros, zeros_kind, bias, mc, K, N,
-                                       group_size, dtype, workspace, BF16_STAGE_OFFSET, rs, st))
-          return rc;
-      }
-      return 0;
-    }
+  // and take the fp16 loops (the bf16 loop has no room for the pipeline: it spills)
+  if (allow_ring && dtype == MI355Q_BF16 && bf16_stage_pays(M, N)) {
+    const int rc = w4a16_bf16_staged_launch(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, workspace,
+                                            workspace_bytes, -1, st);
+    if (rc != BF16_STAGE_NOT_TAKEN) return rc;
   }
   return tile_launch_dense(out, x, qweight, scales, zeros, zeros_kind, bias, M, K, N, group_size, dtype, workspace,
                            workspace_bytes, nullptr, st);
