@@ -346,7 +346,10 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
  * the same shape.  With it, W4A16 launches whose grid would leave most of the chip idle (a long K
  * with few column tiles: the second expert GEMM of a gated MLP at prefill token counts) split K
  * into fp32 partial tiles and add them up in a second kernel; without it they run unsplit.  The
- * result differs between the two only in the order of the fp32 additions.
+ * result differs between the two only in the order of the fp32 additions.  W4A16 with bf16
+ * activations, blocks of 64 slots and two million outputs or more also stages the rows of `a` there
+ * as fp16 times a power of two each (exact) for the fp16 loop; without the room the bf16 loop runs:
+ * same tolerance, other bits.
  *
  * Size limits (the kernels address operands with 32-bit offsets; exceeding one is an error, not a
  * silent wrap): one expert's weights N * K elements and the activation matrix (numel / topk + 1) * K

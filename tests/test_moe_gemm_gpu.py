@@ -97,6 +97,41 @@ def test_grouped_w4a16_both_gemms(fmoe, rearrange, block, dtype, g):
     np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("K,N", [(512, 2048), (4096, 2048)])
+def test_grouped_w4a16_bf16_rows_staged_as_fp16(fmoe, rearrange, K, N):
+    """bf16 at prefill token counts (blocks of 64 slots, two million outputs or more): the activation rows
+    are staged in the workspace as fp16 times a power of two each and take the pipelined fp16 loop; a
+    slot's multiplier is that of the row it was gathered from.  Rows from 2^-40 to 2^40, both GEMM forms,
+    every output compared at the magnitude of its row; K = 4096 also splits K two ways."""
+    print(f"case grouped w4a16 bf16 staged K={K} N={N}", flush=True)
+    rng = np.random.default_rng(K)
+    M, E, T, g, block, dtype = 600, 4, 2, 128, 64, torch.bfloat16
+    q, z, s = make_int4_experts(rng, E, K, N, g)
+    w, zp = int4_to_device(rearrange, q, z)
+    sd = torch.from_numpy(s).to(dtype)
+    tw, ids, _ = om.topk_softmax(rng.standard_normal((M, E)).astype(np.float32), T, True)
+    wf = lambda e: ow4.dequantize(q[e], z[e], sd[e].float().numpy(), g)
+    mag = (2.0 ** rng.integers(-40, 41, size=M)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32) * mag[:, None]).to(dtype)
+    C = torch.full((M, T, N), 7.0, dtype=dtype, device="cuda")
+    run_grouped(fmoe, x.cuda(), w, C, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, False, T,
+                use_int4_w4a16=True, block_shape=[0, g])
+    want = om.fused_moe_gemm(x.float().numpy(), wf, ids, T)
+    norm = np.repeat(mag, T)[:, None]
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy() / norm, want / norm, rtol=RTOL, atol=ATOL)
+    mag2 = (2.0 ** rng.integers(-40, 41, size=M * T)).astype(np.float32)
+    x2 = torch.from_numpy(rng.standard_normal((M * T, K)).astype(np.float32) * mag2[:, None]).to(dtype)
+    C2 = torch.empty((M, T, N), dtype=dtype, device="cuda")
+    run_grouped(fmoe, x2.cuda(), w, C2, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, True, 1,
+                use_int4_w4a16=True, block_shape=[0, g])
+    want2 = om.fused_moe_gemm(x2.float().numpy(), wf, ids, 1, tw, True)
+    np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy() / mag2[:, None], want2 / mag2[:, None], rtol=RTOL, atol=ATOL)
+    C3 = torch.empty_like(C2)
+    run_grouped(fmoe, x2.cuda(), w, C3, None, sd.cuda(), zp, dev(tw), dev(ids), E, block, True, 1,
+                use_int4_w4a16=True, block_shape=[0, g])
+    assert torch.equal(C2, C3)
+
+
 @pytest.mark.parametrize("block", [16, 32, 64])
 def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe, block):
     # what the reference's moe_wna16 loader leaves on the layer: uint8 [E, N, K/2]

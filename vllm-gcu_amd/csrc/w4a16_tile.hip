@@ -118,7 +118,7 @@ template <> struct TileMma<MI355Q_BF16> {
 // SIMD keep the matrix pipe fed while one of them waits or dequantises).
 // GPB = quantisation groups per K block of 128: 1 for group sizes that are multiples of 128, 2 / 4 for
 // groups of 64 / 32 (plain loop only: each group's steps accumulate into a partial tile of their own).
-// IOBF (with DT = fp16, dense): the activations are bf16 rows that a pass before this kernel scaled by a
+// IOBF (with DT = fp16; grouped: the multiplier belongs to the row the slot was gathered from): the activations are bf16 rows that a pass before this kernel scaled by a
 // power of two each and stored as fp16 (exact: eight mantissa bits into eleven); scales, pre-scaled
 // zero-points, bias and output are bf16, and the epilogue multiplies each row by its power of two.
 template <int DT, int ZK, int MT, bool GROUPED, int WM, bool SF32 = false, int GPB = 1, bool IOBF = false>
@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(256 * WM, WM == 1 ? 2 : 1)
 w4a16_tile_kernel(TileArgs a) {
   typedef TileMma<DT> MM;
   typedef typename MM::vec vec;
-  static_assert(!IOBF || (DT == MI355Q_F16 && !GROUPED), "bf16 in and out around the fp16 loop: dense only");
+  static_assert(!IOBF || (DT == MI355Q_F16 && MT == 4 && WM == 1), "bf16 in and out around the fp16 loop: 64-row tiles");
   typedef Elem<IOBF ? MI355Q_BF16 : DT> IO;       // the type of scales, pre-scaled zero-points, bias and output
   static_assert(MT % WM == 0, "row tiles split evenly over the wavefront rows");
   constexpr int BM = 16 * MT;
@@ -477,6 +477,7 @@ w4a16_tile_kernel(TileArgs a) {
         m = tok[(wmh * MTW + mt) * 16 + 4 * kq + i];
         ok = m < a.numel;
         if (ok && a.topk_weights) rw *= a.topk_weights[m];
+        if (IOBF && ok && !a.partial) rw *= a.row_scale[a.topk == 1 ? m : m / a.topk];
       } else {
         m = m0 + (wmh * MTW + mt) * 16 + 4 * kq + i;
         ok = m < M;
@@ -537,7 +538,8 @@ w4a16_splitk_reduce_kernel(uint16_t* out, const float* partial, const uint16_t* 
 template <int DT>
 __global__ void __launch_bounds__(256)
 w4a16_grouped_reduce_kernel(uint16_t* out, const float* partial, const float* row_weight,
-                            const int32_t* sorted_ids, const int32_t* npp, int numel, int N, int splits) {
+                            const int32_t* sorted_ids, const int32_t* npp, int numel, int N, int splits,
+                            const float* row_scale, int topk) {
   const int n4 = N >> 2;
   const long t = (long)blockIdx.x * 256 + threadIdx.x;
   const long p = t / n4;
@@ -558,6 +560,7 @@ w4a16_grouped_reduce_kernel(uint16_t* out, const float* partial, const float* ro
   }
   for (; s < splits; ++s) v += *(const f4*)(partial + (size_t)s * MN + i);
   if (row_weight) v *= row_weight[id];
+  if (row_scale) v *= row_scale[id / topk];          // bf16 rows staged as fp16: the gathered row's power of two
   uint2 o;
   o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
   o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);
@@ -825,22 +828,23 @@ hipError_t launch_mt(const TileArgs& a, int zk, int mt, int row_blocks, hipStrea
 }
 
 // bf16 activations staged as fp16 rows: 64-row tiles on the pipelined fp16 loop, bf16 in and out
+template <bool GROUPED>
 hipError_t launch_iobf(const TileArgs& a, int zk, int row_blocks, hipStream_t st) {
   const int G = a.K >> 7;
   dim3 grid((a.N + BN - 1) / BN, row_blocks, (G + a.kper - 1) / a.kper), block(256);
   const size_t shmem = 2 * 64 * A_ROW;
   if (zk == MI355Q_ZP_NONE) {
     static hipError_t attr = hipFuncSetAttribute(
-        (const void*)w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_NONE, 4, false, 1, false, 1, true>,
+        (const void*)w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_NONE, 4, GROUPED, 1, false, 1, true>,
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL((w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_NONE, 4, false, 1, false, 1, true>), grid, block, shmem, st, a);
+    hipLaunchKernelGGL((w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_NONE, 4, GROUPED, 1, false, 1, true>), grid, block, shmem, st, a);
   } else {
     static hipError_t attr = hipFuncSetAttribute(
-        (const void*)w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_PACKED, 4, false, 1, false, 1, true>,
+        (const void*)w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_PACKED, 4, GROUPED, 1, false, 1, true>,
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
     if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL((w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_PACKED, 4, false, 1, false, 1, true>), grid, block, shmem, st, a);
+    hipLaunchKernelGGL((w4a16_tile_kernel<MI355Q_F16, MI355Q_ZP_PACKED, 4, GROUPED, 1, false, 1, true>), grid, block, shmem, st, a);
   }
   return hipSuccess;
 }
@@ -1259,7 +1263,7 @@ static int tile_launch_dense(void* out, const void* x, const int32_t* qweight, c
   const uint32_t gpk = (uint32_t)group_size / 128u;
   a.gpk_magic = gpk > 1 ? (uint32_t)((((uint64_t)1 << 32) + gpk - 1) / gpk) : 0u;
   if (row_scale)
-    e = launch_iobf(a, zeros_kind, row_blocks, st);
+    e = launch_iobf<false>(a, zeros_kind, row_blocks, st);
   else if (small_groups)
     e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 4, false>(a, zeros_kind, 128 / group_size, row_blocks, st)
                               : launch_small_groups<MI355Q_BF16, 4, false>(a, zeros_kind, 128 / group_size, row_blocks, st);
@@ -1299,9 +1303,22 @@ static int grouped_splits(int numel, int block_size, int max_blocks, int E, int 
   while (s > 1 && (size_t)s * numel * N * sizeof(float) > TILE_SPLITK_BYTES * 2) --s;
   return s < 1 ? 1 : (int)s;
 }
+// bf16 activations of a grouped launch staged as fp16 rows (blocks of 64 slots, outputs of two million
+// elements or more): the area follows the partial tiles of the launch's split-K plan
+static bool grouped_stage_pays(int numel, int block_size, int N) {
+  return block_size == 64 && (long)numel * N >= (1L << 21);
+}
+static size_t grouped_partial_bytes(int splits, int numel, int N) {
+  return splits > 1 ? (((size_t)splits * numel * N * sizeof(float)) + 255) & ~(size_t)255 : 0;
+}
 size_t w4a16_grouped_workspace_bytes(int numel, int block_size, int max_blocks, int E, int K, int N) {
   const int s = grouped_splits(numel, block_size, max_blocks, E, K, N);
-  return s > 1 ? (size_t)s * numel * N * sizeof(float) : 0;
+  size_t need = s > 1 ? (size_t)s * numel * N * sizeof(float) : 0;
+  // (neither the dtype nor topk is known here: room for bf16 rows of one slot each)
+  // (asked for while everything stays within 128 MiB; a larger workspace is used when it is there)
+  const size_t staged = grouped_partial_bytes(s, numel, N) + BF16_STAGE_SCALE_BYTES + (size_t)numel * K * 2;
+  if (grouped_stage_pays(numel, block_size, N) && staged <= 2 * BF16_STAGE_BYTES) need = staged;
+  return need;
 }
 
 int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const void* scales,
@@ -1344,11 +1361,36 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
   a.kper = (G + splits - 1) / splits;
   splits = (G + a.kper - 1) / a.kper;              // no empty splits
   a.partial = splits > 1 ? (float*)workspace : nullptr;
+  // bf16 at prefill token counts: the rows staged as fp16 times a power of two each take the pipelined
+  // fp16 loop (see w4a16_bf16_staged_launch); the multiplier of a slot is that of the row it was gathered from
+  bool staged = false;
+  if (dtype == MI355Q_BF16 && !small_groups && !scales_f32 && !out_scale && zeros_kind != MI355Q_ZP_PRESCALED &&
+      grouped_stage_pays(numel, block_size, N) && workspace && topk > 0) {
+    const size_t poff = grouped_partial_bytes(splits, numel, N);
+    const int rows = numel / topk;
+    if (rows > 0 && rows <= (int)(BF16_STAGE_SCALE_BYTES / sizeof(float)) &&
+        poff + BF16_STAGE_SCALE_BYTES + (size_t)rows * K * 2 <= workspace_bytes) {
+      float* rs = (float*)((char*)workspace + poff);
+      uint16_t* x16 = (uint16_t*)((char*)workspace + poff + BF16_STAGE_SCALE_BYTES);
+      if (K <= 16384)
+        hipLaunchKernelGGL(bf16_rows_to_f16_kernel<true>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x, x16, rs, K, rows,
+                           (const u4*)nullptr, 0L, (uint32_t*)nullptr);
+      else
+        hipLaunchKernelGGL(bf16_rows_to_f16_kernel<false>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x, x16, rs, K, rows,
+                           (const u4*)nullptr, 0L, (uint32_t*)nullptr);
+      MQ_LAUNCH_CHECK("moe_w4a16(bf16 rows to fp16)");
+      a.x = x16;
+      a.row_scale = rs;
+      staged = true;
+    }
+  }
   a.w_stride = (long)(K / 8) * N / 4;              // u4 elements per expert
   a.s_stride = (long)(K / group_size) * N;
   a.z_stride = zeros_kind == MI355Q_ZP_PACKED ? (long)(K / group_size) * (N / 8) : (long)(K / group_size) * N;
   hipError_t e;
-  if (small_groups) {
+  if (staged) {
+    e = launch_iobf<true>(a, zeros_kind, max_blocks, st);
+  } else if (small_groups) {
     const int gpb = 128 / group_size;
     if (block_size == 16)
       e = (dtype == MI355Q_F16) ? launch_small_groups<MI355Q_F16, 1, true>(a, zeros_kind, gpb, max_blocks, st)
@@ -1375,10 +1417,10 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
     const unsigned blocks = (unsigned)((threads + 255) / 256);
     if (dtype == MI355Q_F16)
       hipLaunchKernelGGL((w4a16_grouped_reduce_kernel<MI355Q_F16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, topk_weights, sorted_ids, npp, numel, N, splits);
+                         (const float*)workspace, topk_weights, sorted_ids, npp, numel, N, splits, (const float*)nullptr, 1);
     else
       hipLaunchKernelGGL((w4a16_grouped_reduce_kernel<MI355Q_BF16>), dim3(blocks), dim3(256), 0, st, (uint16_t*)out,
-                         (const float*)workspace, topk_weights, sorted_ids, npp, numel, N, splits);
+                         (const float*)workspace, topk_weights, sorted_ids, npp, numel, N, splits, a.row_scale, topk);
     MQ_LAUNCH_CHECK("moe_w4a16(split-K reduce)");
   }
   return 0;
