@@ -11,6 +11,15 @@ from oracle import w4 as ow4
 from oracle import w8a8 as o8
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(params=[False, True], ids=["zeros-as-given", "zeros-recovered"])
+def zero_reading(request, monkeypatch):
+    """Pre-scaled zero-points either reach the kernels as given or, the default, are turned back into
+    the packed integers once per tensor."""
+    from vllm_gcu_amd.kernels import _custom_ops
+    monkeypatch.setattr(_custom_ops, "_RECOVER_INTEGER_ZEROS", request.param)
+    return request.param
 RTOL = ATOL = 1e-2
 
 
@@ -133,7 +142,7 @@ def test_grouped_w4a16_bf16_rows_staged_as_fp16(fmoe, rearrange, K, N):
 
 
 @pytest.mark.parametrize("block", [16, 32, 64])
-def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe, block):
+def test_grouped_w4a16_reference_layout_and_prescaled_zeros(fmoe, block, zero_reading):
     # what the reference's moe_wna16 loader leaves on the layer: uint8 [E, N, K/2]
     # half-group bytes (moe_wna16.py:464-466) and fp16 zeros = z * scales
     # (blocks of 16 / 32 slots run the weight-streaming kernel, 64 the MFMA tile kernel)

@@ -29,6 +29,16 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+@pytest.fixture(params=[False, True], ids=["zeros-as-given", "zeros-recovered"])
+def zero_reading(request, monkeypatch):
+    """Pre-scaled zero-points (z * s in the activation type) either reach the kernels as given
+    (w = q * s - zeros: the kernels' pre-scaled variants) or, the default, are turned back into the packed
+    integers once per tensor (w = (q - z) * s: the integer variants)."""
+    from vllm_gcu_amd.kernels import _custom_ops
+    monkeypatch.setattr(_custom_ops, "_RECOVER_INTEGER_ZEROS", request.param)
+    return request.param
+
+
 def make_case(seed, M, K, N, g, dtype=np.float16, exact=False):
     rng = np.random.default_rng(seed)
     G = K // (K if g == -1 else g)
@@ -233,7 +243,7 @@ def test_symmetric_default_zero_point(ops, rearrange):
 
 
 @pytest.mark.parametrize("M", [2, 48])
-def test_reference_layout_drop_in(ops, M):
+def test_reference_layout_drop_in(ops, M, zero_reading):
     # exactly what the reference's GPTQ loader leaves on the layer
     # (gptq.py:229-261): uint8 half-group weights, fp16 zeros = z * scales
     K, N, g = 512, 256, 128
@@ -322,7 +332,7 @@ def test_tile_gemm_three_way_split_between_half_and_full_round(ops, rearrange):
     assert torch.equal(got[torch.from_numpy(rows)], want)
 
 
-def test_tile_gemm_zero_kinds_and_group_256(ops, rearrange):
+def test_tile_gemm_zero_kinds_and_group_256(ops, rearrange, zero_reading):
     M, K, N, g = 130, 512, 256, 256
     q, z, s, x = make_case(77, M, K, N, g)
     got = run_gemm(ops, rearrange, q, z, s, x, g, torch.float16).float().cpu().numpy()
@@ -394,7 +404,7 @@ def test_ring_gemm_parity(ops, rearrange, M, K, N, g, split, tw):
 
 @pytest.mark.parametrize("tw", [2, 1, 4])
 @pytest.mark.parametrize("M", [32, 64, 128, 200])
-def test_ring_gemm_zero_kinds(ops, rearrange, M, tw):
+def test_ring_gemm_zero_kinds(ops, rearrange, M, tw, zero_reading):
     """No zero-points (z = 8) and the reference's pre-scaled fp16 zero-points, where the kernel forms
     q * s - zs in one fused multiply-add: the oracle of that form is dequantize_prescaled_zeros."""
     K, N, g = 1024, 384, 128
@@ -601,7 +611,7 @@ def test_tile_gemm_groups_of_64_and_32(ops, rearrange, M, K, N, g, dtype):
 
 
 @pytest.mark.parametrize("g", [64, 32])
-def test_tile_gemm_small_groups_zero_kinds(ops, rearrange, g):
+def test_tile_gemm_small_groups_zero_kinds(ops, rearrange, g, zero_reading):
     """No zero-points and pre-scaled 16-bit zero-points with groups of 64 and 32 on the MFMA kernel."""
     M, K, N = 200, 1024, 384
     print(f"case small groups zero kinds g={g}", flush=True)
@@ -635,7 +645,7 @@ def _random_cases():
 
 
 @pytest.mark.parametrize("seed,M,K,N,g,dt,zk,with_bias", _random_cases())
-def test_random_shapes_through_the_library_s_own_choice(ops, rearrange, seed, M, K, N, g, dt, zk, with_bias):
+def test_random_shapes_through_the_library_s_own_choice(ops, rearrange, seed, M, K, N, g, dt, zk, with_bias, zero_reading):
     """Seeded random shapes, group sizes, types, zero-point kinds and bias through mi355q_w4a16_gemm as a
     caller uses it (no family forced): whichever kernel and split the dispatcher takes, the result is the
     oracle's within the tolerance and run-to-run identical."""
@@ -667,6 +677,34 @@ def test_random_shapes_through_the_library_s_own_choice(ops, rearrange, seed, M,
         if bias is not None:
             want = want + to_act(bias, dtype).float().numpy()[None, :]
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_integer_zero_points_are_recovered_only_when_exact(ops, rearrange, dtype):
+    """zeros == z.to(dtype) * scales bit for bit with z in 0..15 (what the reference's loaders store) comes
+    back as the packed integers; one element one step off, a zero-point of 16, or a non-integer multiple
+    keeps the tensor as given.  A scale of 0 with a zero of 0 is an integer zero-point (any: 0 is taken)."""
+    rng = np.random.default_rng(17)
+    G, N = 6, 256
+    z = rng.integers(0, 16, size=(G, N), dtype=np.uint8)
+    s = to_act(rng.uniform(0.001, 0.01, size=(G, N)).astype(np.float32), dtype).cuda()
+    s[2, 5] = 0.0
+    zt = torch.from_numpy(z).cuda()
+    zs = zt.to(dtype) * s
+    packed = ops._integer_zeros(zs, s)
+    assert packed is not None and packed.dtype == torch.int32 and packed.shape == (G, N // 8)
+    z_expect = z.copy()
+    z_expect[2, 5] = 0
+    assert torch.equal(packed, rearrange.pack_int8_zeros(torch.from_numpy(z_expect).cuda()))
+    assert ops._integer_zeros(zs, s) is packed                       # cached on the tensor
+    z_kind = ops._zero_points(zs, dtype, s)
+    assert z_kind[1] == ops._lib.ZP_PACKED and z_kind[0] is packed
+    off = zs.clone()
+    off[1, 7] = (off[1, 7].view(torch.int16) + 1).view(dtype)           # one step of the type
+    assert ops._integer_zeros(off, s) is None and ops._zero_points(off, dtype, s)[1] == ops._lib.ZP_PRESCALED
+    assert ops._integer_zeros((zt.to(dtype) + 16) * s, s) is None       # out of the int4 range
+    assert ops._integer_zeros(zs * 0.5 + s * 0.25, s) is None           # not integers
+    assert ops._zero_points(zs, dtype, s.float())[1] == ops._lib.ZP_PRESCALED   # scales the caller holds in another type
 
 
 def test_operand_shapes_are_checked_on_the_host(ops, rearrange):

@@ -79,8 +79,40 @@ def _slab_weight(qweight: torch.Tensor, transposed: bool = False) -> torch.Tenso
     return _converted(qweight, lambda t: rearrange.from_reference_layout(t, transposed=transposed))
 
 
-def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype):
-    """-> (tensor or None, zeros_kind)"""
+# Pre-scaled zero-points that are bit for bit (integer 0..15) x scale in the activation type are what the
+# reference's loaders leave on a layer (rearrange.py:33-34, 103-105: ``zeros = z * scales``).  They are
+# turned back into the packed integers once per tensor: w = (q - z) * s is the operator's definition
+# (gptq_gemm_gcu), every kernel then takes the same reading of it, and prefill takes the pipelined loops,
+# which exist for integer zero-points only.  Anything else stays as given (w = q * s - zeros).
+_RECOVER_INTEGER_ZEROS = True
+
+
+def _integer_zeros(zeros: torch.Tensor, scales: torch.Tensor) -> Optional[torch.Tensor]:
+    """Packed int32 zero-points [..., G, N/8] if ``zeros == z.to(dtype) * scales`` bit for bit for
+    integers z in 0..15 (where the scale is 0: zeros 0), else None.  Cached on ``zeros``; the check
+    reads one flag back from the device, so it never runs while a graph is being captured."""
+    tag = (zeros.data_ptr(), zeros._version, tuple(zeros.shape), scales.data_ptr(), scales._version)
+    hit = getattr(zeros, "_mi355q_integer_zeros", None)
+    if hit is not None and hit[0] == tag:
+        return hit[1]
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    packed = None
+    if zeros.shape == scales.shape and zeros.shape[-1] % 8 == 0:
+        s32 = scales.float()
+        z = torch.where(s32 != 0, torch.round(zeros.float() / s32), torch.zeros_like(s32))
+        ok = (z >= 0) & (z <= 15)
+        zi = torch.nan_to_num(z, nan=0.0).clamp_(0, 15)
+        ok &= (zi.to(scales.dtype) * scales) == zeros
+        if bool(ok.all()):
+            packed = rearrange.pack_int8_zeros(zi.to(torch.uint8)).contiguous()
+    zeros._mi355q_integer_zeros = (tag, packed)
+    return packed
+
+
+def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype, scales: Optional[torch.Tensor] = None):
+    """-> (tensor or None, zeros_kind); ``scales``: the group scales as the caller holds them (in the
+    activation type), for the recovery of integer zero-points from pre-scaled ones"""
     if zeros is None or zeros.numel() == 0:
         return None, _lib.ZP_NONE
     if zeros.dtype == torch.int32:
@@ -88,6 +120,10 @@ def _zero_points(zeros: Optional[torch.Tensor], act_dtype: torch.dtype):
     if zeros.dtype in (torch.int8, torch.uint8):
         return _converted(zeros, rearrange.pack_int8_zeros), _lib.ZP_PACKED
     if zeros.dtype == act_dtype:
+        if _RECOVER_INTEGER_ZEROS and scales is not None and scales.dtype == act_dtype and scales.is_cuda:
+            packed = _integer_zeros(zeros, scales)
+            if packed is not None:
+                return packed, _lib.ZP_PACKED
         return zeros, _lib.ZP_PRESCALED
     raise TypeError(f"zero-points of dtype {zeros.dtype} do not match activations of dtype {act_dtype}")
 
@@ -115,10 +151,10 @@ def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     if qw.shape[-2] * 8 != K:
         raise RuntimeError(f"w4a16_gemm: activation K={K} does not match weight K={qw.shape[-2] * 8}")
     x = x.contiguous()
+    z, zk = _zero_points(zeros, x.dtype, scales)
     scales = scales.contiguous()
     if scales.dtype != x.dtype:
         scales = scales.to(x.dtype)
-    z, zk = _zero_points(zeros, x.dtype)
     if z is not None:
         z = z.contiguous()
     if bias is not None:
@@ -1039,10 +1075,10 @@ def _moe_gemm(C, A, B, A_scale, B_scale, gs, B_zp, topk_weights, topk_ids, sorte
         w = _slab_weight(B, transposed=True)
         if w.shape[-2] * 8 != K or w.shape[-1] != N:
             raise RuntimeError(f"fused_moe: int4 experts of shape {tuple(w.shape)} do not fit K={K}, N={N}")
+        zp, zk = _zero_points(B_zp, A.dtype, B_scale)
         w_scale = B_scale.contiguous()
         if w_scale.dtype != A.dtype:
             w_scale = w_scale.to(A.dtype)
-        zp, zk = _zero_points(B_zp, A.dtype)
         if zp is not None:
             zp = zp.contiguous()
         if group <= 0:
