@@ -77,7 +77,7 @@ int mi355q_w4_unpack(const int32_t* packed, uint8_t* dst, int batch, int K, int 
  * streaming kernel, larger M the LDS-staged MFMA kernels (groups of 32, 64 and
  * multiples of 128; other sizes go through the streaming kernel 32 rows at a
  * time), which split K over two kernels when their grid would leave most of
- * the chip idle.  bf16 activations of 129 rows or more on outputs of two million
+ * the chip idle.  bf16 activations of 65 rows or more on outputs of about two million
  * elements or more are first stored in the workspace as fp16 rows, each times a
  * power of two of its own (exact), and take the fp16 kernels (group sizes that
  * are multiples of 128, zero-points not pre-scaled); with a workspace too small

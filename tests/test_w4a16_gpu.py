@@ -467,7 +467,7 @@ def test_ring_gemm_is_fp16_only_and_tile_family_still_forced(ops, rearrange):
     np.testing.assert_allclose(b, want, rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("M,K,N,zeros", [(129, 512, 16384, True), (300, 4096, 7168, True), (640, 1024, 3328, False),
+@pytest.mark.parametrize("M,K,N,zeros", [(65, 256, 28672, True), (129, 512, 16384, True), (300, 4096, 7168, True), (640, 1024, 3328, False),
                                          (2400, 14336, 1024, True), (256, 16512, 8192, True)])
 def test_bf16_rows_staged_as_fp16_for_the_pipelined_loop(ops, rearrange, M, K, N, zeros):
     """bf16 from 129 rows on, the library's own choice with the operator's workspace: each row times a

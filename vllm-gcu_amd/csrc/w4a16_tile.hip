@@ -1110,12 +1110,13 @@ size_t w4a16_tile_workspace_bytes(int M, int K, int N) {
 constexpr size_t BF16_STAGE_OFFSET = TILE_SPLITK_BYTES;
 constexpr size_t BF16_STAGE_SCALE_BYTES = (size_t)64 << 10;          // one multiplier per staged row
 constexpr size_t BF16_STAGE_BYTES = (size_t)64 << 20;
-constexpr int BF16_STAGE_MIN_M = 129;
+constexpr int BF16_STAGE_MIN_M = 65;
 // (measured, us, staged against the bf16 loop: K 4096 x N 28672 at M = 129 / 2048 / 8192: 68 / 477 / 1812
 // against 85 / 578 / 2202; K 4096 x N 6144 at 256 / 512 / 2048: 34 / 49 / 119 against 35 / 55 / 136; K 4096 x
 // N 4096 at 512 / 1024 / 4096: 38 / 53 / 151 against 39 / 58 / 170; K 14336 x N 4096 at 512 / 2048: 85 / 258
-// against 91 / 299: the conversion pass costs 5-25 us, so the output has to have about two million elements)
-static bool bf16_stage_pays(int M, int N) { return M >= BF16_STAGE_MIN_M && (long)M * N >= (1L << 21); }
+// against 91 / 299; 65..128 rows, K 4096 x N 28672 at M = 80 / 100 / 128: 49 / 51 / 51 against 60: the conversion
+// pass costs 5-25 us, so the output has to have about two million elements)
+static bool bf16_stage_pays(int M, int N) { return M >= BF16_STAGE_MIN_M && (long)M * N >= (7L << 18); }
 
 size_t w4a16_bf16_stage_workspace_bytes(int M, int K) {
   if (M < BF16_STAGE_MIN_M) return 0;
