@@ -357,6 +357,8 @@ def main():
         torch.cuda.empty_cache()
     if args.extras:
         out["moe_w4a16_decode"] = moe_bench(ops, dev, stream, "w4a16", tokens=16)
+        import torch as _torch
+        out["moe_w4a16_bf16"] = moe_bench(ops, dev, stream, "w4a16", tokens=512, act_dtype=_torch.bfloat16)
         torch.cuda.empty_cache()
         out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")
         torch.cuda.empty_cache()
@@ -516,7 +518,7 @@ def cpu_baseline_moe_fp8(x, tw, ids, w13, s13, w2, s2, tokens=2):
                       f"experts' weights"}
 
 
-def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False):
+def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False, act_dtype=None):
     """BASELINE configs[3] (Mixtral-8x7B layer, W4A16) and configs[4]
     (DeepSeek-V3-style layer, fp8 block-scaled): routing + the whole
     fused-experts sequence, one layer."""
@@ -535,9 +537,10 @@ def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False):
         M, H, E, I, T = tokens or 512, 4096, 8, 14336, 2
         w13, w2 = rnd_i32(E, H // 8, 2 * I), rnd_i32(E, I // 8, H)
         z13, z2 = rnd_i32(E, H // 128, 2 * I // 8), rnd_i32(E, I // 128, H // 8)
-        s13 = (torch.rand(E, H // 128, 2 * I, device=dev) * 0.009 + 0.001).half()
-        s2 = (torch.rand(E, I // 128, H, device=dev) * 0.009 + 0.001).half()
-        x = torch.randn(M, H, generator=g).half().to(dev)
+        adt = act_dtype or torch.float16             # (configs[3] states fp16; bf16 is the type Mixtral ships in)
+        s13 = (torch.rand(E, H // 128, 2 * I, device=dev) * 0.009 + 0.001).to(adt)
+        s2 = (torch.rand(E, I // 128, H, device=dev) * 0.009 + 0.001).to(adt)
+        x = torch.randn(M, H, generator=g).to(adt).to(dev)
         logits = torch.randn(M, E, generator=g).to(dev)
         moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad(use_int4_w4a16=True, block_shape=[0, 128]))
         kw = dict(w1_scale=s13, w2_scale=s2, w1_zp=z13, w2_zp=z2)
@@ -548,7 +551,8 @@ def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False):
         flops = 2.0 * M * T * (H * 2 * I + I * H)
         bytes_ = E * (H * 2 * I + I * H) // 2 + E * (H // 128 * 2 * I + I // 128 * H) * 2 \
             + E * (H // 128 * 2 * I + I // 128 * H) // 2 + 2 * M * H * 2
-        name = f"fused MoE W4A16, Mixtral-8x7B layer: {M} tok, hidden 4096, 8 experts, inter 14336, top-2"
+        name = f"fused MoE W4A16, Mixtral-8x7B layer: {M} tok, hidden 4096, 8 experts, inter 14336, top-2" + \
+            (", bf16 activations" if adt == torch.bfloat16 else "")
     elif which == "w4a8":
         # the Mixtral-8x7B layer of configs[3] with w4a8-fp8 experts: fp8 activations with one
         # static scale per GEMM, symmetric int4 weights, fp32 group scales
@@ -752,7 +756,7 @@ def variants_bench(ops, dev, stream):
         for dt, g in ((torch.float16, 128), (torch.bfloat16, 128), (torch.float16, 64), (torch.float16, 32)):
             zp = torch.randint(-2**31, 2**31 - 1, (K // g, N // 8), dtype=torch.int32, generator=gen).to(dev)
             sc = (torch.rand(K // g, N, generator=gen) * 0.009 + 0.001).to(dt).to(dev)
-            for M in (128, 2048):
+            for M in ((128, 2048, 8192) if dt == torch.bfloat16 else (128, 2048)):
                 x = torch.randn(M, K, dtype=dt, device=dev)
                 fns = [(lambda qw=qw: ops.w4a16_gemm(x, qw, sc, zp, None, g)) for qw in qws]
                 n = 30
