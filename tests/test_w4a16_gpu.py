@@ -640,7 +640,10 @@ def _random_cases():
         cases.append((i, M, K, N, g, ["f16", "bf16"][int(rng.integers(0, 2))], int(rng.integers(0, 3)), bool(rng.integers(0, 2))))
     # wide enough for the 512-column ring workgroups and for several rounds of every kernel
     cases += [(100, 2048, 1024, 8192, 128, "f16", 1, True), (101, 1536, 512, 12288, 128, "f16", 0, False),
-              (102, 1300, 2048, 4096, 128, "bf16", 1, True), (103, 640, 1024, 16384, 64, "f16", 1, False)]
+              (102, 1300, 2048, 4096, 128, "bf16", 1, True), (103, 640, 1024, 16384, 64, "f16", 1, False),
+              # bf16 rows staged as fp16: the 512-column ring workgroups, 64-row tiles with and without zero-points
+              (104, 1024, 1024, 16384, 128, "bf16", 2, True), (105, 200, 512, 12288, 128, "bf16", 0, False),
+              (106, 90, 768, 28672, 256, "bf16", 1, True)]
     return cases
 
 
