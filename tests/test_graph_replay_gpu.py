@@ -83,6 +83,31 @@ def test_replay_survives_a_larger_eager_plan_on_the_capture_stream():
         between=lambda: ops.w4a16_gemm(big, qw, sc, zp, None, g))
 
 
+@pytest.mark.parametrize("M,K,N", [(300, 4096, 7168), (1024, 512, 16384)])
+def test_bf16_rows_staged_in_the_workspace_replay(M, K, N):
+    """bf16 prefill stages its rows as fp16 in the stream's workspace (64-row tiles at 300 rows, the
+    512-column ring workgroups with their scale maxima at 1024 x 16384).  Between the replays another bf16
+    launch of another height overwrites the staging area and a split-K launch the partial tiles before it."""
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    g = 128
+    gen = torch.Generator(device="cpu").manual_seed(M)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 8, N), dtype=torch.int32, generator=gen).cuda()
+    zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, generator=gen).cuda()
+    sc = (torch.rand(K // g, N, generator=gen) * 0.009 + 0.001).bfloat16().cuda()
+    x = torch.randn(M, K, generator=gen).bfloat16().cuda()
+    other = (torch.randn(777, K, generator=gen) * 1000.0).bfloat16().cuda()
+    small = torch.randn(128, K, generator=gen).bfloat16().cuda()
+    print(f"case graph replay w4a16 bf16 staged M={M} K={K} N={N}", flush=True)
+
+    def between():
+        ops.w4a16_gemm(other, qw, sc, zp, None, g)
+        ops.w4a16_gemm(small, qw, sc, zp, None, g)
+    _replay_against_eager(
+        lambda: ops.w4a16_gemm(x, qw, sc, zp, None, g),
+        [x], lambda i: [(torch.randn(M, K, generator=gen) * (4.0 ** i)).bfloat16()],
+        between=between)
+
+
 def test_workspace_refuses_to_allocate_under_capture(monkeypatch):
     from vllm_gcu_amd.kernels import _runtime as rt
     dev = torch.device("cuda", torch.cuda.current_device())
