@@ -114,7 +114,7 @@ def test_equals_block_scaled_gemm_when_block_scales_are_constant():
 
 
 @pytest.mark.parametrize("M,K,N", [(128, 4096, 1024), (300, 8192, 512), (700, 2048, 1024), (65, 7168, 1536),
-                                   (17, 7168, 1536), (25, 7168, 4096), (49, 4096, 1024)])
+                                   (33, 7168, 1536), (33, 7168, 4096), (25, 14336, 1024)])
 @pytest.mark.parametrize("kslab", [False, True])
 def test_few_tiles_behind_a_long_k_are_split_into_k_ranges(M, K, N, kslab):
     """Both fp8 tile kernels on layers with few 256 x 128 tiles: K ranges run side by side, their fp32 sums

@@ -103,6 +103,34 @@ def test_int8_gemm_kslab_weights(ops, M, K, N):
         np.testing.assert_allclose(a.float().cpu().numpy(), wantf, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("N", [1536, 7168, 16384])
+@pytest.mark.parametrize("M", [1, 16, 17, 32, 33, 64])
+def test_int8_streaming_kernel_16_32_and_64_columns_per_workgroup(ops, M, N, monkeypatch):
+    """The weight-streaming kernel gives a layer of few columns 16 (N = 1536) or 32 (N = 7168) columns
+    per workgroup instead of 64 (N = 16384), so that about every CU streams a share of the weights.
+    Kslab and row-major weights, every row-tile count: against the exact integer oracle through the
+    epilogue, and bit for bit equal to the MFMA tile kernel on the same operands."""
+    from vllm_gcu_amd.kernels import _custom_ops
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print(f"case i8 streaming narrow groups M={M} N={N}", flush=True)
+    K = 1024
+    rng = np.random.default_rng(M + N)
+    x = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    w_nk = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    xs = rng.uniform(0.001, 0.01, size=(M, 1)).astype(np.float32)
+    ws = rng.uniform(0.001, 0.02, N).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.float16).cuda()
+    want = o8.scaled_mm_epilogue(o8.int8_gemm_i32(x, np.ascontiguousarray(w_nk.T)), xs, ws, bias.float().cpu().numpy())
+    wk = rearrange.to_kslab(dev(w_nk))
+    monkeypatch.setattr(_custom_ops, "_INT8_STREAM_MAX_M", 1 << 20)           # the streaming kernel whatever the shape
+    got = ops.cutlass_scaled_mm(dev(x), wk.t(), dev(xs), dev(ws), torch.float16, bias)
+    row_major = ops.cutlass_scaled_mm(dev(x), dev(w_nk).t(), dev(xs), dev(ws), torch.float16, bias)
+    np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    monkeypatch.setattr(_custom_ops, "_INT8_STREAM_MAX_M", 0)                 # the tile kernel
+    tile = ops.cutlass_scaled_mm(dev(x), wk.t(), dev(xs), dev(ws), torch.float16, bias)
+    assert torch.equal(got, tile) and torch.equal(got, row_major)
+
+
 @pytest.mark.parametrize("M,K,N,splits", [(128, 4096, 1024, 4), (200, 8192, 512, 8), (700, 2048, 1024, 2),
                                             (64, 14336, 4096, 8), (1000, 3072, 768, 3)])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])

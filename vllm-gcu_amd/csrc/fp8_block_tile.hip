@@ -474,14 +474,17 @@ int launch_f8_splitk(const F8Args& a, int splits, void* workspace, hipStream_t s
 }
 
 // Rows from which the tile kernel with K ranges side by side is ahead of the weight-streaming kernel,
-// whose time grows with the rows while the split tile kernel's hardly does (measured, us at 16 / 32 /
-// 48 / 64 rows, streaming against split: K 16384 N 7168 33/41/52/62 against 33/33/33/35; K 7168 N 4096
-// 16/20/26/30 against 16/17/17/18; K 8192 N 8192 21/24/29/34 against 23/24/24/24; K 4096 N 4096
-// 10/13/17/20 against 15/15/16/17; K 2048 N 7168 7/9/11/12 against 14/15/15/16).
+// whose time grows with the rows (in steps at 17 and 33: its row tiles) while the split tile kernel's
+// hardly does (measured, us at 16 / 24 / 32 / 40 / 64 rows, streaming against split: K 28672 N 8192
+// 43/53/60/72/92 against 53/52/53/53/54; K 16384 N 7168 24/31/31/39/53 against 34/32/32/32/34; K 14336
+// N 4096 17/21/25/32/45 against 20/21/21/21/23; K 7168 N 4096 9/12/14/18/25 against 16/16/17/17/18;
+// K 8192 N 8192 14/18/19/23/30 against 23/23/22/23/24; K 8192 N 10240, three ranges, 23/29/33/42/55 against
+// 31/31/31/32/33; K 4096 N 4096 7/9/10/13/16 against 15/15/15/16/17).
 int fp8_split_min_rows(int N, int K, int splits) {
-  if (splits < 4) return 64;
-  if (K >= 7168) return K >= 2 * N ? 16 : (N <= 4096 ? 24 : 32);
-  if (K >= 4096) return 48;
+  (void)N;
+  if (splits < 3) return 64;
+  if (K >= 12288) return 24;
+  if (K >= 7168) return 32;
   return 64;
 }
 
@@ -587,11 +590,11 @@ extern "C" int mi355q_fp8_scaled_gemm_ws(void* out, const void* x, const void* w
                        (size_t)128 * (size_t)(kslab ? K : ldw) < ((size_t)1 << 32);
   const bool stream_ok = ldx == K && (kslab || ldw == K) && ldo == N && (size_t)N * K * 2 < ((size_t)1 << 32) &&
                          (size_t)M * K * 2 < ((size_t)1 << 32);
-  // (from 41 rows on layers of 128 tiles or more: the wavefronts without rows only copy there)
+  // (from 33 rows on layers of 128 tiles or more: the wavefronts without rows only copy there)
   // (and, with a workspace, wherever the split plan asks for one: K ranges side by side fill the chip)
   const size_t split_bytes = mi355q_fp8_gemm_workspace_bytes(M, N, K);
   const bool split_ok = tile_ok && workspace && split_bytes > 0 && workspace_bytes >= split_bytes;
-  if (tile_ok && ((M > 64 && tiles >= 64) || (M > 40 && tiles >= 128) || split_ok || !stream_ok)) {
+  if (tile_ok && ((M > 64 && tiles >= 64) || (M > 32 && tiles >= 128) || split_ok || !stream_ok)) {
     F8Args a;
     a.out = out; a.x = (const uint8_t*)x; a.w = (const uint8_t*)w; a.x_scale = x_scale; a.w_scale = w_scale;
     a.bias = bias; a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldw = ldw; a.ldo = ldo;

@@ -116,9 +116,13 @@ __device__ __forceinline__ void s8x16_to_bf16(const u4& v, u4& lo, u4& hi) {
 // columns and take its K blocks round-robin, partial sums meet in LDS.  With one or two row blocks
 // there are only a few hundred wavefronts of 64 columns each; that leaves most of the chip idle
 // and every wavefront with the whole of K as one dependent chain of loads.
-template <int MODE, int ODT, int MT, bool GROUPED, bool KS = false>
+// NI (KS only): 16-column tiles per workgroup, 4, 2 or 1 -- a layer of a few thousand columns has only 64
+// to 128 groups of 64 columns, a quarter to half of the CUs; with 32 or 16 columns per workgroup every
+// CU streams a share of the weights (and reads the activations once more per workgroup).
+template <int MODE, int ODT, int MT, bool GROUPED, bool KS = false, int NI = 4>
 __global__ void __launch_bounds__(256, 1)
 kcontig_gemm_kernel(KcArgs a) {
+  static_assert(NI == 4 || (KS && (NI == 1 || NI == 2)), "narrow column groups exist for the K-split form only");
   typedef Kc<MODE> T;
   typedef typename T::acc_t acc_t;
   constexpr int BM = 16 * MT;
@@ -153,7 +157,7 @@ kcontig_gemm_kernel(KcArgs a) {
       return;
     }
   }
-  const int n0 = KS ? blockIdx.x * 64 : blockIdx.x * 256 + wave * 64;
+  const int n0 = KS ? blockIdx.x * (16 * NI) : blockIdx.x * 256 + wave * 64;
   if (n0 >= N) return;
   // Operands are addressed through buffer descriptors: a 32-bit lane offset plus a scalar K-block offset
   // per load (no 64-bit address arithmetic in the loop; the host checks that one expert's weights, the
@@ -161,11 +165,12 @@ kcontig_gemm_kernel(KcArgs a) {
   const rsrc_t wres = make_rsrc((const char*)a.w + expert * a.w_stride * T::WBYTES, (uint32_t)((size_t)N * K * T::WBYTES));
   const uint32_t kstride = a.kslab ? 4 * 2048 * T::WBYTES : 128 * T::WBYTES;   // bytes between K blocks
   const uint32_t vstride = a.kslab ? 1024 : 16;                                 // ... between the 16-byte vectors of a lane
-  uint32_t woff[4];
+  uint32_t woff[NI];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < NI; ++i) {
     if (a.kslab) {
-      woff[i] = (uint32_t)((((size_t)(n0 >> 6) * KB) * 4 + i) * (2048 * T::WBYTES) + lane * 16);
+      // (tile (n0 >> 4) + i of the layer: group of 64 columns, tile within the group)
+      woff[i] = (uint32_t)((((size_t)(n0 >> 6) * KB) * 4 + ((n0 >> 4) & 3) + i) * (2048 * T::WBYTES) + lane * 16);
     } else {
       const int n = min(n0 + 16 * i + r16, N - 1);
       woff[i] = (uint32_t)(((size_t)n * K + 32 * q) * T::WBYTES);
@@ -177,18 +182,18 @@ kcontig_gemm_kernel(KcArgs a) {
   uint32_t aoff[MT];
   int arow[MT];
 
-  acc_t acc[4][MT];
+  acc_t acc[NI][MT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < MT; ++j) acc[i][j] = (acc_t){0, 0, 0, 0};
 
   struct Blk {
-    u4 w[4][WV];
+    u4 w[NI][WV];
     u4 x[MT][AV];
     float as[MODE == KC_FP8_BLOCK ? MT : 1];
     float ws;
-    uint2 gs[GW ? 4 : 1][2];   // group-wise scales of this lane's 4 columns per row tile, per 64-wide half
+    uint2 gs[GW ? NI : 1][2];   // group-wise scales of this lane's 4 columns per row tile, per 64-wide half
   };
   const uint16_t* ws16 = (const uint16_t*)a.w_scale + expert * a.ws_stride;
   const int gper = GW ? 128 / a.wgroup : 1;        // scale groups per K block
@@ -197,7 +202,7 @@ kcontig_gemm_kernel(KcArgs a) {
   const int wsrow = (n0 >> 7) * KB;
   auto load_w = [&](Blk& b, int kb) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int v = 0; v < WV; ++v)     // streamed once: non-temporal
         b.w[i][v] = bitcast<u4>(__builtin_amdgcn_raw_buffer_load_b128(wres, (int)woff[i], (int)(kb * kstride + v * vstride), 2));
@@ -205,7 +210,7 @@ kcontig_gemm_kernel(KcArgs a) {
     if (MODE == KC_FP8_BLOCK) b.ws = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(wsres, 0, (wsrow + kb) * 4, 0));
     if (GW) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < NI; ++i) {
         const int n = min(n0 + 16 * i + 4 * q, N - 4);
 #pragma unroll
         for (int h = 0; h < 2; ++h)
@@ -233,7 +238,7 @@ kcontig_gemm_kernel(KcArgs a) {
   auto compute_blk = [&](const Blk& b, int kb) {
     if (MODE == KC_FP8_BLOCK) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
           f4 part = {0.f, 0.f, 0.f, 0.f};
@@ -253,7 +258,7 @@ kcontig_gemm_kernel(KcArgs a) {
     } else if (MODE == KC_FP8_PC) {
       // scales live outside the K sum: the products of all K blocks go into one fp32 accumulator
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
           f4 sum = bitcast<f4>(acc[i][j]);
@@ -271,7 +276,7 @@ kcontig_gemm_kernel(KcArgs a) {
         }
     } else if (MODE == KC_INT8) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < MT; ++j)
 #pragma unroll
@@ -281,7 +286,7 @@ kcontig_gemm_kernel(KcArgs a) {
     } else {
       // 16-bit activations; weights 16-bit, or int8 converted on the fly
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < NI; ++i) {
         u4 wv[4];
         if (MODE == KC_F16 || MODE == KC_BF16) {
 #pragma unroll
@@ -375,13 +380,13 @@ kcontig_gemm_kernel(KcArgs a) {
   // KS: wavefront w sums the four partial sums of column tile w (in wavefront order) and stores
   // it; two row tiles at a time go through LDS
   constexpr int RJ = MT < 2 ? MT : 2;
-  __shared__ uint32_t red[KS ? 4 : 1][KS ? 16 * RJ : 1][64];
+  __shared__ uint32_t red[KS ? 4 : 1][KS ? 4 * NI * RJ : 1][64];
   if (KS) {
 #pragma unroll
     for (int jc = 0; jc < MT; jc += RJ) {
       if (jc) __syncthreads();
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < RJ; ++j)
 #pragma unroll
@@ -390,6 +395,7 @@ kcontig_gemm_kernel(KcArgs a) {
       __syncthreads();
 #pragma unroll
       for (int j = 0; j < RJ; ++j) {
+        if (NI < 4 && wave >= NI) break;             // (fewer column tiles than wavefronts: the others only contributed)
         u4 t;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -413,6 +419,7 @@ kcontig_gemm_kernel(KcArgs a) {
 
   // ---- epilogue: lane holds row (l % 16) of each row tile and columns
   // n0 + 16 i + 4 q + {0..3}
+  if (KS && NI < 4 && wave >= NI) return;
   const bool wide = !KS && a.wide_stores;
   const rsrc_t ores = make_rsrc(a.out, (uint32_t)((size_t)(GROUPED ? a.numel : a.M) * N * 2));
 #pragma unroll
@@ -510,6 +517,22 @@ void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
     // (64-row launches only for one-byte weights x one-byte activations: the others run out of registers)
     if ((mt <= 2 || MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8) &&
         (a.N + 255) / 256 * row_blocks < 2 * device_cu_count()) {
+      // a layer of few columns: 32 or 16 columns per workgroup, so that about every CU has one (8-bit
+      // weights and activations, up to 64 rows)
+      if constexpr (MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8) {
+        const long cus = device_cu_count(), groups = (long)((a.N + 63) / 64) * row_blocks;
+        if (mt <= 4 && groups * 4 < cus * 3) {
+          const bool one = groups * 8 < cus * 3;       // even 32-column workgroups would leave a quarter of the CUs idle
+          dim3 gn(one ? (a.N + 15) / 16 : (a.N + 31) / 32, row_blocks);
+          if (mt == 1 && one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true, 1>), gn, block, 0, st, a);
+          else if (mt == 1) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true, 2>), gn, block, 0, st, a);
+          else if (mt == 2 && one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true, 1>), gn, block, 0, st, a);
+          else if (mt == 2) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true, 2>), gn, block, 0, st, a);
+          else if (one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true, 1>), gn, block, 0, st, a);
+          else hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true, 2>), gn, block, 0, st, a);
+          return;
+        }
+      }
       dim3 gks((a.N + 63) / 64, row_blocks);
       if (mt == 1) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true>), gks, block, 0, st, a);
       else if (mt == 2) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true>), gks, block, 0, st, a);

@@ -267,21 +267,26 @@ _INT8_STREAM_MAX_M = 64      # measured on MI355X (K 8192, N 28672): 40-51 us ag
 
 def _int8_stream_rows(K: int, N: int) -> int:
     """Up to how many rows the weight-streaming kernel takes a kslab layer (measured on MI355X, us,
-    streaming / MFMA tile kernel).  The tile kernel's wavefronts without rows only copy, and on layers of
-    at most 128 column tiles it cuts K into ranges that fill the chip:
-    a long K behind a narrow N (down projections) is its case from a handful of rows on --
-    28672 x 8192: M = 16 52.7 / 48.2, M = 64 82.6 / 50.7; 14336 x 4096: M = 16 25.2 / 19.7, M = 64 42.1 / 21.0;
-    square layers from about 40 rows -- 8192 x 8192: M = 32 20.2 / 20.6, M = 48 23.8 / 21.3;
-    wide layers (128 column tiles or more, no split) from 49 -- 8192 x 28672: M = 48 49.4 / 49.9, M = 64 55.3 / 50.8;
-    a short K in front of a wide N stays with the streaming kernel -- 4096 x 14336: M = 64 18.1 / 21.4."""
+    streaming / MFMA tile kernel).  The streaming kernel gives a layer of few columns 32 or 16 columns per
+    workgroup, so every CU streams a share; the tile kernel's wavefronts without rows only copy, and on
+    layers of at most 128 column tiles it cuts K into ranges that fill the chip.  The streaming kernel's
+    time grows with the rows (in steps at 17, 33), the split tile kernel's hardly does: they cross at
+    25..32 rows behind a very long K -- 28672 x 8192: M = 24 45.4 / 50.5, M = 32 51.5 / 50.7, M = 64 67.1 / 49.7;
+    at 33..40 where K >= 2 N -- 16384 x 7168: M = 32 26.2 / 29.6, M = 40 31.0 / 30.3; 14336 x 4096: M = 32 19.5 / 20.1,
+    M = 40 24.4 / 20.2; at 41..48 for other K >= 7168 -- 7168 x 4096: M = 40 14.9 / 15.9, M = 48 16.2 / 16.1;
+    8192 x 8192: M = 48 19.5 / 21.3, M = 64 23.0 / 22.0; on wide layers (128 column tiles or more, no split)
+    -- 8192 x 28672: M = 40 49.8 / 52.3, M = 48 51.9 / 49.1; a short K stays with the streaming kernel --
+    4096 x 4096: M = 64 13.4 / 15.6."""
     top = _INT8_STREAM_MAX_M
     if N % 128 != 0:
         return top
     if N >= 128 * 128:
-        return top * 3 // 4
-    if K >= 2 * N:
-        return top // 8
-    if K >= N:
+        return top * 5 // 8
+    if K >= 24576:
+        return top * 3 // 8
+    if K >= 2 * N and K >= 7168:
+        return top // 2
+    if K >= 7168:
         return top * 5 // 8
     return top
 
@@ -1252,14 +1257,14 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
         raise RuntimeError("linear_quant: operands must be float8_e4m3fn")
     M, N, K = lhs.numel() // lhs.shape[-1], rhs.shape[0], lhs.shape[-1]
     tiles = -(-M // 256) * (N // 128)               # 256 x 128 output tiles, one workgroup each
-    # (from 41 rows on a layer of 128 tiles or more: the tile kernel's wavefronts without rows only copy,
-    # K 8192 x N 28672 at M = 48 / 64: 59.6 / 68.4 -> 52.9 / 55.1 us; 112 tiles: the streamer stays ahead)
+    # (from 33 rows on a layer of 128 tiles or more: the tile kernel's wavefronts without rows only copy,
+    # K 8192 x N 28672 at M = 40 / 48 / 64: 59.0 / 62.3 / 68.7 -> 55.5 / 56.3 / 53.6 us; 112 tiles: the streamer stays ahead)
     # (and, whatever the tile count, where the library plans K ranges side by side that fill the chip:
-    # from 65 rows, and from 17 / 25 / 33 / 49 rows on where K is long, see fp8_split_min_rows)
+    # from 65 rows, and from 25 / 33 rows on where K is long, see fp8_split_min_rows)
     need = _lib.load().mi355q_fp8_gemm_workspace_bytes(M, N, K) \
         if M > _FP8_TILE_MIN_M // 4 and N % 128 == 0 and K % 128 == 0 else 0
     if (need or (M > _FP8_TILE_MIN_M and tiles >= _FP8_TILE_MIN_TILES)
-            or (M > _FP8_TILE_MIN_M * 5 // 8 and tiles >= 2 * _FP8_TILE_MIN_TILES)) \
+            or (M > _FP8_TILE_MIN_M // 2 and tiles >= 2 * _FP8_TILE_MIN_TILES)) \
             and N % 128 == 0 and K % 128 == 0 \
             and out.dtype in (torch.float16, torch.bfloat16) \
             and rhs.dim() == 2 and rhs.is_contiguous() and out.is_contiguous():
