@@ -517,19 +517,22 @@ void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
     // (64-row launches only for one-byte weights x one-byte activations: the others run out of registers)
     if ((mt <= 2 || MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8) &&
         (a.N + 255) / 256 * row_blocks < 2 * device_cu_count()) {
-      // a layer of few columns: 32 or 16 columns per workgroup, so that about every CU has one (8-bit
-      // weights and activations, up to 64 rows)
-      if constexpr (MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8) {
+      // a layer of few columns: 32 or 16 columns per workgroup, so that about every CU has one (up to
+      // 64 rows with 8-bit weights and activations, up to 32 rows otherwise)
+      constexpr bool BYTES = MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8;
+      {
         const long cus = device_cu_count(), groups = (long)((a.N + 63) / 64) * row_blocks;
-        if (mt <= 4 && groups * 4 < cus * 3) {
+        if (mt <= (BYTES ? 4 : 2) && groups * 4 < cus * 3) {
           const bool one = groups * 8 < cus * 3;       // even 32-column workgroups would leave a quarter of the CUs idle
           dim3 gn(one ? (a.N + 15) / 16 : (a.N + 31) / 32, row_blocks);
           if (mt == 1 && one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true, 1>), gn, block, 0, st, a);
           else if (mt == 1) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 1, false, true, 2>), gn, block, 0, st, a);
           else if (mt == 2 && one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true, 1>), gn, block, 0, st, a);
           else if (mt == 2) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 2, false, true, 2>), gn, block, 0, st, a);
-          else if (one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true, 1>), gn, block, 0, st, a);
-          else hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true, 2>), gn, block, 0, st, a);
+          else if constexpr (BYTES) {
+            if (one) hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true, 1>), gn, block, 0, st, a);
+            else hipLaunchKernelGGL((kcontig_gemm_kernel<MODE, ODT, 4, false, true, 2>), gn, block, 0, st, a);
+          }
           return;
         }
       }
