@@ -511,6 +511,17 @@ kslab_repack_kernel(const u4* src, u4* dst, long chunks, int N, int K, int wb) {
 
 template <int MODE, int ODT, bool GROUPED>
 void launch_mt(const KcArgs& a, int mt, int row_blocks, hipStream_t st) {
+  if constexpr (!GROUPED && !(MODE == KC_FP8_BLOCK || MODE == KC_FP8_PC || MODE == KC_INT8)) {
+    // 16-bit activations have no 64-row form with K split inside the workgroup (registers), and 64-row
+    // blocks of 256 columns are few on all but the widest layers at a few hundred rows (N 4096 at
+    // M = 64: 16 workgroups, 79 us): 32-row blocks with the split instead, while they are too few
+    // (K 4096, W8A16, us: N 4096 at M = 64 / 128 / 512: 79 / 78 / 80 -> 14 / 16 / 53; N 14336 at 64 / 128: 81 / 80 -> 31 / 57;
+    // at 512 rows, 448 workgroups of 64 x 256, the 64-row blocks are ahead again: 156 against 169)
+    if (mt == 4 && (long)((a.N + 255) / 256) * row_blocks * 2 < 3L * device_cu_count()) {
+      mt = 2;
+      row_blocks = (a.M + 31) / 32;
+    }
+  }
   dim3 grid((a.N + 255) / 256, row_blocks), block(256);
   if constexpr (!GROUPED) {
     // too few workgroups to fill the chip: split K inside the workgroup
