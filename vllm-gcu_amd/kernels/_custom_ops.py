@@ -348,14 +348,20 @@ def _scaled_int8_mm(out, x, weight, x_scale, w_scale, bias, acc_out=None):
             bias_f32 = 1
         bias = bias.contiguous()
     stream_rows = _int8_stream_rows(K, N)
-    if ldw == 0 and M <= stream_rows and acc_out is None and ws_col and (xs is None or xs_row or M == 1) \
+    # (row-major [N, K] weights: the tile kernel with its K ranges is level with the streaming kernel on
+    # large layers -- 8192 x 28672 at M = 16: 54 against 58 us -- and behind it on small ones up to 32
+    # rows: 4096 x 4096 at M = 16: 13.8 against 7.7 us)
+    small_row_major = ldw == K and M <= stream_rows // 2 and K * N <= (1 << 25) and N % 4 == 0 and K % 128 == 0
+    if (ldw == 0 and M <= stream_rows or small_row_major) and acc_out is None and ws_col \
+            and (xs is None or xs_row or M == 1) \
             and not bias_f32 and out.dtype in (torch.float16, torch.bfloat16) and x2.is_contiguous() \
             and out2.stride(0) == N:
         # decode-sized M on kslab weights: the weight-streaming kernel (same int32 sums, same
         # epilogue order: bit-identical results) reads them about twice as fast
         with torch.cuda.device(x.device):
             _lib.call("mi355q_kcontig_gemm", out2.data_ptr(), x2.data_ptr(), w.data_ptr(), rt.ptr(xs), ws.data_ptr(),
-                      rt.ptr(bias), _lib.Q_INT8, 0, M, K, N, _lib.F16, rt.dtype_code(out.dtype), 1, rt.stream_ptr())
+                      rt.ptr(bias), _lib.Q_INT8, 0, M, K, N, _lib.F16, rt.dtype_code(out.dtype),
+                      1 if ldw == 0 else 0, rt.stream_ptr())
         return
     with torch.cuda.device(x.device):
         # (few output tiles behind a long K: K ranges side by side through the stream's workspace, bit-identical)
