@@ -360,6 +360,10 @@ def main():
         import torch as _torch
         out["moe_w4a16_bf16"] = moe_bench(ops, dev, stream, "w4a16", tokens=512, act_dtype=_torch.bfloat16)
         torch.cuda.empty_cache()
+        # the DeepSeek-V3-style layer at a prefill token count (128 rows per expert: blocks of 256 slots on the
+        # MFMA tile kernel with gathered rows)
+        out["moe_fp8_block_prefill"] = moe_bench(ops, dev, stream, "fp8", iters=6, tokens=4096)
+        torch.cuda.empty_cache()
         out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")
         torch.cuda.empty_cache()
         out["norm_quant"] = glue_bench(ops, dev, stream)
@@ -573,7 +577,7 @@ def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False, act_dty
         bytes_ = E * (H * 2 * I + I * H) // 2 + E * (H // 128 * 2 * I + I // 128 * H) * 4 + 2 * M * H * 2
         name = "fused MoE w4a8-fp8, Mixtral-8x7B layer shape: 512 tok, hidden 4096, 8 experts, inter 14336, top-2"
     else:
-        M, H, E, I, T = 256, 7168, 256, 2048, 8
+        M, H, E, I, T = tokens or 256, 7168, 256, 2048, 8
 
         def block_fp8(n, k):
             """[E, n, k] weights ~ N(0, 0.02) quantised to fp8-e4m3 with one fp32 scale per 128 x 128 block
@@ -603,7 +607,7 @@ def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False, act_dty
         flops = 2.0 * M * T * (H * 2 * I + I * H)
         bytes_ = hit * (2 * I * H + H * I + 4 * (2 * I // 128 * H // 128 + H // 128 * I // 128)) \
             + M * H + M * H // 128 * 4 + M * H * 2
-        name = (f"fused MoE fp8 block-scaled, DeepSeek-V3-style layer: 256 tok, hidden 7168, 256 experts ({hit} hit), inter 2048, "
+        name = (f"fused MoE fp8 block-scaled, DeepSeek-V3-style layer: {M} tok, hidden 7168, 256 experts ({hit} hit), inter 2048, "
                 "top-8; weights ~ N(0, 0.02) quantised per 128 x 128 block")
     time_graph([step], 5, 3, stream)
     t = time_graph([step], iters, 0, stream) / iters

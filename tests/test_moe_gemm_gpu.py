@@ -192,6 +192,59 @@ def test_grouped_fp8_block(fmoe, ops, block):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("kslab", [False, True])
+@pytest.mark.parametrize("M,E,T,K,N", [(300, 6, 3, 512, 384), (40, 4, 2, 384, 128), (700, 3, 1, 1024, 256)])
+def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, kslab):
+    """Blocks of 256 slot ids (prefill token counts) run the MFMA tile kernel with its rows gathered through
+    the ids.  Both GEMM forms (rows t // topk without routing weight; one row per slot with it), row-major
+    and kslab weights, an expert that no token chose, one that expert_map sends elsewhere (its rows come
+    back as zeros); against the oracle and against the weight-streaming kernel on blocks of 64."""
+    print(f"case grouped fp8 tiles M={M} E={E} T={T} K={K} N={N} kslab={kslab}", flush=True)
+    rng = np.random.default_rng(M + K)
+    wq = np.stack([of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 2, -448, 448).astype(np.float32)) for _ in range(E)])
+    ws = rng.uniform(0.005, 0.02, size=(E, N // 128, K // 128)).astype(np.float32)
+    wd = dev(wq).view(torch.float8_e4m3fn)
+    if kslab:
+        wd = rearrange.to_kslab(wd)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    logits[:, E - 1] -= 50.0                                   # nobody routes to the last expert
+    tw, ids, _ = om.topk_softmax(logits, T, True)
+    flat = ids.reshape(-1)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16)
+    xq, xs = ops.per_token_group_quant_fp8(x.cuda(), 128)
+    xq_c, xs_c = xq.view(torch.uint8).cpu().numpy(), xs.cpu().numpy()
+    want = np.zeros((M * T, N), dtype=np.float32)
+    for t in range(M * T):
+        want[t] = of8.block_fp8_gemm(xq_c[t // T:t // T + 1], xs_c[t // T:t // T + 1], wq[flat[t]], ws[flat[t]])[0]
+    C = torch.full((M, T, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    run_grouped(fmoe, xq, wd, C, xs, dev(ws), None, dev(tw), dev(ids), E, 256, False, T,
+                use_fp8_w8a8=True, block_shape=[128, 128])
+    got = C.view(-1, N).float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+    C64 = torch.empty_like(C)
+    run_grouped(fmoe, xq, wd, C64, xs, dev(ws), None, dev(tw), dev(ids), E, 64, False, T,
+                use_fp8_w8a8=True, block_shape=[128, 128])
+    assert (C.float() - C64.float()).abs().max().item() <= 2 ** -6 * max(1.0, float(np.abs(want).max()))
+    # second form: one activation row per slot, routing weights applied; expert 0 mapped away
+    x2 = torch.from_numpy(rng.standard_normal((M * T, K)).astype(np.float32)).to(torch.bfloat16)
+    x2q, x2s = ops.per_token_group_quant_fp8(x2.cuda(), 128)
+    emap = torch.arange(E, dtype=torch.int32)
+    emap[0] = -1
+    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), 256, E, emap.cuda())
+    C2 = torch.full((M, T, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    fmoe.invoke_fused_moe_kernel(x2q, wd, C2, x2s, dev(ws), None, dev(tw), dev(ids), s_, e_, n_, True, 1,
+                                 {"BLOCK_SIZE_M": 256}, use_fp8_w8a8=True, use_int8_w8a8=False, use_int8_w8a16=False,
+                                 use_int4_w4a16=False, block_shape=[128, 128])
+    torch.cuda.synchronize()
+    x2q_c, x2s_c = x2q.view(torch.uint8).cpu().numpy(), x2s.cpu().numpy()
+    want2 = np.zeros((M * T, N), dtype=np.float32)
+    twf = tw.reshape(-1)
+    for t in range(M * T):
+        if flat[t] != 0:
+            want2[t] = of8.block_fp8_gemm(x2q_c[t:t + 1], x2s_c[t:t + 1], wq[flat[t]], ws[flat[t]])[0] * twf[t]
+    np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("N", [260, 264, 200])
 def test_grouped_int8_and_fp16_and_w8a16(fmoe, ops, N):
     # widths that end inside a 64-column group: 260 takes the 8-byte output stores (not a multiple of 8),
@@ -436,20 +489,25 @@ def test_fused_experts_w4a16_sequence(ops, rearrange, M, E, T, H, I):
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 
 
-def test_fused_experts_fp8_block_sequence(ops, fmoe):
-    print("case fused fp8", flush=True)
+@pytest.mark.parametrize("M,E,T,H,I", [(48, 16, 4, 512, 256), (400, 8, 2, 512, 256)])
+def test_fused_experts_fp8_block_sequence(ops, fmoe, M, E, T, H, I):
+    """The whole fused-experts sequence on fp8 block-scaled experts; the second case has 100 rows per expert
+    on average, where the configuration takes align blocks of 256 slots and both GEMMs run the MFMA tile
+    kernel with gathered rows."""
+    print(f"case fused fp8 M={M} E={E}", flush=True)
+    assert (fmoe.get_default_config(M, E, 2 * I, H, T, None, False, [128, 128])["BLOCK_SIZE_M"] == 256) == (M == 400)
     rng = np.random.default_rng(3)
-    M, E, T, H, I = 48, 16, 4, 512, 256
     w13 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, 2 * I, H)) * 0.5, -448, 448).astype(np.float32))
     w2 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, H, I)) * 0.5, -448, 448).astype(np.float32))
     s13 = rng.uniform(0.02, 0.1, size=(E, 2 * I // 128, H // 128)).astype(np.float32)
     s2 = rng.uniform(0.02, 0.1, size=(E, H // 128, I // 128)).astype(np.float32)
     x = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).to(torch.bfloat16)
     logits = rng.standard_normal((M, E)).astype(np.float32)
-    tw, ids = fmoe.grouped_topk(x.cuda(), dev(logits), T, True, 4, 2, "sigmoid", None)
+    groups = 4 if E >= 16 else 2
+    tw, ids = fmoe.grouped_topk(x.cuda(), dev(logits), T, True, groups, 2, "sigmoid", None)
     out = build_moe("fp8")(x.cuda(), dev(w13).view(torch.float8_e4m3fn), dev(w2).view(torch.float8_e4m3fn), tw, ids,
                            w1_scale=dev(s13), w2_scale=dev(s2))
-    two, ido = om.grouped_topk(logits, T, True, 4, 2, "sigmoid", None)
+    two, ido = om.grouped_topk(logits, T, True, groups, 2, "sigmoid", None)
     assert np.array_equal(ids.cpu().numpy(), ido)
 
     def deq(codes, sc):

@@ -46,6 +46,13 @@ struct F8Args {
   int n_panels_swizzle;
   int ksplits;              // > 1: every output tile is worked on by `ksplits` workgroups, each a range of K blocks,
   float* partial;           //      which leave their fp32 sums in partial[split][M][N]; the epilogue is a second launch
+  // grouped (MoE) launches: a row tile is one align block of 256 slot ids of one expert
+  const int32_t* sorted_ids;   // [blocks * 256] flat (token, slot) ids, pad = numel
+  const int32_t* expert_ids;   // [blocks]
+  const int32_t* npp;          // device scalar: padded id count
+  const float* topk_weights;   // [numel] or null
+  int numel, topk, E, max_blocks;
+  long w_stride, ws_stride;    // per expert: bytes of weights, floats of weight scales
 };
 
 __device__ __forceinline__ void dma16(const void* gptr, void* lds_wave_base) {
@@ -60,9 +67,15 @@ __device__ __forceinline__ void dma4(const void* gptr, void* lds_wave_base) {
 
 typedef int i8v __attribute__((ext_vector_type(8)));
 
-template <int DT, bool PC>
+// GROUPED: the fused-MoE grouped GEMM at prefill token counts.  Row tile b is align block b (256 slot
+// ids of expert expert_ids[b]): x rows and their scales are gathered through the ids (row id / topk),
+// weights and weight scales are the expert's, output row id gets the result (times its routing weight).
+// Blocks past num_tokens_post_pad do not exist (the tile count is read on the device); a block of an
+// expert outside [0, E) writes zeros.  No K ranges, no bias.
+template <int DT, bool PC, bool GROUPED = false>
 __global__ void __launch_bounds__(F8_THREADS, 1)
 fp8_block_gemm_kernel(F8Args a) {
+  static_assert(!GROUPED || !PC, "the grouped form exists for block scales");
   constexpr int WN = 2, NI = 4, NJ = 4;                 // 4 x 2 wavefronts of 64 x 64
   constexpr int X_BYTES = FTM * FTKB, W_BYTES = FTN * FTKB, XS_BYTES = FTM * 4;
   constexpr int WS_BYTES = 256;                         // the tile's weight scale of a K block, 64 copies
@@ -74,13 +87,22 @@ fp8_block_gemm_kernel(F8Args a) {
   const int wm = wave / WN, wn = wave % WN;
   const int M = a.M, N = a.N, K = a.K, KB = K >> 7;
 
-  const int mtiles = (M + FTM - 1) / FTM;
+  int mtiles = (M + FTM - 1) / FTM;
+  if (GROUPED) {
+    const int blocks = (*a.npp + FTM - 1) / FTM;
+    mtiles = __builtin_amdgcn_readfirstlane(blocks < a.max_blocks ? blocks : a.max_blocks);
+  }
   const int ntiles_n = N / FTN;
-  const int ksplits = a.ksplits > 1 ? a.ksplits : 1;
+  const int ksplits = (!GROUPED && a.ksplits > 1) ? a.ksplits : 1;
   const int total_tiles = mtiles * ntiles_n * ksplits;   // (split K: tile ids count (output tile, K range) pairs)
+  if (GROUPED && (int)blockIdx.x >= total_tiles) return;  // (the grid is sized for the largest block count the ids can fill)
   auto tile_origin = [&](int tile, int& m0, int& n0) {
     int tm, tn;
-    if (ksplits > 1) {
+    if (GROUPED) {
+      // block-major: neighbouring workgroups share a block's activation rows
+      tm = tile / ntiles_n;
+      tn = tile - tm * ntiles_n;
+    } else if (ksplits > 1) {
       const int t = tile / ksplits;
       tm = t % mtiles;
       tn = t / mtiles;
@@ -119,10 +141,25 @@ fp8_block_gemm_kernel(F8Args a) {
   auto set_copy_tile = [&](int tile) {
     int m0, n0;
     tile_origin(tile, m0, n0);
+    long ebytes = 0;
+    int escales = 0;
+    if (GROUPED) {
+      const int* ids = a.sorted_ids + m0;
 #pragma unroll
-    for (int p = 0; p < XCOPIES; ++p) {
-      const int r = (wave + 8 * p) * 8 + crow;
-      xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * cchunk);
+      for (int p = 0; p < XCOPIES; ++p) {
+        const int id = ids[(wave + 8 * p) * 8 + crow];
+        xo[p] = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)a.ldx + (uint32_t)(16 * cchunk);   // pads read a valid row
+      }
+      int e = a.expert_ids[m0 / FTM];
+      e = __builtin_amdgcn_readfirstlane((e < 0 || e >= a.E) ? 0 : e);     // (a foreign expert's block is computed and zeroed)
+      ebytes = (long)e * a.w_stride;
+      escales = e * (int)a.ws_stride;
+    } else {
+#pragma unroll
+      for (int p = 0; p < XCOPIES; ++p) {
+        const int r = (wave + 8 * p) * 8 + crow;
+        xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * cchunk);
+      }
     }
 #pragma unroll
     for (int p = 0; p < WCOPIES; ++p) {
@@ -139,10 +176,15 @@ fp8_block_gemm_kernel(F8Args a) {
     // activation scales: wavefronts 0..3 copy 64 rows each (index in floats)
     // (split K: the tile's range starts kb0 K blocks into every row; 64 kslab rows interleave their K blocks)
     const int kb0 = ksplits > 1 ? (tile % ksplits) * (KB / ksplits) : 0;
-    xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB + (uint32_t)kb0;
-    wsbase = (n0 >> 7) * KB + kb0;                 // wavefront 4 copies the tile's weight scale
-    xtile = a.x + (long)m0 * a.ldx + (long)kb0 * FTKB;
-    wtile = a.w_kslab ? a.w + (long)kb0 * FTKB * 64 : a.w + (long)n0 * a.ldw + (long)kb0 * FTKB;
+    if (GROUPED) {
+      const int id = a.sorted_ids[m0 + 64 * (wave & 3) + lane];
+      xso = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)KB;
+    } else {
+      xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB + (uint32_t)kb0;
+    }
+    wsbase = escales + (n0 >> 7) * KB + kb0;       // wavefront 4 copies the tile's weight scale
+    xtile = GROUPED ? a.x : a.x + (long)m0 * a.ldx + (long)kb0 * FTKB;
+    wtile = a.w + ebytes + (a.w_kslab ? (long)kb0 * FTKB * 64 : (long)n0 * a.ldw + (long)kb0 * FTKB);
   };
   constexpr int NSLOT = XCOPIES + WCOPIES + 1;
   auto copy_slot = [&](int s, int stage, int kt) {
@@ -314,7 +356,7 @@ fp8_block_gemm_kernel(F8Args a) {
   // One row tile in all (M <= 256) and none of its rows in this wavefront's share: the wavefront only
   // copies.  It keeps the workgroup's barriers and its own copy slots, and leaves the matrix pipe and
   // the LDS read port of its SIMD to the wavefront that has rows (65 .. 128 rows: half the wavefronts).
-  if (mtiles == 1 && wm * (16 * NJ) >= M) {
+  if (!GROUPED && mtiles == 1 && wm * (16 * NJ) >= M) {
     for (; tile < total_tiles; tile += gdim) {
       for (int T = 0; T < nt; ++T) {
         const int kt = ahead_kt(T, 3);
@@ -374,6 +416,29 @@ fp8_block_gemm_kernel(F8Args a) {
         if (m >= M) continue;
 #pragma unroll
         for (int i = 0; i < NI; ++i) *(f4*)(part + (long)m * N + n0 + wn * (16 * NI) + i * 16 + 4 * kq) = acc[i][j];
+      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0), as below
+      continue;
+    }
+    if (GROUPED) {
+      const int e = a.expert_ids[m0 / FTM];
+      const bool foreign = e < 0 || e >= a.E;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int id = a.sorted_ids[m0 + wm * (16 * NJ) + j * 16 + l16];
+        if (id >= a.numel || id < 0) continue;
+        const float rw = foreign ? 0.0f : (a.topk_weights ? a.topk_weights[id] : 1.0f);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+          float v[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] = foreign ? 0.0f : acc[i][j][c] * rw;
+          u2 o;
+          o.x = (uint32_t)Elem<DT>::from_f32(v[0]) | ((uint32_t)Elem<DT>::from_f32(v[1]) << 16);
+          o.y = (uint32_t)Elem<DT>::from_f32(v[2]) | ((uint32_t)Elem<DT>::from_f32(v[3]) << 16);
+          *(u2*)((uint16_t*)a.out + (long)id * a.ldo + n) = o;
+        }
       }
       __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0), as below
       continue;
@@ -516,7 +581,45 @@ int launch_f8(const F8Args& a, hipStream_t st) {
   return 0;
 }
 
+template <int DT>
+int launch_f8_grouped(const F8Args& a, hipStream_t st) {
+  const size_t shmem = 3 * (size_t)(FTM * FTKB + FTN * FTKB + FTM * 4 + 256);
+  static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT, false, true>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  MQ_REQUIRE(attr == hipSuccess, "moe_gemm(fp8 tiles): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
+  long grid = (long)a.max_blocks * (a.N / FTN);
+  const long cus = device_cu_count();
+  if (grid > cus) grid = cus;
+  hipLaunchKernelGGL((fp8_block_gemm_kernel<DT, false, true>), dim3((unsigned)grid), dim3(F8_THREADS), shmem, st, a);
+  MQ_LAUNCH_CHECK("moe_gemm(fp8 tiles)");
+  return 0;
+}
+
 }  // namespace
+
+// The fused-MoE grouped GEMM with 128 x 128 block scales on align blocks of 256 slot ids: the MFMA tile
+// kernel above with its rows gathered through the ids (prefill token counts; smaller blocks take the
+// weight-streaming kernel).  Arguments as mi355q_moe_gemm's; checked by the caller.
+int fp8_block_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, const float* w_scale,
+                             const float* topk_weights, const int32_t* sorted_ids, const int32_t* expert_ids,
+                             const int32_t* npp, int numel, int topk, int max_blocks, int E, int K, int N,
+                             int out_dtype, int w_kslab, hipStream_t st) {
+  MQ_REQUIRE(N % 128 == 0 && K % 128 == 0, "moe_gemm(fp8 tiles): N=%d and K=%d must be multiples of 128", N, K);
+  MQ_REQUIRE(out_dtype == MI355Q_F16 || out_dtype == MI355Q_BF16, "moe_gemm(fp8 tiles): output dtype %d", out_dtype);
+  MQ_REQUIRE(((size_t)numel / topk + 1) * K < ((size_t)1 << 32) && (size_t)N * K < ((size_t)1 << 32),
+             "moe_gemm(fp8 tiles): activations and one expert's weights must each stay below 4 GiB");
+  F8Args g = {};
+  g.out = out; g.x = (const uint8_t*)a; g.w = (const uint8_t*)w; g.x_scale = a_scale; g.w_scale = w_scale;
+  g.M = numel; g.N = N; g.K = K; g.ldx = K; g.ldw = K; g.ldo = N;
+  g.w_kslab = w_kslab;
+  g.ksplits = 1;
+  g.sorted_ids = sorted_ids; g.expert_ids = expert_ids; g.npp = npp; g.topk_weights = topk_weights;
+  g.numel = numel; g.topk = topk; g.E = E; g.max_blocks = max_blocks;
+  g.w_stride = (long)N * K;
+  g.ws_stride = (long)(N / 128) * (K / 128);
+  return out_dtype == MI355Q_F16 ? launch_f8_grouped<MI355Q_F16>(g, st) : launch_f8_grouped<MI355Q_BF16>(g, st);
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;

@@ -597,6 +597,10 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
                          int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                          int group_size, int dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
 size_t w4a16_grouped_workspace_bytes(int numel, int block_size, int max_blocks, int E, int K, int N);
+int fp8_block_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, const float* w_scale,
+                             const float* topk_weights, const int32_t* sorted_ids, const int32_t* expert_ids,
+                             const int32_t* npp, int numel, int topk, int max_blocks, int E, int K, int N,
+                             int out_dtype, int w_kslab, hipStream_t st);
 
 // fp8 x fp8 with scales outside the K sum (per token or one value; per output channel or one value), M <= 128:
 // the weight-streaming kernel.  Arguments are checked by the caller (mi355q_fp8_scaled_gemm).
@@ -680,6 +684,10 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
   if (quant_mode == 1) {
     MQ_REQUIRE(a_scale && w_scale, "moe_gemm(fp8): scales missing");
     MQ_REQUIRE(group_size == 128, "moe_gemm(fp8): only 128x128 block scales are supported, got %d", group_size);
+    // blocks of 256 slots (prefill token counts): the MFMA tile kernel with gathered rows
+    if (block_size == 256 && N % 128 == 0)
+      return fp8_block_grouped_launch(out, a, w, a_scale, (const float*)w_scale, topk_weights, sorted_token_ids, expert_ids,
+                                      num_tokens_post_pad, numel, topk, max_blocks, E, K, N, out_dtype, w_layout, st);
     mode = KC_FP8_BLOCK;
     g.ws_stride = (long)((N + 127) / 128) * (K / 128);
   } else if (quant_mode == 2) {

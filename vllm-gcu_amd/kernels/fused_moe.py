@@ -12,6 +12,14 @@ import torch
 from . import _custom_ops as ops
 
 
+# Rows per expert from which the fp8 block-scaled grouped GEMM takes 256-slot blocks (measured on MI355X, us,
+# blocks of 64 on the weight-streaming kernel / blocks of 256 on the tile kernel; the tile kernel's time hardly
+# depends on how full its blocks are).  Mixtral shape, K 4096 x N 28672, 8 experts, at 32 / 64 / 128 / 512 rows
+# per expert: 213 / 365 / 569 / 1865 against 283 / 289 / 296 / 769; DeepSeek-V3 shape, K 7168 x N 4096, 256 experts,
+# at 32 / 64 / 128 / 256: 1557 / 2491 / 4320 / 7568 against 2142 / 2202 / 2348 / 3493.
+_FP8_TILE_MIN_ROWS_PER_EXPERT = 48
+
+
 def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optional[str], is_marlin: bool,
                        block_shape: Optional[List[int]] = None) -> Dict[str, int]:
     """Only BLOCK_SIZE_M is consumed (as the align/GEMM block size).  The
@@ -21,6 +29,10 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
     tiles with two workgroups per CU were measured faster than 128-row tiles up
     to 4096 tokens on the Mixtral-8x7B layer, and they pad less)."""
     per_expert = (M * topk) / max(E, 1)
+    if block_shape is not None and list(block_shape) == [128, 128] and per_expert > _FP8_TILE_MIN_ROWS_PER_EXPERT:
+        # fp8 block-scaled experts at prefill token counts: blocks of 256 slots run the MFMA tile kernel
+        # with gathered rows instead of the weight-streaming kernel
+        return {"BLOCK_SIZE_M": 256, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
     if per_expert <= 16:
         bm = 16
     elif per_expert <= 28:      # measured on the Mixtral-8x7B W4A16 layer: at 32 rows per expert on average
