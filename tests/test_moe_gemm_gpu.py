@@ -245,6 +245,56 @@ def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T,
     np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("kslab", [False, True])
+@pytest.mark.parametrize("M,E,T,K,N", [(300, 6, 3, 512, 384), (40, 4, 2, 384, 192), (700, 3, 1, 1024, 256)])
+def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, kslab):
+    """int8 experts (per-token x per-channel scales) on blocks of 256 slot ids: the int8 MFMA tile kernel
+    with its rows gathered through the ids.  Both GEMM forms, row-major and kslab weights, an idle expert
+    and one that expert_map sends elsewhere; the int32 sums are exact, so the outputs equal those of the
+    weight-streaming kernel on blocks of 64 bit for bit."""
+    print(f"case grouped int8 tiles M={M} E={E} T={T} K={K} N={N} kslab={kslab}", flush=True)
+    rng = np.random.default_rng(M + K + 1)
+    wq = rng.integers(-127, 128, size=(E, N, K), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.02, size=(E, N, 1)).astype(np.float32)
+    wd = dev(wq)
+    if kslab:
+        wd = rearrange.to_kslab(wd)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    logits[:, E - 1] -= 50.0
+    tw, ids, _ = om.topk_softmax(logits, T, True)
+    flat = ids.reshape(-1)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    xq, xs = o8.dynamic_scaled_int8_quant(x)
+    want = np.zeros((M * T, N), dtype=np.float32)
+    for t in range(M * T):
+        acc = o8.int8_gemm_i32(xq[t // T:t // T + 1], np.ascontiguousarray(wq[flat[t]].T))
+        want[t] = o8.scaled_mm_epilogue(acc, xs[t // T], ws[flat[t], :, 0])[0]
+    C = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
+    run_grouped(fmoe, dev(xq), wd, C, dev(xs), dev(ws), None, dev(tw), dev(ids), E, 256, False, T, use_int8_w8a8=True)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    C64 = torch.empty_like(C)
+    run_grouped(fmoe, dev(xq), wd, C64, dev(xs), dev(ws), None, dev(tw), dev(ids), E, 64, False, T, use_int8_w8a8=True)
+    assert torch.equal(C, C64)
+    # second form: one activation row per slot, routing weights applied; expert 0 mapped away
+    x2 = rng.standard_normal((M * T, K)).astype(np.float16)
+    x2q, x2s = o8.dynamic_scaled_int8_quant(x2)
+    emap = torch.arange(E, dtype=torch.int32)
+    emap[0] = -1
+    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), 256, E, emap.cuda())
+    C2 = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
+    fmoe.invoke_fused_moe_kernel(dev(x2q), wd, C2, dev(x2s), dev(ws), None, dev(tw), dev(ids), s_, e_, n_, True, 1,
+                                 {"BLOCK_SIZE_M": 256}, use_fp8_w8a8=False, use_int8_w8a8=True, use_int8_w8a16=False,
+                                 use_int4_w4a16=False)
+    torch.cuda.synchronize()
+    want2 = np.zeros((M * T, N), dtype=np.float32)
+    twf = tw.reshape(-1)
+    for t in range(M * T):
+        if flat[t] != 0:
+            acc = o8.int8_gemm_i32(x2q[t:t + 1], np.ascontiguousarray(wq[flat[t]].T))
+            want2[t] = o8.scaled_mm_epilogue(acc, x2s[t], ws[flat[t], :, 0])[0] * twf[t]
+    np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("N", [260, 264, 200])
 def test_grouped_int8_and_fp16_and_w8a16(fmoe, ops, N):
     # widths that end inside a 64-column group: 260 takes the 8-byte output stores (not a multiple of 8),

@@ -42,6 +42,13 @@ struct I8Args {
   int wide_stores;          // N, ldo and the output address allow 16-byte stores of 8 adjacent 16-bit outputs
   int ksplits;              // > 1: every output tile is worked on by `ksplits` workgroups, each a K range of its own,
   int32_t* partial;         //      which leave their int32 sums in partial[split][M][N]; the epilogue is a second launch
+  // grouped (MoE) launches: a row tile is one align block of 256 slot ids of one expert
+  const int32_t* sorted_ids;   // [blocks * 256] flat (token, slot) ids, pad = numel
+  const int32_t* expert_ids;   // [blocks]
+  const int32_t* npp;          // device scalar: padded id count
+  const float* topk_weights;   // [numel] or null
+  int numel, topk, E, max_blocks;
+  long w_stride, ws_stride;    // per expert: bytes of weights, floats of weight scales
 };
 
 template <int DT>
@@ -72,7 +79,12 @@ __device__ __forceinline__ void dma16(const void* gptr, void* lds_wave_base) {
 }
 
 // WM x WN wavefronts, each NJ x NI MFMA tiles of 16 x 16 (rows of x by rows of w)
-template <int DT, int WM, int WN, int NI, int NJ>
+// GROUPED: the fused-MoE grouped GEMM at prefill token counts.  Row tile b is align block b (256 slot
+// ids of expert expert_ids[b]): x rows are gathered through the ids (row id / topk), weights and
+// weight scales are the expert's, output row id gets the result times x_scale of its row, the
+// expert's w_scale and its routing weight.  Blocks past num_tokens_post_pad do not exist (the tile
+// count is read on the device); a block of an expert outside [0, E) writes zeros.  No K ranges, no bias.
+template <int DT, int WM, int WN, int NI, int NJ, bool GROUPED = false>
 __global__ void __launch_bounds__(GEMM_THREADS, 1)
 w8a8_int8_gemm_kernel(I8Args a) {
   static_assert(WM * WN == 8 && WM * NJ * 16 == TM, "eight wavefronts cover 256 rows of x");
@@ -93,13 +105,22 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // Tile coordinates: with the swizzle, the tiles whose id is congruent mod 8
   // (they run on one XCD, the grid being a multiple of 8) sweep all row tiles
   // of the same weight panels.
-  const int mtiles = (M + TM - 1) / TM;
+  int mtiles = (M + TM - 1) / TM;
+  if (GROUPED) {
+    const int blocks = (*a.npp + TM - 1) / TM;
+    mtiles = __builtin_amdgcn_readfirstlane(blocks < a.max_blocks ? blocks : a.max_blocks);
+  }
   const int ntiles_n = (N + TN - 1) / TN;
-  const int ksplits = a.ksplits > 1 ? a.ksplits : 1;
+  const int ksplits = (!GROUPED && a.ksplits > 1) ? a.ksplits : 1;
   const int total_tiles = mtiles * ntiles_n * ksplits;   // (split K: tile ids count (output tile, K range) pairs)
+  if (GROUPED && (int)blockIdx.x >= total_tiles) return;  // (the grid is sized for the largest block count the ids can fill)
   auto tile_origin = [&](int tile, int& m0, int& n0) {
     int tm, tn;
-    if (ksplits > 1) {
+    if (GROUPED) {
+      // block-major: neighbouring workgroups share a block's activation rows
+      tm = tile / ntiles_n;
+      tn = tile - tm * ntiles_n;
+    } else if (ksplits > 1) {
       const int t = tile / ksplits;
       tm = t % mtiles;
       tn = t / mtiles;
@@ -141,10 +162,23 @@ w8a8_int8_gemm_kernel(I8Args a) {
   auto set_copy_tile = [&](int tile) {         // the output tile whose operands the copies fetch
     int m0, n0;
     tile_origin(tile, m0, n0);
+    long ebytes = 0;
+    if (GROUPED) {
+      const int* ids = a.sorted_ids + m0;
 #pragma unroll
-    for (int p = 0; p < XCOPIES; ++p) {
-      const int r = (wave + 8 * p) * 8 + crow;
-      xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * cchunk);
+      for (int p = 0; p < XCOPIES; ++p) {
+        const int id = ids[(wave + 8 * p) * 8 + crow];
+        xo[p] = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)a.ldx + (uint32_t)(16 * cchunk);   // pads read a valid row
+      }
+      int e = a.expert_ids[m0 / TM];
+      e = __builtin_amdgcn_readfirstlane((e < 0 || e >= a.E) ? 0 : e);     // (a foreign expert's block is computed and zeroed)
+      ebytes = (long)e * a.w_stride;
+    } else {
+#pragma unroll
+      for (int p = 0; p < XCOPIES; ++p) {
+        const int r = (wave + 8 * p) * 8 + crow;
+        xo[p] = (uint32_t)((min(m0 + r, M - 1) - m0) * a.ldx + 16 * cchunk);
+      }
     }
 #pragma unroll
     for (int p = 0; p < WCOPIES; ++p) {
@@ -164,8 +198,8 @@ w8a8_int8_gemm_kernel(I8Args a) {
     }
     // (split K: the tile's K range starts kbeg bytes into every row; 64 kslab rows interleave their K tiles)
     const long kbeg = ksplits > 1 ? (long)(tile % ksplits) * (K / ksplits) : 0;
-    xtile = a.x + (long)m0 * a.ldx + kbeg;
-    wtile = a.w_kslab ? a.w + kbeg * 64 : a.w + (long)n0 * a.ldw + kbeg;
+    xtile = GROUPED ? a.x : a.x + (long)m0 * a.ldx + kbeg;
+    wtile = a.w + ebytes + (a.w_kslab ? kbeg * 64 : (long)n0 * a.ldw + kbeg);
   };
   // copy slot s of this wavefront: slots 0 .. XCOPIES-1 are its x row groups,
   // the rest its w row groups (the last one only exists for some wavefronts)
@@ -312,7 +346,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // One row tile in all (M <= 256) and none of its rows in this wavefront's share: the wavefront only
   // copies.  It keeps the workgroup's barriers and its own copy slots, and leaves the matrix pipe and
   // the LDS read port of its SIMD to the wavefront that has rows (65 .. 128 rows: half the wavefronts).
-  if (mtiles == 1 && wm * (16 * NJ) >= M) {
+  if (!GROUPED && mtiles == 1 && wm * (16 * NJ) >= M) {
     for (; tile < total_tiles; tile += gdim) {
       for (int T = 0; T < nt; ++T) {
         wait_landed();
@@ -362,6 +396,45 @@ w8a8_int8_gemm_kernel(I8Args a) {
         for (int i = 0; i < NI; ++i) {
           const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
           if (n < N) *(i4*)(part + (long)m * N + n) = acc[i][j];
+        }
+      }
+      if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f70);
+      read_frag(f0, st, 0);
+      lds_wait(f0);
+      continue;
+    }
+    if (GROUPED) {
+      const int e = a.expert_ids[m0 / TM];
+      const bool foreign = e < 0 || e >= a.E;
+      const float* wsp = a.w_scale + (long)(foreign ? 0 : e) * a.ws_stride;
+      float wsg[NI][4];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int n = min(n0 + wn * (16 * NI) + i * 16 + 4 * kq, N - 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) wsg[i][c] = wsp[n + c];
+      }
+      int idj[NJ];
+      float xsg[NJ], rwg[NJ];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int id = a.sorted_ids[m0 + wm * (16 * NJ) + j * 16 + l16];
+        const bool live = id >= 0 && id < a.numel;
+        idj[j] = live ? id : -1;
+        xsg[j] = a.x_scale[a.x_scale_per_row ? (live ? id / a.topk : 0) : 0];
+        rwg[j] = foreign ? 0.0f : ((live && a.topk_weights) ? a.topk_weights[id] : 1.0f);
+      }
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if (idj[j] < 0) continue;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int n = n0 + wn * (16 * NI) + i * 16 + 4 * kq;
+          if (n >= N) continue;
+          float v[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] = foreign ? 0.0f : scaled_sum((float)acc[i][j][c], xsg[j], wsg[i][c]) * rwg[j];
+          store4<DT>(a.out, (long)idj[j] * a.ldo + n, v);
         }
       }
       if constexpr (STAGES == 3) __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -701,7 +774,47 @@ int launch_gemm(const I8Args& a, hipStream_t st) {
   return launch_tile<DT, 2, 4, 4, 8>(a, st);
 }
 
+template <int DT>
+int launch_tile_grouped(const I8Args& a, hipStream_t st) {
+  const size_t shmem = 3 * (size_t)(TM + 128) * TKB;
+  static hipError_t attr = hipFuncSetAttribute((const void*)w8a8_int8_gemm_kernel<DT, 4, 2, 4, 4, true>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  MQ_REQUIRE(attr == hipSuccess, "moe_gemm(int8 tiles): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
+  long grid = (long)a.max_blocks * ((a.N + 127) / 128);
+  const long cus = device_cu_count();
+  if (grid > cus) grid = cus;
+  hipLaunchKernelGGL((w8a8_int8_gemm_kernel<DT, 4, 2, 4, 4, true>), dim3((unsigned)grid), dim3(GEMM_THREADS), shmem, st, a);
+  MQ_LAUNCH_CHECK("moe_gemm(int8 tiles)");
+  return 0;
+}
+
 }  // namespace
+
+// The fused-MoE grouped GEMM on int8 experts (per-token x per-channel scales) on align blocks of 256 slot
+// ids: the MFMA tile kernel above with its rows gathered through the ids (prefill token counts; smaller
+// blocks take the weight-streaming kernel).  Arguments as mi355q_moe_gemm's; checked by the caller.
+int int8_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, int a_scale_per_row,
+                        const float* w_scale, const float* topk_weights, const int32_t* sorted_ids,
+                        const int32_t* expert_ids, const int32_t* npp, int numel, int topk, int max_blocks, int E,
+                        int K, int N, int out_dtype, int w_kslab, hipStream_t st) {
+  MQ_REQUIRE(N % 4 == 0 && K % 128 == 0 && (!w_kslab || N % 64 == 0), "moe_gemm(int8 tiles): bad shape N=%d K=%d", N, K);
+  MQ_REQUIRE(out_dtype == MI355Q_F16 || out_dtype == MI355Q_BF16, "moe_gemm(int8 tiles): output dtype %d", out_dtype);
+  MQ_REQUIRE(a_scale && w_scale, "moe_gemm(int8 tiles): scales missing");
+  MQ_REQUIRE(((size_t)numel / topk + 1) * K < ((size_t)1 << 32) && (size_t)N * K < ((size_t)1 << 32),
+             "moe_gemm(int8 tiles): activations and one expert's weights must each stay below 4 GiB");
+  I8Args g = {};
+  g.out = out; g.x = (const int8_t*)a; g.w = (const int8_t*)w; g.x_scale = a_scale; g.w_scale = w_scale;
+  g.M = numel; g.N = N; g.K = K; g.ldx = K; g.ldw = K; g.ldo = N;
+  g.x_scale_per_row = a_scale_per_row; g.w_scale_per_col = 1;
+  g.w_kslab = w_kslab;
+  g.ksplits = 1;
+  g.sorted_ids = sorted_ids; g.expert_ids = expert_ids; g.npp = npp; g.topk_weights = topk_weights;
+  g.numel = numel; g.topk = topk; g.E = E; g.max_blocks = max_blocks;
+  g.w_stride = (long)N * K;
+  g.ws_stride = N;
+  return out_dtype == MI355Q_F16 ? launch_tile_grouped<MI355Q_F16>(g, st) : launch_tile_grouped<MI355Q_BF16>(g, st);
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;

@@ -81,7 +81,8 @@ class TritonExpertsPad:
         E, num_tokens, N, K, top_k_num = moe_problem_size(hidden_states, w1, w2, topk_ids, self.use_int4_w4a16)
         if global_num_experts == -1:
             global_num_experts = E
-        config = get_default_config(M=num_tokens, E=E, N=N, K=K, topk=top_k_num, dtype=None, is_marlin=False,
+        config = get_default_config(M=num_tokens, E=E, N=N, K=K, topk=top_k_num,
+                                    dtype="int8_w8a8" if self.use_int8_w8a8 else None, is_marlin=False,
                                     block_shape=self.block_shape)
         act_dtype = workspace2.dtype
         # cache1 and cache3 share workspace2: cache1 is dead once cache2 exists
