@@ -549,31 +549,44 @@ static void launch_mt(const StreamArgs& a, int zk, int nt, hipStream_t st) {
   else launch_zk<DT, 4>(a, zk, nt, st);
 }
 
-// Work split, fitted to measurements on MI355X at M = 16 and 64.  Narrowing
-// the tile group (NT = 8, 4, 2) multiplies the workgroups without any
-// exchange, but every workgroup re-reads its K range of the activations from
-// L2, so long K stops at NT = 4.  Splitting K costs dependent round trips to
-// memory for the partial tiles; the split factor is the one that brings the
-// grid closest to one workgroup per CU with at least 8 K blocks each.
+// Work split: tiles of 16 columns per workgroup (NT = 8, 4, 2, 1) and K ranges (splits) that separate
+// workgroups sum through the workspace.  Chosen by a cost per workgroup, fitted to the measured times of
+// every (NT, splits) pair on 18 layer shapes of five model families at M = 16 and 64 (within 1 % of the
+// best pair on 30 of 35, 14 % at worst; the rule before it -- the grid nearest to one workgroup per CU --
+// was up to 50 % off outside the Llama-3-8B shapes, mostly by overshooting the CU count a little, which
+// costs a second round):
+//   bytes a workgroup pulls into its CU: its share of the packed weights plus half of the activation
+//   bytes of its K range (every workgroup of a slab reads them again, from the L2; narrowing the tile
+//   group multiplies the workgroups without any exchange but not their activation reads),
+//   times the rounds the grid needs on the chip; a K split never goes beyond one round,
+//   plus, for a split, a fixed 45 KB (the dependent round trips of the exchange) and 2.5 x the partial
+//   tiles the last workgroup of a slab adds up.
 StreamPlan w4a16_stream_auto_plan(int M, int K, int N, int gs) {
   const int slabs = N / 128, G = K / 128, cus = device_cu_count();
-  StreamPlan p = {8, 1};
-  if (gs % 128 == 0) {
-    if (M > 32) p.nt = 4;          // 64 rows x 8 tiles of accumulators do not fit the register file
-    const int floor_nt = K > 8192 ? 4 : 2;
-    while (p.nt > floor_nt && slabs * (8 / p.nt) < cus / 2) p.nt >>= 1;
-    // one tile per workgroup when that fills the chip without splitting K (measured at
-    // K = N = 4096: 6.4 us against 6.9 us for two tiles and two splits)
-    if (p.nt == 2 && K <= 8192 && slabs * 8 <= cus && slabs * 8 > cus / 2) p.nt = 1;
-  }
-  const int wgs = slabs * (8 / p.nt);
   const int maxs = G / 8 > 0 ? (G / 8 < 32 ? G / 8 : 32) : 1;
-  int best = 1, best_d = abs(wgs - cus);
-  for (int s = 2; s <= maxs; ++s) {
-    const int d = abs(wgs * s - cus);
-    if (d < best_d) { best = s; best_d = d; }
+  StreamPlan p = {8, 1};
+  if (gs % 128 != 0) {
+    // groups of 64 / 32: eight tiles per workgroup only; as many K ranges as stay within one round
+    for (int s = 2; s <= maxs; ++s)
+      if ((long)slabs * s <= cus) p.splits = s;
+    return p;
   }
-  p.splits = best;
+  const double Mp = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+  double best = -1.0;
+  // (64 rows x 8 tiles of accumulators do not fit the register file; one tile per workgroup reads the
+  // activations of all of K per 16 columns: up to K = 8192)
+  for (int nt = M > 32 ? 4 : 8; nt >= 1; nt >>= 1) {
+    if (nt == 1 && K > 8192) continue;
+    const long wg = (long)slabs * (8 / nt);
+    for (int s = 1; s <= maxs; ++s) {
+      const long W = wg * s;
+      if (s > 1 && W > cus) break;
+      const long rounds = (W + cus - 1) / cus;
+      const double bw = (double)K * N / 2 / (double)W, bx = Mp * K * 2 / s;
+      const double cost = (double)rounds * (bw + 0.5 * bx) + (s > 1 ? 45000.0 + 2.5 * s * nt * Mp * 64 : 0.0);
+      if (best < 0 || cost < best) { best = cost; p.nt = nt; p.splits = s; }
+    }
+  }
   return p;
 }
 
