@@ -193,8 +193,9 @@ def test_grouped_fp8_block(fmoe, ops, block):
 
 
 @pytest.mark.parametrize("kslab", [False, True])
-@pytest.mark.parametrize("M,E,T,K,N", [(300, 6, 3, 512, 384), (40, 4, 2, 384, 128), (700, 3, 1, 1024, 256)])
-def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, kslab):
+@pytest.mark.parametrize("M,E,T,K,N,blk", [(300, 6, 3, 512, 384, 256), (40, 4, 2, 384, 128, 256), (700, 3, 1, 1024, 256, 256),
+                                           (300, 6, 3, 512, 384, 128), (700, 3, 1, 1024, 256, 128)])
+def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, blk, kslab):
     """Blocks of 256 slot ids (prefill token counts) run the MFMA tile kernel with its rows gathered through
     the ids.  Both GEMM forms (rows t // topk without routing weight; one row per slot with it), row-major
     and kslab weights, an expert that no token chose, one that expert_map sends elsewhere (its rows come
@@ -217,7 +218,7 @@ def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T,
     for t in range(M * T):
         want[t] = of8.block_fp8_gemm(xq_c[t // T:t // T + 1], xs_c[t // T:t // T + 1], wq[flat[t]], ws[flat[t]])[0]
     C = torch.full((M, T, N), float("nan"), dtype=torch.bfloat16, device="cuda")
-    run_grouped(fmoe, xq, wd, C, xs, dev(ws), None, dev(tw), dev(ids), E, 256, False, T,
+    run_grouped(fmoe, xq, wd, C, xs, dev(ws), None, dev(tw), dev(ids), E, blk, False, T,
                 use_fp8_w8a8=True, block_shape=[128, 128])
     got = C.view(-1, N).float().cpu().numpy()
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
@@ -230,10 +231,10 @@ def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T,
     x2q, x2s = ops.per_token_group_quant_fp8(x2.cuda(), 128)
     emap = torch.arange(E, dtype=torch.int32)
     emap[0] = -1
-    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), 256, E, emap.cuda())
+    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), blk, E, emap.cuda())
     C2 = torch.full((M, T, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     fmoe.invoke_fused_moe_kernel(x2q, wd, C2, x2s, dev(ws), None, dev(tw), dev(ids), s_, e_, n_, True, 1,
-                                 {"BLOCK_SIZE_M": 256}, use_fp8_w8a8=True, use_int8_w8a8=False, use_int8_w8a16=False,
+                                 {"BLOCK_SIZE_M": blk}, use_fp8_w8a8=True, use_int8_w8a8=False, use_int8_w8a16=False,
                                  use_int4_w4a16=False, block_shape=[128, 128])
     torch.cuda.synchronize()
     x2q_c, x2s_c = x2q.view(torch.uint8).cpu().numpy(), x2s.cpu().numpy()
@@ -246,8 +247,9 @@ def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T,
 
 
 @pytest.mark.parametrize("kslab", [False, True])
-@pytest.mark.parametrize("M,E,T,K,N", [(300, 6, 3, 512, 384), (40, 4, 2, 384, 192), (700, 3, 1, 1024, 256)])
-def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, kslab):
+@pytest.mark.parametrize("M,E,T,K,N,blk", [(300, 6, 3, 512, 384, 256), (40, 4, 2, 384, 192, 256), (700, 3, 1, 1024, 256, 256),
+                                           (300, 6, 3, 512, 384, 128), (700, 3, 1, 1024, 256, 128)])
+def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, blk, kslab):
     """int8 experts (per-token x per-channel scales) on blocks of 256 slot ids: the int8 MFMA tile kernel
     with its rows gathered through the ids.  Both GEMM forms, row-major and kslab weights, an idle expert
     and one that expert_map sends elsewhere; the int32 sums are exact, so the outputs equal those of the
@@ -270,7 +272,7 @@ def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N
         acc = o8.int8_gemm_i32(xq[t // T:t // T + 1], np.ascontiguousarray(wq[flat[t]].T))
         want[t] = o8.scaled_mm_epilogue(acc, xs[t // T], ws[flat[t], :, 0])[0]
     C = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
-    run_grouped(fmoe, dev(xq), wd, C, dev(xs), dev(ws), None, dev(tw), dev(ids), E, 256, False, T, use_int8_w8a8=True)
+    run_grouped(fmoe, dev(xq), wd, C, dev(xs), dev(ws), None, dev(tw), dev(ids), E, blk, False, T, use_int8_w8a8=True)
     np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
     C64 = torch.empty_like(C)
     run_grouped(fmoe, dev(xq), wd, C64, dev(xs), dev(ws), None, dev(tw), dev(ids), E, 64, False, T, use_int8_w8a8=True)
@@ -280,10 +282,10 @@ def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N
     x2q, x2s = o8.dynamic_scaled_int8_quant(x2)
     emap = torch.arange(E, dtype=torch.int32)
     emap[0] = -1
-    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), 256, E, emap.cuda())
+    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), blk, E, emap.cuda())
     C2 = torch.full((M, T, N), float("nan"), dtype=torch.float16, device="cuda")
     fmoe.invoke_fused_moe_kernel(dev(x2q), wd, C2, dev(x2s), dev(ws), None, dev(tw), dev(ids), s_, e_, n_, True, 1,
-                                 {"BLOCK_SIZE_M": 256}, use_fp8_w8a8=False, use_int8_w8a8=True, use_int8_w8a16=False,
+                                 {"BLOCK_SIZE_M": blk}, use_fp8_w8a8=False, use_int8_w8a8=True, use_int8_w8a16=False,
                                  use_int4_w4a16=False)
     torch.cuda.synchronize()
     want2 = np.zeros((M * T, N), dtype=np.float32)
@@ -542,10 +544,12 @@ def test_fused_experts_w4a16_sequence(ops, rearrange, M, E, T, H, I):
 @pytest.mark.parametrize("M,E,T,H,I", [(48, 16, 4, 512, 256), (400, 8, 2, 512, 256)])
 def test_fused_experts_fp8_block_sequence(ops, fmoe, M, E, T, H, I):
     """The whole fused-experts sequence on fp8 block-scaled experts; the second case has 100 rows per expert
-    on average, where the configuration takes align blocks of 256 slots and both GEMMs run the MFMA tile
-    kernel with gathered rows."""
+    on average, where the configuration takes align blocks of 128 slots and both GEMMs run the MFMA tile
+    kernel with gathered rows (the upper half of every row tile only copies)."""
     print(f"case fused fp8 M={M} E={E}", flush=True)
-    assert (fmoe.get_default_config(M, E, 2 * I, H, T, None, False, [128, 128])["BLOCK_SIZE_M"] == 256) == (M == 400)
+    assert fmoe.get_default_config(M, E, 2 * I, H, T, None, False, [128, 128])["BLOCK_SIZE_M"] == (128 if M == 400 else 16)
+    assert fmoe.get_default_config(4 * M, E, 2 * I, H, T, None, False, [128, 128])["BLOCK_SIZE_M"] == (256 if M == 400 else 128)
+    assert fmoe.get_default_config(3 * M, E, 2 * I, H, T, None, False, [0, 128])["BLOCK_SIZE_M"] == 64      # (W4A16 experts: 64)
     rng = np.random.default_rng(3)
     w13 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, 2 * I, H)) * 0.5, -448, 448).astype(np.float32))
     w2 = of8.to_e4m3fn(np.clip(rng.standard_normal((E, H, I)) * 0.5, -448, 448).astype(np.float32))

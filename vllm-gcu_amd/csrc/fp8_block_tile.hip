@@ -52,6 +52,8 @@ struct F8Args {
   const int32_t* npp;          // device scalar: padded id count
   const float* topk_weights;   // [numel] or null
   int numel, topk, E, max_blocks;
+  int block_rows;              // slot ids per align block: 256, or 128 (the upper half of every row tile is empty:
+                               // its wavefronts only copy, as in a dense launch of up to 128 rows)
   long w_stride, ws_stride;    // per expert: bytes of weights, floats of weight scales
 };
 
@@ -89,7 +91,7 @@ fp8_block_gemm_kernel(F8Args a) {
 
   int mtiles = (M + FTM - 1) / FTM;
   if (GROUPED) {
-    const int blocks = (*a.npp + FTM - 1) / FTM;
+    const int blocks = (*a.npp + a.block_rows - 1) / a.block_rows;
     mtiles = __builtin_amdgcn_readfirstlane(blocks < a.max_blocks ? blocks : a.max_blocks);
   }
   const int ntiles_n = N / FTN;
@@ -144,10 +146,11 @@ fp8_block_gemm_kernel(F8Args a) {
     long ebytes = 0;
     int escales = 0;
     if (GROUPED) {
-      const int* ids = a.sorted_ids + m0;
+      const int* ids = a.sorted_ids + (m0 / FTM) * a.block_rows;
 #pragma unroll
       for (int p = 0; p < XCOPIES; ++p) {
-        const int id = ids[(wave + 8 * p) * 8 + crow];
+        // (blocks of 128: the upper half of the tile copies the lower half's rows once more; nobody multiplies them)
+        const int id = ids[((wave + 8 * p) * 8 + crow) & (a.block_rows - 1)];
         xo[p] = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)a.ldx + (uint32_t)(16 * cchunk);   // pads read a valid row
       }
       int e = a.expert_ids[m0 / FTM];
@@ -177,7 +180,7 @@ fp8_block_gemm_kernel(F8Args a) {
     // (split K: the tile's range starts kb0 K blocks into every row; 64 kslab rows interleave their K blocks)
     const int kb0 = ksplits > 1 ? (tile % ksplits) * (KB / ksplits) : 0;
     if (GROUPED) {
-      const int id = a.sorted_ids[m0 + 64 * (wave & 3) + lane];
+      const int id = a.sorted_ids[(m0 / FTM) * a.block_rows + ((64 * (wave & 3) + lane) & (a.block_rows - 1))];
       xso = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)KB;
     } else {
       xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB + (uint32_t)kb0;
@@ -356,7 +359,7 @@ fp8_block_gemm_kernel(F8Args a) {
   // One row tile in all (M <= 256) and none of its rows in this wavefront's share: the wavefront only
   // copies.  It keeps the workgroup's barriers and its own copy slots, and leaves the matrix pipe and
   // the LDS read port of its SIMD to the wavefront that has rows (65 .. 128 rows: half the wavefronts).
-  if (!GROUPED && mtiles == 1 && wm * (16 * NJ) >= M) {
+  if (GROUPED ? wm * (16 * NJ) >= a.block_rows : (mtiles == 1 && wm * (16 * NJ) >= M)) {
     for (; tile < total_tiles; tile += gdim) {
       for (int T = 0; T < nt; ++T) {
         const int kt = ahead_kt(T, 3);
@@ -425,7 +428,7 @@ fp8_block_gemm_kernel(F8Args a) {
       const bool foreign = e < 0 || e >= a.E;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const int id = a.sorted_ids[m0 + wm * (16 * NJ) + j * 16 + l16];
+        const int id = a.sorted_ids[(m0 / FTM) * a.block_rows + wm * (16 * NJ) + j * 16 + l16];
         if (id >= a.numel || id < 0) continue;
         const float rw = foreign ? 0.0f : (a.topk_weights ? a.topk_weights[id] : 1.0f);
 #pragma unroll
@@ -597,14 +600,15 @@ int launch_f8_grouped(const F8Args& a, hipStream_t st) {
 
 }  // namespace
 
-// The fused-MoE grouped GEMM with 128 x 128 block scales on align blocks of 256 slot ids: the MFMA tile
-// kernel above with its rows gathered through the ids (prefill token counts; smaller blocks take the
+// The fused-MoE grouped GEMM with 128 x 128 block scales on align blocks of 256 or 128 slot ids: the MFMA
+// tile kernel above with its rows gathered through the ids (prefill token counts; smaller blocks take the
 // weight-streaming kernel).  Arguments as mi355q_moe_gemm's; checked by the caller.
 int fp8_block_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, const float* w_scale,
                              const float* topk_weights, const int32_t* sorted_ids, const int32_t* expert_ids,
-                             const int32_t* npp, int numel, int topk, int max_blocks, int E, int K, int N,
+                             const int32_t* npp, int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                              int out_dtype, int w_kslab, hipStream_t st) {
   MQ_REQUIRE(N % 128 == 0 && K % 128 == 0, "moe_gemm(fp8 tiles): N=%d and K=%d must be multiples of 128", N, K);
+  MQ_REQUIRE(block_size == 256 || block_size == 128, "moe_gemm(fp8 tiles): block_size=%d must be 128 or 256", block_size);
   MQ_REQUIRE(out_dtype == MI355Q_F16 || out_dtype == MI355Q_BF16, "moe_gemm(fp8 tiles): output dtype %d", out_dtype);
   MQ_REQUIRE(((size_t)numel / topk + 1) * K < ((size_t)1 << 32) && (size_t)N * K < ((size_t)1 << 32),
              "moe_gemm(fp8 tiles): activations and one expert's weights must each stay below 4 GiB");
@@ -615,6 +619,7 @@ int fp8_block_grouped_launch(void* out, const void* a, const void* w, const floa
   g.ksplits = 1;
   g.sorted_ids = sorted_ids; g.expert_ids = expert_ids; g.npp = npp; g.topk_weights = topk_weights;
   g.numel = numel; g.topk = topk; g.E = E; g.max_blocks = max_blocks;
+  g.block_rows = block_size;
   g.w_stride = (long)N * K;
   g.ws_stride = (long)(N / 128) * (K / 128);
   return out_dtype == MI355Q_F16 ? launch_f8_grouped<MI355Q_F16>(g, st) : launch_f8_grouped<MI355Q_BF16>(g, st);

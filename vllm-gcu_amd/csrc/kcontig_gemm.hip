@@ -599,11 +599,11 @@ int w4a16_grouped_launch(void* out, const void* x, const int32_t* qweight, const
 size_t w4a16_grouped_workspace_bytes(int numel, int block_size, int max_blocks, int E, int K, int N);
 int int8_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, int a_scale_per_row,
                         const float* w_scale, const float* topk_weights, const int32_t* sorted_ids,
-                        const int32_t* expert_ids, const int32_t* npp, int numel, int topk, int max_blocks, int E,
-                        int K, int N, int out_dtype, int w_kslab, hipStream_t st);
+                        const int32_t* expert_ids, const int32_t* npp, int numel, int topk, int block_size, int max_blocks,
+                        int E, int K, int N, int out_dtype, int w_kslab, hipStream_t st);
 int fp8_block_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, const float* w_scale,
                              const float* topk_weights, const int32_t* sorted_ids, const int32_t* expert_ids,
-                             const int32_t* npp, int numel, int topk, int max_blocks, int E, int K, int N,
+                             const int32_t* npp, int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                              int out_dtype, int w_kslab, hipStream_t st);
 
 // fp8 x fp8 with scales outside the K sum (per token or one value; per output channel or one value), M <= 128:
@@ -689,17 +689,20 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
     MQ_REQUIRE(a_scale && w_scale, "moe_gemm(fp8): scales missing");
     MQ_REQUIRE(group_size == 128, "moe_gemm(fp8): only 128x128 block scales are supported, got %d", group_size);
     // blocks of 256 slots (prefill token counts): the MFMA tile kernel with gathered rows
-    if (block_size == 256 && N % 128 == 0)
+    // (blocks of 128 -- also a block size of the weight-streaming kernel -- from 40 rows per expert on average)
+    if ((block_size == 256 || (block_size == 128 && (long)numel >= 40L * E)) && N % 128 == 0)
       return fp8_block_grouped_launch(out, a, w, a_scale, (const float*)w_scale, topk_weights, sorted_token_ids, expert_ids,
-                                      num_tokens_post_pad, numel, topk, max_blocks, E, K, N, out_dtype, w_layout, st);
+                                      num_tokens_post_pad, numel, topk, block_size, max_blocks, E, K, N, out_dtype,
+                                      w_layout, st);
     mode = KC_FP8_BLOCK;
     g.ws_stride = (long)((N + 127) / 128) * (K / 128);
   } else if (quant_mode == 2) {
     MQ_REQUIRE(w_scale, "moe_gemm(int8): weight scales missing");
     // blocks of 256 slots (prefill token counts): the MFMA tile kernel with gathered rows
-    if (block_size == 256 && a_scale)
+    if ((block_size == 256 || (block_size == 128 && (long)numel >= 40L * E)) && a_scale)
       return int8_grouped_launch(out, a, w, a_scale, 1, (const float*)w_scale, topk_weights, sorted_token_ids, expert_ids,
-                                 num_tokens_post_pad, numel, topk, max_blocks, E, K, N, out_dtype, w_layout, st);
+                                 num_tokens_post_pad, numel, topk, block_size, max_blocks, E, K, N, out_dtype,
+                                 w_layout, st);
     mode = KC_INT8;
     g.ws_stride = N;
   } else if (quant_mode == 3) {

@@ -48,6 +48,8 @@ struct I8Args {
   const int32_t* npp;          // device scalar: padded id count
   const float* topk_weights;   // [numel] or null
   int numel, topk, E, max_blocks;
+  int block_rows;              // slot ids per align block: 256, or 128 (the upper half of every row tile is empty:
+                               // its wavefronts only copy, as in a dense launch of up to 128 rows)
   long w_stride, ws_stride;    // per expert: bytes of weights, floats of weight scales
 };
 
@@ -107,7 +109,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // of the same weight panels.
   int mtiles = (M + TM - 1) / TM;
   if (GROUPED) {
-    const int blocks = (*a.npp + TM - 1) / TM;
+    const int blocks = (*a.npp + a.block_rows - 1) / a.block_rows;
     mtiles = __builtin_amdgcn_readfirstlane(blocks < a.max_blocks ? blocks : a.max_blocks);
   }
   const int ntiles_n = (N + TN - 1) / TN;
@@ -164,10 +166,11 @@ w8a8_int8_gemm_kernel(I8Args a) {
     tile_origin(tile, m0, n0);
     long ebytes = 0;
     if (GROUPED) {
-      const int* ids = a.sorted_ids + m0;
+      const int* ids = a.sorted_ids + (m0 / TM) * a.block_rows;
 #pragma unroll
       for (int p = 0; p < XCOPIES; ++p) {
-        const int id = ids[(wave + 8 * p) * 8 + crow];
+        // (blocks of 128: the upper half of the tile copies the lower half's rows once more; nobody multiplies them)
+        const int id = ids[((wave + 8 * p) * 8 + crow) & (a.block_rows - 1)];
         xo[p] = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)a.ldx + (uint32_t)(16 * cchunk);   // pads read a valid row
       }
       int e = a.expert_ids[m0 / TM];
@@ -346,7 +349,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
   // One row tile in all (M <= 256) and none of its rows in this wavefront's share: the wavefront only
   // copies.  It keeps the workgroup's barriers and its own copy slots, and leaves the matrix pipe and
   // the LDS read port of its SIMD to the wavefront that has rows (65 .. 128 rows: half the wavefronts).
-  if (!GROUPED && mtiles == 1 && wm * (16 * NJ) >= M) {
+  if (GROUPED ? wm * (16 * NJ) >= a.block_rows : (mtiles == 1 && wm * (16 * NJ) >= M)) {
     for (; tile < total_tiles; tile += gdim) {
       for (int T = 0; T < nt; ++T) {
         wait_landed();
@@ -418,7 +421,7 @@ w8a8_int8_gemm_kernel(I8Args a) {
       float xsg[NJ], rwg[NJ];
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const int id = a.sorted_ids[m0 + wm * (16 * NJ) + j * 16 + l16];
+        const int id = a.sorted_ids[(m0 / TM) * a.block_rows + wm * (16 * NJ) + j * 16 + l16];
         const bool live = id >= 0 && id < a.numel;
         idj[j] = live ? id : -1;
         xsg[j] = a.x_scale[a.x_scale_per_row ? (live ? id / a.topk : 0) : 0];
@@ -790,13 +793,14 @@ int launch_tile_grouped(const I8Args& a, hipStream_t st) {
 
 }  // namespace
 
-// The fused-MoE grouped GEMM on int8 experts (per-token x per-channel scales) on align blocks of 256 slot
+// The fused-MoE grouped GEMM on int8 experts (per-token x per-channel scales) on align blocks of 256 or 128 slot
 // ids: the MFMA tile kernel above with its rows gathered through the ids (prefill token counts; smaller
 // blocks take the weight-streaming kernel).  Arguments as mi355q_moe_gemm's; checked by the caller.
 int int8_grouped_launch(void* out, const void* a, const void* w, const float* a_scale, int a_scale_per_row,
                         const float* w_scale, const float* topk_weights, const int32_t* sorted_ids,
-                        const int32_t* expert_ids, const int32_t* npp, int numel, int topk, int max_blocks, int E,
-                        int K, int N, int out_dtype, int w_kslab, hipStream_t st) {
+                        const int32_t* expert_ids, const int32_t* npp, int numel, int topk, int block_size, int max_blocks,
+                        int E, int K, int N, int out_dtype, int w_kslab, hipStream_t st) {
+  MQ_REQUIRE(block_size == 256 || block_size == 128, "moe_gemm(int8 tiles): block_size=%d must be 128 or 256", block_size);
   MQ_REQUIRE(N % 4 == 0 && K % 128 == 0 && (!w_kslab || N % 64 == 0), "moe_gemm(int8 tiles): bad shape N=%d K=%d", N, K);
   MQ_REQUIRE(out_dtype == MI355Q_F16 || out_dtype == MI355Q_BF16, "moe_gemm(int8 tiles): output dtype %d", out_dtype);
   MQ_REQUIRE(a_scale && w_scale, "moe_gemm(int8 tiles): scales missing");
@@ -810,6 +814,7 @@ int int8_grouped_launch(void* out, const void* a, const void* w, const float* a_
   g.ksplits = 1;
   g.sorted_ids = sorted_ids; g.expert_ids = expert_ids; g.npp = npp; g.topk_weights = topk_weights;
   g.numel = numel; g.topk = topk; g.E = E; g.max_blocks = max_blocks;
+  g.block_rows = block_size;
   g.w_stride = (long)N * K;
   g.ws_stride = N;
   return out_dtype == MI355Q_F16 ? launch_tile_grouped<MI355Q_F16>(g, st) : launch_tile_grouped<MI355Q_BF16>(g, st);

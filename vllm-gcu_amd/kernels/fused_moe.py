@@ -12,12 +12,15 @@ import torch
 from . import _custom_ops as ops
 
 
-# Rows per expert from which the fp8 block-scaled grouped GEMM takes 256-slot blocks (measured on MI355X, us,
-# blocks of 64 on the weight-streaming kernel / blocks of 256 on the tile kernel; the tile kernel's time hardly
-# depends on how full its blocks are).  Mixtral shape, K 4096 x N 28672, 8 experts, at 32 / 64 / 128 / 512 rows
-# per expert: 213 / 365 / 569 / 1865 against 283 / 289 / 296 / 769; DeepSeek-V3 shape, K 7168 x N 4096, 256 experts,
-# at 32 / 64 / 128 / 256: 1557 / 2491 / 4320 / 7568 against 2142 / 2202 / 2348 / 3493.
-_FP8_TILE_MIN_ROWS_PER_EXPERT = 48
+# Rows per expert from which the fp8 block-scaled and int8 grouped GEMMs take blocks of 128 and of 256 slots, i.e.
+# the MFMA tile kernels with gathered rows instead of the weight-streaming kernel on blocks of 64 (measured on
+# MI355X, us per GEMM, blocks of 64 / 128 / 256; a tile costs about the same however full it is, one of 128 slots
+# about 0.8 of one of 256).  Mixtral shape, fp8, K 4096 x N 28672, 8 experts, at 48 / 64 / 96 / 128 / 192 rows per
+# expert: 253 / 315 / 475 / 570 / 794 -- 221 / 233 / 251 / 357 / 420 -- 279 / 278 / 283 / 287 / 315; DeepSeek-V3 shape,
+# K 7168 x N 4096, 256 experts, at 64 / 96 / 128 / 192: 2504 / 3538 / 4313 / 5962 -- 1734 / 1896 / 2576 / 4063 --
+# 2177 / 2241 / 2278 / 2477.  (The library takes the tile kernels for blocks of 128 from 40 rows per expert on.)
+_FP8_TILE_MIN_ROWS_PER_EXPERT = 40
+_TILE_256_ROWS_PER_EXPERT = 110
 
 
 def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optional[str], is_marlin: bool,
@@ -31,9 +34,10 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
     per_expert = (M * topk) / max(E, 1)
     tiles = (block_shape is not None and list(block_shape) == [128, 128]) or dtype == "int8_w8a8"
     if tiles and per_expert > _FP8_TILE_MIN_ROWS_PER_EXPERT:
-        # fp8 block-scaled and int8 experts at prefill token counts: blocks of 256 slots run the MFMA tile
-        # kernels with gathered rows instead of the weight-streaming kernel
-        return {"BLOCK_SIZE_M": 256, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
+        # fp8 block-scaled and int8 experts at prefill token counts: blocks of 128 or 256 slots run the MFMA
+        # tile kernels with gathered rows instead of the weight-streaming kernel
+        return {"BLOCK_SIZE_M": 256 if per_expert > _TILE_256_ROWS_PER_EXPERT else 128, "BLOCK_SIZE_N": 64,
+                "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
     if per_expert <= 16:
         bm = 16
     elif per_expert <= 28:      # measured on the Mixtral-8x7B W4A16 layer: at 32 rows per expert on average
