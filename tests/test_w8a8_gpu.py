@@ -132,7 +132,9 @@ def test_int8_streaming_kernel_16_32_and_64_columns_per_workgroup(ops, M, N, mon
 
 
 @pytest.mark.parametrize("M,K,N,splits", [(128, 4096, 1024, 4), (200, 8192, 512, 8), (700, 2048, 1024, 2),
-                                            (64, 14336, 4096, 8), (1000, 3072, 768, 3)])
+                                            (64, 14336, 4096, 8), (1000, 3072, 768, 3),
+                                            # several row tiles on a layer of few columns: K ranges of 256 x 256 tiles
+                                            (520, 8192, 5632, 2)])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_int8_gemm_split_k_is_bit_identical(ops, M, K, N, splits, out_dtype):
     """Few output tiles behind a long K: the operator cuts K into ranges that run side by side (int32

@@ -719,12 +719,30 @@ int int8_ksplits(int M, int N, int K) {
   return s < 1 ? 1 : (int)s;
 }
 
+// The same for several row tiles on a layer of few columns (a few thousand rows on N 4096: 128 tiles of
+// 256 x 256, half a round): K ranges of 256 x 256 tiles, which move a third fewer bytes per multiply-add
+// than the 256 x 128 tiles that would fill the round unsplit (us, K 14336 x N 4096 at M = 1536 / 2048: 146 / 145 ->
+// 110 / 122; K 18944 x N 3584: 186 / 187 -> 130 / 137; K 28672 x N 8192 at M = 768 / 1024: 309 / 320 -> 219 / 247;
+// K 8192 x N 8192 at M = 512 / 768: 63 / 94 -> 53 / 83).  0: not this case.
+int int8_ksplits_wide(int M, int N, int K) {
+  const long cus = device_cu_count(), mtiles = (M + TM - 1) / TM;
+  const long t256 = mtiles * ((N + 255) / 256), t128 = mtiles * ((N + 127) / 128);
+  const int nt = K / TKB;
+  if (N % 4 != 0 || mtiles < 2 || t128 * 2 <= cus || t256 * 2 > cus) return 0;
+  long s = cus / t256;
+  if (s > nt / 32) s = nt / 32;                      // (ranges of 4096 bytes of K or more: K = 4096 stays unsplit, 49 against 61 us)
+  if (s > 8) s = 8;
+  if (s > nt / 8) s = nt / 8;
+  while (s > 1 && (nt % s != 0 || (size_t)s * M * N * sizeof(int32_t) > I8_SPLITK_BYTES)) --s;
+  return s < 2 ? 0 : (int)s;
+}
+
 template <int DT>
-int launch_gemm_splitk(const I8Args& a, int splits, void* workspace, hipStream_t st) {
+int launch_gemm_splitk(const I8Args& a, int splits, void* workspace, hipStream_t st, bool wide = false) {
   I8Args b = a;
   b.ksplits = splits;
   b.partial = (int32_t*)((char*)workspace + I8_WS_OFFSET);
-  if (int rc = launch_tile<DT, 4, 2, 4, 4>(b, st)) return rc;
+  if (int rc = wide ? launch_tile<DT, 2, 4, 4, 8>(b, st) : launch_tile<DT, 4, 2, 4, 4>(b, st)) return rc;
   const long quads = (long)a.M * (a.N / 4);
   hipLaunchKernelGGL((w8a8_splitk_epilogue_kernel<DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, b);
   MQ_LAUNCH_CHECK("w8a8_int8_gemm(split-K epilogue)");
@@ -826,7 +844,8 @@ using namespace mi355q;
 
 extern "C" size_t mi355q_w8a8_int8_workspace_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
-  const int s = int8_ksplits(M, N, K);
+  int s = int8_ksplits(M, N, K);
+  if (s <= 1) s = int8_ksplits_wide(M, N, K);
   return s > 1 ? I8_WS_OFFSET + (size_t)s * M * N * sizeof(int32_t) : 0;
 }
 
@@ -864,11 +883,13 @@ extern "C" int mi355q_w8a8_int8_gemm_ws(void* out, int32_t* acc_out, const int8_
   a.wide_stores = (N % 8 == 0 && ldo % 8 == 0 && ((size_t)out & 15) == 0) ? 1 : 0;
   a.ksplits = 1;
   a.partial = nullptr;
-  const int splits = int8_ksplits(M, N, K);
+  int splits = int8_ksplits(M, N, K);
+  const bool wide = splits <= 1;
+  if (wide) splits = int8_ksplits_wide(M, N, K);
   if (splits > 1 && workspace && workspace_bytes >= I8_WS_OFFSET + (size_t)splits * M * N * sizeof(int32_t)) {
-    if (out_dtype == MI355Q_F16) return launch_gemm_splitk<MI355Q_F16>(a, splits, workspace, as_stream(stream));
-    if (out_dtype == MI355Q_BF16) return launch_gemm_splitk<MI355Q_BF16>(a, splits, workspace, as_stream(stream));
-    return launch_gemm_splitk<MI355Q_F32>(a, splits, workspace, as_stream(stream));
+    if (out_dtype == MI355Q_F16) return launch_gemm_splitk<MI355Q_F16>(a, splits, workspace, as_stream(stream), wide);
+    if (out_dtype == MI355Q_BF16) return launch_gemm_splitk<MI355Q_BF16>(a, splits, workspace, as_stream(stream), wide);
+    return launch_gemm_splitk<MI355Q_F32>(a, splits, workspace, as_stream(stream), wide);
   }
   if (out_dtype == MI355Q_F16) return launch_gemm<MI355Q_F16>(a, as_stream(stream));
   if (out_dtype == MI355Q_BF16) return launch_gemm<MI355Q_BF16>(a, as_stream(stream));
