@@ -195,12 +195,13 @@ def test_grouped_fp8_block(fmoe, ops, block):
 @pytest.mark.parametrize("kslab", [False, True])
 @pytest.mark.parametrize("M,E,T,K,N,blk", [(300, 6, 3, 512, 384, 256), (40, 4, 2, 384, 128, 256), (700, 3, 1, 1024, 256, 256),
                                            (300, 6, 3, 512, 384, 128), (700, 3, 1, 1024, 256, 128)])
-def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, blk, kslab):
+def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, monkeypatch, M, E, T, K, N, blk, kslab):
     """Blocks of 256 slot ids (prefill token counts) run the MFMA tile kernel with its rows gathered through
     the ids.  Both GEMM forms (rows t // topk without routing weight; one row per slot with it), row-major
     and kslab weights, an expert that no token chose, one that expert_map sends elsewhere (its rows come
     back as zeros); against the oracle and against the weight-streaming kernel on blocks of 64."""
     print(f"case grouped fp8 tiles M={M} E={E} T={T} K={K} N={N} kslab={kslab}", flush=True)
+    monkeypatch.setattr(ops, "_AUTO_KSLAB", False)       # (row-major weights stay row-major)
     rng = np.random.default_rng(M + K)
     wq = np.stack([of8.to_e4m3fn(np.clip(rng.standard_normal((N, K)) * 2, -448, 448).astype(np.float32)) for _ in range(E)])
     ws = rng.uniform(0.005, 0.02, size=(E, N // 128, K // 128)).astype(np.float32)
@@ -249,12 +250,13 @@ def test_grouped_fp8_block_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T,
 @pytest.mark.parametrize("kslab", [False, True])
 @pytest.mark.parametrize("M,E,T,K,N,blk", [(300, 6, 3, 512, 384, 256), (40, 4, 2, 384, 192, 256), (700, 3, 1, 1024, 256, 256),
                                            (300, 6, 3, 512, 384, 128), (700, 3, 1, 1024, 256, 128)])
-def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N, blk, kslab):
+def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, monkeypatch, M, E, T, K, N, blk, kslab):
     """int8 experts (per-token x per-channel scales) on blocks of 256 slot ids: the int8 MFMA tile kernel
     with its rows gathered through the ids.  Both GEMM forms, row-major and kslab weights, an idle expert
     and one that expert_map sends elsewhere; the int32 sums are exact, so the outputs equal those of the
     weight-streaming kernel on blocks of 64 bit for bit."""
     print(f"case grouped int8 tiles M={M} E={E} T={T} K={K} N={N} kslab={kslab}", flush=True)
+    monkeypatch.setattr(ops, "_AUTO_KSLAB", False)       # (row-major weights stay row-major)
     rng = np.random.default_rng(M + K + 1)
     wq = rng.integers(-127, 128, size=(E, N, K), dtype=np.int8)
     ws = rng.uniform(0.001, 0.02, size=(E, N, 1)).astype(np.float32)
@@ -294,6 +296,59 @@ def test_grouped_int8_on_blocks_of_256_slots(fmoe, ops, rearrange, M, E, T, K, N
         if flat[t] != 0:
             acc = o8.int8_gemm_i32(x2q[t:t + 1], np.ascontiguousarray(wq[flat[t]].T))
             want2[t] = o8.scaled_mm_epilogue(acc, x2s[t], ws[flat[t], :, 0])[0] * twf[t]
+    np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("kslab", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,E,T,K,N,blk", [(300, 6, 3, 512, 384, 256), (40, 4, 2, 384, 256, 256), (700, 3, 1, 1152, 256, 256),
+                                           (300, 6, 3, 512, 384, 128), (700, 3, 1, 1152, 256, 128)])
+def test_grouped_16bit_on_blocks_of_256_slots(fmoe, ops, rearrange, monkeypatch, M, E, T, K, N, blk, dtype, kslab):
+    """Unquantised fp16 / bf16 experts on blocks of 256 or 128 slot ids: the MFMA tile kernel with its rows
+    gathered through the ids, two 32-deep 16-bit MFMAs per 128-byte K tile.  Both GEMM forms, row-major and
+    kslab weights, an odd and an even number of K tiles, an idle expert and one that expert_map sends
+    elsewhere; against the fp32 oracle, and against the weight-streaming kernel on blocks of 64 (another
+    order of the same fp32 additions)."""
+    print(f"case grouped 16-bit tiles M={M} E={E} T={T} K={K} N={N} blk={blk} {dtype} kslab={kslab}", flush=True)
+    monkeypatch.setattr(ops, "_AUTO_KSLAB", False)       # (row-major weights stay row-major)
+    rng = np.random.default_rng(M + K + 2)
+    w = torch.from_numpy((rng.standard_normal((E, N, K)) * 0.05).astype(np.float32)).to(dtype)
+    wd = w.cuda()
+    if kslab:
+        wd = rearrange.to_kslab(wd)
+    logits = rng.standard_normal((M, E)).astype(np.float32)
+    logits[:, E - 1] -= 50.0
+    tw, ids, _ = om.topk_softmax(logits, T, True)
+    flat = ids.reshape(-1)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    wf, xf = w.float().numpy(), x.float().numpy()
+    want = np.zeros((M * T, N), dtype=np.float32)
+    for e in range(E):
+        rows = np.nonzero(flat == e)[0]
+        if rows.size:
+            want[rows] = xf[rows // T] @ wf[e].T
+    C = torch.full((M, T, N), float("nan"), dtype=dtype, device="cuda")
+    run_grouped(fmoe, x.cuda(), wd, C, None, None, None, dev(tw), dev(ids), E, blk, False, T)
+    np.testing.assert_allclose(C.view(-1, N).float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    C64 = torch.empty_like(C)
+    run_grouped(fmoe, x.cuda(), wd, C64, None, None, None, dev(tw), dev(ids), E, 64, False, T)
+    np.testing.assert_allclose(C.float().cpu().numpy(), C64.float().cpu().numpy(), rtol=RTOL, atol=ATOL)
+    # second form: one activation row per slot, routing weights applied; expert 0 mapped away
+    x2 = torch.from_numpy(rng.standard_normal((M * T, K)).astype(np.float32)).to(dtype)
+    emap = torch.arange(E, dtype=torch.int32)
+    emap[0] = -1
+    s_, e_, n_ = fmoe.moe_align_block_size(dev(ids), blk, E, emap.cuda())
+    C2 = torch.full((M, T, N), float("nan"), dtype=dtype, device="cuda")
+    fmoe.invoke_fused_moe_kernel(x2.cuda(), wd, C2, None, None, None, dev(tw), dev(ids), s_, e_, n_, True, 1,
+                                 {"BLOCK_SIZE_M": blk}, use_fp8_w8a8=False, use_int8_w8a8=False, use_int8_w8a16=False,
+                                 use_int4_w4a16=False)
+    torch.cuda.synchronize()
+    x2f, twf = x2.float().numpy(), tw.reshape(-1)
+    want2 = np.zeros((M * T, N), dtype=np.float32)
+    for e in range(1, E):
+        rows = np.nonzero(flat == e)[0]
+        if rows.size:
+            want2[rows] = (x2f[rows] @ wf[e].T) * twf[rows, None]
     np.testing.assert_allclose(C2.view(-1, N).float().cpu().numpy(), want2, rtol=RTOL, atol=ATOL)
 
 

@@ -21,6 +21,12 @@
 // PC variant (per-token x per-channel scales, cutlass_scaled_mm on fp8 operands): the scales live
 // outside the K sum, so every MFMA accumulates straight into the running sum, no scales travel
 // through LDS, and the epilogue multiplies by x_scale[m] (or one value) and w_scale[n] (or one value).
+//
+// OP16 variant (unquantised fp16 / bf16 experts at prefill token counts, grouped launches only): the
+// same tiles of 128 bytes per row hold 64 elements of 16 bits; a lane's two 16-byte chunks are the
+// operands of two 32-deep 16-bit MFMAs (chunk kq: elements 8 kq .. 8 kq + 7 of the first 32, chunk
+// 4 + kq: of the second 32), which take as long as the one 128-deep fp8 MFMA.  No scales anywhere.
+// The host passes K and the row strides in bytes.
 #include "common.h"
 
 namespace mi355q {
@@ -42,7 +48,7 @@ struct F8Args {
   const void* bias;         // [N] in the output dtype or null
   int M, N, K;
   long ldx, ldw, ldo;
-  int w_kslab;
+  int w_kslab;              // 1: kslab order of 1-byte elements; 2: of 2-byte elements (OP16; K blocks of 256 bytes)
   int n_panels_swizzle;
   int ksplits;              // > 1: every output tile is worked on by `ksplits` workgroups, each a range of K blocks,
   float* partial;           //      which leave their fp32 sums in partial[split][M][N]; the epilogue is a second launch
@@ -74,10 +80,11 @@ typedef int i8v __attribute__((ext_vector_type(8)));
 // weights and weight scales are the expert's, output row id gets the result (times its routing weight).
 // Blocks past num_tokens_post_pad do not exist (the tile count is read on the device); a block of an
 // expert outside [0, E) writes zeros.  No K ranges, no bias.
-template <int DT, bool PC, bool GROUPED = false>
+template <int DT, bool PC, bool GROUPED = false, bool OP16 = false>
 __global__ void __launch_bounds__(F8_THREADS, 1)
 fp8_block_gemm_kernel(F8Args a) {
-  static_assert(!GROUPED || !PC, "the grouped form exists for block scales");
+  static_assert(!GROUPED || !PC || OP16, "the grouped form exists for block scales and for 16-bit operands");
+  static_assert(!OP16 || (PC && GROUPED), "16-bit operands: grouped launches, no scales");
   constexpr int WN = 2, NI = 4, NJ = 4;                 // 4 x 2 wavefronts of 64 x 64
   constexpr int X_BYTES = FTM * FTKB, W_BYTES = FTN * FTKB, XS_BYTES = FTM * 4;
   constexpr int WS_BYTES = 256;                         // the tile's weight scale of a K block, 64 copies
@@ -166,7 +173,14 @@ fp8_block_gemm_kernel(F8Args a) {
     }
 #pragma unroll
     for (int p = 0; p < WCOPIES; ++p) {
-      if (a.w_kslab) {
+      if (OP16 && a.w_kslab) {
+        // 2-byte elements: a K block of the kslab order is 256 bytes per row = two of this kernel's K
+        // tiles; chunk c of K tile h is vector c & 3 of lane quarter 2 h + (c >> 2)
+        const uint32_t n = (uint32_t)(n0 + (wave + 8 * p) * 8 + (lane & 7));
+        const uint32_t c = (uint32_t)((lane >> 3) ^ (wave & 1));
+        wo[p] = ((n >> 6) * (uint32_t)(K >> 8) * 4u + ((n & 63u) >> 4)) * 4096u + (c & 3u) * 1024u +
+                ((c >> 2) * 16u + (n & 15u)) * 16u;
+      } else if (a.w_kslab) {
         const uint32_t n = (uint32_t)(n0 + (wave + 8 * p) * 8 + (lane & 7));
         const uint32_t c = (uint32_t)((lane >> 3) ^ (wave & 1));
         wo[p] = ((n >> 6) * (uint32_t)(K >> 7) * 4u + ((n & 63u) >> 4)) * 2048u + (c & 1u) * 1024u +
@@ -196,8 +210,9 @@ fp8_block_gemm_kernel(F8Args a) {
       dma16(xtile + (long)kt * FTKB + xo[s], xs + (wave + 8 * s) * 1024);
     } else if (s < XCOPIES + WCOPIES) {
       const int p = s - XCOPIES;
-      dma16(wtile + (a.w_kslab ? (long)kt * FTKB * 64 : (long)kt * FTKB) + wo[p < WCOPIES ? p : 0],
-            xs + X_BYTES + (wave + 8 * p) * 1024);
+      const long koff = (OP16 && a.w_kslab) ? (long)(kt >> 1) * 16384 + (kt & 1) * 512
+                                            : (a.w_kslab ? (long)kt * FTKB * 64 : (long)kt * FTKB);
+      dma16(wtile + koff + wo[p < WCOPIES ? p : 0], xs + X_BYTES + (wave + 8 * p) * 1024);
     } else if (PC) {
       // no scales inside the K sum
     } else if (wave < 4) {
@@ -280,7 +295,15 @@ fp8_block_gemm_kernel(F8Args a) {
         const i4 a0 = i < 3 ? w012[i < 3 ? i : 0][0] : w3cur[0], a1 = i < 3 ? w012[i < 3 ? i : 0][1] : w3cur[1];
         const i8v av = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
         const i8v bv = __builtin_shufflevector(cur.bx[0][j], cur.bx[1][j], 0, 1, 2, 3, 4, 5, 6, 7);
-        if (PC) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[i][j], 0, 0, 0, 0, 0, 0);
+        if constexpr (OP16) {
+          if constexpr (DT == MI355Q_F16) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<h8>(a0), bitcast<h8>(cur.bx[0][j]), acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<h8>(a1), bitcast<h8>(cur.bx[1][j]), acc[i][j], 0, 0, 0);
+          } else {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(a0), bitcast<b8>(cur.bx[0][j]), acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(a1), bitcast<b8>(cur.bx[1][j]), acc[i][j], 0, 0, 0);
+          }
+        } else if (PC) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[i][j], 0, 0, 0, 0, 0, 0);
         else ring[n & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
         if (!PC && n >= 2) {
           const int pn = n - 2;
@@ -584,17 +607,17 @@ int launch_f8(const F8Args& a, hipStream_t st) {
   return 0;
 }
 
-template <int DT>
+template <int DT, bool OP16 = false>
 int launch_f8_grouped(const F8Args& a, hipStream_t st) {
   const size_t shmem = 3 * (size_t)(FTM * FTKB + FTN * FTKB + FTM * 4 + 256);
-  static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT, false, true>,
+  static hipError_t attr = hipFuncSetAttribute((const void*)fp8_block_gemm_kernel<DT, OP16, true, OP16>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-  MQ_REQUIRE(attr == hipSuccess, "moe_gemm(fp8 tiles): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
+  MQ_REQUIRE(attr == hipSuccess, "moe_gemm(MFMA tiles): cannot reserve %zu bytes of LDS: %s", shmem, hipGetErrorString(attr));
   long grid = (long)a.max_blocks * (a.N / FTN);
   const long cus = device_cu_count();
   if (grid > cus) grid = cus;
-  hipLaunchKernelGGL((fp8_block_gemm_kernel<DT, false, true>), dim3((unsigned)grid), dim3(F8_THREADS), shmem, st, a);
-  MQ_LAUNCH_CHECK("moe_gemm(fp8 tiles)");
+  hipLaunchKernelGGL((fp8_block_gemm_kernel<DT, OP16, true, OP16>), dim3((unsigned)grid), dim3(F8_THREADS), shmem, st, a);
+  MQ_LAUNCH_CHECK("moe_gemm(MFMA tiles)");
   return 0;
 }
 
@@ -623,6 +646,28 @@ int fp8_block_grouped_launch(void* out, const void* a, const void* w, const floa
   g.w_stride = (long)N * K;
   g.ws_stride = (long)(N / 128) * (K / 128);
   return out_dtype == MI355Q_F16 ? launch_f8_grouped<MI355Q_F16>(g, st) : launch_f8_grouped<MI355Q_BF16>(g, st);
+}
+
+// The same for unquantised fp16 / bf16 experts ([E, N, K] row-major, or the kslab order of 2-byte elements):
+// out[id] = x[id / topk] . w[e]^T (times the routing weight), fp32 sums.
+int half_grouped_tile_launch(void* out, const void* a, const void* w, const float* topk_weights,
+                             const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp, int numel, int topk,
+                             int block_size, int max_blocks, int E, int K, int N, int dtype, int w_kslab, hipStream_t st) {
+  MQ_REQUIRE(N % 128 == 0 && K % 128 == 0, "moe_gemm(16-bit tiles): N=%d and K=%d must be multiples of 128", N, K);
+  MQ_REQUIRE(block_size == 256 || block_size == 128, "moe_gemm(16-bit tiles): block_size=%d must be 128 or 256", block_size);
+  MQ_REQUIRE(dtype == MI355Q_F16 || dtype == MI355Q_BF16, "moe_gemm(16-bit tiles): dtype %d", dtype);
+  MQ_REQUIRE(((size_t)numel / topk + 1) * K * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32),
+             "moe_gemm(16-bit tiles): activations and one expert's weights must each stay below 4 GiB");
+  F8Args g = {};
+  g.out = out; g.x = (const uint8_t*)a; g.w = (const uint8_t*)w;
+  g.M = numel; g.N = N; g.K = 2 * K; g.ldx = 2L * K; g.ldw = 2L * K; g.ldo = N;     // K and operand strides in bytes
+  g.w_kslab = w_kslab ? 2 : 0;
+  g.ksplits = 1;
+  g.sorted_ids = sorted_ids; g.expert_ids = expert_ids; g.npp = npp; g.topk_weights = topk_weights;
+  g.numel = numel; g.topk = topk; g.E = E; g.max_blocks = max_blocks;
+  g.block_rows = block_size;
+  g.w_stride = 2L * N * K;
+  return dtype == MI355Q_F16 ? launch_f8_grouped<MI355Q_F16, true>(g, st) : launch_f8_grouped<MI355Q_BF16, true>(g, st);
 }
 
 }  // namespace mi355q

@@ -606,6 +606,10 @@ int fp8_block_grouped_launch(void* out, const void* a, const void* w, const floa
                              const int32_t* npp, int numel, int topk, int block_size, int max_blocks, int E, int K, int N,
                              int out_dtype, int w_kslab, hipStream_t st);
 
+int half_grouped_tile_launch(void* out, const void* a, const void* w, const float* topk_weights,
+                             const int32_t* sorted_ids, const int32_t* expert_ids, const int32_t* npp, int numel, int topk,
+                             int block_size, int max_blocks, int E, int K, int N, int dtype, int w_kslab, hipStream_t st);
+
 // fp8 x fp8 with scales outside the K sum (per token or one value; per output channel or one value), M <= 128:
 // the weight-streaming kernel.  Arguments are checked by the caller (mi355q_fp8_scaled_gemm).
 int kcontig_fp8_pc_launch(void* out, const void* a, const void* w, const float* a_scale, int scale_per_row,
@@ -706,6 +710,10 @@ extern "C" int mi355q_moe_gemm(void* out, const void* a, const void* w, const fl
     mode = KC_INT8;
     g.ws_stride = N;
   } else if (quant_mode == 3) {
+    // blocks of 256 / 128 slots (prefill token counts): the MFMA tile kernel with gathered rows
+    if ((block_size == 256 || (block_size == 128 && (long)numel >= 40L * E)) && N % 128 == 0 && out_dtype == act_dtype)
+      return half_grouped_tile_launch(out, a, w, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, numel,
+                                      topk, block_size, max_blocks, E, K, N, act_dtype, w_layout, st);
     mode = act_dtype == MI355Q_F16 ? KC_F16 : KC_BF16;
   } else if (quant_mode == 4) {
     MQ_REQUIRE(w_scale, "moe_gemm(w8a16): weight scales missing");

@@ -32,7 +32,7 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
     tiles with two workgroups per CU were measured faster than 128-row tiles up
     to 4096 tokens on the Mixtral-8x7B layer, and they pad less)."""
     per_expert = (M * topk) / max(E, 1)
-    tiles = (block_shape is not None and list(block_shape) == [128, 128]) or dtype == "int8_w8a8"
+    tiles = (block_shape is not None and list(block_shape) == [128, 128]) or dtype in ("int8_w8a8", "w16a16")
     if tiles and per_expert > _FP8_TILE_MIN_ROWS_PER_EXPERT:
         # fp8 block-scaled and int8 experts at prefill token counts: blocks of 128 or 256 slots run the MFMA
         # tile kernels with gathered rows instead of the weight-streaming kernel

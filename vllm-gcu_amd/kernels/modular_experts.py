@@ -81,9 +81,10 @@ class TritonExpertsPad:
         E, num_tokens, N, K, top_k_num = moe_problem_size(hidden_states, w1, w2, topk_ids, self.use_int4_w4a16)
         if global_num_experts == -1:
             global_num_experts = E
+        unquantised = w1.dtype == hidden_states.dtype and w1.dtype in (torch.float16, torch.bfloat16)
         config = get_default_config(M=num_tokens, E=E, N=N, K=K, topk=top_k_num,
-                                    dtype="int8_w8a8" if self.use_int8_w8a8 else None, is_marlin=False,
-                                    block_shape=self.block_shape)
+                                    dtype="int8_w8a8" if self.use_int8_w8a8 else "w16a16" if unquantised else None,
+                                    is_marlin=False, block_shape=self.block_shape)
         act_dtype = workspace2.dtype
         # cache1 and cache3 share workspace2: cache1 is dead once cache2 exists
         cache1 = workspace2.reshape(-1)[:num_tokens * top_k_num * N].view(num_tokens, top_k_num, N)
