@@ -366,6 +366,9 @@ def main():
         torch.cuda.empty_cache()
         out["moe_w4a8"] = moe_bench(ops, dev, stream, "w4a8")
         torch.cuda.empty_cache()
+        # unquantised experts at prefill token counts (blocks of 256 slots on the MFMA tile kernel, 16-bit operands)
+        out["moe_f16_prefill"] = {str(t): moe_bench(ops, dev, stream, "f16", iters=8, tokens=t) for t in (512, 2048)}
+        torch.cuda.empty_cache()
         out["norm_quant"] = glue_bench(ops, dev, stream)
         torch.cuda.empty_cache()
         out["fp8_dense"] = fp8_dense_bench(ops, dev, stream)
@@ -557,6 +560,22 @@ def moe_bench(ops, dev, stream, which, iters=20, tokens=None, cpu=False, act_dty
             + E * (H // 128 * 2 * I + I // 128 * H) // 2 + 2 * M * H * 2
         name = f"fused MoE W4A16, Mixtral-8x7B layer: {M} tok, hidden 4096, 8 experts, inter 14336, top-2" + \
             (", bf16 activations" if adt == torch.bfloat16 else "")
+    elif which == "f16":
+        # the Mixtral-8x7B layer of configs[3] with unquantised fp16 experts (fused_moe_kernel)
+        M, H, E, I, T = tokens or 512, 4096, 8, 14336, 2
+        w13 = torch.empty(E, 2 * I, H, device=dev, dtype=torch.float16).normal_(0, 0.02)
+        w2 = torch.empty(E, H, I, device=dev, dtype=torch.float16).normal_(0, 0.02)
+        x = torch.randn(M, H, generator=g).half().to(dev)
+        logits = torch.randn(M, E, generator=g).to(dev)
+        moe = FusedMoEModularKernel(MoEPrepareAndFinalizeNoEP(), TritonExpertsPad())
+        kw = {}
+
+        def step():
+            tw, ids = ops.fused_topk(x, logits, T, True)
+            return moe(x, w13, w2, tw, ids, **kw)
+        flops = 2.0 * M * T * (H * 2 * I + I * H)
+        bytes_ = E * (H * 2 * I + I * H) * 2 + 2 * M * H * 2
+        name = f"fused MoE, unquantised fp16 experts, Mixtral-8x7B layer shape: {M} tok, hidden 4096, 8 experts, inter 14336, top-2"
     elif which == "w4a8":
         # the Mixtral-8x7B layer of configs[3] with w4a8-fp8 experts: fp8 activations with one
         # static scale per GEMM, symmetric int4 weights, fp32 group scales

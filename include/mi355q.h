@@ -337,9 +337,10 @@ int mi355q_moe_sum(void* out, const void* in, long rows, int topk, int K, int in
  * block b < num_tokens_post_pad / block_size with e = expert_ids[b] and every
  * id t < numel in the block,  out[t, :] = a[t / topk, :] @ W[e]^T  (times
  * topk_weights[t] when that pointer is given).  max_blocks = entries of
- * expert_ids.  block_size in {16, 32, 64, 128}; fp8 block-scaled and int8 experts also 256.  For those two,
- * blocks of 256 -- and blocks of 128 from 40 rows per expert on average (numel >= 40 E) -- run the MFMA tile
- * kernels with gathered rows (prefill token counts; fp8: N % 128 == 0), smaller ones the weight-streaming kernel.  sorted_token_ids must hold at least
+ * expert_ids.  block_size in {16, 32, 64, 128}; fp8 block-scaled, int8 and unquantised experts also 256.  For
+ * those three, blocks of 256 -- and blocks of 128 from 40 rows per expert on average (numel >= 40 E) -- run the
+ * MFMA tile kernels with gathered rows (prefill token counts; fp8 and unquantised: N % 128 == 0), smaller ones
+ * the weight-streaming kernel.  sorted_token_ids must hold at least
  * max_blocks * block_size entries (the kernels load a block's ids before they compare the block
  * with num_tokens_post_pad).  Rows of ids that appear in no block below num_tokens_post_pad (ids
  * the alignment dropped) are not written, with or without a workspace.
