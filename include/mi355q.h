@@ -164,7 +164,11 @@ int mi355q_fp8_scaled_gemm(void* out, const void* x, const void* w, const float*
  * applies bias (and, for the scaled GEMM, the scales): run-to-run identical, and equal to the unsplit
  * launch up to the order of the fp32 additions.  The workspace follows the rules of
  * mi355q_w4a16_gemm's (its first MiB is left alone); without one, or with a smaller one, the unsplit
- * launch (or, for the scaled GEMM on few tiles, the streaming kernel) runs. */
+ * launch (or, for the scaled GEMM on few tiles, the streaming kernel) runs.
+ * mi355q_fp8_block_gemm_ws also uses ceil16(M) * (K / 128) * 4 bytes behind the partial sums (behind the first
+ * MiB where nothing is split), when the workspace has them, on layers of 128 column tiles or 384 output tiles
+ * and more: the activation scales re-ordered K block major by a small launch of its own, so that a workgroup's
+ * 256 scales of a K block are 1 KiB in a row instead of one value per cache line.  Same output bits. */
 size_t mi355q_fp8_gemm_workspace_bytes(int M, int N, int K);
 int mi355q_fp8_block_gemm_ws(void* out, const void* x, const void* w, const float* x_scale,
                              const float* w_scale, const void* bias, int M, int N, int K, long ldx,

@@ -161,6 +161,35 @@ def test_few_tiles_behind_a_long_k_are_split_into_k_ranges(M, K, N, kslab):
     np.testing.assert_allclose(blk.float().cpu().numpy(), wantb, rtol=RTOL, atol=RTOL * max(1.0, float(np.abs(wantb).max())))
 
 
+@pytest.mark.parametrize("M,K,N", [(300, 256, 16384), (200, 2048, 16384), (1300, 384, 9728), (70, 512, 16512)])
+@pytest.mark.parametrize("kslab", [False, True])
+def test_block_scales_of_the_activations_staged_k_block_major(M, K, N, kslab, monkeypatch):
+    """On a layer of many column tiles the block-scaled tile kernel first re-orders the activation scales K block
+    major in the workspace (a workgroup's 256 scales of a K block side by side): the same numbers from another
+    address, so the output equals the unstaged launch bit for bit -- unsplit, with K ranges side by side (the
+    second shape), with a ragged last row tile -- and meets the oracle."""
+    from vllm_gcu_amd.kernels import _custom_ops as ops
+    from vllm_gcu_amd.kernels.quantization import rearrange
+    print(f"case fp8 block scales staged M={M} K={K} N={N} kslab={kslab}", flush=True)
+    rng = np.random.default_rng(M + K + N + 7)
+    xq, _, w, _ = _operands(rng, M, K, N)
+    xsb = rng.uniform(0.01, 0.05, size=(M, K // 128)).astype(np.float32)
+    wsb = rng.uniform(0.01, 0.05, size=(N // 128, K // 128)).astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal(N).astype(np.float32)).to(torch.bfloat16).cuda()
+    xd = dev(xq).view(torch.float8_e4m3fn)
+    wd = dev(w).view(torch.float8_e4m3fn)
+    wk = rearrange.to_kslab(wd) if kslab else wd
+    staged = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(staged, xd, wk, bias, dev(xsb), dev(wsb))
+    monkeypatch.setattr(ops, "_FP8_STAGE_SCALES", False)
+    plain = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.ops._C.linear_quant(plain, xd, wk, bias, dev(xsb), dev(wsb))
+    torch.cuda.synchronize()
+    assert torch.equal(staged, plain)
+    want = of8.block_fp8_gemm(xq, xsb, w, wsb, bias=bias.float().cpu().numpy())
+    np.testing.assert_allclose(staged.float().cpu().numpy(), want, rtol=RTOL, atol=RTOL * max(1.0, float(np.abs(want).max())))
+
+
 @pytest.mark.parametrize("M", [1, 16, 128, 2048])
 def test_full_size_layer_sampled(M):
     """K = 8192, N = 28672 (one Llama-3-70B MLP projection): sampled rows and columns against the oracle, the whole

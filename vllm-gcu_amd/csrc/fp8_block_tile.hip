@@ -45,6 +45,8 @@ struct F8Args {
   const float* x_scale;     // [M, K / 128]; PC: [M] or one value
   const float* w_scale;     // [N / 128, K / 128]; PC: [N] or one value
   int xs_mul, ws_mul;       // PC: index multipliers of x_scale / w_scale (1 = per token / per channel, 0 = one value)
+  const float* xs_t;        // block scales of the activations, K block major: xs_t[kb * xs_ld + r], r = row m (dense) or
+  long xs_ld;               // position in sorted_ids (grouped); null: x_scale as given (a row's K blocks side by side)
   const void* bias;         // [N] in the output dtype or null
   int M, N, K;
   long ldx, ldw, ldo;
@@ -147,6 +149,8 @@ fp8_block_gemm_kernel(F8Args a) {
   uint32_t xo[XCOPIES], wo[WCOPIES], xso = 0;
   int wsbase = 0;
   const uint8_t *xtile, *wtile;
+  const float* xsbase = a.x_scale;
+  const long xs_kstride = a.xs_t ? a.xs_ld : 1;       // floats between the K blocks of a row's scale
   auto set_copy_tile = [&](int tile) {
     int m0, n0;
     tile_origin(tile, m0, n0);
@@ -193,11 +197,18 @@ fp8_block_gemm_kernel(F8Args a) {
     // activation scales: wavefronts 0..3 copy 64 rows each (index in floats)
     // (split K: the tile's range starts kb0 K blocks into every row; 64 kslab rows interleave their K blocks)
     const int kb0 = ksplits > 1 ? (tile % ksplits) * (KB / ksplits) : 0;
-    if (GROUPED) {
+    if (a.xs_t) {
+      // K block major: the 64 scales of a copy lie side by side (4 cache lines instead of 64)
+      if (GROUPED) xso = (uint32_t)((m0 / FTM) * a.block_rows + ((64 * (wave & 3) + lane) & (a.block_rows - 1)));
+      else xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1);
+      xsbase = a.xs_t + (long)kb0 * a.xs_ld;
+    } else if (GROUPED) {
       const int id = a.sorted_ids[(m0 / FTM) * a.block_rows + ((64 * (wave & 3) + lane) & (a.block_rows - 1))];
       xso = (uint32_t)(max(0, min(id, a.numel - 1)) / a.topk) * (uint32_t)KB;
+      xsbase = a.x_scale;
     } else {
       xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1) * (uint32_t)KB + (uint32_t)kb0;
+      xsbase = a.x_scale;
     }
     wsbase = escales + (n0 >> 7) * KB + kb0;       // wavefront 4 copies the tile's weight scale
     xtile = GROUPED ? a.x : a.x + (long)m0 * a.ldx + (long)kb0 * FTKB;
@@ -216,7 +227,7 @@ fp8_block_gemm_kernel(F8Args a) {
     } else if (PC) {
       // no scales inside the K sum
     } else if (wave < 4) {
-      dma4(a.x_scale + xso + kt, xs + X_BYTES + W_BYTES + wave * 256);
+      dma4(xsbase + xso + (long)kt * xs_kstride, xs + X_BYTES + W_BYTES + wave * 256);
     } else if (wave == 4) {
       dma4(a.w_scale + wsbase + kt, xs + X_BYTES + W_BYTES + XS_BYTES);
     }
@@ -308,6 +319,9 @@ fp8_block_gemm_kernel(F8Args a) {
         if (!PC && n >= 2) {
           const int pn = n - 2;
           acc[pn / NJ][pn % NJ] += sc[pn % NJ] * ring[pn & 3];
+          // (pinned here: left alone, the compiler gives every MFMA a result tile of its own and sinks all
+          // sixty-four multiply-adds behind the last MFMA, where the matrix pipe waits for them)
+          asm volatile("" : "+v"(acc[pn / NJ][pn % NJ]));
         }
         __builtin_amdgcn_sched_barrier(0);
         if (n == 0) read_w(w3nxt, 3, rso);
@@ -533,6 +547,39 @@ fp8_splitk_epilogue_kernel(F8Args a) {
   *(u2*)((uint16_t*)a.out + (long)m * a.ldo + n) = o;
 }
 
+// Activation block scales [rows, KB] -> K block major [KB, ld] for the tile kernel's copies: a workgroup's 256
+// scales of a K block then lie side by side instead of one per cache line (every column tile of a row tile reads
+// them again).  Grouped: entry p is the row that position p of sorted_ids gathers (pads: any valid row).
+__global__ void __launch_bounds__(256)
+fp8_scales_kmajor_kernel(const float* xs, float* out, int rows, int KB, long ld, const int32_t* sorted_ids, int numel, int topk) {
+  __shared__ float t[32][33];
+  const int p0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;       // 32 x 8
+  for (int r = ty; r < 32; r += 8) {
+    const int p = p0 + r, kb = k0 + tx;
+    float v = 0.0f;
+    if (p < rows && kb < KB) {
+      int src = p;
+      if (sorted_ids) src = max(0, min(sorted_ids[p], numel - 1)) / topk;
+      v = xs[(long)src * KB + kb];
+    }
+    t[r][tx] = v;
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) {
+    const int kb = k0 + r, p = p0 + tx;
+    if (p < rows && kb < KB) out[(long)kb * ld + p] = t[tx][r];
+  }
+}
+
+int fp8_scales_kmajor_launch(const float* xs, float* out, int rows, int KB, long ld, const int32_t* sorted_ids, int numel,
+                             int topk, hipStream_t st) {
+  hipLaunchKernelGGL(fp8_scales_kmajor_kernel, dim3((unsigned)((rows + 31) / 32), (unsigned)((KB + 31) / 32)), dim3(256), 0, st,
+                     xs, out, rows, KB, ld, sorted_ids, numel, topk);
+  MQ_LAUNCH_CHECK("fp8 gemm (scales, K block major)");
+  return 0;
+}
+
 constexpr size_t F8_SPLITK_BYTES = (size_t)64 << 20;
 constexpr size_t F8_WS_OFFSET = (size_t)1 << 20;     // the first MiB of a workspace belongs to the W4A16 arrival counters
 
@@ -580,13 +627,33 @@ int fp8_split_min_rows(int N, int K, int splits) {
 }
 
 // with a workspace that holds the plan's partial sums: K ranges side by side; else the plain launch
+// bytes of the K block major copy of the activation scales (rows padded to whole 64-byte lines)
+size_t fp8_scales_kmajor_bytes(long rows, int K) { return (size_t)((rows + 15) / 16 * 16) * (K / FTKB) * sizeof(float); }
+
 template <int DT, bool PC>
 int launch_f8_auto(F8Args& a, void* workspace, size_t workspace_bytes, hipStream_t st) {
   a.ksplits = 1;
   a.partial = nullptr;
+  a.xs_t = nullptr;
+  a.xs_ld = 0;
   const int splits = fp8_ksplits(a.M, a.N, a.K);
-  if (splits > 1 && workspace && workspace_bytes >= F8_WS_OFFSET + (size_t)splits * a.M * a.N * sizeof(float))
-    return launch_f8_splitk<DT, PC>(a, splits, workspace, st);
+  const bool split = splits > 1 && workspace && workspace_bytes >= F8_WS_OFFSET + (size_t)splits * a.M * a.N * sizeof(float);
+  // (it pays where many column tiles read a row tile's scales again: measured, us, K 8192 x N 28672 at M = 128 / 256 /
+  // 2048: 75 / 97 / 549 -> 67 / 86 / 529; K 16384 x N 7168 at 2048 / 8192: 289 / 1063 -> 277 / 997; layers of fewer
+  // tiles gain nothing and pay for the extra launch)
+  const long ntiles = a.N / FTN, tiles = (long)((a.M + FTM - 1) / FTM) * ntiles;
+  if (!PC && workspace && (ntiles >= 128 || tiles >= 384)) {
+    // block scales: with room behind the partial sums, the activation scales are re-ordered K block major first
+    const size_t off = F8_WS_OFFSET + (split ? (size_t)splits * a.M * a.N * sizeof(float) : 0);
+    if (workspace_bytes >= off + fp8_scales_kmajor_bytes(a.M, a.K)) {
+      float* xt = (float*)((char*)workspace + off);
+      const long ld = (a.M + 15) / 16 * 16;
+      if (int rc = fp8_scales_kmajor_launch(a.x_scale, xt, a.M, a.K / FTKB, ld, nullptr, 0, 1, st)) return rc;
+      a.xs_t = xt;
+      a.xs_ld = ld;
+    }
+  }
+  if (split) return launch_f8_splitk<DT, PC>(a, splits, workspace, st);
   return launch_f8<DT, PC>(a, st);
 }
 

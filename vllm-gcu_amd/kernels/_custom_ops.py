@@ -1251,6 +1251,7 @@ def _kcontig(out, a, w, a_scale, w_scale, bias, mode, group):
 # 48..64 tiles (K 7168 N 4096: 32 tiles 56 against 31 us, 64 tiles 55 against 58 us, 96 tiles 56
 # against 85 us; the same on K 4096 N 4096, K 2048 N 7168 and K 7168 N 2048)
 _FP8_TILE_MIN_M = 64
+_FP8_STAGE_SCALES = True      # room in the workspace for the activation scales in K block major order (tile kernel)
 _FP8_TILE_MIN_TILES = 64
 
 
@@ -1285,7 +1286,10 @@ def _linear_quant_impl(out, lhs, rhs, bias, lhs_scale, rhs_scale):
                                f"M={M} N={N} K={K} with 128 x 128 blocks")
         b = None if bias is None else bias.to(out.dtype).contiguous()
         with torch.cuda.device(lhs.device):
-            wsp = rt.workspace(lhs.device, need) if need else None
+            # behind the partial sums of a K split (or the first MiB): room for the activation scales in K block major order
+            stage = (M + 15) // 16 * 16 * (K // 128) * 4 if _FP8_STAGE_SCALES else 0
+            total = (need or ((1 << 20) if stage else 0)) + stage
+            wsp = rt.workspace(lhs.device, total) if total else None
             _lib.call("mi355q_fp8_block_gemm_ws", out.data_ptr(), a2.data_ptr(), rhs.data_ptr(), xs.data_ptr(),
                       ws.data_ptr(), rt.ptr(b), M, N, K, K, 0 if rearrange.is_kslab(rhs) else K, N,
                       rt.dtype_code(out.dtype), rt.ptr(wsp), 0 if wsp is None else wsp.numel(), rt.stream_ptr())
