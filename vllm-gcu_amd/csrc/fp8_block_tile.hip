@@ -45,8 +45,8 @@ struct F8Args {
   const float* x_scale;     // [M, K / 128]; PC: [M] or one value
   const float* w_scale;     // [N / 128, K / 128]; PC: [N] or one value
   int xs_mul, ws_mul;       // PC: index multipliers of x_scale / w_scale (1 = per token / per channel, 0 = one value)
-  const float* xs_t;        // block scales of the activations, K block major: xs_t[kb * xs_ld + r], r = row m (dense) or
-  long xs_ld;               // position in sorted_ids (grouped); null: x_scale as given (a row's K blocks side by side)
+  const float* xs_t;        // dense launches: block scales of the activations, K block major, xs_t[kb * xs_ld + m];
+  long xs_ld;               // null: x_scale as given (a row's K blocks side by side)
   const void* bias;         // [N] in the output dtype or null
   int M, N, K;
   long ldx, ldw, ldo;
@@ -150,7 +150,7 @@ fp8_block_gemm_kernel(F8Args a) {
   int wsbase = 0;
   const uint8_t *xtile, *wtile;
   const float* xsbase = a.x_scale;
-  const long xs_kstride = a.xs_t ? a.xs_ld : 1;       // floats between the K blocks of a row's scale
+  const long xs_kstride = (!GROUPED && a.xs_t) ? a.xs_ld : 1;       // floats between the K blocks of a row's scale
   auto set_copy_tile = [&](int tile) {
     int m0, n0;
     tile_origin(tile, m0, n0);
@@ -197,10 +197,9 @@ fp8_block_gemm_kernel(F8Args a) {
     // activation scales: wavefronts 0..3 copy 64 rows each (index in floats)
     // (split K: the tile's range starts kb0 K blocks into every row; 64 kslab rows interleave their K blocks)
     const int kb0 = ksplits > 1 ? (tile % ksplits) * (KB / ksplits) : 0;
-    if (a.xs_t) {
+    if (!GROUPED && a.xs_t) {
       // K block major: the 64 scales of a copy lie side by side (4 cache lines instead of 64)
-      if (GROUPED) xso = (uint32_t)((m0 / FTM) * a.block_rows + ((64 * (wave & 3) + lane) & (a.block_rows - 1)));
-      else xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1);
+      xso = (uint32_t)min(m0 + 64 * (wave & 3) + lane, M - 1);
       xsbase = a.xs_t + (long)kb0 * a.xs_ld;
     } else if (GROUPED) {
       const int id = a.sorted_ids[(m0 / FTM) * a.block_rows + ((64 * (wave & 3) + lane) & (a.block_rows - 1))];
@@ -549,20 +548,16 @@ fp8_splitk_epilogue_kernel(F8Args a) {
 
 // Activation block scales [rows, KB] -> K block major [KB, ld] for the tile kernel's copies: a workgroup's 256
 // scales of a K block then lie side by side instead of one per cache line (every column tile of a row tile reads
-// them again).  Grouped: entry p is the row that position p of sorted_ids gathers (pads: any valid row).
+// them again).
 __global__ void __launch_bounds__(256)
-fp8_scales_kmajor_kernel(const float* xs, float* out, int rows, int KB, long ld, const int32_t* sorted_ids, int numel, int topk) {
+fp8_scales_kmajor_kernel(const float* xs, float* out, int rows, int KB, long ld) {
   __shared__ float t[32][33];
   const int p0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;       // 32 x 8
   for (int r = ty; r < 32; r += 8) {
     const int p = p0 + r, kb = k0 + tx;
     float v = 0.0f;
-    if (p < rows && kb < KB) {
-      int src = p;
-      if (sorted_ids) src = max(0, min(sorted_ids[p], numel - 1)) / topk;
-      v = xs[(long)src * KB + kb];
-    }
+    if (p < rows && kb < KB) v = xs[(long)p * KB + kb];
     t[r][tx] = v;
   }
   __syncthreads();
@@ -572,10 +567,9 @@ fp8_scales_kmajor_kernel(const float* xs, float* out, int rows, int KB, long ld,
   }
 }
 
-int fp8_scales_kmajor_launch(const float* xs, float* out, int rows, int KB, long ld, const int32_t* sorted_ids, int numel,
-                             int topk, hipStream_t st) {
+int fp8_scales_kmajor_launch(const float* xs, float* out, int rows, int KB, long ld, hipStream_t st) {
   hipLaunchKernelGGL(fp8_scales_kmajor_kernel, dim3((unsigned)((rows + 31) / 32), (unsigned)((KB + 31) / 32)), dim3(256), 0, st,
-                     xs, out, rows, KB, ld, sorted_ids, numel, topk);
+                     xs, out, rows, KB, ld);
   MQ_LAUNCH_CHECK("fp8 gemm (scales, K block major)");
   return 0;
 }
@@ -648,7 +642,7 @@ int launch_f8_auto(F8Args& a, void* workspace, size_t workspace_bytes, hipStream
     if (workspace_bytes >= off + fp8_scales_kmajor_bytes(a.M, a.K)) {
       float* xt = (float*)((char*)workspace + off);
       const long ld = (a.M + 15) / 16 * 16;
-      if (int rc = fp8_scales_kmajor_launch(a.x_scale, xt, a.M, a.K / FTKB, ld, nullptr, 0, 1, st)) return rc;
+      if (int rc = fp8_scales_kmajor_launch(a.x_scale, xt, a.M, a.K / FTKB, ld, st)) return rc;
       a.xs_t = xt;
       a.xs_ld = ld;
     }
