@@ -34,8 +34,9 @@ def get_default_config(M: int, E: int, N: int, K: int, topk: int, dtype: Optiona
     per_expert = (M * topk) / max(E, 1)
     tiles = (block_shape is not None and list(block_shape) == [128, 128]) or dtype in ("int8_w8a8", "w16a16")
     if tiles and per_expert > _FP8_TILE_MIN_ROWS_PER_EXPERT:
-        # fp8 block-scaled and int8 experts at prefill token counts: blocks of 128 or 256 slots run the MFMA
-        # tile kernels with gathered rows instead of the weight-streaming kernel
+        # fp8 block-scaled, int8 and unquantised 16-bit experts ("w16a16": this build's name for them, the
+        # reference passes None) at prefill token counts: blocks of 128 or 256 slots run the MFMA tile
+        # kernels with gathered rows instead of the weight-streaming kernel
         return {"BLOCK_SIZE_M": 256 if per_expert > _TILE_256_ROWS_PER_EXPERT else 128, "BLOCK_SIZE_N": 64,
                 "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
     if per_expert <= 16:
